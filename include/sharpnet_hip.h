@@ -1,0 +1,137 @@
+/*
+ * libsharpnet_hip - C ABI of the MI355X (gfx950) matrix-multiplication path
+ * that stands in for the cuBLAS / nvcuda entry points SharpNet's GPUTensor<float>
+ * binds through P/Invoke for Tensor.Dot and Tensor.BatchMatrixMultiplication.
+ *
+ * Conventions (chosen so the C# side needs no change beyond the DllImport name):
+ *   - every function returns an int that uses the cublasStatus_t numbering of
+ *     /root/reference/Prod/GPU/CublasWrapper.cs:8-20, so GPUWrapper.CheckStatus
+ *     (Prod/GPU/GPUWrapper.cs:662-668) keeps working;
+ *   - transpose flags use cublasOperation_t numbering, N=0 T=1 C=2
+ *     (CublasWrapper.cs:22-27); C is treated as T (real data);
+ *   - all matrix pointers are raw device addresses (hipMalloc, or any offset
+ *     into such an allocation: only 4-byte alignment is required);
+ *   - alpha / beta are read from HOST memory at call time;
+ *   - calls are asynchronous on the handle's stream (the null stream unless
+ *     snhip_set_stream was called) and are ordered with earlier work on it;
+ *   - a handle belongs to the device that was current when it was created and
+ *     must be used by one host thread at a time (GPUWrapper.cs:824-832);
+ *   - when beta == 0 the destination is never read.
+ */
+#ifndef SHARPNET_HIP_H
+#define SHARPNET_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SNHIP_STATUS_SUCCESS 0
+#define SNHIP_STATUS_NOT_INITIALIZED 1
+#define SNHIP_STATUS_ALLOC_FAILED 3
+#define SNHIP_STATUS_INVALID_VALUE 7
+#define SNHIP_STATUS_ARCH_MISMATCH 8
+#define SNHIP_STATUS_MAPPING_ERROR 11
+#define SNHIP_STATUS_EXECUTION_FAILED 13
+#define SNHIP_STATUS_INTERNAL_ERROR 14
+#define SNHIP_STATUS_NOT_SUPPORTED 15
+
+#define SNHIP_OP_N 0
+#define SNHIP_OP_T 1
+#define SNHIP_OP_C 2
+
+/* ---- handle lifetime --------------------------------------------------- */
+
+/* Replaces cublasCreate_v2 (CublasWrapper.cs:223, called at GPUWrapper.cs:100). */
+int snhip_create(void** handle);
+/* Replaces cublasDestroy_v2 (CublasWrapper.cs:225). Frees the split-K workspace. */
+int snhip_destroy(void* handle);
+/* No counterpart is bound by the reference (it never calls cublasSetStream, so
+ * GEMMs run on the legacy default stream); offered for callers with their own
+ * hipStream_t.  stream == NULL selects the null stream again. */
+int snhip_set_stream(void* handle, void* stream);
+/* Replaces cublasGetVersion_v2 (CublasWrapper.cs:250): major*10000+minor*100+patch. */
+int snhip_get_version(void* handle, int* version);
+
+/* ---- cuBLAS-shaped GEMM (column-major semantics) ------------------------- */
+
+/* Replaces cublasSgemm_v2 (CublasWrapper.cs:229), call site GpuTensor.cs:1218.
+ * Column-major: C(m x n, ldc) = alpha * op(A) * op(B) + beta * C. */
+int snhip_sgemm(void* handle, int transa, int transb, int m, int n, int k, const float* alpha, const void* A, int lda,
+                const void* B, int ldb, const float* beta, void* C, int ldc);
+
+/* Replaces cublasSgemmStridedBatched (CublasWrapper.cs:231-244), call site
+ * GpuTensor.cs:1192.  Strides are element counts (C# long). */
+int snhip_sgemm_strided_batched(void* handle, int transa, int transb, int m, int n, int k, const float* alpha,
+                                const void* A, int lda, long long strideA, const void* B, int ldb, long long strideB,
+                                const float* beta, void* C, int ldc, long long strideC, int batchCount);
+
+/* ---- row-major entry points (parameter list of BlasServices.DotMkl) ------ */
+
+/* Same parameters as BlasServices.DotMkl (Prod/Data/BlasServices.cs:10):
+ * A is aH x aW, B is bH x bW, both row-major and dense; M,N,K and the leading
+ * dimensions are derived exactly as lines 14-19 do; C is M x N with ldc = N.
+ * transposeA / transposeB are 0 or 1. */
+int snhip_dot(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
+              int transposeB, float* C, float alpha, float beta);
+
+/* snhip_dot followed by C[m][n] += bias[n], in one kernel.  Replaces the pair
+ * Dot + BroadcastAddVectorToOutput of Linear.DenseForwardPropagation
+ * (Prod/Layers/Linear.cs:130-131; GPU bias add at GpuTensor.cs:633-644).
+ * bias may be NULL. */
+int snhip_dot_bias(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
+                   int transposeB, float* C, float alpha, float beta, const float* bias);
+
+/* Row-major strided batch: for i in [0,batch): C_i = alpha op(A_i) op(B_i) + beta C_i
+ * with X_i = X + i*strideX.  Parameters as CpuTensor.BatchMatrixMultiplication
+ * derives them (Prod/CPU/CpuTensor.cs:3004-3025): aH=Shape[1], aW=MultDim1,
+ * stride=MultDim0. */
+int snhip_bmm(void* handle, const float* A, int aH, int aW, int transposeA, long long strideA, const float* B, int bH,
+              int bW, int transposeB, long long strideB, float* C, long long strideC, int batch, float alpha,
+              float beta);
+
+/* General row-major form with explicit leading dimensions (views / slices,
+ * e.g. attention heads addressed in place).  op(A) is M x K, op(B) is K x N. */
+int snhip_gemm_rm(void* handle, int transposeA, int transposeB, int M, int N, int K, float alpha, const float* A,
+                  int lda, long long strideA, const float* B, int ldb, long long strideB, float beta, float* C,
+                  int ldc, long long strideC, int batch, const float* bias);
+
+/* ---- device memory / stream shims --------------------------------------- */
+/* Replace the nvcuda calls GPUTensor makes: cuMemAlloc_v2 (GpuTensor.cs:41),
+ * cuMemFree_v2 (:1634), cuMemsetD32 (:1583), cuMemcpyHtoDAsync (:77),
+ * cuMemcpyDtoH (:1668), cuMemcpyDtoDAsync (:1499), cuStreamSynchronize
+ * (Prod/GPU/StreamWrapper.cs:20). */
+int snhip_malloc(void** dptr, size_t bytes);
+int snhip_free(void* dptr);
+int snhip_memset32(void* handle, void* dptr, unsigned int value, size_t count);
+int snhip_memcpy_htod_async(void* handle, void* dst, const void* src, size_t bytes);
+int snhip_memcpy_dtoh(void* handle, void* dst, const void* src, size_t bytes);
+int snhip_memcpy_dtod_async(void* handle, void* dst, const void* src, size_t bytes);
+int snhip_stream_synchronize(void* handle);
+
+/* ---- measurement helpers (no reference counterpart) ---------------------- */
+/* hipEvent wrappers recording on the handle's stream, for timing launches. */
+int snhip_event_create(void** event);
+int snhip_event_destroy(void* event);
+int snhip_event_record(void* handle, void* event);
+int snhip_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for stop */
+
+/* Device facts: info[0]=compute units, [1]=max engine clock kHz, [2]=memory
+ * clock kHz, [3]=memory bus width bits, [4]=LDS bytes per workgroup (opt-in max),
+ * [5]=gfx architecture number (950 for MI355X). */
+int snhip_device_info(void* handle, int info[6]);
+
+/* Tuning hooks: force the tile configuration / split-K factor used by the next
+ * calls on this handle (-1 / 0 = automatic), and read back what the last GEMM
+ * call selected.  config ids index the table in sharpnet_hip.hip. */
+int snhip_set_tuning(void* handle, int config, int splitk);
+int snhip_get_last_tuning(void* handle, int* config, int* splitk);
+int snhip_config_count(void);
+/* desc[0..4] = BM, BN, BK, threads, LDS bytes */
+int snhip_config_desc(int config, int desc[5]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SHARPNET_HIP_H */

@@ -1,0 +1,284 @@
+"""TEST INFRASTRUCTURE - not part of the product.
+
+Only tests/, ``__graft_entry__.smoke()`` and bench.py's ``cpu_baseline`` leg may
+import this module.  Nothing under sharpnet_amd/ does.
+
+CPU restatement of the reference path behind ``Tensor.Dot`` /
+``Tensor.BatchMatrixMultiplication`` and of the layer code that calls it.
+The GEMM arithmetic of the reference lives in a third-party binary that is not
+part of the reference tree: Intel MKL ``cblas_sgemm`` bound as ``mkl_rt.dll``
+with no pinned version (Prod/Data/BlasServices.cs:44-45; README.md:22).  The
+functions below restate the reference's own code around that call:
+
+======================================  ==========================================  =======
+function                                follows                                      pinned by
+======================================  ==========================================  =======
+dot_shapes / dot / dot_f64              Prod/Data/BlasServices.cs:10-21,             TestGpuTensor.cs:53-109 known answers, QR
+                                        Prod/CPU/CpuTensor.cs:2991-3002              identity (TestCpuTensor.cs:826-863), brute force
+bmm                                     Prod/CPU/CpuTensor.cs:3004-3025              looped 2-D oracle == its definition; attention
+                                                                                     fixture ParallelRunWithPyTorch.cs:963-1010
+sgemm_colmajor                          cuBLAS SGEMM as called at                    transposition identity against dot_f64
+                                        Prod/GPU/GpuTensor.cs:1192,1218
+dense_forward / dense_backward          Prod/Layers/Linear.cs:125-191                loss fixture ParallelRunWithPyTorch.cs:102-138,
+                                                                                     TestNetworkPropagation.cs:36-105
+softmax_last_dim                        Prod/CPU/CpuTensorActivationFunctions.cs     attention loss fixture (same file :963-1010)
+                                        :19-46
+sdpa_forward                            Prod/Layers/ScaledDotProductAttention        same
+                                        Layer.cs:46-91
+mkl_dot (baseline only)                 the same cblas_sgemm call the reference      compared with dot_f64 within the fp32 bound
+                                        makes, through this image's own MKL
+======================================  ==========================================  =======
+
+Every function is pinned (tests/test_oracle.py); none is "parity unpinned".
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+_f32p = ctypes.POINTER(ctypes.c_float)
+
+
+def build(force=False):
+    """Compile dot_oracle.c with gcc (see Makefile)."""
+    so = os.path.join(_HERE, "liboracle.so")
+    src = os.path.join(_HERE, "dot_oracle.c")
+    if force or not os.path.exists(so) or os.path.getmtime(so) < os.path.getmtime(src):
+        if force and os.path.exists(so):
+            os.remove(so)
+        subprocess.run(["make", "-C", _HERE, "liboracle.so"], check=True, stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT)
+    return so
+
+
+def _lib():
+    global _LIB
+    if _LIB is None:
+        so = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(so):
+            build()
+        lib = ctypes.CDLL(so)
+        i, f = ctypes.c_int, ctypes.c_float
+        lib.oracle_dot.argtypes = [_f32p, i, i, i, _f32p, i, i, i, _f32p, f, f]
+        lib.oracle_dot.restype = None
+        lib.oracle_bmm.argtypes = [_f32p, i, i, i, _f32p, i, i, i, _f32p, i, f, f]
+        lib.oracle_bmm.restype = None
+        lib.oracle_sgemm_colmajor.argtypes = [i, i, i, i, i, f, _f32p, i, _f32p, i, f, _f32p, i]
+        lib.oracle_sgemm_colmajor.restype = None
+        _LIB = lib
+    return _LIB
+
+
+def _p(a):
+    return a.ctypes.data_as(_f32p)
+
+
+def _as2d(x):
+    """Operands with >= 2 dims are read as (Shape[0], MultDim0) (CpuTensor.cs:2998, Tensor.cs:1521-1526)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.ndim >= 2
+    return x.reshape(x.shape[0], -1)
+
+
+def dot_shapes(aH, aW, transposeA, bH, bW, transposeB):
+    """M, N, K, lda, ldb, ldc as BlasServices.DotMkl derives them (BlasServices.cs:14-19)."""
+    M = aW if transposeA else aH
+    N = bH if transposeB else bW
+    K = aH if transposeA else aW
+    return M, N, K, aW, bW, N
+
+
+def dot(a, transposeA, b, transposeB, alpha=1.0, beta=0.0, c=None):
+    """C restatement (double accumulator, one rounding).  Returns a new (M, N) float32 array."""
+    a2, b2 = _as2d(a), _as2d(b)
+    M, N, K, _, _, _ = dot_shapes(a2.shape[0], a2.shape[1], transposeA, b2.shape[0], b2.shape[1], transposeB)
+    Kb = b2.shape[1] if transposeB else b2.shape[0]
+    assert K == Kb, "inner dimensions differ: %d vs %d" % (K, Kb)
+    if c is None:
+        assert beta == 0.0
+        out = np.empty((M, N), dtype=np.float32)
+    else:
+        out = np.array(c, dtype=np.float32, copy=True).reshape(M, N)
+    _lib().oracle_dot(_p(a2), a2.shape[0], a2.shape[1], int(transposeA), _p(b2), b2.shape[0], b2.shape[1],
+                      int(transposeB), _p(out), float(alpha), float(beta))
+    return out
+
+
+def dot_f64(a, transposeA, b, transposeB, alpha=1.0, beta=0.0, c=None):
+    """The same contract in numpy float64 (not rounded): the closed form the C code is checked against."""
+    a2 = _as2d(a).astype(np.float64)
+    b2 = _as2d(b).astype(np.float64)
+    opa = a2.T if transposeA else a2
+    opb = b2.T if transposeB else b2
+    r = float(np.float32(alpha)) * (opa @ opb)
+    if beta != 0.0:
+        r = r + float(np.float32(beta)) * np.asarray(c, dtype=np.float64).reshape(r.shape)
+    return r
+
+
+def bmm(a3, transposeA, b3, transposeB, alpha=1.0, beta=0.0, c3=None):
+    """CpuTensor.BatchMatrixMultiplication (CpuTensor.cs:3004-3025): serial loop of Dot over Shape[0]."""
+    a3 = np.ascontiguousarray(a3, dtype=np.float32)
+    b3 = np.ascontiguousarray(b3, dtype=np.float32)
+    assert a3.ndim == 3 and b3.ndim == 3 and a3.shape[0] == b3.shape[0]
+    batch, aH, aW = a3.shape
+    _, bH, bW = b3.shape
+    M, N, _, _, _, _ = dot_shapes(aH, aW, transposeA, bH, bW, transposeB)
+    if c3 is None:
+        assert beta == 0.0
+        out = np.empty((batch, M, N), dtype=np.float32)
+    else:
+        out = np.array(c3, dtype=np.float32, copy=True).reshape(batch, M, N)
+    _lib().oracle_bmm(_p(a3), aH, aW, int(transposeA), _p(b3), bH, bW, int(transposeB), _p(out), batch,
+                      float(alpha), float(beta))
+    return out
+
+
+def sgemm_colmajor(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc):
+    """Column-major SGEMM on flat float32 buffers; returns the updated copy of C."""
+    A = np.ascontiguousarray(A, dtype=np.float32).reshape(-1)
+    B = np.ascontiguousarray(B, dtype=np.float32).reshape(-1)
+    out = np.array(C, dtype=np.float32, copy=True).reshape(-1)
+    _lib().oracle_sgemm_colmajor(int(transa), int(transb), m, n, k, float(alpha), _p(A), lda, _p(B), ldb, float(beta),
+                                 _p(out), ldc)
+    return out
+
+
+def tolerance(K, a, b):
+    """fp32 parity bound: 1e-4 * sqrt(K) * max|a| * max|b| (at least one ulp-scale floor for empty K)."""
+    amax = float(np.max(np.abs(a))) if np.size(a) else 0.0
+    bmax = float(np.max(np.abs(b))) if np.size(b) else 0.0
+    return 1e-4 * np.sqrt(max(K, 1)) * amax * bmax
+
+
+# ---------------------------------------------------------------------------
+# Layer-level restatements (callers of Dot)
+# ---------------------------------------------------------------------------
+
+def dense_forward(x, weights, bias=None, flatten_last=False):
+    """Linear.DenseForwardPropagation (Linear.cs:125-132): y2D = x2D . W^T, then y2D[n,:] += bias."""
+    x = np.asarray(x, dtype=np.float32)
+    x2 = x.reshape(-1, x.shape[-1]) if flatten_last else x.reshape(x.shape[0], -1)
+    y = dot(x2, False, weights, True, 1.0, 0.0)
+    if bias is not None:
+        y = (y + np.asarray(bias, dtype=np.float32).reshape(1, -1)).astype(np.float32)  # CpuTensor.cs:1468-1487
+    return y
+
+
+def dense_backward(x, dy, weights, multiplier=1.0, prev_is_input=False, flatten_last=False):
+    """Linear.DenseBackwardPropagation (Linear.cs:142-191) without weight decay.
+
+    Returns (dW, db, dx): dW = multiplier * dy^T . x (:158), db = column sums of dy (:164),
+    dx = dy . W (:190) or None when the previous layer is the input layer (:184-187).
+    """
+    x = np.asarray(x, dtype=np.float32)
+    dy = np.asarray(dy, dtype=np.float32)
+    x2 = x.reshape(-1, x.shape[-1]) if flatten_last else x.reshape(x.shape[0], -1)
+    dy2 = dy.reshape(-1, dy.shape[-1]) if flatten_last else dy.reshape(dy.shape[0], -1)
+    dW = dot(dy2, True, x2, False, multiplier, 0.0)
+    db = dy2.astype(np.float64).sum(axis=0).astype(np.float32)
+    dx = None if prev_is_input else dot(dy2, False, weights, False, 1.0, 0.0)
+    return dW, db, dx
+
+
+def softmax_last_dim(x):
+    """Max-subtracted softmax over the last dimension in float32 (CpuTensorActivationFunctions.cs:19-46)."""
+    x = np.asarray(x, dtype=np.float32)
+    m = x.max(axis=-1, keepdims=True)
+    e = np.exp((x - m).astype(np.float32)).astype(np.float32)
+    return (e / e.sum(axis=-1, keepdims=True, dtype=np.float32)).astype(np.float32)
+
+
+def sdpa_forward(Q, K, V, use_scale=True, is_causal=False):
+    """ScaledDotProductAttentionForwardPropagation (ScaledDotProductAttentionLayer.cs:46-91).
+
+    Q, K, V: (batch, T, d).  scores = scaling * Q.K^T (:71), entries above the main diagonal set to
+    -1e12 when causal (:73-76), weights = softmax over the last dim (:81), y = weights . V (:85).
+    Returns (y, weights).
+    """
+    d = Q.shape[-1]
+    scaling = 1.0 / np.sqrt(np.float32(d)) if use_scale else 1.0
+    scores = bmm(Q, False, K, True, float(scaling), 0.0)
+    if is_causal:
+        T1, T2 = scores.shape[1], scores.shape[2]
+        mask = np.triu(np.ones((T1, T2), dtype=bool), k=1)
+        scores[:, mask] = np.float32(-1e12)
+    weights = softmax_last_dim(scores)
+    y = bmm(weights, False, V, False, 1.0, 0.0)
+    return y, weights
+
+
+# ---------------------------------------------------------------------------
+# CPU baseline: the reference's own CPU route, MKL cblas_sgemm RowMajor
+# ---------------------------------------------------------------------------
+_MKL = None
+
+
+def _find_mkl():
+    global _MKL
+    if _MKL is not None:
+        return _MKL or None
+    _MKL = False
+    cands = [os.environ.get("MKL_RT_PATH"), "/opt/conda/lib/libmkl_rt.so", "/opt/conda/lib/libmkl_rt.so.2",
+             "/opt/conda/lib/libmkl_rt.so.1", "/usr/lib/x86_64-linux-gnu/libmkl_rt.so", "libmkl_rt.so"]
+    for c in cands:
+        if not c:
+            continue
+        try:
+            lib = ctypes.CDLL(c)
+            fn = lib.cblas_sgemm
+            i, f = ctypes.c_int, ctypes.c_float
+            fn.argtypes = [i, i, i, i, i, i, f, _f32p, i, _f32p, i, f, _f32p, i]
+            fn.restype = None
+            _MKL = lib
+            break
+        except (OSError, AttributeError):
+            continue
+    return _MKL or None
+
+
+def mkl_available():
+    return _find_mkl() is not None
+
+
+def mkl_dot(a2, transposeA, b2, transposeB, out, alpha=1.0, beta=0.0):
+    """The call BlasServices.DotMkl makes (BlasServices.cs:20): cblas_sgemm(RowMajor=101, 111|112, ...).
+
+    Uses libmkl_rt from this image when it is installed, else torch's CPU matmul (MKL-backed build).
+    a2, b2, out must be C-contiguous float32 2-D arrays; out is updated in place.
+    """
+    aH, aW = a2.shape
+    bH, bW = b2.shape
+    M, N, K, lda, ldb, ldc = dot_shapes(aH, aW, transposeA, bH, bW, transposeB)
+    lib = _find_mkl()
+    if lib is not None:
+        lib.cblas_sgemm(101, 112 if transposeA else 111, 112 if transposeB else 111, M, N, K, float(alpha), _p(a2),
+                        lda, _p(b2), ldb, float(beta), _p(out), ldc)
+        return "libmkl_rt cblas_sgemm"
+    import torch
+    ta, tb, to = torch.from_numpy(a2), torch.from_numpy(b2), torch.from_numpy(out)
+    opa = ta.t() if transposeA else ta
+    opb = tb.t() if transposeB else tb
+    with torch.backends.mkldnn.flags(enabled=False):
+        if beta == 0.0:
+            torch.mm(opa, opb, out=to)
+            if alpha != 1.0:
+                to.mul_(alpha)
+        else:
+            torch.addmm(to, opa, opb, beta=beta, alpha=alpha, out=to)
+    return "torch.mm (MKL build)"
+
+
+def mkl_threads():
+    lib = _find_mkl()
+    if lib is not None:
+        try:
+            lib.mkl_get_max_threads.restype = ctypes.c_int
+            return int(lib.mkl_get_max_threads())
+        except AttributeError:
+            pass
+    import torch
+    return torch.get_num_threads()

@@ -1,0 +1,500 @@
+// C ABI of libsharpnet_hip: argument checking, tile-configuration choice and
+// kernel launch for the fp32 GEMM path.  Declarations and the reference entry
+// point each function replaces are in include/sharpnet_hip.h.
+#include "../../include/sharpnet_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#include <new>
+
+#include "sgemm_mfma.hpp"
+
+using namespace snhip;
+
+namespace {
+
+constexpr int kVersion = 100;  // 0.1.0
+
+struct Handle {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    float* ws = nullptr;
+    size_t ws_bytes = 0;
+    int num_cu = 256;
+    int force_cfg = -1;
+    int force_splitk = 0;
+    int last_cfg = -1;
+    int last_splitk = 0;
+};
+
+// Upper bound for the split-K workspace; larger requests fall back to fewer splits.
+constexpr size_t kMaxWorkspaceBytes = size_t(1) << 30;
+
+typedef void (*KernelFn)(const GemmParams);
+
+struct ConfigEntry {
+    int BM, BN, BK, NT, lds_bytes;
+    int mfma_per_k2;  // MFMA instructions one wavefront issues per 2 k
+    KernelFn fn[2][2];  // [transposeA][transposeB]
+};
+
+template <class CFG>
+constexpr ConfigEntry make_entry() {
+    return ConfigEntry{CFG::BM,
+                       CFG::BN,
+                       CFG::BK,
+                       CFG::NT,
+                       CFG::LDS_BYTES,
+                       CFG::TM * CFG::TN,
+                       {{sgemm_mfma_kernel<CFG, false, false>, sgemm_mfma_kernel<CFG, false, true>},
+                        {sgemm_mfma_kernel<CFG, true, false>, sgemm_mfma_kernel<CFG, true, true>}}};
+}
+
+// Tile configurations, largest first.  <TM,TN,WM,WN,BK>: a wavefront owns
+// TM x TN MFMA tiles of 32x32, a workgroup is WM x WN wavefronts.
+const ConfigEntry kConfigs[] = {
+    make_entry<TileCfg<4, 4, 2, 2, 16>>(),  // 0: 256 x 256
+    make_entry<TileCfg<2, 4, 2, 2, 16>>(),  // 1: 128 x 256
+    make_entry<TileCfg<4, 2, 2, 2, 16>>(),  // 2: 256 x 128
+    make_entry<TileCfg<2, 2, 2, 2, 16>>(),  // 3: 128 x 128
+    make_entry<TileCfg<1, 2, 2, 2, 16>>(),  // 4: 64 x 128
+    make_entry<TileCfg<2, 1, 2, 2, 16>>(),  // 5: 128 x 64
+    make_entry<TileCfg<1, 1, 2, 2, 16>>(),  // 6: 64 x 64
+};
+constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
+
+int hip_to_status(hipError_t e) {
+    switch (e) {
+        case hipSuccess:
+            return SNHIP_STATUS_SUCCESS;
+        case hipErrorOutOfMemory:
+            return SNHIP_STATUS_ALLOC_FAILED;
+        case hipErrorInvalidValue:
+        case hipErrorInvalidDevicePointer:
+            return SNHIP_STATUS_INVALID_VALUE;
+        case hipErrorNotInitialized:
+        case hipErrorNoDevice:
+            return SNHIP_STATUS_NOT_INITIALIZED;
+        default:
+            return SNHIP_STATUS_EXECUTION_FAILED;
+    }
+}
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+struct Choice {
+    int cfg;
+    int splitk;
+};
+
+// Estimated run time in MFMA-pipe cycles of one SIMD.  The chip executes
+// num_cu workgroups of 4 wavefronts at a time (one wavefront per SIMD); a
+// workgroup needs (k/2) * mfma_per_k2 MFMA issues of 64 cycles.  Smaller tiles
+// re-read operands more often and expose more latency, modelled by a
+// per-configuration efficiency.  Split-K adds a second pass over M*N*splitk.
+double estimate_cycles(const ConfigEntry& c, int cfg_id, int M, int N, int K, int batch, int splitk, int num_cu) {
+    static const double eff[kNumConfigs] = {0.92, 0.85, 0.85, 0.75, 0.6, 0.6, 0.45};
+    const long long tiles = (long long)ceil_div(M, c.BM) * ceil_div(N, c.BN) * batch * splitk;
+    const long long rounds = (tiles + num_cu - 1) / num_cu;
+    const int kchunk = ceil_div(ceil_div(K, splitk), c.BK) * c.BK;
+    const double tile_cycles = (kchunk / 2.0) * c.mfma_per_k2 * 64.0 / eff[cfg_id] + 3000.0;
+    double total = rounds * tile_cycles;
+    if (splitk > 1) {
+        // reduce pass: (splitk + 1) reads/writes of M*N floats at ~1.5 kB/cycle, plus a launch
+        total += 12000.0 + (double)M * N * batch * (splitk + 2) * 4.0 / 1500.0;
+    }
+    return total;
+}
+
+Choice choose(const Handle* h, int M, int N, int K, int batch) {
+    Choice best{kNumConfigs - 1, 1};
+    double best_cost = 1e300;
+    for (int c = 0; c < kNumConfigs; ++c) {
+        if (h->force_cfg >= 0 && c != h->force_cfg) continue;
+        const ConfigEntry& e = kConfigs[c];
+        for (int s = 1; s <= 32; s *= 2) {
+            if (h->force_splitk > 0 && s != h->force_splitk) continue;
+            if (s > 1) {
+                if (h->force_splitk <= 0 && K / s < 4 * e.BK) break;
+                if ((size_t)M * N * batch * s * sizeof(float) > kMaxWorkspaceBytes) break;
+                const int kchunk = ceil_div(ceil_div(K, s), e.BK) * e.BK;
+                if ((long long)kchunk * (s - 1) >= K) continue;  // would leave an empty split
+            }
+            const double cost = estimate_cycles(e, c, M, N, K, batch, s, h->num_cu);
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = Choice{c, s};
+            }
+        }
+    }
+    return best;
+}
+
+int ensure_workspace(Handle* h, size_t bytes) {
+    if (bytes <= h->ws_bytes) return SNHIP_STATUS_SUCCESS;
+    if (h->ws != nullptr) {
+        // kernels still in flight may be using the old buffer
+        hipError_t e = hipStreamSynchronize(h->stream);
+        if (e != hipSuccess) return hip_to_status(e);
+        (void)hipFree(h->ws);
+        h->ws = nullptr;
+        h->ws_bytes = 0;
+    }
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return SNHIP_STATUS_ALLOC_FAILED;
+    }
+    h->ws = static_cast<float*>(p);
+    h->ws_bytes = bytes;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+// Row-major core: C[M x N] (ldc) = alpha * op(A)[M x K] * op(B)[K x N] + beta * C (+ bias), per batch.
+int gemm_rm(Handle* h, bool tA, bool tB, int M, int N, int K, float alpha, const float* A, int lda, long long sA,
+            const float* B, int ldb, long long sB, float beta, float* C, int ldc, long long sC, int batch,
+            const float* bias) {
+    if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (M < 0 || N < 0 || K < 0 || batch < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (M == 0 || N == 0 || batch == 0) return SNHIP_STATUS_SUCCESS;
+    if (C == nullptr || ldc < N) return SNHIP_STATUS_INVALID_VALUE;
+    if (batch > 65535 * 1) {
+        // grid.y carries batch * splitk
+        if (batch > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
+    }
+
+    hipError_t e;
+    if (K == 0 || alpha == 0.0f) {
+        // BLAS semantics: A and B are not referenced, C = beta * C.
+        if (beta == 1.0f && bias == nullptr) return SNHIP_STATUS_SUCCESS;
+        const long long total = (long long)M * N * batch;
+        const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+        hipLaunchKernelGGL(scale_c_kernel, dim3(blocks), dim3(256), 0, h->stream, C, bias, M, N, ldc, sC, batch, beta);
+        e = hipGetLastError();
+        return hip_to_status(e);
+    }
+    if (A == nullptr || B == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    if (lda < (tA ? M : K) || ldb < (tB ? K : N)) return SNHIP_STATUS_INVALID_VALUE;
+
+    Choice ch = choose(h, M, N, K, batch);
+    const ConfigEntry& cfg = kConfigs[ch.cfg];
+    if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
+
+    GemmParams p;
+    p.A = A;
+    p.B = B;
+    p.C = C;
+    p.bias = bias;
+    p.ws = nullptr;
+    p.M = M;
+    p.N = N;
+    p.K = K;
+    p.lda = lda;
+    p.ldb = ldb;
+    p.ldc = ldc;
+    p.strideA = sA;
+    p.strideB = sB;
+    p.strideC = sC;
+    p.tiles_m = ceil_div(M, cfg.BM);
+    p.tiles_n = ceil_div(N, cfg.BN);
+    p.splitk = ch.splitk;
+    p.kchunk = ceil_div(ceil_div(K, ch.splitk), cfg.BK) * cfg.BK;
+    p.alpha = alpha;
+    p.beta = beta;
+    p.group_m = 8;
+    p.flags = 0;
+    if (ch.splitk > 1) {
+        const size_t need = (size_t)M * N * batch * ch.splitk * sizeof(float);
+        int st = ensure_workspace(h, need);
+        if (st != SNHIP_STATUS_SUCCESS) return st;
+        p.ws = h->ws;
+        if (N % 4 == 0) p.flags |= GEMM_FLAG_C_VEC;
+    } else {
+        const bool c_vec = ((uintptr_t)C % 16 == 0) && (ldc % 4 == 0) && (batch == 1 || sC % 4 == 0) &&
+                           (bias == nullptr || (uintptr_t)bias % 16 == 0);
+        if (c_vec) p.flags |= GEMM_FLAG_C_VEC;
+    }
+    const long long ntiles = (long long)p.tiles_m * p.tiles_n;
+    if (ntiles > 0x7fffffffLL) return SNHIP_STATUS_NOT_SUPPORTED;
+
+    h->last_cfg = ch.cfg;
+    h->last_splitk = ch.splitk;
+
+    KernelFn fn = cfg.fn[tA ? 1 : 0][tB ? 1 : 0];
+    hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)(batch * ch.splitk)), dim3(cfg.NT), cfg.lds_bytes,
+                       h->stream, p);
+    e = hipGetLastError();
+    if (e != hipSuccess) return hip_to_status(e);
+
+    if (ch.splitk > 1) {
+        const long long total = (long long)M * N * batch;
+        const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, h->stream, h->ws, C, bias, M, N, ldc, sC,
+                           ch.splitk, batch, alpha, beta);
+        e = hipGetLastError();
+        if (e != hipSuccess) return hip_to_status(e);
+    }
+    return SNHIP_STATUS_SUCCESS;
+}
+
+inline bool op_is_trans(int op, bool* ok) {
+    *ok = (op == SNHIP_OP_N || op == SNHIP_OP_T || op == SNHIP_OP_C);
+    return op != SNHIP_OP_N;
+}
+
+}  // namespace
+
+extern "C" {
+
+int snhip_create(void** handle) {
+    if (handle == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    *handle = nullptr;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    // The code objects in this library exist for gfx950 only.
+    if (prop.gcnArchName[0] == '\0' || __builtin_strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return SNHIP_STATUS_ARCH_MISMATCH;
+    // Kernels whose LDS stage exceeds the 64 KiB default need an explicit opt-in.
+    for (int c = 0; c < kNumConfigs; ++c) {
+        for (int ta = 0; ta < 2; ++ta)
+            for (int tb = 0; tb < 2; ++tb) {
+                e = hipFuncSetAttribute(reinterpret_cast<const void*>(kConfigs[c].fn[ta][tb]),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kConfigs[c].lds_bytes);
+                if (e != hipSuccess) return hip_to_status(e);
+            }
+    }
+    Handle* h = new (std::nothrow) Handle();
+    if (h == nullptr) return SNHIP_STATUS_ALLOC_FAILED;
+    h->device = dev;
+    h->num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    *handle = h;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_destroy(void* handle) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    Handle* h = static_cast<Handle*>(handle);
+    if (h->ws != nullptr) {
+        (void)hipStreamSynchronize(h->stream);
+        (void)hipFree(h->ws);
+    }
+    delete h;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_set_stream(void* handle, void* stream) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    static_cast<Handle*>(handle)->stream = static_cast<hipStream_t>(stream);
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_get_version(void* handle, int* version) {
+    (void)handle;
+    if (version == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    *version = kVersion;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_sgemm_strided_batched(void* handle, int transa, int transb, int m, int n, int k, const float* alpha,
+                                const void* A, int lda, long long strideA, const void* B, int ldb, long long strideB,
+                                const float* beta, void* C, int ldc, long long strideC, int batchCount) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (alpha == nullptr || beta == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    bool oka, okb;
+    const bool ta = op_is_trans(transa, &oka), tb = op_is_trans(transb, &okb);
+    if (!oka || !okb) return SNHIP_STATUS_INVALID_VALUE;
+    if (m < 0 || n < 0 || k < 0 || batchCount < 0) return SNHIP_STATUS_INVALID_VALUE;
+    // cuBLAS leading-dimension rules for column-major storage
+    const int rows_a = ta ? k : m, rows_b = tb ? n : k;
+    if (lda < (rows_a > 1 ? rows_a : 1) || ldb < (rows_b > 1 ? rows_b : 1) || ldc < (m > 1 ? m : 1))
+        return SNHIP_STATUS_INVALID_VALUE;
+    // A column-major matrix with leading dimension ld is the row-major transpose
+    // with row pitch ld.  C^T (n x m) = op(B)^T * op(A)^T, so in row-major terms the
+    // left operand is B (transposed iff transb) and the right operand is A.
+    return gemm_rm(static_cast<Handle*>(handle), tb, ta, n, m, k, *alpha, static_cast<const float*>(B), ldb, strideB,
+                   static_cast<const float*>(A), lda, strideA, *beta, static_cast<float*>(C), ldc, strideC, batchCount,
+                   nullptr);
+}
+
+int snhip_sgemm(void* handle, int transa, int transb, int m, int n, int k, const float* alpha, const void* A, int lda,
+                const void* B, int ldb, const float* beta, void* C, int ldc) {
+    return snhip_sgemm_strided_batched(handle, transa, transb, m, n, k, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1);
+}
+
+int snhip_gemm_rm(void* handle, int transposeA, int transposeB, int M, int N, int K, float alpha, const float* A,
+                  int lda, long long strideA, const float* B, int ldb, long long strideB, float beta, float* C,
+                  int ldc, long long strideC, int batch, const float* bias) {
+    return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha, A, lda, strideA, B,
+                   ldb, strideB, beta, C, ldc, strideC, batch, bias);
+}
+
+int snhip_dot_bias(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
+                   int transposeB, float* C, float alpha, float beta, const float* bias) {
+    if (aH < 0 || aW < 0 || bH < 0 || bW < 0) return SNHIP_STATUS_INVALID_VALUE;
+    // BlasServices.DotMkl, Prod/Data/BlasServices.cs:14-19
+    const int M = transposeA ? aW : aH;
+    const int N = transposeB ? bH : bW;
+    const int K = transposeA ? aH : aW;
+    const int Kb = transposeB ? bW : bH;
+    if (K != Kb) return SNHIP_STATUS_INVALID_VALUE;
+    return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha, A, aW, 0, B, bW, 0,
+                   beta, C, N, 0, 1, bias);
+}
+
+int snhip_dot(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
+              int transposeB, float* C, float alpha, float beta) {
+    return snhip_dot_bias(handle, A, aH, aW, transposeA, B, bH, bW, transposeB, C, alpha, beta, nullptr);
+}
+
+int snhip_bmm(void* handle, const float* A, int aH, int aW, int transposeA, long long strideA, const float* B, int bH,
+              int bW, int transposeB, long long strideB, float* C, long long strideC, int batch, float alpha,
+              float beta) {
+    if (aH < 0 || aW < 0 || bH < 0 || bW < 0) return SNHIP_STATUS_INVALID_VALUE;
+    const int M = transposeA ? aW : aH;
+    const int N = transposeB ? bH : bW;
+    const int K = transposeA ? aH : aW;
+    const int Kb = transposeB ? bW : bH;
+    if (K != Kb) return SNHIP_STATUS_INVALID_VALUE;
+    return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha, A, aW, strideA, B,
+                   bW, strideB, beta, C, N, strideC, batch, nullptr);
+}
+
+/* ---- memory / stream shims ---- */
+
+int snhip_malloc(void** dptr, size_t bytes) {
+    if (dptr == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    *dptr = nullptr;
+    if (bytes < 8) bytes = 8;  // GPUTensor never allocates less (GpuTensor.cs:38)
+    hipError_t e = hipMalloc(dptr, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return SNHIP_STATUS_ALLOC_FAILED;
+    }
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_free(void* dptr) {
+    if (dptr == nullptr) return SNHIP_STATUS_SUCCESS;
+    return hip_to_status(hipFree(dptr));
+}
+
+int snhip_memset32(void* handle, void* dptr, unsigned int value, size_t count) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (count == 0) return SNHIP_STATUS_SUCCESS;
+    if (dptr == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    return hip_to_status(hipMemsetD32Async((hipDeviceptr_t)dptr, (int)value, count, static_cast<Handle*>(handle)->stream));
+}
+
+int snhip_memcpy_htod_async(void* handle, void* dst, const void* src, size_t bytes) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (bytes == 0) return SNHIP_STATUS_SUCCESS;
+    if (dst == nullptr || src == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    return hip_to_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<Handle*>(handle)->stream));
+}
+
+int snhip_memcpy_dtoh(void* handle, void* dst, const void* src, size_t bytes) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (bytes == 0) return SNHIP_STATUS_SUCCESS;
+    if (dst == nullptr || src == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipStream_t s = static_cast<Handle*>(handle)->stream;
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) return hip_to_status(e);
+    return hip_to_status(hipStreamSynchronize(s));
+}
+
+int snhip_memcpy_dtod_async(void* handle, void* dst, const void* src, size_t bytes) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (bytes == 0) return SNHIP_STATUS_SUCCESS;
+    if (dst == nullptr || src == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    return hip_to_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<Handle*>(handle)->stream));
+}
+
+int snhip_stream_synchronize(void* handle) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    return hip_to_status(hipStreamSynchronize(static_cast<Handle*>(handle)->stream));
+}
+
+/* ---- measurement helpers ---- */
+
+int snhip_event_create(void** event) {
+    if (event == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipEvent_t ev;
+    hipError_t e = hipEventCreate(&ev);
+    if (e != hipSuccess) return hip_to_status(e);
+    *event = ev;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_event_destroy(void* event) {
+    if (event == nullptr) return SNHIP_STATUS_SUCCESS;
+    return hip_to_status(hipEventDestroy(static_cast<hipEvent_t>(event)));
+}
+
+int snhip_event_record(void* handle, void* event) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (event == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    return hip_to_status(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<Handle*>(handle)->stream));
+}
+
+int snhip_event_elapsed_ms(void* start, void* stop, float* ms) {
+    if (start == nullptr || stop == nullptr || ms == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipError_t e = hipEventSynchronize(static_cast<hipEvent_t>(stop));
+    if (e != hipSuccess) return hip_to_status(e);
+    return hip_to_status(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+}
+
+int snhip_device_info(void* handle, int info[6]) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (info == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipDeviceProp_t prop;
+    hipError_t e = hipGetDeviceProperties(&prop, static_cast<Handle*>(handle)->device);
+    if (e != hipSuccess) return hip_to_status(e);
+    info[0] = prop.multiProcessorCount;
+    info[1] = prop.clockRate;
+    info[2] = prop.memoryClockRate;
+    info[3] = prop.memoryBusWidth;
+    info[4] = (int)prop.sharedMemPerBlockOptin;
+    int arch = 0;
+    for (const char* c = prop.gcnArchName + 3; *c >= '0' && *c <= '9'; ++c) arch = arch * 10 + (*c - '0');
+    info[5] = arch;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_set_tuning(void* handle, int config, int splitk) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (config >= kNumConfigs || splitk < 0 || splitk > 64) return SNHIP_STATUS_INVALID_VALUE;
+    Handle* h = static_cast<Handle*>(handle);
+    h->force_cfg = config < 0 ? -1 : config;
+    h->force_splitk = splitk;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_get_last_tuning(void* handle, int* config, int* splitk) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    Handle* h = static_cast<Handle*>(handle);
+    if (config != nullptr) *config = h->last_cfg;
+    if (splitk != nullptr) *splitk = h->last_splitk;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_config_count(void) { return kNumConfigs; }
+
+int snhip_config_desc(int config, int desc[5]) {
+    if (config < 0 || config >= kNumConfigs || desc == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    desc[0] = kConfigs[config].BM;
+    desc[1] = kConfigs[config].BN;
+    desc[2] = kConfigs[config].BK;
+    desc[3] = kConfigs[config].NT;
+    desc[4] = kConfigs[config].lds_bytes;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+}  // extern "C"

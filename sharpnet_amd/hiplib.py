@@ -1,0 +1,107 @@
+"""ctypes binding of libsharpnet_hip.so - the Python twin of the P/Invoke shim a
+SharpNet maintainer would write in place of Prod/GPU/CublasWrapper.cs:221-250.
+
+Nothing here computes: every function forwards raw device addresses to the C
+ABI declared in include/sharpnet_hip.h.  There is no CPU fallback; if the
+library is missing, ``load_library`` raises.
+"""
+import ctypes
+import enum
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+class CublasStatus(enum.IntEnum):
+    """Status numbering shared with cublasStatus_t (Prod/GPU/CublasWrapper.cs:8-20)."""
+    CUBLAS_STATUS_SUCCESS = 0
+    CUBLAS_STATUS_NOT_INITIALIZED = 1
+    CUBLAS_STATUS_ALLOC_FAILED = 3
+    CUBLAS_STATUS_INVALID_VALUE = 7
+    CUBLAS_STATUS_ARCH_MISMATCH = 8
+    CUBLAS_STATUS_MAPPING_ERROR = 11
+    CUBLAS_STATUS_EXECUTION_FAILED = 13
+    CUBLAS_STATUS_INTERNAL_ERROR = 14
+    CUBLAS_STATUS_NOT_SUPPORTED = 15
+
+
+class SharpNetHipError(Exception):
+    """Raised for any non-zero status, like GPUWrapper.CheckStatus (Prod/GPU/GPUWrapper.cs:662-668)."""
+
+    def __init__(self, status, where=""):
+        try:
+            name = CublasStatus(status).name
+        except ValueError:
+            name = "status %d" % status
+        super().__init__(name + (" in " + where if where else ""))
+        self.status = status
+
+
+def check_status(status, where=""):
+    if status != 0:
+        raise SharpNetHipError(status, where)
+
+
+def library_path():
+    return os.environ.get("SHARPNET_HIP_LIB", os.path.join(_HERE, "libsharpnet_hip.so"))
+
+
+_c_int_p = ctypes.POINTER(ctypes.c_int)
+_c_float_p = ctypes.POINTER(ctypes.c_float)
+_vp = ctypes.c_void_p
+_vpp = ctypes.POINTER(ctypes.c_void_p)
+_i = ctypes.c_int
+_ll = ctypes.c_longlong
+_f = ctypes.c_float
+_sz = ctypes.c_size_t
+
+# name -> argtypes; every function returns int.  Must list every symbol of include/sharpnet_hip.h.
+SIGNATURES = {
+    "snhip_create": [_vpp],
+    "snhip_destroy": [_vp],
+    "snhip_set_stream": [_vp, _vp],
+    "snhip_get_version": [_vp, _c_int_p],
+    "snhip_sgemm": [_vp, _i, _i, _i, _i, _i, _c_float_p, _vp, _i, _vp, _i, _c_float_p, _vp, _i],
+    "snhip_sgemm_strided_batched": [_vp, _i, _i, _i, _i, _i, _c_float_p, _vp, _i, _ll, _vp, _i, _ll, _c_float_p, _vp,
+                                    _i, _ll, _i],
+    "snhip_dot": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f],
+    "snhip_dot_bias": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f, _vp],
+    "snhip_bmm": [_vp, _vp, _i, _i, _i, _ll, _vp, _i, _i, _i, _ll, _vp, _ll, _i, _f, _f],
+    "snhip_gemm_rm": [_vp, _i, _i, _i, _i, _i, _f, _vp, _i, _ll, _vp, _i, _ll, _f, _vp, _i, _ll, _i, _vp],
+    "snhip_malloc": [_vpp, _sz],
+    "snhip_free": [_vp],
+    "snhip_memset32": [_vp, _vp, ctypes.c_uint, _sz],
+    "snhip_memcpy_htod_async": [_vp, _vp, _vp, _sz],
+    "snhip_memcpy_dtoh": [_vp, _vp, _vp, _sz],
+    "snhip_memcpy_dtod_async": [_vp, _vp, _vp, _sz],
+    "snhip_stream_synchronize": [_vp],
+    "snhip_event_create": [_vpp],
+    "snhip_event_destroy": [_vp],
+    "snhip_event_record": [_vp, _vp],
+    "snhip_event_elapsed_ms": [_vp, _vp, _c_float_p],
+    "snhip_device_info": [_vp, _c_int_p],
+    "snhip_set_tuning": [_vp, _i, _i],
+    "snhip_get_last_tuning": [_vp, _c_int_p, _c_int_p],
+    "snhip_config_count": [],
+    "snhip_config_desc": [_i, _c_int_p],
+}
+
+
+def load_library(path=None):
+    """dlopen libsharpnet_hip.so and attach the prototypes.  Raises if it is absent."""
+    global _LIB
+    if _LIB is not None and path is None:
+        return _LIB
+    path = path or library_path()
+    if not os.path.exists(path):
+        raise FileNotFoundError(
+            "%s not found: build it with `python -m sharpnet_amd.build` (hipcc, gfx950). "
+            "There is no CPU fallback for this path." % path)
+    lib = ctypes.CDLL(path)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_int
+    _LIB = lib
+    return lib

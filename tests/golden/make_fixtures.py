@@ -1,0 +1,130 @@
+"""Writes tests/golden/reference_vectors.json from the literals the reference's own tests hold.
+
+Run once in a container that has the reference tree:  python tests/golden/make_fixtures.py
+The reference files are opened as TEXT only (nothing is compiled, imported or
+executed); the output holds numbers - inputs and expected outputs - never source.
+The GPU box has no reference tree: tests read the committed JSON.
+"""
+import json
+import os
+import re
+import sys
+
+REF = os.environ.get("SHARPNET_REFERENCE", "/root/reference")
+OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_vectors.json")
+
+
+def read(rel):
+    with open(os.path.join(REF, rel), encoding="utf-8-sig") as f:
+        return f.read()
+
+
+def lines(text, lo, hi):
+    """1-based inclusive line range."""
+    return "\n".join(text.split("\n")[lo - 1:hi])
+
+
+def numpy_literals(block):
+    """All FromNumpyArray-style literals in a block of C#: "[[...]]" or "numpy.array([...], numpy.float)"."""
+    out = []
+    for m in re.finditer(r'"\s*(?:numpy\.array\()?\s*(\[[^"]*?\])\s*(?:,\s*numpy\.float\))?\s*"', block):
+        out.append(json.loads(m.group(1)))
+    return out
+
+
+def const_literal(text, name):
+    m = re.search(r'const string ' + re.escape(name) + r'\s*=\s*@?"([^"]*)"', text)
+    body = m.group(1)
+    arr = re.search(r'(\[.*\])', body, re.S).group(1)
+    return json.loads(arr)
+
+
+def main():
+    fx = {}
+
+    # ---- Tests/GPU/TestGpuTensor.cs:50-120  TestDot known answers (tolerance 1e-9) ----
+    fx["TestDot"] = {
+        "source": "Tests/GPU/TestGpuTensor.cs:53-109",
+        "tolerance": 1e-9,
+        "cases": [
+            {"a_shape": [1, 1], "a": [2], "b_shape": [1, 1], "b": [5], "c_shape": [1, 1], "expected": [10]},
+            {"a_shape": [2, 2], "a": [1, 2, 3, 4], "b_shape": [2, 2], "b": [1, 2, 3, 4], "c_shape": [2, 2],
+             "expected": [7, 10, 15, 22]},
+            {"a_shape": [1, 2], "a": [1, 2], "b_shape": [2, 1], "b": [3, 4], "c_shape": [1, 1], "expected": [11]},
+            {"a_shape": [2, 1], "a": [1, 2], "b_shape": [1, 2], "b": [3, 4], "c_shape": [2, 2],
+             "expected": [3, 4, 6, 8]},
+            {"a_shape": [2, 1, 1], "a": [1, 2], "b_shape": [1, 1, 2], "b": [3, 4], "c_shape": [2, 2],
+             "expected": [3, 4, 6, 8]},
+            {"a_shape": [10, 1, 28, 28], "a": "zeros", "b_shape": [784, 100], "b": "zeros", "c_shape": [10, 1, 1, 100],
+             "expected": "zeros"},
+            {"a_shape": [35, 124], "a": "zeros", "b_shape": [124, 21], "b": "zeros", "c_shape": [35, 21],
+             "expected": "zeros"},
+        ],
+    }
+
+    # ---- Tests/CPU/TestCpuTensor.cs:826-866  QR factorisation of the Rosetta-code matrix ----
+    cpu = read("Tests/CPU/TestCpuTensor.cs")
+    qr_cases = []
+    for m in re.finditer(r'\[TestCase\("(\[\[[^"]*\]\])",\s*"\s*(\[\[[^"]*\]\])"\)\]', lines(cpu, 855, 870)):
+        qr_cases.append({"A": json.loads(m.group(1)), "Q": json.loads(m.group(2))})
+    assert len(qr_cases) == 2, qr_cases
+    fx["QR"] = {
+        "source": "Tests/CPU/TestCpuTensor.cs:826-866 (A at :830, expected Q at :861-863); "
+                  "asserts Dot(Q,R)~A within 1e-4 and max|QtQ-I| < 1e-6",
+        "cases": qr_cases,
+    }
+
+    # ---- Tests/NonReg/TestNetworkPropagation.cs  Linear + sigmoid predictions ----
+    tnp = read("Tests/NonReg/TestNetworkPropagation.cs")
+    fx["Linear_1_1_1_1"] = {
+        "source": "Tests/NonReg/TestNetworkPropagation.cs:36-61",
+        "x": [[[[1.0]]]],
+        "w": numpy_literals(lines(tnp, 47, 48))[0],
+        "sigmoid_prediction": numpy_literals(lines(tnp, 50, 51))[0],
+        "tolerance": 1e-6,
+    }
+    fx["Linear_1_1_4_4"] = {
+        "source": "Tests/NonReg/TestNetworkPropagation.cs:24,34,80-105 (weights literal is (in=16, out=3): "
+                  "prediction = sigmoid(x[1x16] . W[16x3]))",
+        "x": const_literal(tnp, "X_1_1_4_4"),
+        "w_in_out": const_literal(tnp, "W_N_1_4_4"),
+        "sigmoid_prediction": numpy_literals(lines(tnp, 95, 95))[0],
+        "tolerance": 1e-6,
+    }
+
+    # ---- Tests/NonReg/ParallelRunWithPyTorch.cs:102-138  two Linear layers, MSE, SGD momentum ----
+    prp = read("Tests/NonReg/ParallelRunWithPyTorch.cs")
+    blk = lines(prp, 102, 138)
+    w = numpy_literals(blk)
+    assert len(w) == 2 and len(w[0]) == 3 and len(w[0][0]) == 5 and len(w[1][0]) == 36
+    losses = [float(v) for v in re.findall(r'Assert\.AreEqual\(([0-9.eE+-]+), loss_', blk)]
+    fx["PyTorch_Mse"] = {
+        "source": "Tests/NonReg/ParallelRunWithPyTorch.cs:102-138; inputs numpy_array_for_tests(2,3,4,5) and "
+                  "y_numpy_array_for_tests(2,3), Tests/NonReg/TestNetworkPropagation.cs:167-186",
+        "x_shape": [2, 3, 4, 5], "y_shape": [2, 3],
+        "linear1_weight_out_in": w[0], "linear2_weight_out_in": w[1],
+        "lr": 0.1, "momentum": 0.9, "epochs": 10,
+        "loss_before": losses[0], "loss_after": losses[1], "tolerance": 1e-6,
+    }
+
+    # ---- same file :963-1010  scaled-dot-product attention chain ----
+    blk = lines(prp, 961, 1010)
+    w = numpy_literals(blk)
+    assert len(w) == 4, len(w)
+    cases = re.findall(r'\[TestCase\((false|true),\s*([0-9.eE+-]+),\s*([0-9.eE+-]+)\)\]', blk)
+    fx["PyTorch_DotProductAttention"] = {
+        "source": "Tests/NonReg/ParallelRunWithPyTorch.cs:963-1010 (use_scale=false); X = numpy_array_for_tests(6,4,5) "
+                  "read as (N, C=4, L=5); conv1D kernels of width 1 = per-sample (2x4).(4x5) products",
+        "x_shape": [6, 4, 5], "y_shape": [6, 3],
+        "conv_q": w[0], "conv_k": w[1], "conv_v": w[2], "dense_weight_out_in": w[3],
+        "cases": [{"is_causal": c[0] == "true", "loss_before": float(c[1]), "loss_after": float(c[2])} for c in cases],
+        "tolerance": 1e-6,
+    }
+
+    with open(OUT, "w") as f:
+        json.dump(fx, f, indent=1)
+    print("wrote", OUT, os.path.getsize(OUT), "bytes")
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,304 @@
+"""GPU parity tests of Tensor.Dot / BatchMatrixMultiplication through the C ABI.
+
+Shaped like the reference's own harness (Tests/TestParallelRunCpuVersusGpu.cs:1449-1465):
+the same seeded host inputs go to the oracle and to the device, and every output is
+compared.  fp32 bar (written out in `tol`): max|C_gpu - C_ref| <= 1e-4*sqrt(K)*max|a|*max|b|.
+"""
+import ctypes
+import itertools
+
+import numpy as np
+import pytest
+
+from tests.helpers import random_tensor
+
+pytestmark = pytest.mark.gpu
+
+
+def tol(K, a, b, alpha=1.0, beta=0.0, c=None):
+    t = 1e-4 * np.sqrt(max(K, 1)) * float(np.max(np.abs(a))) * float(np.max(np.abs(b))) * max(abs(alpha), 1e-30)
+    if beta != 0.0 and c is not None:
+        t += 1e-6 * abs(beta) * float(np.max(np.abs(c)))
+    return max(t, 1e-30)
+
+
+def gpu_dot(w, a, tA, b, tB, alpha=1.0, beta=0.0, c=None, c_shape=None, prefill=None):
+    from sharpnet_amd import GPUTensor
+    ga, gb = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w)
+    if c is not None:
+        gc = GPUTensor(c.shape, c, w)
+    else:
+        gc = GPUTensor(c_shape, None, w)
+        if prefill is not None:
+            gc.SetValue(prefill)
+    gc.Dot(ga, tA, gb, tB, alpha, beta)
+    out = gc.ToNumpy()
+    for t in (ga, gb, gc):
+        t.Dispose()
+    return out
+
+
+def mnk(a, tA, b, tB):
+    a2, b2 = a.reshape(a.shape[0], -1), b.reshape(b.shape[0], -1)
+    M = a2.shape[1] if tA else a2.shape[0]
+    N = b2.shape[0] if tB else b2.shape[1]
+    K = a2.shape[0] if tA else a2.shape[1]
+    return M, N, K
+
+
+# ---------------------------------------------------------------------------
+# reference known answers
+# ---------------------------------------------------------------------------
+def test_TestDot_known_answers(golden, gpu_wrapper):
+    """Tests/GPU/TestGpuTensor.cs:50-120, tolerance 1e-9."""
+    for case in golden["TestDot"]["cases"]:
+        def arr(v, shape):
+            return np.zeros(shape, np.float32) if v == "zeros" else np.array(v, np.float32).reshape(shape)
+        a, b = arr(case["a"], case["a_shape"]), arr(case["b"], case["b_shape"])
+        got = gpu_dot(gpu_wrapper, a, False, b, False, 1, 0, c_shape=case["c_shape"], prefill=float("nan"))
+        expected = arr(case["expected"], case["c_shape"])
+        assert got.shape == expected.shape
+        assert np.max(np.abs(got - expected)) <= golden["TestDot"]["tolerance"], case
+
+
+def test_QR_identity_on_device(golden, gpu_wrapper):
+    """Tests/GPU/TestGpuTensor.cs:18-47: Dot(Q,R) ~ A (1e-4), max|QtQ - I| < 1e-6."""
+    for case in golden["QR"]["cases"]:
+        A, Q = np.array(case["A"], np.float32), np.array(case["Q"], np.float32)
+        n = A.shape[1]
+        R = gpu_dot(gpu_wrapper, Q, True, A, False, c_shape=[n, n])
+        QR = gpu_dot(gpu_wrapper, Q, False, R, False, c_shape=list(A.shape))
+        assert np.max(np.abs(QR - A)) < 1e-4
+        QtQ = gpu_dot(gpu_wrapper, Q, True, Q, False, c_shape=[n, n])
+        assert np.max(np.abs(QtQ - np.eye(n))) < 1e-6
+
+
+# ---------------------------------------------------------------------------
+# CPU-versus-GPU harness cases
+# ---------------------------------------------------------------------------
+def test_cpu_vs_gpu_TestDot_cases(oracle, gpu_wrapper):
+    """TestDot 8x10x12 (:368-375), TestDotV2 (:436-443), TestDotV3 2x20000x2 (:445-456)."""
+    rng = np.random.default_rng(0)
+    for (M, K, N) in [(8, 10, 12), (8, 10, 12), (2, 20000, 2)]:
+        a, b = random_tensor(rng, (M, K)), random_tensor(rng, (K, N))
+        got = gpu_dot(gpu_wrapper, a, False, b, False, 1, 0, c_shape=[M, N], prefill=float("nan"))
+        ref = oracle.dot(a, False, b, False)
+        err = np.max(np.abs(got - ref))
+        assert err <= tol(K, a, b), (M, N, K, err)
+        assert err <= 1e-2   # the reference's own acceptance (:1440-1447)
+
+
+def test_cpu_vs_gpu_BatchMatrixMultiplication(oracle, gpu_wrapper):
+    """Tests/TestParallelRunCpuVersusGpu.cs:377-401: batch 3, L=12, d=7; NT alpha=0.25, NN, TN."""
+    from sharpnet_amd import GPUTensor
+    rng = np.random.default_rng(1)
+    batch, L, d = 3, 12, 7
+    V, dy, K_, Q = (random_tensor(rng, (batch, L, d)) for _ in range(4))
+    S = random_tensor(rng, (batch, L, L))
+    cases = [((batch, L, L), dy, False, V, True, 0.25),
+             ((batch, L, d), S, False, K_, False, 1.0),
+             ((batch, L, d), S, True, Q, False, 1.0)]
+    for c_shape, a, tA, b, tB, alpha in cases:
+        ga, gb = GPUTensor(a.shape, a, gpu_wrapper), GPUTensor(b.shape, b, gpu_wrapper)
+        gc = GPUTensor(c_shape, None, gpu_wrapper)
+        gc.SetValue(float("nan"))
+        gc.BatchMatrixMultiplication(ga, tA, gb, tB, alpha, 0.0)
+        got = gc.ToNumpy()
+        ref = oracle.bmm(a, tA, b, tB, alpha, 0.0)
+        Kdim = a.shape[1] if tA else a.shape[2]
+        assert np.max(np.abs(got - ref)) <= tol(Kdim, a, b, alpha)
+
+
+# ---------------------------------------------------------------------------
+# every tile configuration x transpose x alpha/beta on ragged shapes
+# ---------------------------------------------------------------------------
+SHAPES = [(35, 21, 124), (33, 17, 65), (129, 257, 63), (256, 256, 64), (300, 130, 200), (64, 64, 16), (1, 1, 1),
+          (257, 100, 33), (5, 300, 1000)]
+
+
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_all_configs_all_transposes(oracle, gpu_wrapper, tA, tB):
+    rng = np.random.default_rng(100 + 2 * tA + tB)
+    ncfg = len(gpu_wrapper.configs())
+    try:
+        for (M, N, K) in SHAPES:
+            a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
+            b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
+            c = random_tensor(rng, (M, N), -1, 1)
+            refs = {}
+            for alpha, beta in [(1.0, 0.0), (0.25, 0.0), (-1.0, 1.0), (0.5, 1.0)]:
+                refs[(alpha, beta)] = oracle.dot(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
+            for cfg in range(ncfg):
+                for splitk in (1, 2, 4):
+                    if splitk > 1 and K < 64:
+                        continue
+                    gpu_wrapper.set_tuning(cfg, splitk)
+                    for (alpha, beta), ref in refs.items():
+                        if beta == 0.0:
+                            got = gpu_dot(gpu_wrapper, a, tA, b, tB, alpha, beta, c_shape=[M, N],
+                                          prefill=float("nan"))
+                        else:
+                            got = gpu_dot(gpu_wrapper, a, tA, b, tB, alpha, beta, c=c)
+                        err = np.max(np.abs(got - ref))
+                        assert np.all(np.isfinite(got)), (M, N, K, cfg, splitk, alpha, beta)
+                        assert err <= tol(K, a, b, alpha, beta, c), (M, N, K, cfg, splitk, alpha, beta, err)
+    finally:
+        gpu_wrapper.set_tuning(-1, 0)
+
+
+def test_beta_zero_never_reads_destination(oracle, gpu_wrapper):
+    """TensorMemoryPool hands out uninitialised memory (Prod/Data/TensorMemoryPool.cs:59-64)."""
+    rng = np.random.default_rng(2)
+    for (M, N, K) in [(128, 256, 784), (300, 300, 300), (1000, 64, 2048)]:
+        a, b = random_tensor(rng, (M, K)), random_tensor(rng, (K, N))
+        for fill in (float("nan"), float("inf")):
+            got = gpu_dot(gpu_wrapper, a, False, b, False, 1, 0, c_shape=[M, N], prefill=fill)
+            assert np.all(np.isfinite(got))
+            assert np.max(np.abs(got - oracle.dot(a, False, b, False))) <= tol(K, a, b)
+
+
+def test_aliased_operands_VanillaSgdOrtho_pattern(oracle, gpu_wrapper):
+    """Prod/Optimizers/VanillaSgdOrtho.cs:83: buffer = I - W.W^T via Dot(W,false,W,true,-1,1) on an identity."""
+    from sharpnet_amd import GPUTensor
+    rng = np.random.default_rng(3)
+    m, n = 37, 53
+    W = random_tensor(rng, (m, n), -1, 1)
+    gW = GPUTensor(W.shape, W, gpu_wrapper)
+    gI = GPUTensor([m, m], np.eye(m, dtype=np.float32), gpu_wrapper)
+    gI.Dot(gW, False, gW, True, -1.0, 1.0)
+    got = gI.ToNumpy()
+    ref = oracle.dot(W, False, W, True, -1.0, 1.0, np.eye(m, dtype=np.float32))
+    assert np.max(np.abs(got - ref)) <= tol(n, W, W, 1.0, 1.0, np.eye(m))
+    # alpha = 0.5, beta = 1 accumulation (:88)
+    X = random_tensor(rng, (m, n), -1, 1)
+    gX = GPUTensor(X.shape, X, gpu_wrapper)
+    gX.Dot(gI, False, gW, False, 0.5, 1.0)
+    ref2 = oracle.dot(ref, False, W, False, 0.5, 1.0, X)
+    assert np.max(np.abs(gX.ToNumpy() - ref2)) <= tol(m, ref, W, 0.5, 1.0, X) + 1e-5
+
+
+def test_views_at_odd_element_offsets(oracle, gpu_wrapper):
+    """Slices are views at Pointer + 4*startIndex (GpuTensor.cs:616): only 4-byte alignment may be assumed."""
+    from sharpnet_amd import GPUTensor
+    rng = np.random.default_rng(4)
+    M, N, K = 130, 260, 70
+    for off in (1, 2, 3, 5):
+        bufA = random_tensor(rng, (M * K + 8,), -1, 1)
+        bufB = random_tensor(rng, (K * N + 8,), -1, 1)
+        bufC = random_tensor(rng, (M * N + 8,), -1, 1)
+        gA, gB, gC = (GPUTensor([x.size], x, gpu_wrapper) for x in (bufA, bufB, bufC))
+        a, b, c = gA.Slice(off, [M, K]), gB.Slice(off, [K, N]), gC.Slice(off, [M, N])
+        c.Dot(a, False, b, False, 1.0, 1.0)
+        out = gC.ToNumpy()
+        ref = oracle.dot(bufA[off:off + M * K].reshape(M, K), False, bufB[off:off + K * N].reshape(K, N), False, 1.0,
+                         1.0, bufC[off:off + M * N].reshape(M, N))
+        assert np.max(np.abs(out[off:off + M * N].reshape(M, N) - ref)) <= tol(K, bufA, bufB, 1, 1, bufC)
+        # nothing outside the view was written
+        assert np.array_equal(out[:off], bufC[:off]) and np.array_equal(out[off + M * N:], bufC[off + M * N:])
+        # transposed operands through views as well
+        at, bt = gA.Slice(off, [K, M]), gB.Slice(off, [N, K])
+        c.Dot(at, True, bt, True, 1.0, 0.0)
+        ref = oracle.dot(bufA[off:off + M * K].reshape(K, M), True, bufB[off:off + K * N].reshape(N, K), True)
+        assert np.max(np.abs(c.ToNumpy() - ref)) <= tol(K, bufA, bufB)
+
+
+def test_colmajor_sgemm_with_padded_leading_dimensions(oracle, gpu_wrapper):
+    """snhip_sgemm has cublasSgemm_v2's column-major meaning incl. lda/ldb/ldc > rows; padding stays untouched."""
+    from sharpnet_amd import GPUTensor
+    lib, h = gpu_wrapper.lib, gpu_wrapper.handle
+    rng = np.random.default_rng(5)
+    m, n, k = 70, 45, 130
+    for ta, tb in itertools.product([0, 1], repeat=2):
+        lda = (k if ta else m) + 3
+        ldb = (n if tb else k) + 2
+        ldc = m + 5
+        A = random_tensor(rng, ((m if ta else k), lda), -1, 1)
+        B = random_tensor(rng, ((k if tb else n), ldb), -1, 1)
+        C = random_tensor(rng, (n, ldc), -1, 1)
+        gA, gB, gC = (GPUTensor(list(x.shape), x, gpu_wrapper) for x in (A, B, C))
+        al, be = ctypes.c_float(0.5), ctypes.c_float(-1.0)
+        st = lib.snhip_sgemm(h, ta, tb, m, n, k, ctypes.byref(al), gA.Pointer, lda, gB.Pointer, ldb, ctypes.byref(be),
+                             gC.Pointer, ldc)
+        assert st == 0
+        got = gC.ToNumpy()
+        ref = oracle.sgemm_colmajor(ta, tb, m, n, k, 0.5, A, lda, B, ldb, -1.0, C, ldc).reshape(n, ldc)
+        assert np.max(np.abs(got - ref)) <= tol(k, A, B, 0.5, 1.0, C)
+        assert np.array_equal(got[:, m:], C[:, m:])
+
+
+def test_row_major_entry_points_agree(oracle, gpu_wrapper):
+    """snhip_dot / snhip_dot_bias / snhip_bmm / snhip_gemm_rm give the oracle's numbers."""
+    from sharpnet_amd import GPUTensor
+    lib, h = gpu_wrapper.lib, gpu_wrapper.handle
+    rng = np.random.default_rng(6)
+    M, N, K = 128, 256, 784
+    x = rng.uniform(0, 1, (M, K)).astype(np.float32)
+    w = random_tensor(rng, (N, K), -0.076, 0.076)
+    bias = random_tensor(rng, (N,), -1, 1)
+    gx, gw, gb = GPUTensor([M, K], x, gpu_wrapper), GPUTensor([N, K], w, gpu_wrapper), GPUTensor([N], bias, gpu_wrapper)
+    gy = GPUTensor([M, N], None, gpu_wrapper)
+    gy.SetValue(float("nan"))
+    gy.DotRowMajor(gx, False, gw, True, 1.0, 0.0, bias=gb)
+    ref = oracle.dense_forward(x, w, bias)
+    assert np.max(np.abs(gy.ToNumpy() - ref)) <= tol(K, x, w) + 1e-6
+    # inner-dimension mismatch is rejected, not computed
+    assert lib.snhip_dot(h, gx.Pointer, M, K, 0, gw.Pointer, N, K, 0, gy.Pointer, 1.0, 0.0) == 7
+    # strided batch through snhip_bmm
+    batch, T, d = 5, 40, 24
+    Q, Kt = random_tensor(rng, (batch, T, d)), random_tensor(rng, (batch, T, d))
+    gq, gk = GPUTensor(Q.shape, Q, gpu_wrapper), GPUTensor(Kt.shape, Kt, gpu_wrapper)
+    gs = GPUTensor([batch, T, T], None, gpu_wrapper)
+    st = lib.snhip_bmm(h, gq.Pointer, T, d, 0, T * d, gk.Pointer, T, d, 1, T * d, gs.Pointer, T * T, batch, 0.125, 0.0)
+    assert st == 0
+    assert np.max(np.abs(gs.ToNumpy() - oracle.bmm(Q, False, Kt, True, 0.125))) <= tol(d, Q, Kt, 0.125)
+    # sub-matrix views with explicit leading dimensions through snhip_gemm_rm
+    big = random_tensor(rng, (90, 200), -1, 1)
+    gbig = GPUTensor(list(big.shape), big, gpu_wrapper)
+    sub_a = big[10:70, 20:120]        # 60 x 100, lda = 200
+    sub_b = big[0:50, 60:160]         # 50 x 100, ldb = 200, used transposed -> K=100, N=50
+    gout = GPUTensor([60, 64], np.zeros((60, 64), np.float32), gpu_wrapper)
+    st = lib.snhip_gemm_rm(h, 0, 1, 60, 50, 100, 1.0, gbig.Pointer + 4 * (10 * 200 + 20), 200, 0,
+                           gbig.Pointer + 4 * 60, 200, 0, 0.0, gout.Pointer, 64, 0, 1, None)
+    assert st == 0
+    got = gout.ToNumpy()
+    ref = oracle.dot(np.ascontiguousarray(sub_a), False, np.ascontiguousarray(sub_b), True)
+    assert np.max(np.abs(got[:, :50] - ref)) <= tol(100, sub_a, sub_b)
+    assert np.all(got[:, 50:] == 0)
+
+
+def test_degenerate_products(oracle, gpu_wrapper):
+    """alpha == 0 or K == 0: C = beta*C and A, B are not referenced; M or N == 0: no-op."""
+    from sharpnet_amd import GPUTensor
+    lib, h = gpu_wrapper.lib, gpu_wrapper.handle
+    rng = np.random.default_rng(7)
+    c = random_tensor(rng, (9, 11))
+    gc = GPUTensor([9, 11], c, gpu_wrapper)
+    nan = np.full((9, 5), np.nan, np.float32)
+    ga, gb = GPUTensor([9, 5], nan, gpu_wrapper), GPUTensor([5, 11], np.full((5, 11), np.nan, np.float32), gpu_wrapper)
+    gc.Dot(ga, False, gb, False, 0.0, 0.5)
+    assert np.allclose(gc.ToNumpy(), 0.5 * c, atol=1e-7)
+    gc.Dot(ga, False, gb, False, 0.0, 0.0)
+    assert np.all(gc.ToNumpy() == 0)
+    assert lib.snhip_dot(h, ga.Pointer, 0, 5, 0, gb.Pointer, 5, 11, 0, gc.Pointer, 1.0, 0.0) == 0
+    # invalid arguments come back as status codes, nothing is thrown or aborted
+    one = ctypes.c_float(1.0)
+    assert lib.snhip_sgemm(h, 5, 0, 4, 4, 4, ctypes.byref(one), ga.Pointer, 4, gb.Pointer, 4, ctypes.byref(one),
+                           gc.Pointer, 4) == 7
+    assert lib.snhip_sgemm(h, 0, 0, 4, 4, 4, ctypes.byref(one), ga.Pointer, 2, gb.Pointer, 4, ctypes.byref(one),
+                           gc.Pointer, 4) == 7
+    assert lib.snhip_sgemm(h, 0, 0, -1, 4, 4, ctypes.byref(one), ga.Pointer, 4, gb.Pointer, 4, ctypes.byref(one),
+                           gc.Pointer, 4) == 7
+
+
+def test_run_to_run_determinism(gpu_wrapper):
+    """The reference opts into deterministic cuBLAS (GPUWrapper.cs:78-80); split-K must not use float atomics."""
+    rng = np.random.default_rng(8)
+    try:
+        for (M, N, K, cfg, sk) in [(300, 200, 4096, -1, 0), (64, 64, 8192, 6, 8), (512, 512, 512, 0, 1)]:
+            gpu_wrapper.set_tuning(cfg, sk)
+            a, b = random_tensor(rng, (M, K)), random_tensor(rng, (K, N))
+            first = gpu_dot(gpu_wrapper, a, False, b, False, c_shape=[M, N])
+            for _ in range(3):
+                assert np.array_equal(first, gpu_dot(gpu_wrapper, a, False, b, False, c_shape=[M, N]))
+    finally:
+        gpu_wrapper.set_tuning(-1, 0)

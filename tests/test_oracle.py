@@ -1,0 +1,229 @@
+"""Pins the CPU oracle (oracle/dot_oracle.*) before anything is compared against it.
+
+Each check is chosen so that a plausible slip (a transposed operand, lda/ldb mixed
+up, beta applied to the product, C read when beta == 0, a wrong flatten rule)
+fails at least one of them:
+  * the reference's known answers (Tests/GPU/TestGpuTensor.cs:53-109),
+  * brute-force triple loops on tiny ragged shapes,
+  * the numpy float64 closed form on random ragged shapes,
+  * the QR identity of Tests/CPU/TestCpuTensor.cs:826-866,
+  * network-level losses the reference stores (ParallelRunWithPyTorch.cs).
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from tests.helpers import numpy_array_for_tests, y_numpy_array_for_tests, random_tensor, sigmoid
+
+
+def test_known_answers_TestDot(golden, oracle):
+    for case in golden["TestDot"]["cases"]:
+        def arr(v, shape):
+            return np.zeros(shape, np.float32) if v == "zeros" else np.array(v, np.float32).reshape(shape)
+        a = arr(case["a"], case["a_shape"])
+        b = arr(case["b"], case["b_shape"])
+        got = oracle.dot(a, False, b, False, 1, 0)
+        expected = arr(case["expected"], case["c_shape"]).reshape(got.shape)
+        assert np.max(np.abs(got - expected), initial=0.0) <= golden["TestDot"]["tolerance"]
+
+
+def _brute(a, tA, b, tB, alpha, beta, c):
+    aH, aW = a.shape
+    bH, bW = b.shape
+    M = aW if tA else aH
+    N = bH if tB else bW
+    K = aH if tA else aW
+    out = np.zeros((M, N), np.float64)
+    for m in range(M):
+        for n in range(N):
+            s = 0.0
+            for k in range(K):
+                av = a[k, m] if tA else a[m, k]
+                bv = b[n, k] if tB else b[k, n]
+                s += float(av) * float(bv)
+            out[m, n] = float(np.float32(alpha)) * s + (float(np.float32(beta)) * float(c[m, n]) if beta != 0 else 0.0)
+    return out
+
+
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_brute_force_tiny(oracle, tA, tB):
+    rng = np.random.default_rng(7)
+    for (M, N, K) in [(1, 1, 1), (3, 2, 5), (5, 7, 3), (2, 9, 4)]:
+        a = random_tensor(rng, (K, M) if tA else (M, K))
+        b = random_tensor(rng, (N, K) if tB else (K, N))
+        c = random_tensor(rng, (M, N))
+        for alpha, beta in [(1.0, 0.0), (0.25, 0.0), (-1.0, 1.0), (0.5, 1.0), (1.0, -0.75)]:
+            got = oracle.dot(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
+            ref = _brute(a, tA, b, tB, alpha, beta, c)
+            assert got.shape == (M, N)
+            assert np.max(np.abs(got - ref)) <= 2e-6 * max(1.0, np.max(np.abs(ref)))
+
+
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_closed_form_ragged(oracle, tA, tB):
+    rng = np.random.default_rng(11)
+    for (M, N, K) in [(35, 21, 124), (33, 17, 65), (8, 12, 10), (2, 2, 20000), (129, 257, 63)]:
+        a = random_tensor(rng, (K, M) if tA else (M, K))
+        b = random_tensor(rng, (N, K) if tB else (K, N))
+        c = random_tensor(rng, (M, N))
+        for alpha, beta in [(1.0, 0.0), (0.25, 0.0), (-1.0, 1.0)]:
+            got = oracle.dot(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
+            ref = oracle.dot_f64(a, tA, b, tB, alpha, beta, c)
+            # one fp32 rounding of a double-accumulated value
+            assert np.max(np.abs(got - ref)) <= 1e-6 * max(1.0, np.max(np.abs(ref)))
+
+
+def test_beta_zero_does_not_read_c(oracle):
+    # the C entry point is handed a NaN-filled destination; beta == 0 must overwrite it
+    import ctypes
+    rng = np.random.default_rng(3)
+    a, b = random_tensor(rng, (4, 6)), random_tensor(rng, (6, 5))
+    out = np.full((4, 5), np.nan, np.float32)
+    p = lambda x: x.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+    oracle._lib().oracle_dot(p(a), 4, 6, 0, p(b), 6, 5, 0, p(out), 1.0, 0.0)
+    assert np.all(np.isfinite(out))
+    assert np.allclose(out, a.astype(np.float64) @ b.astype(np.float64), atol=1e-5)
+
+
+def test_flatten_rule(oracle):
+    # operands with more than 2 dims are (Shape[0], MultDim0) matrices: Tests/GPU/TestGpuTensor.cs:84-101
+    rng = np.random.default_rng(5)
+    a = random_tensor(rng, (10, 1, 4, 7))
+    b = random_tensor(rng, (28, 3, 2))
+    got = oracle.dot(a, False, b, False)
+    assert got.shape == (10, 6)
+    assert np.allclose(got, a.reshape(10, 28).astype(np.float64) @ b.reshape(28, 6).astype(np.float64), atol=1e-5)
+
+
+def test_qr_identity(golden, oracle):
+    for case in golden["QR"]["cases"]:
+        A = np.array(case["A"], np.float32)
+        Q = np.array(case["Q"], np.float32)
+        n = A.shape[1]
+        R = oracle.dot(Q, True, A, False)           # TN, as QRFactorization's tail does (CpuTensor.cs:3078)
+        assert R.shape == (n, n)
+        assert np.max(np.abs(np.tril(R, -1))) < 1e-4   # upper triangular
+        QR = oracle.dot(Q, False, R, False)         # NN
+        assert np.max(np.abs(QR - A)) < 1e-4
+        QtQ = oracle.dot(Q, True, Q, False)         # A == B aliasing
+        assert np.max(np.abs(QtQ - np.eye(n))) < 1e-6
+
+
+def test_bmm_is_loop_of_dot(oracle):
+    rng = np.random.default_rng(13)
+    batch, L, d = 3, 12, 7   # Tests/TestParallelRunCpuVersusGpu.cs:377-401
+    dy, V = random_tensor(rng, (batch, L, d)), random_tensor(rng, (batch, L, d))
+    S = random_tensor(rng, (batch, L, L))
+    for (a, tA, b, tB, alpha) in [(dy, False, V, True, 0.25), (S, False, V, False, 1.0), (S, True, V, False, 1.0)]:
+        got = oracle.bmm(a, tA, b, tB, alpha, 0.0)
+        for i in range(batch):
+            ref = oracle.dot_f64(a[i], tA, b[i], tB, alpha)
+            assert np.max(np.abs(got[i] - ref)) <= 1e-6 * max(1.0, np.max(np.abs(ref)))
+
+
+def test_sgemm_colmajor_identity(oracle):
+    # column-major C(m x n) = op(A) op(B)  <=>  row-major C^T = op(B)^T op(A)^T on the same buffers
+    rng = np.random.default_rng(17)
+    m, n, k = 5, 7, 9
+    for ta, tb in itertools.product([0, 1], repeat=2):
+        lda = (k if ta else m) + 2
+        ldb = (n if tb else k) + 1
+        ldc = m + 3
+        A = random_tensor(rng, ((m if ta else k), lda))   # row-major view: ld is the row pitch
+        B = random_tensor(rng, ((k if tb else n), ldb))
+        C = random_tensor(rng, (n, ldc))
+        out = oracle.sgemm_colmajor(ta, tb, m, n, k, 0.5, A, lda, B, ldb, -1.0, C, ldc).reshape(n, ldc)
+        Acm = A[:, :(k if ta else m)].T.astype(np.float64)   # column-major matrix = transpose of the row-major view
+        Bcm = B[:, :(n if tb else k)].T.astype(np.float64)
+        opA = Acm.T if ta else Acm
+        opB = Bcm.T if tb else Bcm
+        ref = 0.5 * (opA @ opB) - C[:, :m].T.astype(np.float64)
+        assert np.max(np.abs(out[:, :m].T - ref)) < 1e-5
+        assert np.array_equal(out[:, m:], C[:, m:])          # padding untouched
+
+
+def test_linear_sigmoid_predictions(golden, oracle):
+    fx = golden["Linear_1_1_1_1"]
+    x = np.array(fx["x"], np.float32)
+    w_in_out = np.array(fx["w"], np.float32)                  # (in=1, out=2); layout-independent for 1x1 input
+    y = oracle.dense_forward(x, w_in_out.T.copy())
+    assert np.max(np.abs(sigmoid(y) - np.array(fx["sigmoid_prediction"]))) < fx["tolerance"]
+
+    fx = golden["Linear_1_1_4_4"]
+    x = np.array(fx["x"], np.float32)                          # (1,1,4,4)
+    w_in_out = np.array(fx["w_in_out"], np.float32)            # (16, 3)
+    y_nn = oracle.dot(x, False, w_in_out, False)               # NN reading of the stored literal
+    assert np.max(np.abs(sigmoid(y_nn) - np.array(fx["sigmoid_prediction"]))) < 2e-6
+    y_nt = oracle.dense_forward(x, np.ascontiguousarray(w_in_out.T))   # same numbers through the NT path
+    assert np.max(np.abs(y_nn - y_nt)) < 1e-6
+
+
+def test_dense_chain_losses(golden, oracle):
+    """Two Linear layers trained for 10 epochs reproduce the stored losses
+    (Tests/NonReg/ParallelRunWithPyTorch.cs:102-138): pins NT forward, TN dW, NN dx, bias gradient."""
+    fx = golden["PyTorch_Mse"]
+    X = numpy_array_for_tests(*fx["x_shape"])
+    Y = y_numpy_array_for_tests(*fx["y_shape"])
+    W1 = np.array(fx["linear1_weight_out_in"], np.float32)
+    W2 = np.array(fx["linear2_weight_out_in"], np.float32)
+    b1 = np.zeros(W1.shape[0], np.float32)
+    b2 = np.zeros(W2.shape[0], np.float32)
+    params = [W1, b1, W2, b2]
+    vel = [np.zeros_like(p) for p in params]
+
+    def forward():
+        h = oracle.dense_forward(X, params[0], params[1], flatten_last=True)    # (24, 3)
+        r = np.maximum(h, 0)
+        f = r.reshape(X.shape[0], -1)                                            # Flatten -> (2, 36)
+        out = oracle.dense_forward(f, params[2], params[3])
+        return h, r, f, out
+
+    def mse(out):
+        return float(np.mean((out.astype(np.float64) - Y) ** 2))
+
+    loss_before = mse(forward()[3])
+    assert abs(loss_before - fx["loss_before"]) < fx["tolerance"]
+    for _ in range(fx["epochs"]):
+        h, r, f, out = forward()
+        dout = (2.0 * (out - Y) / out.size).astype(np.float32)
+        dW2, db2, df = oracle.dense_backward(f, dout, params[2])
+        dr = df.reshape(r.shape)
+        dh = (dr * (h > 0)).astype(np.float32)
+        dW1, db1, _ = oracle.dense_backward(X, dh, params[0], prev_is_input=True, flatten_last=True)
+        for i, g in enumerate([dW1, db1, dW2, db2]):
+            vel[i] = (fx["momentum"] * vel[i] + g).astype(np.float32)
+            params[i] = (params[i] - fx["lr"] * vel[i]).astype(np.float32)
+    loss_after = mse(forward()[3])
+    assert abs(loss_after - fx["loss_after"]) < fx["tolerance"]
+
+
+def test_attention_chain_losses(golden, oracle):
+    """loss_before of Test_DotProductAttention (ParallelRunWithPyTorch.cs:963-1010): batched NT -> softmax -> NN."""
+    fx = golden["PyTorch_DotProductAttention"]
+    X = numpy_array_for_tests(*fx["x_shape"])                  # (6, 4, 5) = (N, C, L)
+    Y = y_numpy_array_for_tests(*fx["y_shape"])
+    Wq, Wk, Wv = [np.array(fx[k], np.float32)[:, :, 0] for k in ("conv_q", "conv_k", "conv_v")]   # (2, 4)
+    Wd = np.array(fx["dense_weight_out_in"], np.float32)      # (3, 10)
+    conv = lambda W: np.stack([oracle.dot(W, False, X[n], False) for n in range(X.shape[0])])    # (6, 2, 5)
+    Q, K, V = conv(Wq), conv(Wk), conv(Wv)
+    for case in fx["cases"]:
+        y, _ = oracle.sdpa_forward(Q, K, V, use_scale=False, is_causal=case["is_causal"])
+        logits = oracle.dense_forward(y.reshape(X.shape[0], -1), Wd)
+        p = oracle.softmax_last_dim(logits).astype(np.float64)
+        loss = float(np.mean(-np.sum(Y * np.log(p), axis=1)))
+        assert abs(loss - case["loss_before"]) < 2e-6, (case, loss)
+
+
+def test_mkl_route_matches_closed_form(oracle):
+    """The baseline route (the cblas_sgemm call of BlasServices.cs:20) agrees with float64 within the fp32 bound."""
+    rng = np.random.default_rng(19)
+    for tA, tB in itertools.product([False, True], repeat=2):
+        M, N, K = 65, 47, 130
+        a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
+        b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
+        c = random_tensor(rng, (M, N), -1, 1)
+        out = c.copy()
+        oracle.mkl_dot(a, tA, b, tB, out, alpha=0.5, beta=1.0)
+        ref = oracle.dot_f64(a, tA, b, tB, 0.5, 1.0, c)
+        assert np.max(np.abs(out - ref)) <= oracle.tolerance(K, a, b)
