@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Benchmark of the Tensor.Dot hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+A "step" is one Tensor.Dot of the headline workload: fp32, M = N = K = 8192,
+no transposes, alpha = 1, beta = 0, A and B ~ U(-1, 1) (seeded), operands resident
+in HBM before the timed region.  Prints ONE JSON line on stdout:
+  value      TFLOP/s = 2*M*N*K / (wall time of K steps / K), device synchronised on both sides;
+  roofline   the same algorithmic flops over the kernel's average launch duration measured with
+             HIP events on the stream the kernel runs on, against the 157.3 TFLOP/s fp32 MFMA peak;
+  cpu_baseline  the reference's CPU route (MKL cblas_sgemm RowMajor, the call of
+             Prod/Data/BlasServices.cs:20) timed on this box's host cores on a bounded sample;
+  extra      GPU TFLOP/s and roofline fraction of the other benchmark configurations
+             (dense layer, sweep, MLP step, LSTM projections, attention matmuls).
+Everything but the JSON line goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
+    ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--probe", action="store_true",
+                    help="counter-collection mode for rocprofv3 --pmc: 3 plain copies of 1 GiB, then 3 headline GEMMs")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on ONE GPU only (no collectives, no sharding); run with --gpus 1")
+
+    from sharpnet_amd import GPUWrapper, GPUTensor, workloads as wl
+    w = GPUWrapper.FromDeviceId(0)
+    info = w.device_info()
+    log("[bench] device:", info)
+
+    def upload(arr):
+        return GPUTensor(arr.shape, arr, w)
+
+    def time_gemm(g, a, b, c, steps, warmup, bias=None):
+        """Returns (wall ms/step, event ms/launch, GPUTensor C)."""
+        ga, gb = upload(a), upload(b)
+        gc = upload(c) if c is not None else GPUTensor(g.c_shape, None, w)
+        gbias = upload(bias) if bias is not None else None
+
+        def launch():
+            if g.batch > 1:
+                gc.BatchMatrixMultiplication(ga, g.tA, gb, g.tB, g.alpha, g.beta)
+            elif gbias is not None:
+                gc.DotRowMajor(ga, g.tA, gb, g.tB, g.alpha, g.beta, bias=gbias)
+            else:
+                gc.Dot(ga, g.tA, gb, g.tB, g.alpha, g.beta)
+        for _ in range(warmup):
+            launch()
+        e0, e1 = w.new_event(), w.new_event()
+        w.synchronize()
+        t0 = time.perf_counter()
+        w.record(e0)
+        for _ in range(steps):
+            launch()
+        w.record(e1)
+        w.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        ev_ms = w.elapsed_ms(e0, e1) / steps
+        w.destroy_event(e0)
+        w.destroy_event(e1)
+        ga.Dispose()
+        gb.Dispose()
+        if gbias is not None:
+            gbias.Dispose()
+        return wall_ms, ev_ms, gc
+
+    if args.probe:
+        # known-size launch: copy_f32_kernel reads 2**30 bytes and writes 2**30 bytes
+        n = 1 << 28
+        src, dst = GPUTensor([n], None, w), GPUTensor([n], None, w)
+        src.SetValue(1.0)
+        for _ in range(3):
+            from sharpnet_amd.hiplib import check_status
+            check_status(w.lib.snhip_copy_f32(w.handle, dst.Pointer, src.Pointer, n), "snhip_copy_f32")
+        w.synchronize()
+        src.Dispose()
+        dst.Dispose()
+        g = wl.HEADLINE
+        a, b, _ = wl.uniform_operands(g, seed=2)
+        _, ev_ms, gc = time_gemm(g, a, b, None, 3, 0)
+        log("[bench] probe: 3 x copy of 2^30 bytes, 3 x %s at %.3f ms" % (g.label(), ev_ms))
+        return
+
+    # ------------------------------------------------------------------ headline
+    g = wl.HEADLINE
+    a, b, _ = wl.uniform_operands(g, seed=2)
+    wall_ms, ev_ms, gc = time_gemm(g, a, b, None, args.steps, args.warmup)
+    cfg, splitk = w.last_tuning()
+    tflops = g.flops / (wall_ms * 1e-3) / 1e12
+    achieved = g.flops / (ev_ms * 1e-3) / 1e12
+    log("[bench] headline %s: wall %.3f ms/step, events %.3f ms/launch, %.1f TFLOP/s, tile config %d split-K %d"
+        % (g.label(), wall_ms, ev_ms, tflops, cfg, splitk))
+
+    # parity of the timed configuration: sampled rows and columns against the oracle
+    from oracle import dot_oracle
+    rng = np.random.default_rng(99)
+    rows = np.sort(rng.choice(g.M, 16, replace=False))
+    got = gc.ToNumpy()[rows]
+    ref = dot_oracle.dot(np.ascontiguousarray(a[rows]), False, b, False)
+    err = float(np.max(np.abs(got - ref)))
+    bound = dot_oracle.tolerance(g.K, a, b)
+    log("[bench] parity of the timed result (16 sampled rows): max|d| = %.3e, bound %.3e" % (err, bound))
+    if not err <= bound:
+        sys.exit("bench.py: timed result is outside the parity bound")
+    gc.Dispose()
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "sgemm_8192_hbm_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+
+    out = {
+        "metric": "fp32 GEMM throughput, Tensor.Dot M=N=K=8192 (GEMM TFLOP/s + % of fp32 MFMA peak at 1 GPU)",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1] sweep, headline size: Tensor.Dot fp32 row-major NN, M=N=K=8192, alpha=1, "
+                               "beta=0, A,B~U(-1,1) seed 2, operands resident in HBM",
+                   "M": g.M, "N": g.N, "K": g.K, "tile_config": cfg, "splitk": splitk,
+                   "device": {"cu": info["compute_units"], "clock_mhz": info["clock_khz"] / 1000.0}},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": wl.FP32_MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / wl.FP32_MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
+                     "flops_per_launch": g.flops, "ms_per_launch_hip_events": round(ev_ms, 4)},
+        "parity": {"max_abs_err": err, "bound": bound, "rows_checked": 16},
+    }
+
+    # ------------------------------------------------------------------ CPU baseline (bounded sample)
+    if not args.no_cpu:
+        cores = dot_oracle.mkl_threads()
+        cpu_out = np.empty((g.M, g.N), np.float32)
+        route = dot_oracle.mkl_dot(a, False, b, False, cpu_out)          # warm-up, also the full-size oracle
+        ts = []
+        for _ in range(args.cpu_reps):
+            t0 = time.perf_counter()
+            dot_oracle.mkl_dot(a, False, b, False, cpu_out)
+            ts.append(time.perf_counter() - t0)
+        cpu_s = float(np.median(ts))
+        out["cpu_baseline"] = {
+            "value": round(g.flops / cpu_s / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": "%d timed + 1 warm-up calls of the full headline GEMM (8192^3) through %s, "
+                      "median %.2f s per call; os.cpu_count()=%d" % (args.cpu_reps, route, cpu_s, os.cpu_count()),
+        }
+        log("[bench] cpu baseline:", out["cpu_baseline"])
+        del cpu_out
+    del a, b
+
+    # ------------------------------------------------------------------ the other configurations (GPU side)
+    if not args.no_extra:
+        extra = {}
+
+        def run(gm, seed, steps=10, warmup=3, bias=None):
+            aa, bb, cc = wl.uniform_operands(gm, seed)
+            _, ms, gcx = time_gemm(gm, aa, bb, cc, steps, warmup, bias=bias)
+            gcx.Dispose()
+            tf = gm.flops / (ms * 1e-3) / 1e12
+            return {"gemm": gm.label(), "ms": round(ms, 4), "tflops": round(tf, 2),
+                    "frac_of_roofline": round(gm.roofline_seconds() * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
+                    "splitk": w.last_tuning()[1]}
+
+        extra["config1_dense_layer"] = [run(gm, 1, 50, 10, bias=np.zeros(gm.N, np.float32) if gm.bias else None)
+                                        for gm in wl.dense_layer_gemms()]
+        sweep = []
+        for (M, N, K) in wl.SWEEP_SIZES:
+            for tA in (False, True):
+                for tB in (False, True):
+                    steps = 5 if M * N * K > 1e11 else 20
+                    sweep.append(run(wl.Gemm(M, N, K, tA, tB, 1.0, 0.0), 2, steps, 2))
+            sweep.append(run(wl.Gemm(M, N, K, False, False, 1.0, 1.0), 2, 5, 2))
+        extra["config2_sweep"] = sweep
+        mlp = [run(gm, 3, 5, 2, bias=np.zeros(gm.N, np.float32) if gm.bias else None) for gm in wl.mlp_gemms()]
+        extra["config3_mlp_step"] = {"gemms": mlp, "total_ms": round(sum(r["ms"] for r in mlp), 4),
+                                     "tflops": round(sum(gm.flops for gm in wl.mlp_gemms()) /
+                                                     (sum(r["ms"] for r in mlp) * 1e-3) / 1e12, 2)}
+        proj, rec, seq = wl.lstm_gemms()
+        extra["config4_lstm"] = {"input_projection": run(proj, 4, 10, 2), "recurrent_step": run(rec, 4, seq, 10),
+                                 "recurrent_steps": seq}
+        extra["config5_attention_fp32"] = [run(gm, 5, 20, 3) for gm in wl.attention_gemms()]
+        out["extra"] = extra
+        for k, v in extra.items():
+            log("[bench]", k, json.dumps(v))
+
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -117,6 +117,10 @@ int snhip_event_destroy(void* event);
 int snhip_event_record(void* handle, void* event);
 int snhip_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for stop */
 
+/* Plain copy kernel of `count` floats on the handle's stream: the known-size
+ * launch that rocprof traffic counters (FETCH_SIZE / WRITE_SIZE) are scaled by. */
+int snhip_copy_f32(void* handle, void* dst, const void* src, long long count);
+
 /* Device facts: info[0]=compute units, [1]=max engine clock kHz, [2]=memory
  * clock kHz, [3]=memory bus width bits, [4]=LDS bytes per workgroup (opt-in max),
  * [5]=gfx architecture number (950 for MI355X). */

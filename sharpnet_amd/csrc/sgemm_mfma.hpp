@@ -37,6 +37,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace snhip {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -99,51 +101,63 @@ struct TileStage {
     __device__ __forceinline__ void advance() { gptr += KCONTIG ? (long long)BK : (long long)BK * ld; }
 
     // Unchecked load: every element of the tile is inside the matrix.
+    __device__ __forceinline__ void load_fast_vec(f32x4& r, int v) const {
+        const float* p = gptr + (long long)(v * LINE_STEP) * ld;
+        __builtin_memcpy(&r, p, 16);
+    }
+
     __device__ __forceinline__ void load_fast(f32x4 (&r)[NV]) const {
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const float* p = gptr + (long long)(v * LINE_STEP) * ld;
-            __builtin_memcpy(&r[v], p, 16);
-        }
+        for (int v = 0; v < NV; ++v) load_fast_vec(r[v], v);
     }
 
     // Checked load: elements with m/n >= mn_rem or k >= k_rem read as zero
-    // (mn_rem, k_rem are counted from the tile origin).
-    __device__ __forceinline__ void load_safe(f32x4 (&r)[NV], int mn_rem, int k_rem) const {
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const float* p = gptr + (long long)(v * LINE_STEP) * ld;
-            int nval;
-            if (KCONTIG) {
-                const int mn = mn0 + v * LINE_STEP;
-                nval = (mn < mn_rem) ? (k_rem - k0) : 0;
-            } else {
-                const int k = k0 + v * LINE_STEP;
-                nval = (k < k_rem) ? (mn_rem - mn0) : 0;
-            }
-            f32x4 x;
+    // (mn_rem, k_rem are counted from the tile origin) and touch no memory.
+    __device__ __forceinline__ void load_safe_vec(f32x4& r, int v, int mn_rem, int k_rem) const {
+        const float* p = gptr + (long long)(v * LINE_STEP) * ld;
+        int nval;
+        if (KCONTIG) {
+            const int mn = mn0 + v * LINE_STEP;
+            nval = (mn < mn_rem) ? (k_rem - k0) : 0;
+        } else {
+            const int k = k0 + v * LINE_STEP;
+            nval = (k < k_rem) ? (mn_rem - mn0) : 0;
+        }
+        f32x4 x;
+        if (nval >= 4) {
+            // whole vector inside the matrix: the common case even in edge tiles
+            __builtin_memcpy(&x, p, 16);
+        } else {
             x.x = (nval > 0) ? p[0] : 0.0f;
             x.y = (nval > 1) ? p[1] : 0.0f;
             x.z = (nval > 2) ? p[2] : 0.0f;
-            x.w = (nval > 3) ? p[3] : 0.0f;
-            r[v] = x;
+            x.w = 0.0f;
+        }
+        r = x;
+    }
+
+    __device__ __forceinline__ void load_safe(f32x4 (&r)[NV], int mn_rem, int k_rem) const {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) load_safe_vec(r[v], v, mn_rem, k_rem);
+    }
+
+    // vector v of this thread -> its place in the k-major LDS tile
+    __device__ __forceinline__ void store_lds_vec(float* s, const f32x4& r, int v) const {
+        if (KCONTIG) {
+            float* d = s + k0 * PITCH + (mn0 + v * LINE_STEP);
+            d[0 * PITCH] = r.x;
+            d[1 * PITCH] = r.y;
+            d[2 * PITCH] = r.z;
+            d[3 * PITCH] = r.w;
+        } else {
+            float* d = s + (k0 + v * LINE_STEP) * PITCH + mn0;
+            *reinterpret_cast<f32x4*>(d) = r;
         }
     }
 
     __device__ __forceinline__ void store_lds(float* s, const f32x4 (&r)[NV]) const {
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            if (KCONTIG) {
-                float* d = s + k0 * PITCH + (mn0 + v * LINE_STEP);
-                d[0 * PITCH] = r[v].x;
-                d[1 * PITCH] = r[v].y;
-                d[2 * PITCH] = r[v].z;
-                d[3 * PITCH] = r[v].w;
-            } else {
-                float* d = s + (k0 + v * LINE_STEP) * PITCH + mn0;
-                *reinterpret_cast<f32x4*>(d) = r[v];
-            }
-        }
+        for (int v = 0; v < NV; ++v) store_lds_vec(s, r[v], v);
     }
 };
 
@@ -174,6 +188,28 @@ struct Frag<4> {
         v[3] = t.w;
     }
 };
+
+// Element r of an accumulator tile.  With many tiles per wavefront the
+// accumulators live in AGPRs; reading them one by one where they are consumed
+// (instead of letting the compiler copy all of them to VGPRs when the k loop
+// ends) keeps the epilogue's register footprint small.
+__device__ __forceinline__ float acc_element(const f32x16& t, int r, bool from_agpr) {
+    float x;
+    if (from_agpr) {
+        asm("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(t[r]));
+    } else {
+        x = t[r];
+    }
+    return x;
+}
+
+// Workgroup barrier that orders LDS traffic only: global loads that are still in
+// flight (the register prefetch) must not be waited for here.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  Remap the id
 // so that each XCD (which has a private L2) works on a contiguous range of
@@ -243,7 +279,6 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     sa.init(Ab, p.lda, m0, kbeg, tid);
     sb.init(Bb, p.ldb, n0, kbeg, tid);
 
-    f32x4 ra[StageA::NV], rb[StageB::NV];
     f32x16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -252,71 +287,145 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    auto load_tile = [&](int kt) {
-        if (full_mn && kt < nk_full) {
-            sa.load_fast(ra);
-            sb.load_fast(rb);
-        } else {
-            const int k_rem = klen - kt * BK;
-            sa.load_safe(ra, m_rem, k_rem);
-            sb.load_safe(rb, n_rem, k_rem);
-        }
-        sa.advance();
-        sb.advance();
-    };
-
-    if (nk > 0) {
-        load_tile(0);
-        sa.store_lds(As, ra);
-        sb.store_lds(Bs, rb);
-        __syncthreads();
-    }
-
     const int a_off = wm * (TM * 32) + l32 * TM;
     const int b_off = wn * (TN * 32) + l32 * TN;
+    constexpr int KS = BK / 2;                   // MFMA k steps per tile
+    constexpr int NP = StageA::NV + StageB::NV;  // LDS store pieces per tile
 
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        const bool has_next = (kt + 1 < nk);
-        if (has_next) load_tile(kt + 1);
+    // Two register stages per operand: while tile kt is multiplied out of LDS,
+    // tile kt+1 sits in registers and is written to the other LDS buffer in small
+    // pieces between MFMAs, and tile kt+2 is in flight from global memory.  Each
+    // piece's registers are refilled with tile kt+3 right after they have been
+    // stored, so a global load has two full tiles of MFMA work to land.
+    //
+    // The k loop is one straight-line body of two tiles with no special cases:
+    // tiles at or beyond the end of K are fetched as zeros (no memory access), so
+    // an odd tile count simply multiplies one tile of zeros.
+    f32x4 ra[2][StageA::NV], rb[2][StageB::NV];
+    int fetch = 0;  // index of the k tile the stage pointers address; tiles are fetched in order
 
-        const float* as = As + cur * (BK * PA) + lhi * PA + a_off;
-        const float* bs = Bs + cur * (BK * PB) + lhi * PB + b_off;
+    // MFMA operand fragments, double-buffered over k steps; they live across k
+    // tiles because the first fragments of tile kt+1 are read at the end of tile kt.
+    Frag<TM> fa[2];
+    Frag<TN> fb[2];
+    const float* const a_rd = As + lhi * PA + a_off;
+    const float* const b_rd = Bs + lhi * PB + b_off;
 
-        Frag<TM> fa[2];
-        Frag<TN> fb[2];
-        fa[0].load(as);
-        fb[0].load(bs);
+    {
+        // prologue: tile 0 -> LDS buffer 0, tile 1 -> stage 1, tile 2 -> stage 0
 #pragma unroll
-        for (int s = 0; s < BK / 2; ++s) {
-            // Issue the LDS reads of the next k step right behind the first MFMA of
-            // this one, so their latency is covered by the remaining MFMAs.  The
-            // scheduling fences keep the compiler from sinking them to the end.
+        for (int t = 0; t < 3; ++t) {
+            const int st = (t == 1) ? 1 : 0;
+            const int k_rem = klen - fetch * BK;
+            if (full_mn && fetch < nk_full) {
+                sa.load_fast(ra[st]);
+                sb.load_fast(rb[st]);
+            } else {
+                sa.load_safe(ra[st], m_rem, k_rem);
+                sb.load_safe(rb[st], n_rem, k_rem);
+            }
+            sa.advance();
+            sb.advance();
+            ++fetch;
+            if (t == 0) {
+                sa.store_lds(As, ra[0]);
+                sb.store_lds(Bs, rb[0]);
+            }
+        }
+        lds_barrier();
+        fa[0].load(a_rd);
+        fb[0].load(b_rd);
+    }
+
+    static_assert(KS % 2 == 0, "fragment double-buffering across tiles needs an even number of k steps");
+    constexpr int KSW = (KS > 1) ? KS - 1 : 1;  // k steps that carry LDS stores (the last one carries the barrier)
+    constexpr int MID = (TM * TN) / 2;          // MFMA index of the last k step behind which the barrier sits
+
+    // One k tile.  P selects the LDS buffer read; the register stage P^1 holds the
+    // next tile and is refilled, piece by piece, with tile `fetch`.
+    auto k_tile = [&](auto parity, auto steady) {
+        constexpr int P = decltype(parity)::value;
+        constexpr int Q = P ^ 1;
+        // STEADY: the caller guarantees that tile `fetch` is a full tile of an interior block
+        const bool fast = decltype(steady)::value || (full_mn && (fetch < nk_full));
+        const int k_rem = klen - fetch * BK;
+        const float* as = a_rd + P * (BK * PA);
+        const float* bs = b_rd + P * (BK * PB);
+        float* const as_next = As + Q * (BK * PA);
+        float* const bs_next = Bs + Q * (BK * PB);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1].v[i], fb[s & 1].v[j], acc[i][j], 0, 0, 0);
-                    if (i == 0 && j == 0 && s + 1 < BK / 2) {
+                    if (i == 0 && j == 0) {
+                        // Everything that is not an MFMA is issued right behind the first
+                        // MFMA of a k step and completes under the remaining ones: the LDS
+                        // reads of the next step and this step's share of the LDS stores,
+                        // each followed by the global load that refills its registers.
                         __builtin_amdgcn_sched_barrier(0);
-                        fa[(s + 1) & 1].load(as + (2 * (s + 1)) * PA);
-                        fb[(s + 1) & 1].load(bs + (2 * (s + 1)) * PB);
+                        if (s + 1 < KS) {
+                            fa[(s + 1) & 1].load(as + (2 * (s + 1)) * PA);
+                            fb[(s + 1) & 1].load(bs + (2 * (s + 1)) * PB);
+                        }
+                        if (s < KSW) {
+#pragma unroll
+                            for (int q = (s * NP) / KSW; q < ((s + 1) * NP) / KSW; ++q) {
+                                if (q < StageA::NV) {
+                                    const int v = q < StageA::NV ? q : 0;
+                                    sa.store_lds_vec(as_next, ra[Q][v], v);
+                                    if (fast)
+                                        sa.load_fast_vec(ra[Q][v], v);
+                                    else
+                                        sa.load_safe_vec(ra[Q][v], v, m_rem, k_rem);
+                                } else {
+                                    const int v = q >= StageA::NV ? q - StageA::NV : 0;
+                                    sb.store_lds_vec(bs_next, rb[Q][v], v);
+                                    if (fast)
+                                        sb.load_fast_vec(rb[Q][v], v);
+                                    else
+                                        sb.load_safe_vec(rb[Q][v], v, n_rem, k_rem);
+                                }
+                            }
+                        }
+                        if (s + 1 == KS) {
+                            sa.advance();
+                            sb.advance();
+                            ++fetch;
+                        }
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    // The prefetched tile goes to the other LDS buffer behind the first
-                    // MFMA of the last k step; the rest of that step covers the writes.
-                    if (i == 0 && j == 0 && s + 1 == BK / 2) {
+                    if (s + 1 == KS && i * TN + j == MID) {
+                        // Half way through the last k step: the stores of the next tile were
+                        // issued a whole k step ago, so the barrier finds them complete, and
+                        // the first fragments of the next tile are read under the remaining MFMAs.
                         __builtin_amdgcn_sched_barrier(0);
-                        if (has_next) {
-                            sa.store_lds(As + (cur ^ 1) * (BK * PA), ra);
-                            sb.store_lds(Bs + (cur ^ 1) * (BK * PB), rb);
-                        }
+                        lds_barrier();
+                        fa[0].load(a_rd + Q * (BK * PA));
+                        fb[0].load(b_rd + Q * (BK * PB));
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }
         }
-        __syncthreads();
+    };
+
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
+    int kt = 0;
+    if (full_mn) {
+        // interior blocks: branch-free pairs of tiles while both fetches (tiles kt+3, kt+4) are full tiles
+        for (; kt + 4 < nk_full; kt += 2) {
+            k_tile(P0{}, std::true_type{});
+            k_tile(P1{}, std::true_type{});
+        }
+    }
+    // edge blocks and the last few tiles: same body, each fetch chooses checked or unchecked loads
+    for (; kt < nk; kt += 2) {
+        k_tile(P0{}, std::false_type{});
+        k_tile(P1{}, std::false_type{});
     }
 
     // ---------------- epilogue ----------------
@@ -343,6 +452,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         beta = p.beta;
         bias = p.bias;
     }
+    constexpr bool BIG_ACC = false;
     const bool vec_ok = (TN == 4) && (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
 
     float bv[TN];
@@ -358,7 +468,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             float* crow = out + (long long)row * ldo + col0;
             float v[TN];
 #pragma unroll
-            for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r] + bv[j];
+            for (int j = 0; j < TN; ++j) v[j] = alpha * acc_element(acc[i][j], r, BIG_ACC) + bv[j];
             if (vec_ok) {
                 if constexpr (TN == 4) {
                     f32x4 o = {v[0], v[1], v[2], v[3]};
@@ -420,6 +530,24 @@ __global__ void __launch_bounds__(256) scale_c_kernel(float* C, const float* __r
         float o = (beta != 0.0f) ? beta * *c : 0.0f;
         if (bias != nullptr) o += bias[col];
         *c = o;
+    }
+}
+
+// Plain device-to-device copy of `count` floats (16-byte vectors when both
+// pointers allow it).  Exists as the known-size reference launch against which
+// hardware traffic counters are scaled; it is not on the GEMM path.
+__global__ void __launch_bounds__(256) copy_f32_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                       long long count, int vec) {
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec) {
+        const long long n4 = count / 4;
+        const f32x4* s4 = reinterpret_cast<const f32x4*>(src);
+        f32x4* d4 = reinterpret_cast<f32x4*>(dst);
+        for (long long j = i; j < n4; j += stride) d4[j] = s4[j];
+        for (long long j = n4 * 4 + i; j < count; j += stride) dst[j] = src[j];
+    } else {
+        for (; i < count; i += stride) dst[i] = src[i];
     }
 }
 

@@ -63,6 +63,10 @@ const ConfigEntry kConfigs[] = {
     make_entry<TileCfg<1, 2, 2, 2, 16>>(),  // 4: 64 x 128
     make_entry<TileCfg<2, 1, 2, 2, 16>>(),  // 5: 128 x 64
     make_entry<TileCfg<1, 1, 2, 2, 16>>(),  // 6: 64 x 64
+    make_entry<TileCfg<4, 4, 2, 2, 32>>(),  // 7: 256 x 256, BK 32
+    make_entry<TileCfg<2, 2, 2, 2, 32>>(),  // 8: 128 x 128, BK 32
+    make_entry<TileCfg<2, 1, 2, 2, 32>>(),  // 9: 128 x 64, BK 32
+    make_entry<TileCfg<1, 1, 2, 2, 32>>(),  // 10: 64 x 64, BK 32
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -96,7 +100,7 @@ struct Choice {
 // re-read operands more often and expose more latency, modelled by a
 // per-configuration efficiency.  Split-K adds a second pass over M*N*splitk.
 double estimate_cycles(const ConfigEntry& c, int cfg_id, int M, int N, int K, int batch, int splitk, int num_cu) {
-    static const double eff[kNumConfigs] = {0.92, 0.85, 0.85, 0.75, 0.6, 0.6, 0.45};
+    static const double eff[kNumConfigs] = {0.92, 0.85, 0.85, 0.75, 0.6, 0.6, 0.45, 0.5, 0.5, 0.5, 0.5};
     const long long tiles = (long long)ceil_div(M, c.BM) * ceil_div(N, c.BN) * batch * splitk;
     const long long rounds = (tiles + num_cu - 1) / num_cu;
     const int kchunk = ceil_div(ceil_div(K, splitk), c.BK) * c.BK;
@@ -449,6 +453,20 @@ int snhip_event_elapsed_ms(void* start, void* stop, float* ms) {
     hipError_t e = hipEventSynchronize(static_cast<hipEvent_t>(stop));
     if (e != hipSuccess) return hip_to_status(e);
     return hip_to_status(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+}
+
+int snhip_copy_f32(void* handle, void* dst, const void* src, long long count) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (count < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (count == 0) return SNHIP_STATUS_SUCCESS;
+    if (dst == nullptr || src == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    Handle* h = static_cast<Handle*>(handle);
+    const int vec = ((uintptr_t)dst % 16 == 0 && (uintptr_t)src % 16 == 0) ? 1 : 0;
+    const long long work = vec ? (count + 3) / 4 : count;
+    const int blocks = (int)((work + 255) / 256 < 16384 ? (work + 255) / 256 : 16384);
+    hipLaunchKernelGGL(copy_f32_kernel, dim3(blocks), dim3(256), 0, h->stream, static_cast<const float*>(src),
+                       static_cast<float*>(dst), count, vec);
+    return hip_to_status(hipGetLastError());
 }
 
 int snhip_device_info(void* handle, int info[6]) {

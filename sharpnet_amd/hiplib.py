@@ -80,6 +80,7 @@ SIGNATURES = {
     "snhip_event_destroy": [_vp],
     "snhip_event_record": [_vp, _vp],
     "snhip_event_elapsed_ms": [_vp, _vp, _c_float_p],
+    "snhip_copy_f32": [_vp, _vp, _vp, _ll],
     "snhip_device_info": [_vp, _c_int_p],
     "snhip_set_tuning": [_vp, _i, _i],
     "snhip_get_last_tuning": [_vp, _c_int_p, _c_int_p],
