@@ -97,6 +97,23 @@ int snhip_gemm_rm(void* handle, int transposeA, int transposeB, int M, int N, in
                   int lda, long long strideA, const float* B, int ldb, long long strideB, float beta, float* C,
                   int ldc, long long strideC, int batch, const float* bias);
 
+/* ---- bf16-input / fp32-accumulate variant (no reference counterpart) ------ */
+/* Operands stay fp32 in device memory; they are rounded to bf16 (nearest even)
+ * on their way into LDS and multiplied with v_mfma_f32_32x32x16_bf16, products
+ * accumulated in fp32, C is fp32.  Expected deviation from the fp32 result:
+ * <= 1e-2 * max|C|.  The reference has only the fp32 SGEMM (GpuTensor.cs:1218). */
+#define SNHIP_MATH_FP32 0
+#define SNHIP_MATH_BF16_INPUT 1
+/* Selects the arithmetic used by every GEMM entry point of this handle
+ * (the role cublasSetMathMode plays for cuBLAS handles). Default SNHIP_MATH_FP32. */
+int snhip_set_math_mode(void* handle, int mode);
+/* snhip_dot_bias / snhip_bmm in bf16-input arithmetic regardless of the handle's mode. */
+int snhip_dot_bf16(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
+                   int transposeB, float* C, float alpha, float beta, const float* bias);
+int snhip_bmm_bf16(void* handle, const float* A, int aH, int aW, int transposeA, long long strideA, const float* B,
+                   int bH, int bW, int transposeB, long long strideB, float* C, long long strideC, int batch,
+                   float alpha, float beta);
+
 /* ---- device memory / stream shims --------------------------------------- */
 /* Replace the nvcuda calls GPUTensor makes: cuMemAlloc_v2 (GpuTensor.cs:41),
  * cuMemFree_v2 (:1634), cuMemsetD32 (:1583), cuMemcpyHtoDAsync (:77),
@@ -132,8 +149,8 @@ int snhip_device_info(void* handle, int info[6]);
 int snhip_set_tuning(void* handle, int config, int splitk);
 int snhip_get_last_tuning(void* handle, int* config, int* splitk);
 int snhip_config_count(void);
-/* desc[0..4] = BM, BN, BK, threads, LDS bytes */
-int snhip_config_desc(int config, int desc[5]);
+/* desc[0..5] = BM, BN, BK, threads, LDS bytes, kind (0 fp32 kernel, 1 bf16-input kernel) */
+int snhip_config_desc(int config, int desc[6]);
 
 #ifdef __cplusplus
 }

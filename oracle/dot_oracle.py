@@ -25,6 +25,9 @@ softmax_last_dim                        Prod/CPU/CpuTensorActivationFunctions.cs
                                         :19-46
 sdpa_forward                            Prod/Layers/ScaledDotProductAttention        same
                                         Layer.cs:46-91
+round_to_bf16                           IEEE-754 round-to-nearest-even to a          closed-form ties/neighbours and torch's CPU
+                                        bfloat16 (what v_cvt_pk_bf16_f32 does);      bfloat16 cast (independent implementation)
+                                        no reference counterpart (variant is new)
 mkl_dot (baseline only)                 the same cblas_sgemm call the reference      compared with dot_f64 within the fp32 bound
                                         makes, through this image's own MKL
 ======================================  ==========================================  =======
@@ -144,6 +147,17 @@ def sgemm_colmajor(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc)
     out = np.array(C, dtype=np.float32, copy=True).reshape(-1)
     _lib().oracle_sgemm_colmajor(int(transa), int(transb), m, n, k, float(alpha), _p(A), lda, _p(B), ldb, float(beta),
                                  _p(out), ldc)
+    return out
+
+
+def round_to_bf16(x):
+    """float32 -> nearest bfloat16 (ties to even), returned as float32.  NaN stays NaN."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    rounded = ((u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+    out = rounded.view(np.float32).reshape(x.shape).copy()
+    nan = np.isnan(x)
+    out[nan] = x[nan]
     return out
 
 

@@ -189,20 +189,6 @@ struct Frag<4> {
     }
 };
 
-// Element r of an accumulator tile.  With many tiles per wavefront the
-// accumulators live in AGPRs; reading them one by one where they are consumed
-// (instead of letting the compiler copy all of them to VGPRs when the k loop
-// ends) keeps the epilogue's register footprint small.
-__device__ __forceinline__ float acc_element(const f32x16& t, int r, bool from_agpr) {
-    float x;
-    if (from_agpr) {
-        asm("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(t[r]));
-    } else {
-        x = t[r];
-    }
-    return x;
-}
-
 // Workgroup barrier that orders LDS traffic only: global loads that are still in
 // flight (the register prefetch) must not be waited for here.
 __device__ __forceinline__ void lds_barrier() {
@@ -228,6 +214,72 @@ __device__ __forceinline__ void tile_coords(int bid, int ntiles, int tiles_m, in
     const int in_g = logical - g * per_group;
     tm = first_m + in_g % gsz;
     tn = in_g / gsz;
+}
+
+// Epilogue shared by the fp32 and bf16-input kernels.  acc[i][j][r] holds
+// C[row][col] with  row = row_base + TM*(8*(r/4) + 4*lhi + r%4) + i  and
+// col = col0 + j  (row_base = first row of the wavefront, col0 = first of the
+// TN consecutive columns this lane owns, lhi = lane / 32).  Writes
+// alpha*acc + beta*C + bias to C, or the raw partial sums to the split-K
+// workspace slice `zb`.  C is read only when beta != 0.
+template <int TM, int TN>
+__device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], const GemmParams& p, int row_base,
+                                                   int col0, int lhi, int zb, int batch) {
+    const bool to_ws = (p.splitk > 1);
+    float* out;
+    long long ldo;
+    float alpha, beta;
+    const float* bias;
+    if (to_ws) {
+        out = p.ws + (long long)zb * p.M * p.N;
+        ldo = p.N;
+        alpha = 1.0f;
+        beta = 0.0f;
+        bias = nullptr;
+    } else {
+        out = p.C + (long long)batch * p.strideC;
+        ldo = p.ldc;
+        alpha = p.alpha;
+        beta = p.beta;
+        bias = p.bias;
+    }
+    const bool vec_ok = (TN == 4) && (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
+
+    float bv[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bv[j] = (bias != nullptr && col0 + j < p.N) ? bias[col0 + j] : 0.0f;
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
+            if (row >= p.M) continue;
+            float* crow = out + (long long)row * ldo + col0;
+            float v[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r] + bv[j];
+            if (vec_ok) {
+                if constexpr (TN == 4) {
+                    f32x4 o = {v[0], v[1], v[2], v[3]};
+                    if (beta != 0.0f) {
+                        const f32x4 c = *reinterpret_cast<const f32x4*>(crow);
+                        o += beta * c;
+                    }
+                    *reinterpret_cast<f32x4*>(crow) = o;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if (col0 + j < p.N) {
+                        float o = v[j];
+                        if (beta != 0.0f) o += beta * crow[j];
+                        crow[j] = o;
+                    }
+                }
+            }
+        }
+    }
 }
 
 template <int TM_, int TN_, int WM_, int WN_, int BK_>
@@ -428,68 +480,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         k_tile(P1{}, std::false_type{});
     }
 
-    // ---------------- epilogue ----------------
-    // acc[i][j][r] holds C[row][col] with
-    //   row = m0 + wm*TM*32 + TM*(8*(r/4) + 4*lhi + r%4) + i
-    //   col = n0 + wn*TN*32 + TN*l32 + j
-    const int col0 = n0 + wn * (TN * 32) + TN * l32;
-    const int row_base = m0 + wm * (TM * 32);
-    const bool to_ws = (p.splitk > 1);
-    float* out;
-    long long ldo;
-    float alpha, beta;
-    const float* bias;
-    if (to_ws) {
-        out = p.ws + (long long)zb * p.M * p.N;
-        ldo = p.N;
-        alpha = 1.0f;
-        beta = 0.0f;
-        bias = nullptr;
-    } else {
-        out = p.C + (long long)batch * p.strideC;
-        ldo = p.ldc;
-        alpha = p.alpha;
-        beta = p.beta;
-        bias = p.bias;
-    }
-    constexpr bool BIG_ACC = false;
-    const bool vec_ok = (TN == 4) && (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
-
-    float bv[TN];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) bv[j] = (bias != nullptr && col0 + j < p.N) ? bias[col0 + j] : 0.0f;
-
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
-            if (row >= p.M) continue;
-            float* crow = out + (long long)row * ldo + col0;
-            float v[TN];
-#pragma unroll
-            for (int j = 0; j < TN; ++j) v[j] = alpha * acc_element(acc[i][j], r, BIG_ACC) + bv[j];
-            if (vec_ok) {
-                if constexpr (TN == 4) {
-                    f32x4 o = {v[0], v[1], v[2], v[3]};
-                    if (beta != 0.0f) {
-                        const f32x4 c = *reinterpret_cast<const f32x4*>(crow);
-                        o += beta * c;
-                    }
-                    *reinterpret_cast<f32x4*>(crow) = o;
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    if (col0 + j < p.N) {
-                        float o = v[j];
-                        if (beta != 0.0f) o += beta * crow[j];
-                        crow[j] = o;
-                    }
-                }
-            }
-        }
-    }
+    store_accumulators<TM, TN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch);
 }
 
 // C = alpha * sum_s ws[batch][s] + beta * C + bias, splits summed in index

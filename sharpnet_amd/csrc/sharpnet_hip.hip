@@ -10,6 +10,7 @@
 
 #include <new>
 
+#include "bgemm_mfma.hpp"
 #include "sgemm_mfma.hpp"
 
 using namespace snhip;
@@ -24,6 +25,7 @@ struct Handle {
     float* ws = nullptr;
     size_t ws_bytes = 0;
     int num_cu = 256;
+    int math_mode = 0;  // 0: fp32 MFMA, 1: bf16-input MFMA for every GEMM on this handle
     int force_cfg = -1;
     int force_splitk = 0;
     int last_cfg = -1;
@@ -37,7 +39,8 @@ typedef void (*KernelFn)(const GemmParams);
 
 struct ConfigEntry {
     int BM, BN, BK, NT, lds_bytes;
-    int mfma_per_k2;  // MFMA instructions one wavefront issues per 2 k
+    int mfma_per_k2;    // TM*TN: MFMA instructions one wavefront issues per MFMA k step
+    int kind;           // 0: fp32 kernel (k step 2, 64 cycles per MFMA), 1: bf16-input kernel (k step 16, 32 cycles)
     KernelFn fn[2][2];  // [transposeA][transposeB]
 };
 
@@ -49,8 +52,22 @@ constexpr ConfigEntry make_entry() {
                        CFG::NT,
                        CFG::LDS_BYTES,
                        CFG::TM * CFG::TN,
+                       0,
                        {{sgemm_mfma_kernel<CFG, false, false>, sgemm_mfma_kernel<CFG, false, true>},
                         {sgemm_mfma_kernel<CFG, true, false>, sgemm_mfma_kernel<CFG, true, true>}}};
+}
+
+template <class CFG>
+constexpr ConfigEntry make_entry_bf16() {
+    return ConfigEntry{CFG::BM,
+                       CFG::BN,
+                       CFG::BK,
+                       CFG::NT,
+                       CFG::LDS_BYTES,
+                       CFG::TM * CFG::TN,
+                       1,
+                       {{bgemm_mfma_kernel<CFG, false, false>, bgemm_mfma_kernel<CFG, false, true>},
+                        {bgemm_mfma_kernel<CFG, true, false>, bgemm_mfma_kernel<CFG, true, true>}}};
 }
 
 // Tile configurations, largest first.  <TM,TN,WM,WN,BK>: a wavefront owns
@@ -67,6 +84,11 @@ const ConfigEntry kConfigs[] = {
     make_entry<TileCfg<2, 2, 2, 2, 32>>(),  // 8: 128 x 128, BK 32
     make_entry<TileCfg<2, 1, 2, 2, 32>>(),  // 9: 128 x 64, BK 32
     make_entry<TileCfg<1, 1, 2, 2, 32>>(),  // 10: 64 x 64, BK 32
+    // bf16-input kernels
+    make_entry_bf16<BTileCfg<4, 4, 2, 2, 32>>(),  // 11: 256 x 256, BK 32
+    make_entry_bf16<BTileCfg<2, 2, 2, 2, 32>>(),  // 12: 128 x 128, BK 32
+    make_entry_bf16<BTileCfg<2, 1, 2, 2, 64>>(),  // 13: 128 x 64, BK 64
+    make_entry_bf16<BTileCfg<1, 1, 2, 2, 64>>(),  // 14: 64 x 64, BK 64
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -100,11 +122,12 @@ struct Choice {
 // re-read operands more often and expose more latency, modelled by a
 // per-configuration efficiency.  Split-K adds a second pass over M*N*splitk.
 double estimate_cycles(const ConfigEntry& c, int cfg_id, int M, int N, int K, int batch, int splitk, int num_cu) {
-    static const double eff[kNumConfigs] = {0.92, 0.85, 0.85, 0.75, 0.6, 0.6, 0.45, 0.5, 0.5, 0.5, 0.5};
+    static const double eff[kNumConfigs] = {0.92, 0.85, 0.85, 0.75, 0.6, 0.6, 0.45, 0.5, 0.5, 0.5, 0.5, 0.35, 0.3, 0.25, 0.2};
     const long long tiles = (long long)ceil_div(M, c.BM) * ceil_div(N, c.BN) * batch * splitk;
     const long long rounds = (tiles + num_cu - 1) / num_cu;
     const int kchunk = ceil_div(ceil_div(K, splitk), c.BK) * c.BK;
-    const double tile_cycles = (kchunk / 2.0) * c.mfma_per_k2 * 64.0 / eff[cfg_id] + 3000.0;
+    const double mfma_cycles = c.kind == 0 ? (kchunk / 2.0) * 64.0 : (kchunk / 16.0) * 32.0;
+    const double tile_cycles = mfma_cycles * c.mfma_per_k2 / eff[cfg_id] + 3000.0;
     double total = rounds * tile_cycles;
     if (splitk > 1) {
         // reduce pass: (splitk + 1) reads/writes of M*N floats at ~1.5 kB/cycle, plus a launch
@@ -113,12 +136,14 @@ double estimate_cycles(const ConfigEntry& c, int cfg_id, int M, int N, int K, in
     return total;
 }
 
-Choice choose(const Handle* h, int M, int N, int K, int batch) {
-    Choice best{kNumConfigs - 1, 1};
+Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
+    Choice best{kind == 0 ? 6 : kNumConfigs - 1, 1};
     double best_cost = 1e300;
+    const bool forced = h->force_cfg >= 0 && kConfigs[h->force_cfg].kind == kind;
     for (int c = 0; c < kNumConfigs; ++c) {
-        if (h->force_cfg >= 0 && c != h->force_cfg) continue;
         const ConfigEntry& e = kConfigs[c];
+        if (e.kind != kind) continue;
+        if (forced && c != h->force_cfg) continue;
         for (int s = 1; s <= 32; s *= 2) {
             if (h->force_splitk > 0 && s != h->force_splitk) continue;
             if (s > 1) {
@@ -161,8 +186,9 @@ int ensure_workspace(Handle* h, size_t bytes) {
 // Row-major core: C[M x N] (ldc) = alpha * op(A)[M x K] * op(B)[K x N] + beta * C (+ bias), per batch.
 int gemm_rm(Handle* h, bool tA, bool tB, int M, int N, int K, float alpha, const float* A, int lda, long long sA,
             const float* B, int ldb, long long sB, float beta, float* C, int ldc, long long sC, int batch,
-            const float* bias) {
+            const float* bias, int math = -1) {
     if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (math < 0) math = h->math_mode;
     if (M < 0 || N < 0 || K < 0 || batch < 0) return SNHIP_STATUS_INVALID_VALUE;
     if (M == 0 || N == 0 || batch == 0) return SNHIP_STATUS_SUCCESS;
     if (C == nullptr || ldc < N) return SNHIP_STATUS_INVALID_VALUE;
@@ -184,7 +210,7 @@ int gemm_rm(Handle* h, bool tA, bool tB, int M, int N, int K, float alpha, const
     if (A == nullptr || B == nullptr) return SNHIP_STATUS_INVALID_VALUE;
     if (lda < (tA ? M : K) || ldb < (tB ? K : N)) return SNHIP_STATUS_INVALID_VALUE;
 
-    Choice ch = choose(h, M, N, K, batch);
+    Choice ch = choose(h, M, N, K, batch, math);
     const ConfigEntry& cfg = kConfigs[ch.cfg];
     if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
 
@@ -371,6 +397,38 @@ int snhip_bmm(void* handle, const float* A, int aH, int aW, int transposeA, long
                    bW, strideB, beta, C, N, strideC, batch, nullptr);
 }
 
+int snhip_set_math_mode(void* handle, int mode) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (mode != SNHIP_MATH_FP32 && mode != SNHIP_MATH_BF16_INPUT) return SNHIP_STATUS_INVALID_VALUE;
+    static_cast<Handle*>(handle)->math_mode = mode;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_dot_bf16(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
+                   int transposeB, float* C, float alpha, float beta, const float* bias) {
+    if (aH < 0 || aW < 0 || bH < 0 || bW < 0) return SNHIP_STATUS_INVALID_VALUE;
+    const int M = transposeA ? aW : aH;
+    const int N = transposeB ? bH : bW;
+    const int K = transposeA ? aH : aW;
+    const int Kb = transposeB ? bW : bH;
+    if (K != Kb) return SNHIP_STATUS_INVALID_VALUE;
+    return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha, A, aW, 0, B, bW, 0,
+                   beta, C, N, 0, 1, bias, SNHIP_MATH_BF16_INPUT);
+}
+
+int snhip_bmm_bf16(void* handle, const float* A, int aH, int aW, int transposeA, long long strideA, const float* B,
+                   int bH, int bW, int transposeB, long long strideB, float* C, long long strideC, int batch,
+                   float alpha, float beta) {
+    if (aH < 0 || aW < 0 || bH < 0 || bW < 0) return SNHIP_STATUS_INVALID_VALUE;
+    const int M = transposeA ? aW : aH;
+    const int N = transposeB ? bH : bW;
+    const int K = transposeA ? aH : aW;
+    const int Kb = transposeB ? bW : bH;
+    if (K != Kb) return SNHIP_STATUS_INVALID_VALUE;
+    return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha, A, aW, strideA, B,
+                   bW, strideB, beta, C, N, strideC, batch, nullptr, SNHIP_MATH_BF16_INPUT);
+}
+
 /* ---- memory / stream shims ---- */
 
 int snhip_malloc(void** dptr, size_t bytes) {
@@ -505,13 +563,14 @@ int snhip_get_last_tuning(void* handle, int* config, int* splitk) {
 
 int snhip_config_count(void) { return kNumConfigs; }
 
-int snhip_config_desc(int config, int desc[5]) {
+int snhip_config_desc(int config, int desc[6]) {
     if (config < 0 || config >= kNumConfigs || desc == nullptr) return SNHIP_STATUS_INVALID_VALUE;
     desc[0] = kConfigs[config].BM;
     desc[1] = kConfigs[config].BN;
     desc[2] = kConfigs[config].BK;
     desc[3] = kConfigs[config].NT;
     desc[4] = kConfigs[config].lds_bytes;
+    desc[5] = kConfigs[config].kind;
     return SNHIP_STATUS_SUCCESS;
 }
 

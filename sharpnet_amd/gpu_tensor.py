@@ -63,6 +63,14 @@ class GPUWrapper:
         check_status(self.lib.snhip_get_version(self.handle, ctypes.byref(v)), "snhip_get_version")
         return v.value
 
+    # -- arithmetic ----------------------------------------------------------
+    MATH_FP32 = 0
+    MATH_BF16_INPUT = 1
+
+    def set_math_mode(self, mode):
+        """fp32 MFMA (default) or bf16-input / fp32-accumulate MFMA for every GEMM of this handle."""
+        check_status(self.lib.snhip_set_math_mode(self.handle, mode), "snhip_set_math_mode")
+
     # -- tuning hooks -------------------------------------------------------
     def set_tuning(self, config=-1, splitk=0):
         check_status(self.lib.snhip_set_tuning(self.handle, config, splitk), "snhip_set_tuning")
@@ -75,9 +83,10 @@ class GPUWrapper:
     def configs(self):
         out = []
         for i in range(self.lib.snhip_config_count()):
-            d = (ctypes.c_int * 5)()
+            d = (ctypes.c_int * 6)()
             check_status(self.lib.snhip_config_desc(i, d))
-            out.append({"id": i, "BM": d[0], "BN": d[1], "BK": d[2], "threads": d[3], "lds_bytes": d[4]})
+            out.append({"id": i, "BM": d[0], "BN": d[1], "BK": d[2], "threads": d[3], "lds_bytes": d[4],
+                        "kind": "bf16" if d[5] else "fp32"})
         return out
 
     # -- stream / timing ----------------------------------------------------

@@ -69,6 +69,9 @@ SIGNATURES = {
     "snhip_dot_bias": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f, _vp],
     "snhip_bmm": [_vp, _vp, _i, _i, _i, _ll, _vp, _i, _i, _i, _ll, _vp, _ll, _i, _f, _f],
     "snhip_gemm_rm": [_vp, _i, _i, _i, _i, _i, _f, _vp, _i, _ll, _vp, _i, _ll, _f, _vp, _i, _ll, _i, _vp],
+    "snhip_set_math_mode": [_vp, _i],
+    "snhip_dot_bf16": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f, _vp],
+    "snhip_bmm_bf16": [_vp, _vp, _i, _i, _i, _ll, _vp, _i, _i, _i, _ll, _vp, _ll, _i, _f, _f],
     "snhip_malloc": [_vpp, _sz],
     "snhip_free": [_vp],
     "snhip_memset32": [_vp, _vp, ctypes.c_uint, _sz],

@@ -57,7 +57,7 @@ def test_argument_errors_without_gpu():
     assert lib.snhip_destroy(None) == 1
     assert lib.snhip_create(None) == 7
     assert lib.snhip_config_count() >= 4
-    d = (ctypes.c_int * 5)()
+    d = (ctypes.c_int * 6)()
     assert lib.snhip_config_desc(0, d) == 0 and d[0] > 0 and d[1] > 0
     assert lib.snhip_config_desc(999, d) == 7
 

@@ -227,3 +227,18 @@ def test_mkl_route_matches_closed_form(oracle):
         oracle.mkl_dot(a, tA, b, tB, out, alpha=0.5, beta=1.0)
         ref = oracle.dot_f64(a, tA, b, tB, 0.5, 1.0, c)
         assert np.max(np.abs(out - ref)) <= oracle.tolerance(K, a, b)
+
+
+def test_round_to_bf16(oracle):
+    """Ties go to the even 8-bit significand; agrees with torch's CPU bfloat16 cast on random data."""
+    f = np.float32
+    cases = [(1.0, 1.0), (1 + 2.0 ** -8, 1.0), (1 + 2.0 ** -8 + 2.0 ** -20, 1 + 2.0 ** -7),
+             (1 + 3 * 2.0 ** -8, 1 + 2.0 ** -6), (-(1 + 2.0 ** -8), -1.0), (0.0, 0.0),
+             (2.0 ** -130, 2.0 ** -130)]
+    for x, want in cases:
+        assert oracle.round_to_bf16(np.array([x], f))[0] == f(want), (x, want)
+    import torch
+    rng = np.random.default_rng(23)
+    x = np.concatenate([rng.normal(0, 1, 20000), rng.uniform(-1e-3, 1e-3, 20000), rng.normal(0, 1e4, 20000)]).astype(f)
+    want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(oracle.round_to_bf16(x), want)
