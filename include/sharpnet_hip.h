@@ -114,6 +114,27 @@ int snhip_bmm_bf16(void* handle, const float* A, int aH, int aW, int transposeA,
                    int bH, int bW, int transposeB, long long strideB, float* C, long long strideC, int batch,
                    float alpha, float beta);
 
+/* ---- row / column helpers next to the GEMMs in Linear and attention ------- */
+/* bias_gradient[c] = sum_r dy[r][c].  Replaces Tensor.Compute_BiasGradient_from_dy
+ * (Prod/Layers/Linear.cs:164; GPU: cudnnConvolutionBackwardBias, GpuTensor.cs:686-701). */
+int snhip_bias_gradient(void* handle, const float* dy, int rows, int cols, float* bias_gradient);
+/* y[r][c] += vector[c].  Replaces Tensor.BroadcastAddVectorToOutput (Linear.cs:131; GPU:
+ * cudnnAddTensor, GpuTensor.cs:633-644) for callers that do not use snhip_dot_bias. */
+int snhip_broadcast_add_vector(void* handle, const float* vector, float* y, int rows, int cols);
+/* y += alpha * x.  Replaces Tensor.Update_Adding_Alpha_X (weight decay, Linear.cs:168-181). */
+int snhip_axpy(void* handle, long long n, float alpha, const float* x, float* y);
+/* y = softmax(x) over the last dimension of a (rows, cols) view, max-subtracted fp32.  Replaces
+ * ActivationForward(SOFTMAX_LAST_DIMENSION) between the two attention products
+ * (Prod/Layers/ScaledDotProductAttentionLayer.cs:81; CPU: CpuTensorActivationFunctions.cs:19-46).
+ * x and y may be the same buffer. */
+int snhip_softmax_last_dim(void* handle, const float* x, float* y, long long rows, int cols);
+/* dx = y * (dy - sum_j dy_j y_j) per row, the softmax gradient the reference's GPU path gets from
+ * cuDNN (ScaledDotProductAttentionLayer.cs:125).  dx may alias dy. */
+int snhip_softmax_last_dim_backward(void* handle, const float* y, const float* dy, float* dx, long long rows, int cols);
+/* x[b][r][c] = value for c > r.  Replaces Tensor.SetAllElementsAboveMainDiagonal (causal mask,
+ * ScaledDotProductAttentionLayer.cs:73-76; CPU: CpuTensor.cs:3037-3052). */
+int snhip_set_above_main_diagonal(void* handle, float* x, int matrices, int rows, int cols, float value);
+
 /* ---- device memory / stream shims --------------------------------------- */
 /* Replace the nvcuda calls GPUTensor makes: cuMemAlloc_v2 (GpuTensor.cs:41),
  * cuMemFree_v2 (:1634), cuMemsetD32 (:1583), cuMemcpyHtoDAsync (:77),

@@ -25,6 +25,8 @@ softmax_last_dim                        Prod/CPU/CpuTensorActivationFunctions.cs
                                         :19-46
 sdpa_forward                            Prod/Layers/ScaledDotProductAttention        same
                                         Layer.cs:46-91
+softmax_last_dim_backward /             ScaledDotProductAttentionLayer.cs:111-132    central finite differences of sdpa_forward
+sdpa_backward                           (softmax gradient: cuDNN definition)         (tests/test_oracle.py)
 round_to_bf16                           IEEE-754 round-to-nearest-even to a          closed-form ties/neighbours and torch's CPU
                                         bfloat16 (what v_cvt_pk_bf16_f32 does);      bfloat16 cast (independent implementation)
                                         no reference counterpart (variant is new)
@@ -223,6 +225,30 @@ def sdpa_forward(Q, K, V, use_scale=True, is_causal=False):
     weights = softmax_last_dim(scores)
     y = bmm(weights, False, V, False, 1.0, 0.0)
     return y, weights
+
+
+def softmax_last_dim_backward(y, dy):
+    """Softmax gradient over the last dimension as the reference's GPU path obtains it from cuDNN
+    (ActivationBackward(SOFTMAX_LAST_DIMENSION), ScaledDotProductAttentionLayer.cs:125):
+    dx = y * (dy - sum_j dy_j y_j).  (The reference's CPU helper, CpuTensorActivationFunctions.cs:109-121,
+    is a loss-specific shortcut and is not the Jacobian; this function is pinned by finite differences.)"""
+    y = np.asarray(y, dtype=np.float64)
+    dy = np.asarray(dy, dtype=np.float64)
+    s = np.sum(dy * y, axis=-1, keepdims=True)
+    return (y * (dy - s)).astype(np.float32)
+
+
+def sdpa_backward(Q, K, V, dy, weights, use_scale=True):
+    """ScaledDotProductAttentionBackwardPropagation (ScaledDotProductAttentionLayer.cs:111-132).
+    Returns (dQ, dK, dV)."""
+    d = V.shape[-1]
+    scaling = 1.0 / np.sqrt(np.float32(d)) if use_scale else 1.0
+    dV = bmm(weights, True, dy, False, 1.0, 0.0)                       # :117
+    dW = bmm(dy, False, V, True, float(scaling), 0.0)                  # :123
+    dS = softmax_last_dim_backward(weights, dW)                        # :125
+    dQ = bmm(dS, False, K, False, 1.0, 0.0)                            # :127
+    dK = bmm(dS, True, Q, False, 1.0, 0.0)                             # :128
+    return dQ, dK, dV
 
 
 # ---------------------------------------------------------------------------

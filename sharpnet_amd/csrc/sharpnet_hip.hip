@@ -11,6 +11,7 @@
 #include <new>
 
 #include "bgemm_mfma.hpp"
+#include "rowops.hpp"
 #include "sgemm_mfma.hpp"
 
 using namespace snhip;
@@ -427,6 +428,73 @@ int snhip_bmm_bf16(void* handle, const float* A, int aH, int aW, int transposeA,
     if (K != Kb) return SNHIP_STATUS_INVALID_VALUE;
     return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha, A, aW, strideA, B,
                    bW, strideB, beta, C, N, strideC, batch, nullptr, SNHIP_MATH_BF16_INPUT);
+}
+
+/* ---- row / column helpers of the Linear and attention layers ---- */
+
+static inline int grid_for(long long total) {
+    const long long b = (total + 255) / 256;
+    return (int)(b < 1 ? 1 : (b > 16384 ? 16384 : b));
+}
+
+int snhip_bias_gradient(void* handle, const float* dy, int rows, int cols, float* bias_gradient) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (rows < 0 || cols < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (cols == 0) return SNHIP_STATUS_SUCCESS;
+    if (bias_gradient == nullptr || (rows > 0 && dy == nullptr)) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(column_sum_kernel, dim3((cols + 63) / 64), dim3(256), 0, static_cast<Handle*>(handle)->stream, dy,
+                       bias_gradient, rows, cols);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_broadcast_add_vector(void* handle, const float* vector, float* y, int rows, int cols) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (rows < 0 || cols < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (rows == 0 || cols == 0) return SNHIP_STATUS_SUCCESS;
+    if (vector == nullptr || y == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(broadcast_add_kernel, dim3(grid_for((long long)rows * cols)), dim3(256), 0,
+                       static_cast<Handle*>(handle)->stream, y, vector, (long long)rows, cols);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_axpy(void* handle, long long n, float alpha, const float* x, float* y) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (n < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (n == 0) return SNHIP_STATUS_SUCCESS;
+    if (x == nullptr || y == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(axpy_kernel, dim3(grid_for(n)), dim3(256), 0, static_cast<Handle*>(handle)->stream, y, x, alpha, n);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_softmax_last_dim(void* handle, const float* x, float* y, long long rows, int cols) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (rows < 0 || cols < 0 || rows > 0x7fffffffLL * 4) return SNHIP_STATUS_INVALID_VALUE;
+    if (rows == 0 || cols == 0) return SNHIP_STATUS_SUCCESS;
+    if (x == nullptr || y == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       static_cast<Handle*>(handle)->stream, x, y, rows, cols);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_softmax_last_dim_backward(void* handle, const float* y, const float* dy, float* dx, long long rows, int cols) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (rows < 0 || cols < 0 || rows > 0x7fffffffLL * 4) return SNHIP_STATUS_INVALID_VALUE;
+    if (rows == 0 || cols == 0) return SNHIP_STATUS_SUCCESS;
+    if (y == nullptr || dy == nullptr || dx == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(softmax_rows_bwd_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       static_cast<Handle*>(handle)->stream, y, dy, dx, rows, cols);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_set_above_main_diagonal(void* handle, float* x, int matrices, int rows, int cols, float value) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (matrices < 0 || rows < 0 || cols < 0) return SNHIP_STATUS_INVALID_VALUE;
+    const long long total = (long long)matrices * rows * cols;
+    if (total == 0) return SNHIP_STATUS_SUCCESS;
+    if (x == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(set_above_diagonal_kernel, dim3(grid_for(total)), dim3(256), 0,
+                       static_cast<Handle*>(handle)->stream, x, (long long)matrices, rows, cols, value);
+    return hip_to_status(hipGetLastError());
 }
 
 /* ---- memory / stream shims ---- */

@@ -317,3 +317,50 @@ class GPUTensor:
             self.Dispose()
         except Exception:
             pass
+
+
+# -- element-wise / row helpers next to the GEMMs (same names as the reference's Tensor methods) -----------------
+def _add_tensor_methods():
+    def Compute_BiasGradient_from_dy(self, biasGradient_1D):
+        """biasGradient[c] = sum over rows of this[r][c]  (CpuTensor.cs:1736-1740)."""
+        assert len(biasGradient_1D.Shape) == 1 and biasGradient_1D.Count == self.MultDim0
+        check_status(self._lib.snhip_bias_gradient(self.Wrapper.handle, self.Pointer, self.Shape[0], self.MultDim0,
+                                                   biasGradient_1D.Pointer), "snhip_bias_gradient")
+
+    def BroadcastAddVectorToOutput(self, y):
+        """y[n, :] += this  (this = 1-D bias; CpuTensor.cs:1468-1487)."""
+        assert y.Dimension >= 2 and y.MultDim0 == self.Count
+        check_status(self._lib.snhip_broadcast_add_vector(self.Wrapper.handle, self.Pointer, y.Pointer, y.Shape[0],
+                                                          y.MultDim0), "snhip_broadcast_add_vector")
+
+    def Update_Adding_Alpha_X(self, alpha, x):
+        """this += alpha * x  (Linear.cs:178)."""
+        assert x.Count == self.Count
+        check_status(self._lib.snhip_axpy(self.Wrapper.handle, self.Count, alpha, x.Pointer, self.Pointer), "snhip_axpy")
+
+    def SoftmaxLastDimension(self, y):
+        """y = softmax(this) over the last dimension (ActivationForward(SOFTMAX_LAST_DIMENSION))."""
+        cols = self.Shape[-1]
+        check_status(self._lib.snhip_softmax_last_dim(self.Wrapper.handle, self.Pointer, y.Pointer,
+                                                      self.Count // cols if cols else 0, cols), "snhip_softmax_last_dim")
+
+    def SoftmaxLastDimensionBackward(self, dy, dx):
+        """dx = softmax gradient given this = y (ActivationBackward(SOFTMAX_LAST_DIMENSION), cuDNN semantics)."""
+        cols = self.Shape[-1]
+        check_status(self._lib.snhip_softmax_last_dim_backward(self.Wrapper.handle, self.Pointer, dy.Pointer, dx.Pointer,
+                                                               self.Count // cols if cols else 0, cols),
+                     "snhip_softmax_last_dim_backward")
+
+    def SetAllElementsAboveMainDiagonal(self, value):
+        """CpuTensor.cs:3037-3052; 2-D or 3-D tensors."""
+        assert len(self.Shape) in (2, 3)
+        m, r, c = (self.Shape if len(self.Shape) == 3 else [1] + self.Shape)
+        check_status(self._lib.snhip_set_above_main_diagonal(self.Wrapper.handle, self.Pointer, m, r, c, value),
+                     "snhip_set_above_main_diagonal")
+
+    for f in (Compute_BiasGradient_from_dy, BroadcastAddVectorToOutput, Update_Adding_Alpha_X, SoftmaxLastDimension,
+              SoftmaxLastDimensionBackward, SetAllElementsAboveMainDiagonal):
+        setattr(GPUTensor, f.__name__, f)
+
+
+_add_tensor_methods()

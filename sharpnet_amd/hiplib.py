@@ -72,6 +72,12 @@ SIGNATURES = {
     "snhip_set_math_mode": [_vp, _i],
     "snhip_dot_bf16": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f, _vp],
     "snhip_bmm_bf16": [_vp, _vp, _i, _i, _i, _ll, _vp, _i, _i, _i, _ll, _vp, _ll, _i, _f, _f],
+    "snhip_bias_gradient": [_vp, _vp, _i, _i, _vp],
+    "snhip_broadcast_add_vector": [_vp, _vp, _vp, _i, _i],
+    "snhip_axpy": [_vp, _ll, _f, _vp, _vp],
+    "snhip_softmax_last_dim": [_vp, _vp, _vp, _ll, _i],
+    "snhip_softmax_last_dim_backward": [_vp, _vp, _vp, _vp, _ll, _i],
+    "snhip_set_above_main_diagonal": [_vp, _vp, _i, _i, _i, _f],
     "snhip_malloc": [_vpp, _sz],
     "snhip_free": [_vp],
     "snhip_memset32": [_vp, _vp, ctypes.c_uint, _sz],

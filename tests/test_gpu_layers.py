@@ -1,0 +1,190 @@
+"""GPU tests of the callers of Dot: Linear forward/backward and scaled-dot-product attention,
+driven through the host mirrors of the reference's layer code and checked against the oracle
+and against the losses the reference's own tests store."""
+import numpy as np
+import pytest
+
+from tests.helpers import numpy_array_for_tests, y_numpy_array_for_tests, random_tensor, sigmoid
+
+pytestmark = pytest.mark.gpu
+
+
+def T(w, a):
+    from sharpnet_amd import GPUTensor
+    a = np.asarray(a, np.float32)
+    return GPUTensor(list(a.shape), a, w)
+
+
+def bound(K, a, b, extra=0.0):
+    return 1e-4 * np.sqrt(max(K, 1)) * float(np.max(np.abs(a))) * float(np.max(np.abs(b))) + extra
+
+
+def test_dense_layer_forward_backward_config1(oracle, gpu_wrapper):
+    """Single Dense layer fwd+bwd, batch 128, 784 -> 256 (reference layout W:(out,in), Linear.cs:125-191)."""
+    from sharpnet_amd import GPUTensor, workloads as wl, linear
+    d = wl.dense_layer_inputs(seed=1)
+    x, W, dy = d["x"], d["w_out_in"], d["dy"]
+    bias = np.linspace(-0.5, 0.5, W.shape[0]).astype(np.float32)
+    gx, gW, gb, gdy = T(gpu_wrapper, x), T(gpu_wrapper, W), T(gpu_wrapper, bias), T(gpu_wrapper, dy)
+    ref_y = oracle.dense_forward(x, W, bias)
+    for fuse in (True, False):
+        gy = GPUTensor([x.shape[0], W.shape[0]], None, gpu_wrapper)
+        gy.SetValue(float("nan"))
+        linear.DenseForwardPropagation(gy, gx, gW, gb, False, fuse_bias=fuse)
+        assert np.max(np.abs(gy.ToNumpy() - ref_y)) <= bound(x.shape[1], x, W, 1e-6)
+    gdW, gdb, gdx = GPUTensor(list(W.shape), None, gpu_wrapper), GPUTensor([W.shape[0]], None, gpu_wrapper), \
+        GPUTensor(list(x.shape), None, gpu_wrapper)
+    for t in (gdW, gdb, gdx):
+        t.SetValue(float("nan"))
+    linear.DenseBackwardPropagation(gdx, gdW, gdb, gx, gdy, gW)           # SharpNet mode: multiplier 1/batch
+    rdW, rdb, rdx = oracle.dense_backward(x, dy, W, multiplier=1.0 / x.shape[0])
+    assert np.max(np.abs(gdW.ToNumpy() - rdW)) <= bound(x.shape[0], dy, x) / x.shape[0] + 1e-9
+    assert np.max(np.abs(gdb.ToNumpy() - rdb)) <= 1e-5 * np.sqrt(x.shape[0]) * np.max(np.abs(dy)) + 1e-7
+    assert np.max(np.abs(gdx.ToNumpy() - rdx)) <= bound(W.shape[0], dy, W)
+    # weight decay epilogue (PyTorch mode: dW += batch*wd*W, Linear.cs:168-181) and the input-layer shortcut
+    gdx.SetValue(7.0)
+    linear.DenseBackwardPropagation(gdx, gdW, gdb, gx, gdy, gW, bias_1D=gb, compatibility_mode="PyTorch",
+                                    use_weight_decay_in_backpropagation=True, weight_decay=0.01,
+                                    prevLayerIsInputLayer=True)
+    rdW2, rdb2, _ = oracle.dense_backward(x, dy, W, multiplier=1.0)
+    alpha = 1 * x.shape[0] * 0.01
+    assert np.max(np.abs(gdW.ToNumpy() - (rdW2 + alpha * W))) <= bound(x.shape[0], dy, x) + 1e-5
+    assert np.max(np.abs(gdb.ToNumpy() - (rdb2 + alpha * bias))) <= 1e-4
+    assert np.all(gdx.ToNumpy() == 7.0)                                  # dx untouched when the previous layer is the input
+
+
+def test_linear_sigmoid_predictions_on_device(golden, gpu_wrapper):
+    """Tests/NonReg/TestNetworkPropagation.cs:36-105 predictions through the GPU Dot."""
+    from sharpnet_amd import GPUTensor, linear
+    fx = golden["Linear_1_1_4_4"]
+    x = np.array(fx["x"], np.float32)
+    w_in_out = np.array(fx["w_in_out"], np.float32)
+    gx, gw = T(gpu_wrapper, x), T(gpu_wrapper, w_in_out)
+    gy = GPUTensor([1, 3], None, gpu_wrapper)
+    gy.Dot(gx, False, gw, False, 1.0, 0.0)                                # (1,1,4,4) read as (1,16): flatten rule
+    assert np.max(np.abs(sigmoid(gy.ToNumpy()) - np.array(fx["sigmoid_prediction"]))) < 2e-6
+    gwt = T(gpu_wrapper, np.ascontiguousarray(w_in_out.T))
+    linear.DenseForwardPropagation(gy, gx, gwt, None, False)
+    assert np.max(np.abs(sigmoid(gy.ToNumpy()) - np.array(fx["sigmoid_prediction"]))) < 2e-6
+
+
+def test_dense_chain_training_losses_on_device(golden, gpu_wrapper):
+    """Tests/NonReg/ParallelRunWithPyTorch.cs:102-138 with every Linear product on the GPU:
+    loss 0.297953724861145 before and 0.09050967544317245 after 10 epochs of SGD(0.1, momentum 0.9)."""
+    from sharpnet_amd import GPUTensor, linear
+    w = gpu_wrapper
+    fx = golden["PyTorch_Mse"]
+    X = numpy_array_for_tests(*fx["x_shape"])
+    Y = y_numpy_array_for_tests(*fx["y_shape"])
+    params = [np.array(fx["linear1_weight_out_in"], np.float32), np.zeros(3, np.float32),
+              np.array(fx["linear2_weight_out_in"], np.float32), np.zeros(3, np.float32)]
+    vel = [np.zeros_like(p) for p in params]
+    gX = T(w, X)
+
+    def forward():
+        gW1, gb1, gW2, gb2 = (T(w, p) for p in params)
+        gh = GPUTensor([2, 3, 4, 3], None, w)
+        linear.DenseForwardPropagation(gh, gX, gW1, gb1, True)            # flatten on last dimension: (24,5).(5,3)
+        h = gh.ToNumpy()
+        r = np.maximum(h, 0)
+        gf = T(w, r.reshape(2, 36))
+        gout = GPUTensor([2, 3], None, w)
+        linear.DenseForwardPropagation(gout, gf, gW2, gb2, False)
+        return h, r, gf, gout.ToNumpy(), (gW1, gW2)
+
+    mse = lambda out: float(np.mean((out.astype(np.float64) - Y) ** 2))
+    assert abs(mse(forward()[3]) - fx["loss_before"]) < fx["tolerance"]
+    for _ in range(fx["epochs"]):
+        h, r, gf, out, (gW1, gW2) = forward()
+        dout = (2.0 * (out - Y) / out.size).astype(np.float32)
+        gdW2, gdb2, gdf = GPUTensor([3, 36], None, w), GPUTensor([3], None, w), GPUTensor([2, 36], None, w)
+        linear.DenseBackwardPropagation(gdf, gdW2, gdb2, gf, T(w, dout), gW2, compatibility_mode="PyTorch")
+        dh = (gdf.ToNumpy().reshape(r.shape) * (h > 0)).astype(np.float32)
+        gdW1, gdb1 = GPUTensor([3, 5], None, w), GPUTensor([3], None, w)
+        linear.DenseBackwardPropagation(None, gdW1, gdb1, gX, T(w, dh), gW1, compatibility_mode="PyTorch",
+                                        prevLayerIsInputLayer=True, flattenInputTensorOnLastDimension=True)
+        grads = [gdW1.ToNumpy(), gdb1.ToNumpy(), gdW2.ToNumpy(), gdb2.ToNumpy()]
+        for i, g in enumerate(grads):
+            vel[i] = (fx["momentum"] * vel[i] + g).astype(np.float32)
+            params[i] = (params[i] - fx["lr"] * vel[i]).astype(np.float32)
+    assert abs(mse(forward()[3]) - fx["loss_after"]) < fx["tolerance"]
+
+
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_attention_fixture_loss_on_device(golden, oracle, gpu_wrapper, is_causal):
+    """Tests/NonReg/ParallelRunWithPyTorch.cs:963-1010 loss_before with QK^T, softmax, PV on the GPU."""
+    from sharpnet_amd import GPUTensor, attention, linear
+    w = gpu_wrapper
+    fx = golden["PyTorch_DotProductAttention"]
+    X = numpy_array_for_tests(*fx["x_shape"])
+    Y = y_numpy_array_for_tests(*fx["y_shape"])
+    Wq, Wk, Wv = [np.array(fx[k], np.float32)[:, :, 0] for k in ("conv_q", "conv_k", "conv_v")]
+    Wd = np.array(fx["dense_weight_out_in"], np.float32)
+    gX = T(w, X)
+    qkv = []
+    for Wc in (Wq, Wk, Wv):                       # kernel-1 conv = per-sample (2x4).(4x5): a batched product, W stride 0
+        out = GPUTensor([6, 2, 5], None, w)
+        st = w.lib.snhip_gemm_rm(w.handle, 0, 0, 2, 5, 4, 1.0, T(w, Wc).Pointer, 4, 0, gX.Pointer, 5, 20, 0.0,
+                                 out.Pointer, 5, 10, 6, None)
+        assert st == 0
+        qkv.append(out)
+    gy = GPUTensor([6, 2, 5], None, w)
+    attention.ScaledDotProductAttentionForwardPropagation(qkv[0], qkv[1], qkv[2], gy, False, False, is_causal)
+    glog = GPUTensor([6, 3], None, w)
+    linear.DenseForwardPropagation(glog, gy, T(w, Wd), None, False)
+    p = oracle.softmax_last_dim(glog.ToNumpy()).astype(np.float64)
+    loss = float(np.mean(-np.sum(Y * np.log(p), axis=1)))
+    want = [c for c in fx["cases"] if c["is_causal"] == is_causal][0]["loss_before"]
+    assert abs(loss - want) < 2e-6
+
+
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_sdpa_forward_backward_vs_oracle(oracle, gpu_wrapper, is_causal):
+    """ScaledDotProductAttentionLayer.cs:46-132: all six batched products (NT, NN, TN, NT, NN, TN) + softmax."""
+    from sharpnet_amd import GPUTensor, attention
+    w = gpu_wrapper
+    rng = np.random.default_rng(41)
+    B, Tn, d = 12, 96, 64
+    Q, K, V, dy = (rng.normal(0, 1, (B, Tn, d)).astype(np.float32) for _ in range(4))
+    gQ, gK, gV, gdy = (T(w, t) for t in (Q, K, V, dy))
+    gy = GPUTensor([B, Tn, d], None, w)
+    gweights = attention.ScaledDotProductAttentionForwardPropagation(gQ, gK, gV, gy, True, True, is_causal)
+    ry, rw = oracle.sdpa_forward(Q, K, V, use_scale=True, is_causal=is_causal)
+    assert np.max(np.abs(gweights.ToNumpy() - rw)) <= 2e-5
+    assert np.max(np.abs(gy.ToNumpy() - ry)) <= bound(Tn, rw, V, 1e-5)
+    gdQ, gdK, gdV = (GPUTensor([B, Tn, d], None, w) for _ in range(3))
+    attention.ScaledDotProductAttentionBackwardPropagation(gdQ, gdK, gdV, gQ, gK, gV, gdy, gweights, True)
+    rdQ, rdK, rdV = oracle.sdpa_backward(Q, K, V, dy, rw, use_scale=True)
+    assert np.max(np.abs(gdV.ToNumpy() - rdV)) <= bound(Tn, rw, dy, 1e-4)
+    assert np.max(np.abs(gdQ.ToNumpy() - rdQ)) <= bound(Tn, K, dy, 2e-4)
+    assert np.max(np.abs(gdK.ToNumpy() - rdK)) <= bound(Tn, Q, dy, 2e-4)
+
+
+def test_row_helpers_vs_numpy(gpu_wrapper):
+    """Compute_BiasGradient_from_dy, BroadcastAddVectorToOutput, Update_Adding_Alpha_X, softmax, causal mask
+    (Tests/TestParallelRunCpuVersusGpu.cs:730-736, 938-944, 651-665, 766)."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    rng = np.random.default_rng(43)
+    for rows, cols in [(1, 1), (7, 130), (300, 65), (1000, 1000)]:
+        dy = random_tensor(rng, (rows, cols))
+        gdb = GPUTensor([cols], None, w)
+        T(w, dy).Compute_BiasGradient_from_dy(gdb)
+        assert np.max(np.abs(gdb.ToNumpy() - dy.astype(np.float64).sum(0))) <= 1e-5 * np.sqrt(rows) * 1.5 * 4
+        v = random_tensor(rng, (cols,))
+        gy = T(w, dy)
+        T(w, v).BroadcastAddVectorToOutput(gy)
+        assert np.array_equal(gy.ToNumpy(), dy + v[None, :])
+        gy.Update_Adding_Alpha_X(-0.5, T(w, dy))
+        assert np.max(np.abs(gy.ToNumpy() - ((dy + v[None, :]) - 0.5 * dy))) <= 1e-6
+        gs = GPUTensor([rows, cols], None, w)
+        T(w, dy).SoftmaxLastDimension(gs)
+        e = np.exp(dy.astype(np.float64) - dy.max(1, keepdims=True))
+        assert np.max(np.abs(gs.ToNumpy() - e / e.sum(1, keepdims=True))) <= 2e-6
+    m = random_tensor(rng, (3, 5, 7))
+    gm = T(w, m)
+    gm.SetAllElementsAboveMainDiagonal(-1e12)
+    want = m.copy()
+    for r in range(5):
+        want[:, r, r + 1:] = np.float32(-1e12)
+    assert np.array_equal(gm.ToNumpy(), want)

@@ -1,0 +1,150 @@
+"""The five benchmark configurations at their real shapes, checked through size-independent properties:
+sampled rows / columns / batches of the result against the oracle on the same seeded inputs (any row block of
+C = op(A) op(B) is itself a Dot of a row block of op(A) with B), NaN-prefilled destinations, and linearity in beta."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def bound(K, a, b, extra=0.0):
+    return 1e-4 * np.sqrt(max(K, 1)) * float(np.max(np.abs(a))) * float(np.max(np.abs(b))) + extra
+
+
+def sampled_rows_check(oracle, w, g, a, b, c, nrows=8, seed=0, bf16=False):
+    """Runs g on the device and compares `nrows` sampled rows with the oracle."""
+    from sharpnet_amd import GPUTensor
+    ga, gb = GPUTensor(list(a.shape), a, w), GPUTensor(list(b.shape), b, w)
+    gc = GPUTensor([g.M, g.N], c, w) if c is not None else GPUTensor([g.M, g.N], None, w)
+    if c is None:
+        gc.SetValue(float("nan"))
+    gc.Dot(ga, g.tA, gb, g.tB, g.alpha, g.beta)
+    got = gc.ToNumpy()
+    assert np.all(np.isfinite(got))
+    rows = np.sort(np.random.default_rng(seed).choice(g.M, min(nrows, g.M), replace=False))
+    opa_rows = np.ascontiguousarray(a[:, rows].T if g.tA else a[rows])       # rows of op(A), as a non-transposed operand
+    if bf16:
+        opa_rows, bb = oracle.round_to_bf16(opa_rows), oracle.round_to_bf16(b)
+    else:
+        bb = b
+    ref = oracle.dot(opa_rows, False, bb, g.tB, g.alpha, g.beta, c[rows] if c is not None else None)
+    err = float(np.max(np.abs(got[rows] - ref)))
+    assert err <= bound(g.K, a, b, 1e-6 * (float(np.max(np.abs(c))) if c is not None else 0)), (g.label(), err)
+    for t in (ga, gb, gc):
+        t.Dispose()
+    return got
+
+
+def test_config2_sweep_all_sizes_transposes_betas(oracle, gpu_wrapper):
+    """Square and ragged sweep incl. 8192^3; the same A/B buffers serve all transposes of a square size."""
+    from sharpnet_amd import workloads as wl
+    rng = np.random.default_rng(2)
+    for (M, N, K) in wl.SWEEP_SIZES:
+        bufs = {}
+        for tA in (False, True):
+            for tB in (False, True):
+                sa = (K, M) if tA else (M, K)
+                sb = (N, K) if tB else (K, N)
+                for s in (sa, sb):
+                    if s not in bufs:
+                        bufs[s] = rng.uniform(-1, 1, s).astype(np.float32)
+                a, b = bufs[sa], bufs[sb]
+                if a is b:                                     # square sizes: keep A and B distinct
+                    b = bufs.setdefault((sb, "b"), rng.uniform(-1, 1, sb).astype(np.float32))
+                betas = (0.0, 1.0) if (M * N * K < 3e11 or (not tA and not tB)) else (0.0,)
+                for beta in betas:
+                    c = rng.uniform(-1, 1, (M, N)).astype(np.float32) if beta else None
+                    sampled_rows_check(oracle, gpu_wrapper, wl.Gemm(M, N, K, tA, tB, 1.0, beta), a, b, c, nrows=6)
+
+
+def test_config2_headline_bf16(oracle, gpu_wrapper):
+    from sharpnet_amd import workloads as wl
+    rng = np.random.default_rng(22)
+    a, b = rng.uniform(-1, 1, (4096, 4096)).astype(np.float32), rng.uniform(-1, 1, (4096, 4096)).astype(np.float32)
+    try:
+        gpu_wrapper.set_math_mode(gpu_wrapper.MATH_BF16_INPUT)
+        for tA, tB in [(False, False), (False, True), (True, False), (True, True)]:
+            got = sampled_rows_check(oracle, gpu_wrapper, wl.Gemm(4096, 4096, 4096, tA, tB), a, b, None, bf16=True)
+            # 1e-2 relative to the fp32 result as well
+            rows = slice(0, 4)
+            ref32 = oracle.dot(np.ascontiguousarray(a[:, rows].T if tA else a[rows]), False, b, tB)
+            assert np.max(np.abs(got[rows] - ref32)) / np.max(np.abs(ref32)) <= 1e-2
+    finally:
+        gpu_wrapper.set_math_mode(gpu_wrapper.MATH_FP32)
+
+
+def test_config3_mlp_step_gemms(oracle, gpu_wrapper):
+    """Batch 4096, 3072 -> 4096 -> 4096 -> 1000: every forward (+bias), dW and dX product at full shape."""
+    from sharpnet_amd import GPUTensor, workloads as wl
+    w = gpu_wrapper
+    rng = np.random.default_rng(3)
+    for g in wl.mlp_gemms():
+        a = rng.uniform(0, 1, g.a_shape).astype(np.float32) if g.name.startswith("fwd") else \
+            rng.normal(0, 1e-3, g.a_shape).astype(np.float32)
+        lim = np.sqrt(6.0 / (g.N + g.K))
+        b = rng.uniform(-lim, lim, g.b_shape).astype(np.float32)
+        if not g.bias:
+            sampled_rows_check(oracle, w, g, a, b, None, nrows=4)
+            continue
+        bias = rng.uniform(-1, 1, g.N).astype(np.float32)
+        ga, gb, gbias = GPUTensor(list(a.shape), a, w), GPUTensor(list(b.shape), b, w), GPUTensor([g.N], bias, w)
+        gc = GPUTensor([g.M, g.N], None, w)
+        gc.SetValue(float("nan"))
+        gc.DotRowMajor(ga, g.tA, gb, g.tB, 1.0, 0.0, bias=gbias)
+        rows = np.array([0, 1, g.M // 2, g.M - 1])
+        ref = oracle.dense_forward(a[rows], b, bias)
+        assert np.max(np.abs(gc.ToNumpy()[rows] - ref)) <= bound(g.K, a, b, 1e-6), g.label()
+
+
+def test_config4_lstm_projections(oracle, gpu_wrapper):
+    """Input projection (32768,2048,256) once, then sequential recurrent steps (256,2048,512) accumulating with beta=1."""
+    from sharpnet_amd import GPUTensor, workloads as wl
+    w = gpu_wrapper
+    d = wl.lstm_inputs(seed=4)
+    proj, rec, _ = wl.lstm_gemms()
+    sampled_rows_check(oracle, w, proj, d["x"], d["w"], None, nrows=8)
+    steps = 6
+    rng = np.random.default_rng(44)
+    hs = [np.tanh(rng.normal(0, 1, d["h"].shape)).astype(np.float32) for _ in range(steps)]
+    gates0 = rng.normal(0, 1, (rec.M, rec.N)).astype(np.float32)
+    gg, gu = GPUTensor([rec.M, rec.N], gates0, w), GPUTensor(list(d["u"].shape), d["u"], w)
+    ref = gates0.copy()
+    for h in hs:
+        gg.Dot(GPUTensor(list(h.shape), h, w), False, gu, False, 1.0, 1.0)
+        ref = oracle.dot(h, False, d["u"], False, 1.0, 1.0, ref)
+    assert np.max(np.abs(gg.ToNumpy() - ref)) <= steps * bound(rec.K, hs[0], d["u"], 1e-6)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_config5_attention_batched(oracle, gpu_wrapper, bf16):
+    """512 batches x (256,256,64): S = Q K^T / 8, P = softmax(S) on the host, O = P V; sampled batches vs the oracle."""
+    from sharpnet_amd import GPUTensor, workloads as wl
+    w = gpu_wrapper
+    d = wl.attention_inputs(seed=5)
+    q, k, v = d["q"], d["k"], d["v"]
+    batch, T, dim = q.shape
+    gq, gk, gv = (GPUTensor(list(t.shape), t, w) for t in (q, k, v))
+    gs = GPUTensor([batch, T, T], None, w)
+    gs.SetValue(float("nan"))
+    rnd = oracle.round_to_bf16 if bf16 else (lambda t: t)
+    try:
+        if bf16:
+            w.set_math_mode(w.MATH_BF16_INPUT)
+        gs.BatchMatrixMultiplication(gq, False, gk, True, 0.125, 0.0)
+        s = gs.ToNumpy()
+        sel = [0, 1, 255, 511]
+        ref_s = oracle.bmm(rnd(q[sel]), False, rnd(k[sel]), True, 0.125)
+        assert np.max(np.abs(s[sel] - ref_s)) <= bound(dim, q, k) * 0.125 + 1e-6
+        p = oracle.softmax_last_dim(s)
+        gp, go = GPUTensor([batch, T, T], p, w), GPUTensor([batch, T, dim], None, w)
+        go.SetValue(float("nan"))
+        go.BatchMatrixMultiplication(gp, False, gv, False, 1.0, 0.0)
+        o = go.ToNumpy()
+        assert np.all(np.isfinite(o)) and np.all(np.isfinite(s))
+        ref_o = oracle.bmm(rnd(p[sel]), False, rnd(v[sel]), False)
+        assert np.max(np.abs(o[sel] - ref_o)) <= bound(T, p, v)
+        if bf16:   # and within 1e-2 relative of the fp32 result
+            ref32 = oracle.bmm(p[sel], False, v[sel], False)
+            assert np.max(np.abs(o[sel] - ref32)) / np.max(np.abs(ref32)) <= 1e-2
+    finally:
+        w.set_math_mode(w.MATH_FP32)

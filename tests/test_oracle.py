@@ -242,3 +242,32 @@ def test_round_to_bf16(oracle):
     x = np.concatenate([rng.normal(0, 1, 20000), rng.uniform(-1e-3, 1e-3, 20000), rng.normal(0, 1e4, 20000)]).astype(f)
     want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
     assert np.array_equal(oracle.round_to_bf16(x), want)
+
+
+def test_sdpa_backward_by_finite_differences(oracle):
+    """dQ, dK, dV of the attention chain agree with central differences of sum(y * g) (float64 restatement)."""
+    rng = np.random.default_rng(29)
+    B, T, d = 2, 5, 3
+    Q, K, V = (rng.normal(0, 1, (B, T, d)).astype(np.float32) for _ in range(3))
+    g = rng.normal(0, 1, (B, T, d)).astype(np.float32)
+
+    def f(q, k, v):
+        s = np.einsum("btd,bsd->bts", q, k) / np.sqrt(d)
+        e = np.exp(s - s.max(-1, keepdims=True))
+        p = e / e.sum(-1, keepdims=True)
+        return float(np.sum(np.einsum("bts,bsd->btd", p, v) * g))
+
+    y, w = oracle.sdpa_forward(Q, K, V, use_scale=True, is_causal=False)
+    dQ, dK, dV = oracle.sdpa_backward(Q, K, V, g, w, use_scale=True)
+    eps = 1e-4
+    for name, X, dX in (("Q", Q, dQ), ("K", K, dK), ("V", V, dV)):
+        num = np.zeros_like(X, dtype=np.float64)
+        for idx in np.ndindex(*X.shape):
+            args = {"Q": Q.astype(np.float64), "K": K.astype(np.float64), "V": V.astype(np.float64)}
+            xp, xm = args[name].copy(), args[name].copy()
+            xp[idx] += eps
+            xm[idx] -= eps
+            ap, am = dict(args), dict(args)
+            ap[name], am[name] = xp, xm
+            num[idx] = (f(ap["Q"], ap["K"], ap["V"]) - f(am["Q"], am["K"], am["V"])) / (2 * eps)
+        assert np.max(np.abs(num - dX)) < 2e-4, name
