@@ -186,18 +186,30 @@ def main():
         for (M, N, K) in wl.SWEEP_SIZES:
             for tA in (False, True):
                 for tB in (False, True):
-                    steps = 5 if M * N * K > 1e11 else 20
-                    sweep.append(run(wl.Gemm(M, N, K, tA, tB, 1.0, 0.0), 2, steps, 2))
-            sweep.append(run(wl.Gemm(M, N, K, False, False, 1.0, 1.0), 2, 5, 2))
+                    steps, warm = (5, 3) if M * N * K > 1e11 else (50, 20)
+                    sweep.append(run(wl.Gemm(M, N, K, tA, tB, 1.0, 0.0), 2, steps, warm))
+            sweep.append(run(wl.Gemm(M, N, K, False, False, 1.0, 1.0), 2, steps, warm))
         extra["config2_sweep"] = sweep
-        mlp = [run(gm, 3, 5, 2, bias=np.zeros(gm.N, np.float32) if gm.bias else None) for gm in wl.mlp_gemms()]
+        mlp = [run(gm, 3, 20, 10, bias=np.zeros(gm.N, np.float32) if gm.bias else None) for gm in wl.mlp_gemms()]
         extra["config3_mlp_step"] = {"gemms": mlp, "total_ms": round(sum(r["ms"] for r in mlp), 4),
                                      "tflops": round(sum(gm.flops for gm in wl.mlp_gemms()) /
                                                      (sum(r["ms"] for r in mlp) * 1e-3) / 1e12, 2)}
         proj, rec, seq = wl.lstm_gemms()
-        extra["config4_lstm"] = {"input_projection": run(proj, 4, 10, 2), "recurrent_step": run(rec, 4, seq, 10),
+        extra["config4_lstm"] = {"input_projection": run(proj, 4, 20, 10), "recurrent_step": run(rec, 4, seq, 20),
                                  "recurrent_steps": seq}
-        extra["config5_attention_fp32"] = [run(gm, 5, 20, 3) for gm in wl.attention_gemms()]
+        extra["config5_attention_fp32"] = [run(gm, 5, 50, 10) for gm in wl.attention_gemms()]
+        # bf16-input / fp32-accumulate variant (operands stay fp32 in HBM, rounded on the way into LDS)
+        w.set_math_mode(w.MATH_BF16_INPUT)
+        try:
+            bf = [run(gm, 5, 50, 10) for gm in wl.attention_gemms()]
+            for r, gm in zip(bf, wl.attention_gemms()):   # HBM-bound: roofline = bytes / 8 TB/s vs bf16 MFMA peak
+                r["frac_of_roofline"] = round(gm.roofline_seconds(wl.BF16_MFMA_PEAK_TFLOPS) * 1e3 / r["ms"], 4)
+            extra["config5_attention_bf16_input"] = bf
+            hb = run(wl.Gemm(8192, 8192, 8192, True, False, 1.0, 0.0), 2, 10, 5)
+            hb["frac_of_roofline"] = round(hb["tflops"] / wl.BF16_MFMA_PEAK_TFLOPS, 4)
+            extra["config2_8192_bf16_input_TN"] = hb
+        finally:
+            w.set_math_mode(w.MATH_FP32)
         out["extra"] = extra
         for k, v in extra.items():
             log("[bench]", k, json.dumps(v))

@@ -97,8 +97,10 @@ struct BStage {
         const float* p = vec_ptr(v);
         int nval;
         if (KCONTIG) {
+            // rows past the edge re-read the last valid row (their products are never stored)
             const int mn = row_const(v) + T * line;
-            nval = (mn < mn_rem) ? (k_rem - k0) : 0;
+            if (mn >= mn_rem) p = gptr + (long long)(mn_rem - 1 - T * line) * ld;
+            nval = k_rem - k0;
         } else {
             const int k = 4 * (kb + (v / 4) * KB_STEP) + (v % 4);
             nval = (k < k_rem) ? (mn_rem - 4 * g) : 0;

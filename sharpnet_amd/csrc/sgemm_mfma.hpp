@@ -114,12 +114,18 @@ struct TileStage {
     // Checked load: elements with m/n >= mn_rem or k >= k_rem read as zero
     // (mn_rem, k_rem are counted from the tile origin) and touch no memory.
     __device__ __forceinline__ void load_safe_vec(f32x4& r, int v, int mn_rem, int k_rem) const {
-        const float* p = gptr + (long long)(v * LINE_STEP) * ld;
+        const float* p;
         int nval;
         if (KCONTIG) {
+            // Rows past the edge re-read the last valid row instead of being zeroed: their
+            // products land in rows (columns) of C that are never stored, and the load
+            // stays a plain 16-byte vector for every lane of an edge tile.
             const int mn = mn0 + v * LINE_STEP;
-            nval = (mn < mn_rem) ? (k_rem - k0) : 0;
+            const int mnc = (mn < mn_rem) ? mn : mn_rem - 1;
+            p = gptr + (long long)(mnc - mn0) * ld;
+            nval = k_rem - k0;
         } else {
+            p = gptr + (long long)(v * LINE_STEP) * ld;
             const int k = k0 + v * LINE_STEP;
             nval = (k < k_rem) ? (mn_rem - mn0) : 0;
         }
@@ -206,7 +212,8 @@ __device__ __forceinline__ void tile_coords(int bid, int ntiles, int tiles_m, in
     constexpr int NXCD = 8;
     const int q = ntiles / NXCD, r = ntiles % NXCD;
     const int xcd = bid % NXCD, local = bid / NXCD;
-    const int logical = xcd * q + (xcd < r ? xcd : r) + local;
+    // reversed, so the ragged last tile row / column (slower, bounds-checked) is issued first
+    const int logical = ntiles - 1 - (xcd * q + (xcd < r ? xcd : r) + local);
     const int per_group = group_m * tiles_n;
     const int g = logical / per_group;
     const int first_m = g * group_m;

@@ -43,10 +43,15 @@ struct ConfigEntry {
     int mfma_per_k2;    // TM*TN: MFMA instructions one wavefront issues per MFMA k step
     int kind;           // 0: fp32 kernel (k step 2, 64 cycles per MFMA), 1: bf16-input kernel (k step 16, 32 cycles)
     KernelFn fn[2][2];  // [transposeA][transposeB]
+    // cost-model inputs, calibrated on MI355X
+    int occ;            // workgroups that fit on one CU (registers / LDS)
+    double eff_alone;   // fraction of the MFMA issue rate reached with one workgroup per CU
+    double eff_shared;  // ... with two or more co-resident workgroups hiding each other's stalls
+    double edge_slow;   // slow-down of a tile that needs bounds-checked loads
 };
 
 template <class CFG>
-constexpr ConfigEntry make_entry() {
+constexpr ConfigEntry make_entry(int occ, double eff_alone, double eff_shared, double edge_slow) {
     return ConfigEntry{CFG::BM,
                        CFG::BN,
                        CFG::BK,
@@ -55,11 +60,15 @@ constexpr ConfigEntry make_entry() {
                        CFG::TM * CFG::TN,
                        0,
                        {{sgemm_mfma_kernel<CFG, false, false>, sgemm_mfma_kernel<CFG, false, true>},
-                        {sgemm_mfma_kernel<CFG, true, false>, sgemm_mfma_kernel<CFG, true, true>}}};
+                        {sgemm_mfma_kernel<CFG, true, false>, sgemm_mfma_kernel<CFG, true, true>}},
+                       occ,
+                       eff_alone,
+                       eff_shared,
+                       edge_slow};
 }
 
 template <class CFG>
-constexpr ConfigEntry make_entry_bf16() {
+constexpr ConfigEntry make_entry_bf16(int occ, double eff_alone, double eff_shared, double edge_slow) {
     return ConfigEntry{CFG::BM,
                        CFG::BN,
                        CFG::BK,
@@ -68,28 +77,33 @@ constexpr ConfigEntry make_entry_bf16() {
                        CFG::TM * CFG::TN,
                        1,
                        {{bgemm_mfma_kernel<CFG, false, false>, bgemm_mfma_kernel<CFG, false, true>},
-                        {bgemm_mfma_kernel<CFG, true, false>, bgemm_mfma_kernel<CFG, true, true>}}};
+                        {bgemm_mfma_kernel<CFG, true, false>, bgemm_mfma_kernel<CFG, true, true>}},
+                       occ,
+                       eff_alone,
+                       eff_shared,
+                       edge_slow};
 }
 
 // Tile configurations, largest first.  <TM,TN,WM,WN,BK>: a wavefront owns
 // TM x TN MFMA tiles of 32x32, a workgroup is WM x WN wavefronts.
 const ConfigEntry kConfigs[] = {
-    make_entry<TileCfg<4, 4, 2, 2, 16>>(),  // 0: 256 x 256
-    make_entry<TileCfg<2, 4, 2, 2, 16>>(),  // 1: 128 x 256
-    make_entry<TileCfg<4, 2, 2, 2, 16>>(),  // 2: 256 x 128
-    make_entry<TileCfg<2, 2, 2, 2, 16>>(),  // 3: 128 x 128
-    make_entry<TileCfg<1, 2, 2, 2, 16>>(),  // 4: 64 x 128
-    make_entry<TileCfg<2, 1, 2, 2, 16>>(),  // 5: 128 x 64
-    make_entry<TileCfg<1, 1, 2, 2, 16>>(),  // 6: 64 x 64
-    make_entry<TileCfg<4, 4, 2, 2, 32>>(),  // 7: 256 x 256, BK 32
-    make_entry<TileCfg<2, 2, 2, 2, 32>>(),  // 8: 128 x 128, BK 32
-    make_entry<TileCfg<2, 1, 2, 2, 32>>(),  // 9: 128 x 64, BK 32
-    make_entry<TileCfg<1, 1, 2, 2, 32>>(),  // 10: 64 x 64, BK 32
-    // bf16-input kernels
-    make_entry_bf16<BTileCfg<4, 4, 2, 2, 32>>(),  // 11: 256 x 256, BK 32
-    make_entry_bf16<BTileCfg<2, 2, 2, 2, 32>>(),  // 12: 128 x 128, BK 32
-    make_entry_bf16<BTileCfg<2, 1, 2, 2, 64>>(),  // 13: 128 x 64, BK 64
-    make_entry_bf16<BTileCfg<1, 1, 2, 2, 64>>(),  // 14: 64 x 64, BK 64
+    //                                      occ  alone shared edge
+    make_entry<TileCfg<4, 4, 2, 2, 16>>(1, 0.94, 0.94, 1.7),   // 0: 256 x 256
+    make_entry<TileCfg<2, 4, 2, 2, 16>>(1, 0.91, 0.91, 1.5),   // 1: 128 x 256
+    make_entry<TileCfg<4, 2, 2, 2, 16>>(1, 0.92, 0.92, 1.5),   // 2: 256 x 128
+    make_entry<TileCfg<2, 2, 2, 2, 16>>(2, 0.80, 0.87, 1.3),   // 3: 128 x 128
+    make_entry<TileCfg<1, 2, 2, 2, 16>>(3, 0.70, 0.82, 1.15),  // 4: 64 x 128
+    make_entry<TileCfg<2, 1, 2, 2, 16>>(3, 0.70, 0.82, 1.15),  // 5: 128 x 64
+    make_entry<TileCfg<1, 1, 2, 2, 16>>(5, 0.62, 0.75, 1.1),   // 6: 64 x 64
+    make_entry<TileCfg<4, 4, 2, 2, 32>>(1, 0.94, 0.94, 1.7),   // 7: 256 x 256, BK 32
+    make_entry<TileCfg<2, 2, 2, 2, 32>>(1, 0.80, 0.86, 1.3),   // 8: 128 x 128, BK 32
+    make_entry<TileCfg<2, 1, 2, 2, 32>>(2, 0.72, 0.82, 1.15),  // 9: 128 x 64, BK 32
+    make_entry<TileCfg<1, 1, 2, 2, 32>>(4, 0.60, 0.75, 1.1),   // 10: 64 x 64, BK 32
+    // bf16-input kernels (fp32 operands in memory: bound by the L2 -> LDS path long before the MFMA rate)
+    make_entry_bf16<BTileCfg<4, 4, 2, 2, 32>>(1, 0.80, 0.80, 1.7),   // 11: 256 x 256, BK 32
+    make_entry_bf16<BTileCfg<2, 2, 2, 2, 32>>(2, 0.60, 0.75, 1.3),   // 12: 128 x 128, BK 32
+    make_entry_bf16<BTileCfg<2, 1, 2, 2, 64>>(2, 0.50, 0.65, 1.15),  // 13: 128 x 64, BK 64
+    make_entry_bf16<BTileCfg<1, 1, 2, 2, 64>>(3, 0.40, 0.55, 1.1),   // 14: 64 x 64, BK 64
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -117,24 +131,45 @@ struct Choice {
     int splitk;
 };
 
-// Estimated run time in MFMA-pipe cycles of one SIMD.  The chip executes
-// num_cu workgroups of 4 wavefronts at a time (one wavefront per SIMD); a
-// workgroup needs (k/2) * mfma_per_k2 MFMA issues of 64 cycles.  Smaller tiles
-// re-read operands more often and expose more latency, modelled by a
-// per-configuration efficiency.  Split-K adds a second pass over M*N*splitk.
-double estimate_cycles(const ConfigEntry& c, int cfg_id, int M, int N, int K, int batch, int splitk, int num_cu) {
-    static const double eff[kNumConfigs] = {0.92, 0.85, 0.85, 0.75, 0.6, 0.6, 0.45, 0.5, 0.5, 0.5, 0.5, 0.35, 0.3, 0.25, 0.2};
-    const long long tiles = (long long)ceil_div(M, c.BM) * ceil_div(N, c.BN) * batch * splitk;
-    const long long rounds = (tiles + num_cu - 1) / num_cu;
+// Estimated run time in engine cycles.  The launch is bound by the slowest of
+//  - the MFMA pipes: every CU works off ceil(blocks / num_cu) workgroups, one wavefront per SIMD each;
+//  - the per-tile critical path of a workgroup that has the CU to itself (LDS round trip + barrier);
+//  - HBM (unique operand bytes + C, plus the split-K partial sums);
+//  - the L2 -> LDS path (every workgroup re-reads its A and B panels).
+// Split-K adds a second launch that re-reads the partial sums.  Constants are fits to measurements on MI355X.
+double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int splitk, int num_cu) {
+    constexpr double kTileLatency = 700.0;     // cycles per k tile when nothing hides the LDS/barrier latency
+    constexpr double kFixed = 5000.0;          // prologue + epilogue of one workgroup
+    constexpr double kStoreBytesPerCycle = 40; // C write-out rate of one CU
+    constexpr double kHbmBytesPerCycle = 1600; // ~3.8 TB/s streaming at 2.4 GHz
+    constexpr double kL2BytesPerCycle = 5000;  // ~12 TB/s aggregate L2 -> CU
+    constexpr double kLaunch = 6000.0;
+    constexpr double kSplitFixed = 20000.0;    // second launch + dependency gap
+    const long long tiles_mn = (long long)ceil_div(M, c.BM) * ceil_div(N, c.BN);
+    const long long blocks = tiles_mn * batch * splitk;
+    const long long per_cu = (blocks + num_cu - 1) / num_cu;
     const int kchunk = ceil_div(ceil_div(K, splitk), c.BK) * c.BK;
-    const double mfma_cycles = c.kind == 0 ? (kchunk / 2.0) * 64.0 : (kchunk / 16.0) * 32.0;
-    const double tile_cycles = mfma_cycles * c.mfma_per_k2 / eff[cfg_id] + 3000.0;
-    double total = rounds * tile_cycles;
-    if (splitk > 1) {
-        // reduce pass: (splitk + 1) reads/writes of M*N floats at ~1.5 kB/cycle, plus a launch
-        total += 12000.0 + (double)M * N * batch * (splitk + 2) * 4.0 / 1500.0;
-    }
-    return total;
+    const int nk = ((kchunk / c.BK + 1) / 2) * 2;  // the k loop runs pairs of tiles
+    const double mfma_per_tile = c.kind == 0 ? (c.BK / 2) * 64.0 * c.mfma_per_k2 : (c.BK / 16) * 32.0 * c.mfma_per_k2;
+    const long long resident = per_cu < c.occ ? per_cu : c.occ;
+    const double eff = resident >= 2 ? c.eff_shared : c.eff_alone;
+    const bool has_edge = (M % c.BM != 0) || (N % c.BN != 0);
+    const double edge = !has_edge ? 1.0 : (per_cu <= 2 ? c.edge_slow : 1.0 + (c.edge_slow - 1.0) * 0.15);
+    const double t_mfma = per_cu * nk * mfma_per_tile / eff * edge + kFixed;
+    const double tile_alone = mfma_per_tile / c.eff_alone > kTileLatency ? mfma_per_tile / c.eff_alone : kTileLatency;
+    const double t_lat = (double)((per_cu + c.occ - 1) / c.occ) *
+                         (nk * tile_alone + kFixed + (double)c.BM * c.BN * 4.0 / kStoreBytesPerCycle);
+    const double bytes_hbm = (double)batch * (4.0 * ((double)M * K + (double)K * N) + 4.0 * M * N) +
+                             (splitk > 1 ? (double)batch * M * N * 4.0 * splitk : 0.0);
+    const double t_mem = bytes_hbm / kHbmBytesPerCycle;
+    const double t_l2 = (double)blocks * (c.BM + c.BN) * (double)kchunk * 4.0 / kL2BytesPerCycle;
+    double t = t_mfma;
+    if (t_lat > t) t = t_lat;
+    if (t_mem > t) t = t_mem;
+    if (t_l2 > t) t = t_l2;
+    t += kLaunch;
+    if (splitk > 1) t += kSplitFixed + (double)batch * M * N * (2.0 * splitk + 2.0) * 4.0 / kHbmBytesPerCycle;
+    return t;
 }
 
 Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
@@ -153,7 +188,7 @@ Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
                 const int kchunk = ceil_div(ceil_div(K, s), e.BK) * e.BK;
                 if ((long long)kchunk * (s - 1) >= K) continue;  // would leave an empty split
             }
-            const double cost = estimate_cycles(e, c, M, N, K, batch, s, h->num_cu);
+            const double cost = estimate_cycles(e, M, N, K, batch, s, h->num_cu);
             if (cost < best_cost) {
                 best_cost = cost;
                 best = Choice{c, s};
