@@ -169,6 +169,10 @@ int snhip_device_info(void* handle, int info[6]);
  * call selected.  config ids index the table in sharpnet_hip.hip. */
 int snhip_set_tuning(void* handle, int config, int splitk);
 int snhip_get_last_tuning(void* handle, int* config, int* splitk);
+/* How split-K partial sums are added: 0 = automatic (currently always a second kernel, the faster
+ * choice on MI355X), 1 = a second kernel, 2 = in the GEMM kernel by the last workgroup to arrive for
+ * its tile.  The order of summation is fixed in both, so results are run-to-run identical either way. */
+int snhip_set_splitk_mode(void* handle, int mode);
 int snhip_config_count(void);
 /* desc[0..5] = BM, BN, BK, threads, LDS bytes, kind (0 fp32 kernel, 1 bf16-input kernel) */
 int snhip_config_desc(int config, int desc[6]);

@@ -46,7 +46,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 enum : int {
-    GEMM_FLAG_C_VEC = 1,  // C (and bias) may be accessed as aligned 16-byte vectors
+    GEMM_FLAG_C_VEC = 1,   // C (and bias) may be accessed as aligned 16-byte vectors
+    GEMM_FLAG_WS_VEC = 2,  // split-K workspace rows may be accessed as aligned 16-byte vectors (N % 4 == 0)
 };
 
 struct GemmParams {
@@ -55,6 +56,8 @@ struct GemmParams {
     float* C;           // destination; split-K partial sums go to ws instead
     const float* bias;  // optional, length N, added after alpha/beta
     float* ws;          // split-K workspace [batch][splitk][M][N], or nullptr
+    int* counters;      // split-K arrival counters [batch][tiles], all zero between launches; nullptr = reduce in a
+                        // second kernel
     int M, N, K;
     int lda, ldb, ldc;
     long long strideA, strideB, strideC;  // in elements
@@ -226,9 +229,15 @@ __device__ __forceinline__ void tile_coords(int bid, int ntiles, int tiles_m, in
 // Epilogue shared by the fp32 and bf16-input kernels.  acc[i][j][r] holds
 // C[row][col] with  row = row_base + TM*(8*(r/4) + 4*lhi + r%4) + i  and
 // col = col0 + j  (row_base = first row of the wavefront, col0 = first of the
-// TN consecutive columns this lane owns, lhi = lane / 32).  Writes
-// alpha*acc + beta*C + bias to C, or the raw partial sums to the split-K
-// workspace slice `zb`.  C is read only when beta != 0.
+// TN consecutive columns this lane owns, lhi = lane / 32).
+//
+// Without split-K: C = alpha*acc + beta*C + bias (C is read only when beta != 0).
+// With split-K the raw partial sums go to workspace slice `zb`.  If arrival
+// counters are supplied, the workgroup that arrives last for its tile (per-tile
+// atomic counter, release/acquire fences at device scope) adds the splitk
+// partial tiles in index order - every partial is re-read from memory, so the
+// sum does not depend on which workgroup happens to be last - and writes
+// alpha*sum + beta*C + bias.  Otherwise a second kernel does that reduction.
 template <int TM, int TN>
 __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], const GemmParams& p, int row_base,
                                                    int col0, int lhi, int zb, int batch) {
@@ -237,20 +246,22 @@ __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], 
     long long ldo;
     float alpha, beta;
     const float* bias;
+    bool vec_ok;
     if (to_ws) {
         out = p.ws + (long long)zb * p.M * p.N;
         ldo = p.N;
         alpha = 1.0f;
         beta = 0.0f;
         bias = nullptr;
+        vec_ok = (TN == 4) && (p.flags & GEMM_FLAG_WS_VEC) && (col0 + TN <= p.N);
     } else {
         out = p.C + (long long)batch * p.strideC;
         ldo = p.ldc;
         alpha = p.alpha;
         beta = p.beta;
         bias = p.bias;
+        vec_ok = (TN == 4) && (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
     }
-    const bool vec_ok = (TN == 4) && (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
 
     float bv[TN];
 #pragma unroll
@@ -281,6 +292,78 @@ __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], 
                     if (col0 + j < p.N) {
                         float o = v[j];
                         if (beta != 0.0f) o += beta * crow[j];
+                        crow[j] = o;
+                    }
+                }
+            }
+        }
+    }
+
+    if (!to_ws || p.counters == nullptr) return;
+
+    // ---- in-kernel split-K reduction by the last workgroup to arrive ----
+    __shared__ int s_is_last;
+    __threadfence();  // release: this thread's partial sums are visible device-wide
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int* cnt = p.counters + (long long)batch * gridDim.x + blockIdx.x;
+        const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = (old == p.splitk - 1);
+        if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+        s_is_last = last;
+    }
+    __syncthreads();
+    if (!s_is_last) return;
+    __threadfence();  // acquire: the other workgroups' partial sums are visible to every thread here
+
+    const long long mn = (long long)p.M * p.N;
+    const float* wsb = p.ws + (long long)batch * p.splitk * mn;
+    float* Cb = p.C + (long long)batch * p.strideC;
+    const bool ws_vec = (TN == 4) && (p.flags & GEMM_FLAG_WS_VEC) && (col0 + TN <= p.N);
+    const bool c_vec = (TN == 4) && (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
+    float cb[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) cb[j] = (p.bias != nullptr && col0 + j < p.N) ? p.bias[col0 + j] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
+            if (row >= p.M) continue;
+            const float* wrow = wsb + (long long)row * p.N + col0;
+            float sum[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) sum[j] = 0.0f;
+            for (int sidx = 0; sidx < p.splitk; ++sidx) {
+                const float* w = wrow + (long long)sidx * mn;
+                if (ws_vec) {
+                    if constexpr (TN == 4) {
+                        const f32x4 t = *reinterpret_cast<const f32x4*>(w);
+                        sum[0] += t.x;
+                        sum[1] += t.y;
+                        sum[2] += t.z;
+                        sum[3] += t.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        if (col0 + j < p.N) sum[j] += w[j];
+                }
+            }
+            float* crow = Cb + (long long)row * p.ldc + col0;
+            if (c_vec) {
+                if constexpr (TN == 4) {
+                    f32x4 o = {p.alpha * sum[0] + cb[0], p.alpha * sum[1] + cb[1], p.alpha * sum[2] + cb[2],
+                               p.alpha * sum[3] + cb[3]};
+                    if (p.beta != 0.0f) o += p.beta * *reinterpret_cast<const f32x4*>(crow);
+                    *reinterpret_cast<f32x4*>(crow) = o;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if (col0 + j < p.N) {
+                        float o = p.alpha * sum[j] + cb[j];
+                        if (p.beta != 0.0f) o += p.beta * crow[j];
                         crow[j] = o;
                     }
                 }

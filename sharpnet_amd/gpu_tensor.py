@@ -75,6 +75,10 @@ class GPUWrapper:
     def set_tuning(self, config=-1, splitk=0):
         check_status(self.lib.snhip_set_tuning(self.handle, config, splitk), "snhip_set_tuning")
 
+    def set_splitk_mode(self, mode):
+        """0 automatic, 1 reduce split-K partial sums in a second kernel, 2 in the GEMM kernel."""
+        check_status(self.lib.snhip_set_splitk_mode(self.handle, mode), "snhip_set_splitk_mode")
+
     def last_tuning(self):
         c, s = ctypes.c_int(), ctypes.c_int()
         check_status(self.lib.snhip_get_last_tuning(self.handle, ctypes.byref(c), ctypes.byref(s)))

@@ -93,6 +93,7 @@ SIGNATURES = {
     "snhip_device_info": [_vp, _c_int_p],
     "snhip_set_tuning": [_vp, _i, _i],
     "snhip_get_last_tuning": [_vp, _c_int_p, _c_int_p],
+    "snhip_set_splitk_mode": [_vp, _i],
     "snhip_config_count": [],
     "snhip_config_desc": [_i, _c_int_p],
 }

@@ -290,15 +290,53 @@ def test_degenerate_products(oracle, gpu_wrapper):
                            gc.Pointer, 4) == 7
 
 
-def test_run_to_run_determinism(gpu_wrapper):
-    """The reference opts into deterministic cuBLAS (GPUWrapper.cs:78-80); split-K must not use float atomics."""
+def test_run_to_run_determinism(oracle, gpu_wrapper):
+    """The reference opts into deterministic cuBLAS (GPUWrapper.cs:78-80); split-K must not use float atomics.
+    Both ways of adding the split-K partial sums (second kernel / last workgroup in the GEMM kernel) are covered."""
     rng = np.random.default_rng(8)
     try:
-        for (M, N, K, cfg, sk) in [(300, 200, 4096, -1, 0), (64, 64, 8192, 6, 8), (512, 512, 512, 0, 1)]:
-            gpu_wrapper.set_tuning(cfg, sk)
-            a, b = random_tensor(rng, (M, K)), random_tensor(rng, (K, N))
-            first = gpu_dot(gpu_wrapper, a, False, b, False, c_shape=[M, N])
-            for _ in range(3):
-                assert np.array_equal(first, gpu_dot(gpu_wrapper, a, False, b, False, c_shape=[M, N]))
+        for mode in (1, 2, 0):
+            gpu_wrapper.set_splitk_mode(mode)
+            for (M, N, K, cfg, sk) in [(300, 200, 4096, -1, 0), (64, 64, 8192, 6, 8), (512, 512, 512, 0, 1),
+                                       (256, 2048, 512, 6, 4), (1000, 64, 4096, 5, 16), (130, 70, 3000, 3, 8)]:
+                gpu_wrapper.set_tuning(cfg, sk)
+                a, b = random_tensor(rng, (M, K)), random_tensor(rng, (K, N))
+                c = random_tensor(rng, (M, N))
+                first = gpu_dot(gpu_wrapper, a, False, b, False, 0.5, 1.0, c=c)
+                assert np.max(np.abs(first - oracle.dot(a, False, b, False, 0.5, 1.0, c))) <= tol(K, a, b, 0.5, 1.0, c)
+                for _ in range(4):
+                    assert np.array_equal(first, gpu_dot(gpu_wrapper, a, False, b, False, 0.5, 1.0, c=c))
     finally:
         gpu_wrapper.set_tuning(-1, 0)
+        gpu_wrapper.set_splitk_mode(0)
+
+
+def test_splitk_modes_batched_and_bias(oracle, gpu_wrapper):
+    """In-kernel and two-kernel split-K reductions on a strided batch and with the fused bias."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    lib, h = gpu_wrapper.lib, gpu_wrapper.handle
+    rng = np.random.default_rng(9)
+    try:
+        for mode in (1, 2):
+            gpu_wrapper.set_splitk_mode(mode)
+            for cfg in (0, 3, 6):
+                gpu_wrapper.set_tuning(cfg, 4)
+                batch, M, N, K = 5, 70, 45, 1030
+                a, b = random_tensor(rng, (batch, M, K), -1, 1), random_tensor(rng, (batch, N, K), -1, 1)
+                ga, gb = GPUTensor(a.shape, a, gpu_wrapper), GPUTensor(b.shape, b, gpu_wrapper)
+                gc = GPUTensor([batch, M, N], None, gpu_wrapper)
+                gc.SetValue(float("nan"))
+                gc.BatchMatrixMultiplication(ga, False, gb, True, 0.25, 0.0)
+                assert gpu_wrapper.last_tuning() == (cfg, 4)
+                assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, False, b, True, 0.25))) <= tol(K, a, b, 0.25)
+                x, w_, bias = random_tensor(rng, (128, 784), 0, 1), random_tensor(rng, (256, 784), -0.07, 0.07), \
+                    random_tensor(rng, (256,), -1, 1)
+                gx, gw, gbias = (GPUTensor(t.shape, t, gpu_wrapper) for t in (x, w_, bias))
+                gy = GPUTensor([128, 256], None, gpu_wrapper)
+                gy.SetValue(float("nan"))
+                gy.DotRowMajor(gx, False, gw, True, 1.0, 0.0, bias=gbias)
+                assert np.max(np.abs(gy.ToNumpy() - oracle.dense_forward(x, w_, bias))) <= tol(784, x, w_) + 1e-6
+    finally:
+        gpu_wrapper.set_tuning(-1, 0)
+        gpu_wrapper.set_splitk_mode(0)
