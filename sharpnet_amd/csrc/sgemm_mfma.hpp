@@ -46,7 +46,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 enum : int {
-    GEMM_FLAG_C_VEC = 1,   // C (and bias) may be accessed as aligned 16-byte vectors
+    GEMM_FLAG_C_VEC = 1,   // C rows may be accessed as aligned vectors of up to 16 bytes (pointer, pitch, batch stride)
     GEMM_FLAG_WS_VEC = 2,  // split-K workspace rows may be accessed as aligned 16-byte vectors (N % 4 == 0)
 };
 
@@ -226,6 +226,30 @@ __device__ __forceinline__ void tile_coords(int bid, int ntiles, int tiles_m, in
     tn = in_g / gsz;
 }
 
+// TN consecutive floats as one vector access (TN = 1, 2 or 4); the caller has checked alignment.
+template <int TN>
+__device__ __forceinline__ void load_row_vec(const float* p, float (&v)[TN]) {
+    if constexpr (TN == 4) {
+        const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+        v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+    } else if constexpr (TN == 2) {
+        const f32x2 t = *reinterpret_cast<const f32x2*>(p);
+        v[0] = t.x, v[1] = t.y;
+    } else {
+        v[0] = p[0];
+    }
+}
+template <int TN>
+__device__ __forceinline__ void store_row_vec(float* p, const float (&v)[TN]) {
+    if constexpr (TN == 4) {
+        *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+    } else if constexpr (TN == 2) {
+        *reinterpret_cast<f32x2*>(p) = f32x2{v[0], v[1]};
+    } else {
+        p[0] = v[0];
+    }
+}
+
 // Epilogue shared by the fp32 and bf16-input kernels.  acc[i][j][r] holds
 // C[row][col] with  row = row_base + TM*(8*(r/4) + 4*lhi + r%4) + i  and
 // col = col0 + j  (row_base = first row of the wavefront, col0 = first of the
@@ -253,14 +277,14 @@ __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], 
         alpha = 1.0f;
         beta = 0.0f;
         bias = nullptr;
-        vec_ok = (TN == 4) && (p.flags & GEMM_FLAG_WS_VEC) && (col0 + TN <= p.N);
+        vec_ok = (p.flags & GEMM_FLAG_WS_VEC) && (col0 + TN <= p.N);
     } else {
         out = p.C + (long long)batch * p.strideC;
         ldo = p.ldc;
         alpha = p.alpha;
         beta = p.beta;
         bias = p.bias;
-        vec_ok = (TN == 4) && (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
+        vec_ok = (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
     }
 
     float bv[TN];
@@ -278,14 +302,13 @@ __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], 
 #pragma unroll
             for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r] + bv[j];
             if (vec_ok) {
-                if constexpr (TN == 4) {
-                    f32x4 o = {v[0], v[1], v[2], v[3]};
-                    if (beta != 0.0f) {
-                        const f32x4 c = *reinterpret_cast<const f32x4*>(crow);
-                        o += beta * c;
-                    }
-                    *reinterpret_cast<f32x4*>(crow) = o;
+                if (beta != 0.0f) {
+                    float c[TN];
+                    load_row_vec<TN>(crow, c);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) v[j] += beta * c[j];
                 }
+                store_row_vec<TN>(crow, v);
             } else {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
@@ -319,8 +342,8 @@ __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], 
     const long long mn = (long long)p.M * p.N;
     const float* wsb = p.ws + (long long)batch * p.splitk * mn;
     float* Cb = p.C + (long long)batch * p.strideC;
-    const bool ws_vec = (TN == 4) && (p.flags & GEMM_FLAG_WS_VEC) && (col0 + TN <= p.N);
-    const bool c_vec = (TN == 4) && (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
+    const bool ws_vec = (p.flags & GEMM_FLAG_WS_VEC) && (col0 + TN <= p.N);
+    const bool c_vec = (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
     float cb[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) cb[j] = (p.bias != nullptr && col0 + j < p.N) ? p.bias[col0 + j] : 0.0f;
@@ -337,13 +360,10 @@ __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], 
             for (int sidx = 0; sidx < p.splitk; ++sidx) {
                 const float* w = wrow + (long long)sidx * mn;
                 if (ws_vec) {
-                    if constexpr (TN == 4) {
-                        const f32x4 t = *reinterpret_cast<const f32x4*>(w);
-                        sum[0] += t.x;
-                        sum[1] += t.y;
-                        sum[2] += t.z;
-                        sum[3] += t.w;
-                    }
+                    float t[TN];
+                    load_row_vec<TN>(w, t);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) sum[j] += t[j];
                 } else {
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
@@ -352,12 +372,16 @@ __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], 
             }
             float* crow = Cb + (long long)row * p.ldc + col0;
             if (c_vec) {
-                if constexpr (TN == 4) {
-                    f32x4 o = {p.alpha * sum[0] + cb[0], p.alpha * sum[1] + cb[1], p.alpha * sum[2] + cb[2],
-                               p.alpha * sum[3] + cb[3]};
-                    if (p.beta != 0.0f) o += p.beta * *reinterpret_cast<const f32x4*>(crow);
-                    *reinterpret_cast<f32x4*>(crow) = o;
+                float o[TN];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) o[j] = p.alpha * sum[j] + cb[j];
+                if (p.beta != 0.0f) {
+                    float c[TN];
+                    load_row_vec<TN>(crow, c);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) o[j] += p.beta * c[j];
                 }
+                store_row_vec<TN>(crow, o);
             } else {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
@@ -480,8 +504,10 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     }
 
     static_assert(KS % 2 == 0, "fragment double-buffering across tiles needs an even number of k steps");
-    constexpr int KSW = (KS > 1) ? KS - 1 : 1;  // k steps that carry LDS stores (the last one carries the barrier)
-    constexpr int MID = (TM * TN) / 2;          // MFMA index of the last k step behind which the barrier sits
+    constexpr int MT = TM * TN;                 // MFMAs per k step
+    constexpr int MID = MT / 2;                 // MFMA slot of the last k step behind which the barrier sits
+    constexpr int G = (KS - 1) * MT + MID;      // MFMA slots of a tile that may carry staging work (before the barrier)
+    constexpr int NW = 2 * NP;                  // staging work items per tile: (store, refill) per piece
 
     // One k tile.  P selects the LDS buffer read; the register stage P^1 holds the
     // next tile and is refilled, piece by piece, with tile `fetch`.
@@ -501,54 +527,57 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             for (int i = 0; i < TM; ++i) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
+                    const int m = i * TN + j;      // MFMA slot inside the k step
+                    const int gslot = s * MT + m;  // MFMA slot inside the tile
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1].v[i], fb[s & 1].v[j], acc[i][j], 0, 0, 0);
-                    if (i == 0 && j == 0) {
-                        // Everything that is not an MFMA is issued right behind the first
-                        // MFMA of a k step and completes under the remaining ones: the LDS
-                        // reads of the next step and this step's share of the LDS stores,
-                        // each followed by the global load that refills its registers.
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (s + 1 < KS) {
-                            fa[(s + 1) & 1].load(as + (2 * (s + 1)) * PA);
-                            fb[(s + 1) & 1].load(bs + (2 * (s + 1)) * PB);
-                        }
-                        if (s < KSW) {
+                    // An MFMA occupies its SIMD's matrix pipe for 64 cycles and the wavefront cannot
+                    // issue the next one earlier, so whatever is placed between two MFMAs is free
+                    // as long as it issues within that shadow.  The non-MFMA work of a tile is
+                    // therefore spread thinly over its MFMA slots (the fences pin it there):
+                    __builtin_amdgcn_sched_barrier(0);
+                    // - the LDS reads of the next k step right behind the first MFMA of this one;
+                    if (m == 0 && s + 1 < KS) {
+                        fa[(s + 1) & 1].load(as + (2 * (s + 1)) * PA);
+                        fb[(s + 1) & 1].load(bs + (2 * (s + 1)) * PB);
+                    }
+                    // - the staging work items (store piece q to LDS, then refill its registers
+                    //   from global memory), item w in slot w*G/NW;
+                    if (gslot < G) {
 #pragma unroll
-                            for (int q = (s * NP) / KSW; q < ((s + 1) * NP) / KSW; ++q) {
-                                if (q < StageA::NV) {
-                                    const int v = q < StageA::NV ? q : 0;
+                        for (int w = 0; w < NW; ++w) {
+                            if ((w * G) / NW != gslot) continue;
+                            const int q = w / 2;
+                            const bool is_store = (w % 2 == 0);
+                            if (q < StageA::NV) {
+                                const int v = q < StageA::NV ? q : 0;
+                                if (is_store)
                                     sa.store_lds_vec(as_next, ra[Q][v], v);
-                                    if (fast)
-                                        sa.load_fast_vec(ra[Q][v], v);
-                                    else
-                                        sa.load_safe_vec(ra[Q][v], v, m_rem, k_rem);
-                                } else {
-                                    const int v = q >= StageA::NV ? q - StageA::NV : 0;
+                                else if (fast)
+                                    sa.load_fast_vec(ra[Q][v], v);
+                                else
+                                    sa.load_safe_vec(ra[Q][v], v, m_rem, k_rem);
+                            } else {
+                                const int v = q >= StageA::NV ? q - StageA::NV : 0;
+                                if (is_store)
                                     sb.store_lds_vec(bs_next, rb[Q][v], v);
-                                    if (fast)
-                                        sb.load_fast_vec(rb[Q][v], v);
-                                    else
-                                        sb.load_safe_vec(rb[Q][v], v, n_rem, k_rem);
-                                }
+                                else if (fast)
+                                    sb.load_fast_vec(rb[Q][v], v);
+                                else
+                                    sb.load_safe_vec(rb[Q][v], v, n_rem, k_rem);
                             }
                         }
-                        if (s + 1 == KS) {
-                            sa.advance();
-                            sb.advance();
-                            ++fetch;
-                        }
-                        __builtin_amdgcn_sched_barrier(0);
                     }
-                    if (s + 1 == KS && i * TN + j == MID) {
-                        // Half way through the last k step: the stores of the next tile were
-                        // issued a whole k step ago, so the barrier finds them complete, and
-                        // the first fragments of the next tile are read under the remaining MFMAs.
-                        __builtin_amdgcn_sched_barrier(0);
+                    // - half way through the last k step the barrier (the stores were issued at
+                    //   least half a k step earlier) and the first fragments of the next tile.
+                    if (s + 1 == KS && m == MID) {
+                        sa.advance();
+                        sb.advance();
+                        ++fetch;
                         lds_barrier();
                         fa[0].load(a_rd + Q * (BK * PA));
                         fb[0].load(b_rd + Q * (BK * PB));
-                        __builtin_amdgcn_sched_barrier(0);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
