@@ -150,6 +150,47 @@ struct TileStage {
         for (int v = 0; v < NV; ++v) load_safe_vec(r[v], v, mn_rem, k_rem);
     }
 
+    // Per-thread facts about a tile at the ragged edge of m/n, computed once per workgroup: they do not
+    // change from k tile to k tile, so full-k tiles of an edge block can be loaded without re-deriving them.
+    struct Edge {
+        long long off[KCONTIG ? NV : 1];  // KCONTIG: element offset of vector v from gptr, row clamped to the last valid one
+        int nv;                           // !KCONTIG: how many of this thread's 4 consecutive m/n are inside (<= 0: none)
+    };
+    __device__ __forceinline__ Edge edge_info(int mn_rem) const {
+        Edge e;
+        if (KCONTIG) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const int mn = mn0 + v * LINE_STEP;
+                e.off[v] = (long long)(((mn < mn_rem) ? mn : mn_rem - 1) - mn0) * ld;
+            }
+            e.nv = 4;
+        } else {
+            e.off[0] = 0;
+            e.nv = mn_rem - mn0;
+        }
+        return e;
+    }
+    // Load of a full-k tile of an edge block: plain vectors except for the (at most one per row) vector that
+    // straddles the edge of an m/n-contiguous operand; nothing past the matrix is touched.
+    __device__ __forceinline__ void load_edge_vec(f32x4& r, int v, const Edge& e) const {
+        if (KCONTIG) {
+            __builtin_memcpy(&r, gptr + e.off[v], 16);
+        } else {
+            const float* p = gptr + (long long)(v * LINE_STEP) * ld;
+            if (e.nv >= 4) {
+                __builtin_memcpy(&r, p, 16);
+            } else {
+                f32x4 x;
+                x.x = (e.nv > 0) ? p[0] : 0.0f;
+                x.y = (e.nv > 1) ? p[1] : 0.0f;
+                x.z = (e.nv > 2) ? p[2] : 0.0f;
+                x.w = 0.0f;
+                r = x;
+            }
+        }
+    }
+
     // vector v of this thread -> its place in the k-major LDS tile
     __device__ __forceinline__ void store_lds_vec(float* s, const f32x4& r, int v) const {
         if (KCONTIG) {
@@ -511,11 +552,14 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
 
     // One k tile.  P selects the LDS buffer read; the register stage P^1 holds the
     // next tile and is refilled, piece by piece, with tile `fetch`.
-    auto k_tile = [&](auto parity, auto steady) {
+    // MODE 0: tile `fetch` is a full tile of an interior block (unchecked loads);
+    // MODE 1: a full-k tile of an edge block (loads use the precomputed edge facts ea / eb);
+    // MODE 2: anything (each fetch decides between unchecked and fully checked loads).
+    auto k_tile = [&](auto parity, auto mode, const typename StageA::Edge& ea, const typename StageB::Edge& eb) {
         constexpr int P = decltype(parity)::value;
         constexpr int Q = P ^ 1;
-        // STEADY: the caller guarantees that tile `fetch` is a full tile of an interior block
-        const bool fast = decltype(steady)::value || (full_mn && (fetch < nk_full));
+        constexpr int MODE = decltype(mode)::value;
+        const bool fast = (MODE == 0) || (MODE == 2 && full_mn && (fetch < nk_full));
         const int k_rem = klen - fetch * BK;
         const float* as = a_rd + P * (BK * PA);
         const float* bs = b_rd + P * (BK * PB);
@@ -552,6 +596,8 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                                 const int v = q < StageA::NV ? q : 0;
                                 if (is_store)
                                     sa.store_lds_vec(as_next, ra[Q][v], v);
+                                else if (MODE == 1)
+                                    sa.load_edge_vec(ra[Q][v], v, ea);
                                 else if (fast)
                                     sa.load_fast_vec(ra[Q][v], v);
                                 else
@@ -560,6 +606,8 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                                 const int v = q >= StageA::NV ? q - StageA::NV : 0;
                                 if (is_store)
                                     sb.store_lds_vec(bs_next, rb[Q][v], v);
+                                else if (MODE == 1)
+                                    sb.load_edge_vec(rb[Q][v], v, eb);
                                 else if (fast)
                                     sb.load_fast_vec(rb[Q][v], v);
                                 else
@@ -585,18 +633,25 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
 
     using P0 = std::integral_constant<int, 0>;
     using P1 = std::integral_constant<int, 1>;
+    const typename StageA::Edge ea = sa.edge_info(m_rem);
+    const typename StageB::Edge eb = sb.edge_info(n_rem);
     int kt = 0;
+    // branch-free pairs of tiles while both fetches (tiles kt+3, kt+4) are full k tiles
     if (full_mn) {
-        // interior blocks: branch-free pairs of tiles while both fetches (tiles kt+3, kt+4) are full tiles
         for (; kt + 4 < nk_full; kt += 2) {
-            k_tile(P0{}, std::true_type{});
-            k_tile(P1{}, std::true_type{});
+            k_tile(P0{}, std::integral_constant<int, 0>{}, ea, eb);
+            k_tile(P1{}, std::integral_constant<int, 0>{}, ea, eb);
+        }
+    } else {
+        for (; kt + 4 < nk_full; kt += 2) {
+            k_tile(P0{}, std::integral_constant<int, 1>{}, ea, eb);
+            k_tile(P1{}, std::integral_constant<int, 1>{}, ea, eb);
         }
     }
-    // edge blocks and the last few tiles: same body, each fetch chooses checked or unchecked loads
+    // the last few tiles (K tail included): same body, each fetch chooses checked or unchecked loads
     for (; kt < nk; kt += 2) {
-        k_tile(P0{}, std::false_type{});
-        k_tile(P1{}, std::false_type{});
+        k_tile(P0{}, std::integral_constant<int, 2>{}, ea, eb);
+        k_tile(P1{}, std::integral_constant<int, 2>{}, ea, eb);
     }
 
     store_accumulators<TM, TN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch);

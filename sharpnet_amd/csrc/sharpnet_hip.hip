@@ -91,22 +91,21 @@ constexpr ConfigEntry make_entry_bf16(int occ, double eff_alone, double eff_shar
 // TM x TN MFMA tiles of 32x32, a workgroup is WM x WN wavefronts.
 const ConfigEntry kConfigs[] = {
     //                                      occ  alone shared edge
-    make_entry<TileCfg<4, 4, 2, 2, 16>>(1, 0.94, 0.94, 1.7),   // 0: 256 x 256
-    make_entry<TileCfg<2, 4, 2, 2, 16>>(1, 0.91, 0.91, 1.5),   // 1: 128 x 256
-    make_entry<TileCfg<4, 2, 2, 2, 16>>(1, 0.92, 0.92, 1.5),   // 2: 256 x 128
-    make_entry<TileCfg<2, 2, 2, 2, 16>>(2, 0.80, 0.87, 1.3),   // 3: 128 x 128
-    make_entry<TileCfg<1, 2, 2, 2, 16>>(3, 0.70, 0.82, 1.15),  // 4: 64 x 128
-    make_entry<TileCfg<2, 1, 2, 2, 16>>(3, 0.70, 0.82, 1.15),  // 5: 128 x 64
-    make_entry<TileCfg<1, 1, 2, 2, 16>>(5, 0.62, 0.75, 1.1),   // 6: 64 x 64
-    make_entry<TileCfg<4, 4, 2, 2, 32>>(1, 0.94, 0.94, 1.7),   // 7: 256 x 256, BK 32
-    make_entry<TileCfg<2, 2, 2, 2, 32>>(1, 0.80, 0.86, 1.3),   // 8: 128 x 128, BK 32
-    make_entry<TileCfg<2, 1, 2, 2, 32>>(2, 0.72, 0.82, 1.15),  // 9: 128 x 64, BK 32
-    make_entry<TileCfg<1, 1, 2, 2, 32>>(4, 0.60, 0.75, 1.1),   // 10: 64 x 64, BK 32
+    make_entry<TileCfg<4, 4, 2, 2, 16>>(1, 0.94, 0.94, 1.25),  // 0: 256 x 256
+    make_entry<TileCfg<2, 4, 2, 2, 16>>(1, 0.91, 0.91, 1.2),   // 1: 128 x 256
+    make_entry<TileCfg<4, 2, 2, 2, 16>>(1, 0.92, 0.92, 1.2),   // 2: 256 x 128
+    make_entry<TileCfg<2, 2, 2, 2, 16>>(2, 0.80, 0.87, 1.1),   // 3: 128 x 128
+    make_entry<TileCfg<1, 2, 2, 2, 16>>(3, 0.70, 0.82, 1.05),  // 4: 64 x 128
+    make_entry<TileCfg<2, 1, 2, 2, 16>>(3, 0.70, 0.82, 1.05),  // 5: 128 x 64
+    make_entry<TileCfg<1, 1, 2, 2, 16>>(5, 0.62, 0.75, 1.05),  // 6: 64 x 64
+    make_entry<TileCfg<2, 2, 2, 2, 32>>(1, 0.82, 0.86, 1.1),   // 7: 128 x 128, BK 32
+    make_entry<TileCfg<2, 1, 2, 2, 32>>(2, 0.72, 0.82, 1.05),  // 8: 128 x 64, BK 32
+    make_entry<TileCfg<1, 1, 2, 2, 32>>(4, 0.60, 0.75, 1.05),  // 9: 64 x 64, BK 32
     // bf16-input kernels (fp32 operands in memory: bound by the L2 -> LDS path long before the MFMA rate)
-    make_entry_bf16<BTileCfg<4, 4, 2, 2, 32>>(1, 0.80, 0.80, 1.7),   // 11: 256 x 256, BK 32
-    make_entry_bf16<BTileCfg<2, 2, 2, 2, 32>>(2, 0.60, 0.75, 1.3),   // 12: 128 x 128, BK 32
-    make_entry_bf16<BTileCfg<2, 1, 2, 2, 64>>(2, 0.50, 0.65, 1.15),  // 13: 128 x 64, BK 64
-    make_entry_bf16<BTileCfg<1, 1, 2, 2, 64>>(3, 0.40, 0.55, 1.1),   // 14: 64 x 64, BK 64
+    make_entry_bf16<BTileCfg<4, 4, 2, 2, 32>>(1, 0.80, 0.80, 4.0),   // 10: 256 x 256, BK 32
+    make_entry_bf16<BTileCfg<2, 2, 2, 2, 32>>(2, 0.60, 0.75, 1.3),   // 11: 128 x 128, BK 32
+    make_entry_bf16<BTileCfg<2, 1, 2, 2, 64>>(2, 0.45, 0.60, 1.15),  // 12: 128 x 64, BK 64
+    make_entry_bf16<BTileCfg<1, 1, 2, 2, 64>>(3, 0.45, 0.60, 1.1),   // 13: 64 x 64, BK 64
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -138,14 +137,15 @@ struct Choice {
 //  - the MFMA pipes: every CU works off ceil(blocks / num_cu) workgroups, one wavefront per SIMD each;
 //  - the per-tile critical path of a workgroup that has the CU to itself (LDS round trip + barrier);
 //  - HBM (unique operand bytes + C, plus the split-K partial sums);
-//  - the L2 -> LDS path (every workgroup re-reads its A and B panels).
+//  - the L2 -> LDS path (every workgroup re-reads its A and B panels), chip-wide and per CU.
 // Split-K adds a second launch that re-reads the partial sums.  Constants are fits to measurements on MI355X.
 double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int splitk, int num_cu) {
     constexpr double kTileLatency = 700.0;     // cycles per k tile when nothing hides the LDS/barrier latency
     constexpr double kFixed = 5000.0;          // prologue + epilogue of one workgroup
     constexpr double kStoreBytesPerCycle = 40; // C write-out rate of one CU
-    constexpr double kHbmBytesPerCycle = 1600; // ~3.8 TB/s streaming at 2.4 GHz
-    constexpr double kL2BytesPerCycle = 5000;  // ~12 TB/s aggregate L2 -> CU
+    constexpr double kHbmBytesPerCycle = 2000; // ~4.8 TB/s streaming at 2.4 GHz (what a plain copy reaches)
+    constexpr double kL2BytesPerCycle = 7000;  // ~17 TB/s aggregate L2 -> CU
+    constexpr double kCuBytesPerCycle = 40;    // what one CU can pull from L2 into LDS
     constexpr double kLaunch = 6000.0;
     constexpr double kSplitFixed = 20000.0;    // second launch + dependency gap
     const long long tiles_mn = (long long)ceil_div(M, c.BM) * ceil_div(N, c.BN);
@@ -166,7 +166,9 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
                              (splitk > 1 ? (double)batch * M * N * 4.0 * splitk : 0.0);
     const double t_mem = bytes_hbm / kHbmBytesPerCycle;
     const double t_l2 = (double)blocks * (c.BM + c.BN) * (double)kchunk * 4.0 / kL2BytesPerCycle;
+    const double t_cu = (double)per_cu * (c.BM + c.BN) * (double)kchunk * 4.0 / kCuBytesPerCycle + kFixed;
     double t = t_mfma;
+    if (t_cu > t) t = t_cu;
     if (t_lat > t) t = t_lat;
     if (t_mem > t) t = t_mem;
     if (t_l2 > t) t = t_l2;
