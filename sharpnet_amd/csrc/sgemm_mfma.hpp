@@ -511,10 +511,15 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     f32x4 ra[2][StageA::NV], rb[2][StageB::NV];
     int fetch = 0;  // index of the k tile the stage pointers address; tiles are fetched in order
 
-    // MFMA operand fragments, double-buffered over k steps; they live across k
-    // tiles because the first fragments of tile kt+1 are read at the end of tile kt.
-    Frag<TM> fa[2];
-    Frag<TN> fb[2];
+    // MFMA operand fragments: a ring of NB buffers over k steps, read D = NB-1 steps ahead of their use.
+    // With one or two MFMAs per k step a single step (64-128 cycles) does not cover an LDS round trip, so
+    // those configurations look three steps ahead.  The ring runs on across k tiles.
+    constexpr int MT = TM * TN;           // MFMAs per k step
+    constexpr int NB = (MT <= 2) ? 4 : 2;
+    constexpr int D = NB - 1;
+    static_assert(KS % NB == 0, "the fragment ring must divide the k steps of a tile");
+    Frag<TM> fa[NB];
+    Frag<TN> fb[NB];
     const float* const a_rd = As + lhi * PA + a_off;
     const float* const b_rd = Bs + lhi * PB + b_off;
 
@@ -540,15 +545,22 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             }
         }
         lds_barrier();
-        fa[0].load(a_rd);
-        fb[0].load(b_rd);
+#pragma unroll
+        for (int t = 0; t < D; ++t) {
+            fa[t].load(a_rd + (2 * t) * PA);
+            fb[t].load(b_rd + (2 * t) * PB);
+        }
     }
 
-    static_assert(KS % 2 == 0, "fragment double-buffering across tiles needs an even number of k steps");
-    constexpr int MT = TM * TN;                 // MFMAs per k step
-    constexpr int MID = MT / 2;                 // MFMA slot of the last k step behind which the barrier sits
-    constexpr int G = (KS - 1) * MT + MID;      // MFMA slots of a tile that may carry staging work (before the barrier)
-    constexpr int NW = 2 * NP;                  // staging work items per tile: (store, refill) per piece
+    // The barrier of a tile sits behind the first MFMA of k step SB = KS - D.  By then this wavefront has
+    // issued its last fragment read of the current LDS buffer (for step KS-1, issued at step SB-1) and all its
+    // stores of the next tile; once every wavefront is past it, the next tile may be read - the look-ahead
+    // reads of steps SB.. go there - and the current buffer may be overwritten by the tile after.
+    constexpr int SB = KS - D;
+    constexpr int G = SB * MT - (MT >= 2 ? MT / 2 : 1);  // MFMA slots that carry staging work: they end a little
+                                                         // before the barrier so its wait finds the stores done
+    constexpr int NW = 2 * NP;                           // staging work items per tile: (store, refill) per piece
+    static_assert(G >= 1, "no MFMA slot left for staging");
 
     // One k tile.  P selects the LDS buffer read; the register stage P^1 holds the
     // next tile and is refilled, piece by piece, with tile `fetch`.
@@ -573,16 +585,29 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                 for (int j = 0; j < TN; ++j) {
                     const int m = i * TN + j;      // MFMA slot inside the k step
                     const int gslot = s * MT + m;  // MFMA slot inside the tile
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1].v[i], fb[s & 1].v[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s % NB].v[i], fb[s % NB].v[j], acc[i][j], 0, 0, 0);
                     // An MFMA occupies its SIMD's matrix pipe for 64 cycles and the wavefront cannot
                     // issue the next one earlier, so whatever is placed between two MFMAs is free
                     // as long as it issues within that shadow.  The non-MFMA work of a tile is
                     // therefore spread thinly over its MFMA slots (the fences pin it there):
                     __builtin_amdgcn_sched_barrier(0);
-                    // - the LDS reads of the next k step right behind the first MFMA of this one;
-                    if (m == 0 && s + 1 < KS) {
-                        fa[(s + 1) & 1].load(as + (2 * (s + 1)) * PA);
-                        fb[(s + 1) & 1].load(bs + (2 * (s + 1)) * PB);
+                    // - behind the first MFMA of a k step: the tile's barrier (step SB only) and the
+                    //   LDS reads of the fragments needed D steps later, from this tile or the next;
+                    if (m == 0) {
+                        if (s == SB) {
+                            sa.advance();
+                            sb.advance();
+                            ++fetch;
+                            lds_barrier();
+                        }
+                        const int t = s + D;
+                        if (t < KS) {
+                            fa[t % NB].load(as + (2 * t) * PA);
+                            fb[t % NB].load(bs + (2 * t) * PB);
+                        } else {
+                            fa[t % NB].load(a_rd + Q * (BK * PA) + (2 * (t - KS)) * PA);
+                            fb[t % NB].load(b_rd + Q * (BK * PB) + (2 * (t - KS)) * PB);
+                        }
                     }
                     // - the staging work items (store piece q to LDS, then refill its registers
                     //   from global memory), item w in slot w*G/NW;
@@ -614,16 +639,6 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                                     sb.load_safe_vec(rb[Q][v], v, n_rem, k_rem);
                             }
                         }
-                    }
-                    // - half way through the last k step the barrier (the stores were issued at
-                    //   least half a k step earlier) and the first fragments of the next tile.
-                    if (s + 1 == KS && m == MID) {
-                        sa.advance();
-                        sb.advance();
-                        ++fetch;
-                        lds_barrier();
-                        fa[0].load(a_rd + Q * (BK * PA));
-                        fb[0].load(b_rd + Q * (BK * PB));
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
