@@ -147,6 +147,10 @@ int snhip_memcpy_htod_async(void* handle, void* dst, const void* src, size_t byt
 int snhip_memcpy_dtoh(void* handle, void* dst, const void* src, size_t bytes);
 int snhip_memcpy_dtod_async(void* handle, void* dst, const void* src, size_t bytes);
 int snhip_stream_synchronize(void* handle);
+/* Replace cuStreamCreate(flags 0) / cuStreamDestroy_v2 (Prod/GPU/StreamWrapper.cs:14,45); the stream is
+ * created at the default priority and can be given to snhip_set_stream. */
+int snhip_stream_create(void** stream);
+int snhip_stream_destroy(void* stream);
 
 /* ---- measurement helpers (no reference counterpart) ---------------------- */
 /* hipEvent wrappers recording on the handle's stream, for timing launches. */
@@ -169,6 +173,9 @@ int snhip_device_info(void* handle, int info[6]);
  * call selected.  config ids index the table in sharpnet_hip.hip. */
 int snhip_set_tuning(void* handle, int config, int splitk);
 int snhip_get_last_tuning(void* handle, int* config, int* splitk);
+/* What the automatic choice would be for a row-major M x N x K product of `batch` matrices (no launch, no
+ * device access).  handle may be NULL: the model then assumes an MI355X (256 CUs) and no overrides. */
+int snhip_query_tuning(void* handle, int m, int n, int k, int batch, int math_mode, int* config, int* splitk);
 /* How split-K partial sums are added: 0 = automatic (currently always a second kernel, the faster
  * choice on MI355X), 1 = a second kernel, 2 = in the GEMM kernel by the last workgroup to arrive for
  * its tile.  The order of summation is fixed in both, so results are run-to-run identical either way. */

@@ -263,6 +263,13 @@ int gemm_rm(Handle* h, bool tA, bool tB, int M, int N, int K, float alpha, const
             const float* bias, int math = -1) {
     if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     if (math < 0) math = h->math_mode;
+    {
+        // The handle belongs to one device (GPUWrapper.AssociateCurrentThreadWithDevice, GPUWrapper.cs:782-788);
+        // a caller thread whose current device differs is switched to it, as cudaSetDevice would have been.
+        int cur = -1;
+        if (hipGetDevice(&cur) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+        if (cur != h->device && hipSetDevice(h->device) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    }
     if (M < 0 || N < 0 || K < 0 || batch < 0) return SNHIP_STATUS_INVALID_VALUE;
     if (M == 0 || N == 0 || batch == 0) return SNHIP_STATUS_SUCCESS;
     if (C == nullptr || ldc < N) return SNHIP_STATUS_INVALID_VALUE;
@@ -627,6 +634,21 @@ int snhip_memcpy_dtod_async(void* handle, void* dst, const void* src, size_t byt
     return hip_to_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<Handle*>(handle)->stream));
 }
 
+int snhip_stream_create(void** stream) {
+    if (stream == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipStream_t st = nullptr;
+    // default priority, blocking with respect to the null stream: the flags-0 stream of StreamWrapper.cs:14
+    hipError_t e = hipStreamCreateWithFlags(&st, hipStreamDefault);
+    if (e != hipSuccess) return hip_to_status(e);
+    *stream = st;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_stream_destroy(void* stream) {
+    if (stream == nullptr) return SNHIP_STATUS_SUCCESS;
+    return hip_to_status(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+}
+
 int snhip_stream_synchronize(void* handle) {
     if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     return hip_to_status(hipStreamSynchronize(static_cast<Handle*>(handle)->stream));
@@ -698,6 +720,18 @@ int snhip_set_tuning(void* handle, int config, int splitk) {
     Handle* h = static_cast<Handle*>(handle);
     h->force_cfg = config < 0 ? -1 : config;
     h->force_splitk = splitk;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_query_tuning(void* handle, int m, int n, int k, int batch, int math_mode, int* config, int* splitk) {
+    if (m <= 0 || n <= 0 || k <= 0 || batch <= 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (math_mode != SNHIP_MATH_FP32 && math_mode != SNHIP_MATH_BF16_INPUT) return SNHIP_STATUS_INVALID_VALUE;
+    Handle model;  // without a handle: an MI355X with 256 CUs, no overrides
+    const Handle* h = handle != nullptr ? static_cast<const Handle*>(handle) : &model;
+    Choice ch = choose(h, m, n, k, batch, math_mode);
+    if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
+    if (config != nullptr) *config = ch.cfg;
+    if (splitk != nullptr) *splitk = ch.splitk;
     return SNHIP_STATUS_SUCCESS;
 }
 

@@ -85,6 +85,8 @@ SIGNATURES = {
     "snhip_memcpy_dtoh": [_vp, _vp, _vp, _sz],
     "snhip_memcpy_dtod_async": [_vp, _vp, _vp, _sz],
     "snhip_stream_synchronize": [_vp],
+    "snhip_stream_create": [_vpp],
+    "snhip_stream_destroy": [_vp],
     "snhip_event_create": [_vpp],
     "snhip_event_destroy": [_vp],
     "snhip_event_record": [_vp, _vp],
@@ -94,6 +96,7 @@ SIGNATURES = {
     "snhip_set_tuning": [_vp, _i, _i],
     "snhip_get_last_tuning": [_vp, _c_int_p, _c_int_p],
     "snhip_set_splitk_mode": [_vp, _i],
+    "snhip_query_tuning": [_vp, _i, _i, _i, _i, _i, _c_int_p, _c_int_p],
     "snhip_config_count": [],
     "snhip_config_desc": [_i, _c_int_p],
 }

@@ -66,3 +66,42 @@ def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     from sharpnet_amd import hiplib
     with pytest.raises(FileNotFoundError):
         hiplib.load_library(str(tmp_path / "libsharpnet_hip.so"))
+
+
+def test_tile_choice_model_is_sane_without_gpu():
+    """The configuration/split-K choice is pure host arithmetic: check its invariants over many shapes."""
+    import ctypes
+    import itertools
+    from sharpnet_amd import hiplib
+    lib = hiplib.load_library()
+    ncfg = lib.snhip_config_count()
+    descs = []
+    for i in range(ncfg):
+        d = (ctypes.c_int * 6)()
+        assert lib.snhip_config_desc(i, d) == 0
+        descs.append(list(d))
+    dims = [1, 2, 63, 64, 65, 256, 1000, 1024, 4097, 8192, 32768]
+    for math in (0, 1):
+        for M, N, K in itertools.product(dims, repeat=3):
+            if M * N > (1 << 28):
+                continue
+            for batch in (1, 7, 512):
+                if M * N * batch > (1 << 28):
+                    continue
+                c, s = ctypes.c_int(-1), ctypes.c_int(-1)
+                assert lib.snhip_query_tuning(None, M, N, K, batch, math, ctypes.byref(c), ctypes.byref(s)) == 0
+                BM, BN, BK, NT, lds, kind = descs[c.value]
+                assert kind == math                                  # a kernel of the requested arithmetic
+                assert 1 <= s.value <= 32 and batch * s.value <= 65535
+                assert M * N * batch * s.value * 4 <= (1 << 30) or s.value == 1      # workspace cap
+                if s.value > 1:
+                    kchunk = -(-(-(-K // s.value)) // BK) * BK
+                    assert kchunk * (s.value - 1) < K                # no empty split
+                    assert K // s.value >= 4 * BK                    # splits keep a few k tiles each
+                assert lds <= 160 * 1024
+    # the headline shape gets the largest fp32 tile and no split
+    c, s = ctypes.c_int(), ctypes.c_int()
+    assert lib.snhip_query_tuning(None, 8192, 8192, 8192, 1, 0, ctypes.byref(c), ctypes.byref(s)) == 0
+    assert (descs[c.value][0], descs[c.value][1], s.value) == (256, 256, 1)
+    assert lib.snhip_query_tuning(None, 0, 8, 8, 1, 0, ctypes.byref(c), ctypes.byref(s)) == 7
+    assert lib.snhip_query_tuning(None, 8, 8, 8, 1, 5, ctypes.byref(c), ctypes.byref(s)) == 7

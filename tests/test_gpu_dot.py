@@ -340,3 +340,35 @@ def test_splitk_modes_batched_and_bias(oracle, gpu_wrapper):
     finally:
         gpu_wrapper.set_tuning(-1, 0)
         gpu_wrapper.set_splitk_mode(0)
+
+
+def test_limits_and_user_stream(oracle, gpu_wrapper):
+    """Batch counts beyond the grid limit are refused with a status; a caller-supplied stream is honoured."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    lib, h = gpu_wrapper.lib, gpu_wrapper.handle
+    rng = np.random.default_rng(10)
+    tiny = GPUTensor([70000, 1, 1], np.ones(70000, np.float32), gpu_wrapper)
+    out = GPUTensor([70000, 1, 1], None, gpu_wrapper)
+    # 70000 matrices > 65535: status 15 (NOT_SUPPORTED), nothing launched
+    assert lib.snhip_bmm(h, tiny.Pointer, 1, 1, 0, 1, tiny.Pointer, 1, 1, 0, 1, out.Pointer, 1, 70000, 1.0, 0.0) == 15
+    # the largest supported batch works
+    assert lib.snhip_bmm(h, tiny.Pointer, 1, 1, 0, 1, tiny.Pointer, 1, 1, 0, 1, out.Pointer, 1, 65535, 2.0, 0.0) == 0
+    assert np.all(out.ToNumpy().reshape(-1)[:65535] == 2.0)
+    # K == 0 on a batch: C = beta * C
+    c0 = random_tensor(rng, (4, 3, 5))
+    gc = GPUTensor([4, 3, 5], c0, gpu_wrapper)
+    assert lib.snhip_bmm(h, tiny.Pointer, 3, 0, 0, 0, tiny.Pointer, 0, 5, 0, 0, gc.Pointer, 15, 4, 1.0, 0.5) == 0
+    assert np.allclose(gc.ToNumpy(), 0.5 * c0, atol=1e-7)
+    # caller-supplied stream
+    import ctypes
+    st = ctypes.c_void_p()
+    check_status(lib.snhip_stream_create(ctypes.byref(st)))
+    try:
+        check_status(lib.snhip_set_stream(h, st))
+        a, b = random_tensor(rng, (300, 500)), random_tensor(rng, (500, 200))
+        got = gpu_dot(gpu_wrapper, a, False, b, False, c_shape=[300, 200], prefill=float("nan"))
+        assert np.max(np.abs(got - oracle.dot(a, False, b, False))) <= tol(500, a, b)
+    finally:
+        check_status(lib.snhip_set_stream(h, None))
+        check_status(lib.snhip_stream_destroy(st))
