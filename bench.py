@@ -39,6 +39,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--table", default=None, metavar="PATH",
+                    help="also write the per-configuration figures of `extra` as a markdown table to PATH")
+    ap.add_argument("--pcie", action="store_true",
+                    help="also time the headline GEMM with host->device upload of A, B and device->host download of C")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: 3 plain copies of 1 GiB, then 3 headline GEMMs")
     args = ap.parse_args()
@@ -155,6 +159,26 @@ def main():
         "parity": {"max_abs_err": err, "bound": bound, "rows_checked": 16},
     }
 
+    if args.pcie:
+        # what a caller with host-resident operands would see: upload A and B, multiply, download C (pageable host memory)
+        ga, gb = GPUTensor(list(a.shape), None, w), GPUTensor(list(b.shape), None, w)
+        gcp = GPUTensor([g.M, g.N], None, w)
+        ts = []
+        for _ in range(3):
+            w.synchronize()
+            t0 = time.perf_counter()
+            ga.InitializeFromHostMemory(a)
+            gb.InitializeFromHostMemory(b)
+            gcp.Dot(ga, False, gb, False, 1.0, 0.0)
+            gcp.ContentAsFloatArray()
+            ts.append(time.perf_counter() - t0)
+        t_pcie = float(np.median(ts))
+        out["pcie_inclusive"] = {"ms": round(t_pcie * 1e3, 2), "tflops": round(g.flops / t_pcie / 1e12, 2),
+                                 "note": "H2D of A and B (2 x 268 MB), kernel, D2H of C (268 MB), pageable host memory"}
+        log("[bench] PCIe-inclusive:", out["pcie_inclusive"])
+        for t in (ga, gb, gcp):
+            t.Dispose()
+
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     if not args.no_cpu:
         cores = dot_oracle.mkl_threads()
@@ -222,7 +246,37 @@ def main():
         for k, v in extra.items():
             log("[bench]", k, json.dumps(v))
 
+    if args.table and "extra" in out:
+        write_table(args.table, out)
     print(json.dumps(out), flush=True)
+
+
+def write_table(path, out):
+    """Markdown rendering of the `extra` object (one row per GEMM) plus the headline figures of the same run."""
+    rows = []
+    for name, v in out["extra"].items():
+        items = v if isinstance(v, list) else v.get("gemms") or [x for x in v.values() if isinstance(x, dict)] or [v]
+        if isinstance(v, dict) and "gemm" in v:
+            items = [v]
+        for r in items:
+            rows.append("| %s | %s | %.4f | %.1f | %.3f | %d | %d |" % (name, r["gemm"], r["ms"], r["tflops"],
+                                                                       r["frac_of_roofline"], r["tile_config"], r["splitk"]))
+        if isinstance(v, dict) and "total_ms" in v:
+            rows.append("| %s | all nine GEMMs | %.4f | %.1f | | | |" % (name, v["total_ms"], v["tflops"]))
+    cpu = out.get("cpu_baseline")
+    with open(path, "w") as f:
+        f.write("# Per-configuration GPU figures (MI355X, one GPU, fp32 unless noted)\n\n"
+                "Command: `python bench.py --table %s` (the table is the `extra` object of its JSON line). time = HIP events\n"
+                "around the timed launches; fraction = max(flops / 157.3 TFLOP/s, bytes / 8 TB/s) / time (bf16-input rows:\n"
+                "against the 2.5 PFLOP/s bf16 peak or 8 TB/s); tile config = index into `snhip_config_desc`.\n\n"
+                "| configuration | GEMM | ms | TFLOP/s | fraction of roofline | tile config | split-K |\n"
+                "|---|---|---|---|---|---|---|\n" % path)
+        f.write("\n".join(rows) + "\n\n")
+        f.write("Headline line of the same run: %.2f TFLOP/s (%.1f %% of fp32 MFMA peak)" %
+                (out["value"], 100.0 * out["roofline"]["frac"]))
+        if cpu:
+            f.write(", CPU baseline (%d threads): %.2f TFLOP/s" % (cpu["cores"], cpu["value"]))
+        f.write(".\n")
 
 
 if __name__ == "__main__":

@@ -372,3 +372,53 @@ def test_limits_and_user_stream(oracle, gpu_wrapper):
     finally:
         check_status(lib.snhip_set_stream(h, None))
         check_status(lib.snhip_stream_destroy(st))
+
+
+def test_random_shapes_offsets_and_pitches(oracle, gpu_wrapper):
+    """300 seeded random cases through snhip_gemm_rm: shapes up to 400, all transposes, random alpha/beta, padded
+    leading dimensions, element offsets (4-byte alignment only), strided batches, optional bias; automatic tiling."""
+    from sharpnet_amd import GPUTensor
+    lib, h = gpu_wrapper.lib, gpu_wrapper.handle
+    rng = np.random.default_rng(2024)
+    for case in range(300):
+        M, N, K = (int(rng.integers(1, 400)) for _ in range(3))
+        if case % 7 == 0:
+            K = int(rng.integers(400, 3000))
+        tA, tB = bool(rng.integers(2)), bool(rng.integers(2))
+        batch = int(rng.choice([1, 1, 1, 2, 5]))
+        alpha = float(rng.choice([1.0, -1.0, 0.5, 0.125, 2.0]))
+        beta = float(rng.choice([0.0, 0.0, 1.0, -0.5]))
+        use_bias = bool(rng.integers(2)) and batch == 1
+        ar, ac = (K, M) if tA else (M, K)
+        br, bc = (N, K) if tB else (K, N)
+        lda, ldb, ldc = ac + int(rng.integers(0, 4)), bc + int(rng.integers(0, 4)), N + int(rng.integers(0, 4))
+        offa, offb, offc = (int(rng.integers(0, 4)) for _ in range(3))
+        sA, sB, sC = ar * lda + int(rng.integers(0, 3)), br * ldb + int(rng.integers(0, 3)), M * ldc + int(rng.integers(0, 3))
+        bufA = random_tensor(rng, (offa + batch * sA + 4,), -1, 1)
+        bufB = random_tensor(rng, (offb + batch * sB + 4,), -1, 1)
+        bufC = random_tensor(rng, (offc + batch * sC + 4,), -1, 1)
+        bias = random_tensor(rng, (N,), -1, 1) if use_bias else None
+        gA, gB, gC = (GPUTensor([x.size], x, gpu_wrapper) for x in (bufA, bufB, bufC))
+        gbias = GPUTensor([N], bias, gpu_wrapper) if use_bias else None
+        st = lib.snhip_gemm_rm(h, int(tA), int(tB), M, N, K, alpha, gA.Pointer + 4 * offa, lda, sA,
+                               gB.Pointer + 4 * offb, ldb, sB, beta, gC.Pointer + 4 * offc, ldc, sC, batch,
+                               gbias.Pointer if use_bias else None)
+        assert st == 0, (case, st)
+        got = gC.ToNumpy()
+        want = bufC.copy()
+        for i in range(batch):
+            a = bufA[offa + i * sA: offa + i * sA + ar * lda].reshape(ar, lda)[:, :ac]
+            b = bufB[offb + i * sB: offb + i * sB + br * ldb].reshape(br, ldb)[:, :bc]
+            cview = want[offc + i * sC: offc + i * sC + M * ldc].reshape(M, ldc)
+            ref = oracle.dot(np.ascontiguousarray(a), tA, np.ascontiguousarray(b), tB, alpha, beta,
+                             np.ascontiguousarray(cview[:, :N]) if beta != 0 else None)
+            if use_bias:
+                ref = ref + bias[None, :]
+            gview = got[offc + i * sC: offc + i * sC + M * ldc].reshape(M, ldc)
+            err = float(np.max(np.abs(gview[:, :N] - ref)))
+            assert err <= tol(K, a, b, alpha, beta, cview) + 1e-6, (case, M, N, K, tA, tB, batch, alpha, beta, err)
+            cview[:, :N] = gview[:, :N]
+        # everything outside the M x N windows (padding columns, gaps between matrices, offsets) is untouched
+        assert np.array_equal(got, want), (case, "padding overwritten")
+        for t in (gA, gB, gC):
+            t.Dispose()
