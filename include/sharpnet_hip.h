@@ -97,6 +97,76 @@ int snhip_gemm_rm(void* handle, int transposeA, int transposeB, int M, int N, in
                   int lda, long long strideA, const float* B, int ldb, long long strideB, float beta, float* C,
                   int ldc, long long strideC, int batch, const float* bias);
 
+/* ---- fused Linear-layer forms ---------------------------------------------- */
+/* Element-wise functions the GEMM epilogue can apply; the reference runs them as the ActivationLayer that follows
+ * a Linear layer (cudnnActivationMode_t RELU / LEAKY_RELU / SIGMOID / TANH, Prod/GPU/CudnnWrapper.cs:267-281;
+ * definitions Prod/CPU/CpuTensorActivationFunctions.cs:184-245). */
+#define SNHIP_ACT_NONE 0
+#define SNHIP_ACT_RELU 1
+#define SNHIP_ACT_LEAKY_RELU 2 /* activation_param = slope for x < 0 */
+#define SNHIP_ACT_SIGMOID 3
+#define SNHIP_ACT_TANH 4
+
+/* One launch, everything optional beyond the product itself (row-major, strided batch of `batch` matrices):
+ *     C[z] = act(alpha * op(A[z]) . op(B[z]) + bias[col] + beta * C[z] + gamma * D[z])
+ *     colsum[z][m] = sum_k op(A[z])[m][k]                       (transA = 1 only)
+ * Matrix z of operand X sits at X + (z / batch_inner) * strideX_outer + (z % batch_inner) * strideX; batch_inner = 0
+ * means a single level (strideX only).  The two levels let the heads of a (batch, time, heads * dim) activation be
+ * multiplied in place (lda = heads * dim, strideX = dim, strideX_outer = time * heads * dim), which replaces the
+ * reference's TransposeSecondAndThirdDimension copies (Prod/Layers/MultiheadAttention.cs:207-227).
+ * gamma * D is the weight-decay term of Prod/Layers/Linear.cs:168-178; colsum is Compute_BiasGradient_from_dy
+ * (Linear.cs:160-165) taken from the dy tiles the dW product reads anyway.
+ * Zero-initialise the struct, set struct_size = sizeof(snhip_gemm_desc), then fill what is needed. */
+typedef struct snhip_gemm_desc {
+    int struct_size;
+    int transA, transB;
+    int M, N, K;
+    float alpha, beta;
+    const float* A;
+    const float* B;
+    float* C;
+    int lda, ldb, ldc;
+    int batch;       /* number of matrices (>= 1) */
+    int batch_inner; /* 0, or the number of matrices per outer step (must divide batch) */
+    long long strideA, strideB, strideC;                   /* elements */
+    long long strideA_outer, strideB_outer, strideC_outer; /* elements; used when 0 < batch_inner < batch */
+    const float* bias; /* length N, or NULL */
+    const float* D;    /* M x N addend with row pitch ldd, or NULL */
+    int ldd;
+    long long strideD, strideD_outer;
+    float gamma;
+    int activation; /* SNHIP_ACT_* */
+    float activation_param;
+    float* colsum; /* [batch][M], or NULL */
+    int math;      /* -1: the handle's math mode, else SNHIP_MATH_* */
+} snhip_gemm_desc;
+int snhip_gemm_ex(void* handle, const snhip_gemm_desc* desc);
+/* sizeof(snhip_gemm_desc) as this library was built: lets a binding check its own struct layout (returns the size,
+ * not a status). */
+int snhip_sizeof_gemm_desc(void);
+
+/* y[rows x out] = act(x[rows x in] . W^T + bias), W stored (out, in): Linear.DenseForwardPropagation
+ * (Prod/Layers/Linear.cs:125-132) with the following ActivationLayer folded in (SNHIP_ACT_NONE for none). */
+int snhip_dense_forward(void* handle, float* y, const float* x, const float* weights, const float* bias, int rows,
+                        int in_features, int out_features, int activation, float activation_param);
+
+/* Linear.DenseBackwardPropagation (Prod/Layers/Linear.cs:143-191) in at most two launches:
+ *   weight_gradients = multiplier * dy^T . x + weight_decay_alpha * weights   (Linear.cs:151-158,168-178)
+ *   bias_gradients   = column sums of dy, or NULL to skip                    (Linear.cs:160-165)
+ *   dx               = dy . weights, or NULL when the previous layer is the input (Linear.cs:184-190)
+ * multiplier is 1/batch or 1 by compatibility mode; weight_decay_alpha = k * batch * weight_decay (0: none). */
+int snhip_dense_backward(void* handle, float* dx, float* weight_gradients, float* bias_gradients, const float* x,
+                         const float* dy, const float* weights, int rows, int in_features, int out_features,
+                         float multiplier, float weight_decay_alpha);
+
+/* y = act(x) and dx = dy * act'(x) expressed through y, element-wise over n floats (in place allowed):
+ * Tensor.ActivationForward / ActivationBackward for the modes above (Prod/GPU/GpuTensor.cs ActivationForward,
+ * Prod/CPU/CpuTensorActivationFunctions.cs:184-245). */
+int snhip_activation_forward(void* handle, int activation, float activation_param, const float* x, float* y,
+                             long long n);
+int snhip_activation_backward(void* handle, int activation, float activation_param, const float* y, const float* dy,
+                              float* dx, long long n);
+
 /* ---- bf16-input / fp32-accumulate variant (no reference counterpart) ------ */
 /* Operands stay fp32 in device memory; they are rounded to bf16 (nearest even)
  * on their way into LDS and multiplied with v_mfma_f32_32x32x16_bf16, products

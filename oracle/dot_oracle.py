@@ -21,6 +21,13 @@ sgemm_colmajor                          cuBLAS SGEMM as called at               
                                         Prod/GPU/GpuTensor.cs:1192,1218
 dense_forward / dense_backward          Prod/Layers/Linear.cs:125-191                loss fixture ParallelRunWithPyTorch.cs:102-138,
                                                                                      TestNetworkPropagation.cs:36-105
+activation_forward /                    Prod/CPU/CpuTensorActivationFunctions.cs     relu + its gradient: the loss fixture above (the
+activation_backward                     :184-245 (tanh, relu, leaky relu, sigmoid)   ReLU sits between its two Linear layers); sigmoid:
+                                                                                     stored predictions TestNetworkPropagation.cs:36-105;
+                                                                                     tanh / leaky: identities tanh x = 2 s(2x) - 1,
+                                                                                     leaky(x,a) = relu(x) - a relu(-x); every gradient:
+                                                                                     central finite differences of the forward
+dense_backward(weight_decay_alpha)      Prod/Layers/Linear.cs:168-178                linearity: dW(alpha) - dW(0) == alpha * W exactly
 softmax_last_dim                        Prod/CPU/CpuTensorActivationFunctions.cs     attention loss fixture (same file :963-1010)
                                         :19-46
 sdpa_forward                            Prod/Layers/ScaledDotProductAttention        same
@@ -184,17 +191,56 @@ def dense_forward(x, weights, bias=None, flatten_last=False):
     return y
 
 
-def dense_backward(x, dy, weights, multiplier=1.0, prev_is_input=False, flatten_last=False):
-    """Linear.DenseBackwardPropagation (Linear.cs:142-191) without weight decay.
+def activation_forward(x, mode, alpha=0.0):
+    """Tensor.ActivationForward for 'relu' (max(0,x)), 'leaky_relu' (x >= 0 ? x : alpha x), 'sigmoid', 'tanh'
+    (CpuTensorActivationFunctions.cs:184-245), float32 in and out."""
+    x = np.asarray(x, dtype=np.float32)
+    if mode in (None, "identity"):
+        return x.copy()
+    if mode == "relu":
+        return np.maximum(x, np.float32(0))
+    if mode == "leaky_relu":
+        return np.where(x >= 0, x, np.float32(alpha) * x).astype(np.float32)
+    if mode == "sigmoid":
+        return (1.0 / (1.0 + np.exp(-x.astype(np.float64)))).astype(np.float32)
+    if mode == "tanh":
+        return np.tanh(x.astype(np.float64)).astype(np.float32)
+    raise ValueError(mode)
 
-    Returns (dW, db, dx): dW = multiplier * dy^T . x (:158), db = column sums of dy (:164),
-    dx = dy . W (:190) or None when the previous layer is the input layer (:184-187).
+
+def activation_backward(y, dy, mode, alpha=0.0):
+    """dx from the OUTPUT y of the activation and dy, as the reference's CPU gradients are written
+    (ReluGradient :202-206 y > 0, LeakyReluGradient :214-219 y >= 0 ? dy : alpha dy, SigmoidGradient :240-244
+    dy y (1 - y), TanhGradient :190-194 dy (1 - y^2))."""
+    y = np.asarray(y, dtype=np.float32)
+    dy = np.asarray(dy, dtype=np.float32)
+    if mode in (None, "identity"):
+        return dy.copy()
+    if mode == "relu":
+        return np.where(y > 0, dy, np.float32(0)).astype(np.float32)
+    if mode == "leaky_relu":
+        return np.where(y >= 0, dy, np.float32(alpha) * dy).astype(np.float32)
+    if mode == "sigmoid":
+        return (dy * y * (np.float32(1) - y)).astype(np.float32)
+    if mode == "tanh":
+        return (dy * (np.float32(1) - y * y)).astype(np.float32)
+    raise ValueError(mode)
+
+
+def dense_backward(x, dy, weights, multiplier=1.0, prev_is_input=False, flatten_last=False, weight_decay_alpha=0.0):
+    """Linear.DenseBackwardPropagation (Linear.cs:142-191).
+
+    Returns (dW, db, dx): dW = multiplier * dy^T . x (:158) + weight_decay_alpha * W (:168-178, alpha as computed
+    there: k * batch * weight_decay), db = column sums of dy (:164), dx = dy . W (:190) or None when the previous
+    layer is the input layer (:184-187).
     """
     x = np.asarray(x, dtype=np.float32)
     dy = np.asarray(dy, dtype=np.float32)
     x2 = x.reshape(-1, x.shape[-1]) if flatten_last else x.reshape(x.shape[0], -1)
     dy2 = dy.reshape(-1, dy.shape[-1]) if flatten_last else dy.reshape(dy.shape[0], -1)
     dW = dot(dy2, True, x2, False, multiplier, 0.0)
+    if weight_decay_alpha:
+        dW = (dW + np.float32(weight_decay_alpha) * np.asarray(weights, dtype=np.float32)).astype(np.float32)
     db = dy2.astype(np.float64).sum(axis=0).astype(np.float32)
     dx = None if prev_is_input else dot(dy2, False, weights, False, 1.0, 0.0)
     return dW, db, dx

@@ -348,7 +348,7 @@ __global__ void __launch_bounds__(CFG::NT) bgemm_mfma_kernel(const GemmParams p)
         k_tile(P1{}, std::false_type{});
     }
 
-    store_accumulators<TM, TN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch);
+    store_accumulators_plain<TM, TN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch);
 }
 
 }  // namespace snhip

@@ -10,9 +10,11 @@
 
 #include <new>
 
-#include "bgemm_mfma.hpp"
+#include "kernel_list.hpp"
 #include "rowops.hpp"
-#include "sgemm_mfma.hpp"
+
+// The GEMM kernels are compiled in gemm_kernels.hip; here they are only declared.
+SNHIP_ALL_KERNEL_GROUPS(SNHIP_DECLARE_KERNELS)
 
 using namespace snhip;
 
@@ -46,6 +48,8 @@ struct ConfigEntry {
     int mfma_per_k2;    // TM*TN: MFMA instructions one wavefront issues per MFMA k step
     int kind;           // 0: fp32 kernel (k step 2, 64 cycles per MFMA), 1: bf16-input kernel (k step 16, 32 cycles)
     KernelFn fn[2][2];  // [transposeA][transposeB]
+    KernelFn fn_ext[2][2];  // the same with the extended write-out (addend, ReLU, two-level batch, column sum);
+                            // nullptr if not built
     // cost-model inputs, calibrated on MI355X
     int occ;            // workgroups that fit on one CU (registers / LDS)
     double eff_alone;   // fraction of the MFMA issue rate reached with one workgroup per CU
@@ -64,6 +68,8 @@ constexpr ConfigEntry make_entry(int occ, double eff_alone, double eff_shared, d
                        0,
                        {{sgemm_mfma_kernel<CFG, false, false>, sgemm_mfma_kernel<CFG, false, true>},
                         {sgemm_mfma_kernel<CFG, true, false>, sgemm_mfma_kernel<CFG, true, true>}},
+                       {{sgemm_mfma_kernel<CFG, false, false, true>, sgemm_mfma_kernel<CFG, false, true, true>},
+                        {sgemm_mfma_kernel<CFG, true, false, true>, sgemm_mfma_kernel<CFG, true, true, true>}},
                        occ,
                        eff_alone,
                        eff_shared,
@@ -81,6 +87,7 @@ constexpr ConfigEntry make_entry_bf16(int occ, double eff_alone, double eff_shar
                        1,
                        {{bgemm_mfma_kernel<CFG, false, false>, bgemm_mfma_kernel<CFG, false, true>},
                         {bgemm_mfma_kernel<CFG, true, false>, bgemm_mfma_kernel<CFG, true, true>}},
+                       {{nullptr, nullptr}, {nullptr, nullptr}},
                        occ,
                        eff_alone,
                        eff_shared,
@@ -257,12 +264,34 @@ int ensure_counters(Handle* h, size_t n) {
     return SNHIP_STATUS_SUCCESS;
 }
 
-// Row-major core: C[M x N] (ldc) = alpha * op(A)[M x K] * op(B)[K x N] + beta * C (+ bias), per batch.
-int gemm_rm(Handle* h, bool tA, bool tB, int M, int N, int K, float alpha, const float* A, int lda, long long sA,
-            const float* B, int ldb, long long sB, float beta, float* C, int ldc, long long sC, int batch,
-            const float* bias, int math = -1) {
+// Everything one GEMM launch can be asked to do (row-major):
+//   C[z] = act(alpha * op(A[z]) . op(B[z]) + bias + beta * C[z] + gamma * D[z]),  z = 0 .. batch-1,
+//   optionally colsum[z][m] = sum_k op(A[z])[m][k].
+// Matrix z of a two-level batch sits at base + (z / batch_inner) * stride2 + (z % batch_inner) * stride.
+struct GemmArgs {
+    bool tA = false, tB = false;
+    int M = 0, N = 0, K = 0;
+    float alpha = 1.0f, beta = 0.0f;
+    const float* A = nullptr;
+    const float* B = nullptr;
+    float* C = nullptr;
+    int lda = 0, ldb = 0, ldc = 0;
+    int batch = 1, batch_inner = 0;  // batch_inner 0: single-level batch
+    long long sA = 0, sB = 0, sC = 0, sA2 = 0, sB2 = 0, sC2 = 0;
+    const float* bias = nullptr;
+    const float* D = nullptr;
+    int ldd = 0;
+    long long sD = 0, sD2 = 0;
+    float gamma = 0.0f;
+    int act = ACT_NONE;
+    float act_param = 0.0f;
+    float* colsum = nullptr;
+    int math = -1;  // -1: the handle's math mode
+};
+
+int gemm_core(Handle* h, const GemmArgs& g) {
     if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
-    if (math < 0) math = h->math_mode;
+    const int math = (g.math < 0) ? h->math_mode : g.math;
     {
         // The handle belongs to one device (GPUWrapper.AssociateCurrentThreadWithDevice, GPUWrapper.cs:782-788);
         // a caller thread whose current device differs is switched to it, as cudaSetDevice would have been.
@@ -270,59 +299,142 @@ int gemm_rm(Handle* h, bool tA, bool tB, int M, int N, int K, float alpha, const
         if (hipGetDevice(&cur) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
         if (cur != h->device && hipSetDevice(h->device) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
     }
-    if (M < 0 || N < 0 || K < 0 || batch < 0) return SNHIP_STATUS_INVALID_VALUE;
+    const int M = g.M, N = g.N, K = g.K, batch = g.batch;
+    if (M < 0 || N < 0 || K < 0 || batch < 0 || g.batch_inner < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (math != SNHIP_MATH_FP32 && math != SNHIP_MATH_BF16_INPUT) return SNHIP_STATUS_INVALID_VALUE;
+    if (g.act < ACT_NONE || g.act > ACT_TANH) return SNHIP_STATUS_NOT_SUPPORTED;
+    if (g.colsum != nullptr && !g.tA) return SNHIP_STATUS_NOT_SUPPORTED;  // only sums along the k of a transposed A
     if (M == 0 || N == 0 || batch == 0) return SNHIP_STATUS_SUCCESS;
-    if (C == nullptr || ldc < N) return SNHIP_STATUS_INVALID_VALUE;
-    if (batch > 65535 * 1) {
-        // grid.y carries batch * splitk
-        if (batch > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
-    }
+    if (g.C == nullptr || g.ldc < N) return SNHIP_STATUS_INVALID_VALUE;
+    if (g.D != nullptr && g.ldd < N) return SNHIP_STATUS_INVALID_VALUE;
+    if (batch > 65535) return SNHIP_STATUS_NOT_SUPPORTED;  // grid.y carries batch * splitk
+    const int inner = (g.batch_inner > 0) ? g.batch_inner : batch;
+    if (batch % inner != 0) return SNHIP_STATUS_INVALID_VALUE;
+    const bool multi = batch > 1;
+    const bool two_level = multi && inner < batch;
+
+    // everything that can follow alpha * A.B + bias + beta * C
+    Epilogue ep;
+    ep.bias = g.bias;
+    ep.addend = (g.gamma != 0.0f) ? g.D : nullptr;
+    ep.ldd = g.ldd;
+    ep.strideD = g.sD;
+    ep.strideD2 = g.sD2;
+    ep.gamma = g.gamma;
+    ep.act = g.act;
+    ep.act_param = (g.act == ACT_RELU) ? 0.0f : g.act_param;
 
     hipError_t e;
-    if (K == 0 || alpha == 0.0f) {
-        // BLAS semantics: A and B are not referenced, C = beta * C.
-        if (beta == 1.0f && bias == nullptr) return SNHIP_STATUS_SUCCESS;
+    // C = act(1 * C + gamma * D) as a pass of its own: used for what the chosen GEMM kernel does not apply itself
+    auto after_pass = [&](const float* addend, int act) -> int {
+        Epilogue ea = ep;
+        ea.bias = nullptr;
+        ea.addend = addend;
+        ea.act = act;
         const long long total = (long long)M * N * batch;
         const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
-        hipLaunchKernelGGL(scale_c_kernel, dim3(blocks), dim3(256), 0, h->stream, C, bias, M, N, ldc, sC, batch, beta);
-        e = hipGetLastError();
-        return hip_to_status(e);
+        hipLaunchKernelGGL(scale_c_kernel, dim3(blocks), dim3(256), 0, h->stream, g.C, ea, M, N, g.ldc, g.sC, g.sC2, inner,
+                           batch, 1.0f);
+        return hip_to_status(hipGetLastError());
+    };
+    // op(A) = A^T: A[z] is K x M with row pitch lda, so the sum over k is a plain column sum (zeros when K == 0)
+    auto standalone_colsum = [&]() -> int {
+        if (K > 0 && g.A == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+        for (int zo = 0; zo < batch / inner; ++zo) {
+            hipLaunchKernelGGL(column_sum_kernel, dim3((M + 63) / 64, inner), dim3(256), 0, h->stream,
+                               g.A + (long long)zo * g.sA2, g.colsum + (long long)zo * inner * M, K, M,
+                               (long long)g.lda, g.sA);
+        }
+        return hip_to_status(hipGetLastError());
+    };
+    if (K == 0 || g.alpha == 0.0f) {
+        // BLAS semantics: A and B are not referenced by the product, C = beta * C (then the rest of the epilogue).
+        if (g.colsum != nullptr) {
+            const int st = standalone_colsum();
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
+        if (g.beta == 1.0f && ep.bias == nullptr && ep.addend == nullptr && ep.act == ACT_NONE)
+            return SNHIP_STATUS_SUCCESS;
+        const long long total = (long long)M * N * batch;
+        const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+        hipLaunchKernelGGL(scale_c_kernel, dim3(blocks), dim3(256), 0, h->stream, g.C, ep, M, N, g.ldc, g.sC, g.sC2, inner,
+                           batch, g.beta);
+        return hip_to_status(hipGetLastError());
     }
-    if (A == nullptr || B == nullptr) return SNHIP_STATUS_INVALID_VALUE;
-    if (lda < (tA ? M : K) || ldb < (tB ? K : N)) return SNHIP_STATUS_INVALID_VALUE;
+    if (g.A == nullptr || g.B == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    if (g.lda < (g.tA ? M : K) || g.ldb < (g.tB ? K : N)) return SNHIP_STATUS_INVALID_VALUE;
 
     Choice ch = choose(h, M, N, K, batch, math);
     const ConfigEntry& cfg = kConfigs[ch.cfg];
     if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
 
+    // The extended kernels apply gamma * D and the (leaky) ReLU while writing C, walk a two-level batch, and -
+    // transposed A, plain B, no split-K - add up the column sum on the side.  They are used only when one of
+    // those is asked for; a configuration without them (the bf16-input kernels) gets the same results from the
+    // plain kernel plus passes over C / A, and one launch per outer batch step.
+    const KernelFn fn_ext = cfg.fn_ext[g.tA ? 1 : 0][g.tB ? 1 : 0];
+    const bool relu_family = (ep.act == ACT_RELU || ep.act == ACT_LEAKY_RELU);
+    const bool want_ext = ep.addend != nullptr || relu_family || two_level || g.colsum != nullptr;
+    const bool use_ext = want_ext && fn_ext != nullptr;
+    if (two_level && !use_ext) {
+        GemmArgs part = g;
+        part.batch = inner;
+        part.batch_inner = 0;
+        for (int zo = 0; zo < batch / inner; ++zo) {
+            part.A = g.A + (long long)zo * g.sA2;
+            part.B = g.B + (long long)zo * g.sB2;
+            part.C = g.C + (long long)zo * g.sC2;
+            part.D = (g.D != nullptr) ? g.D + (long long)zo * g.sD2 : nullptr;
+            part.colsum = (g.colsum != nullptr) ? g.colsum + (long long)zo * inner * M : nullptr;
+            const int st = gemm_core(h, part);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
+        return SNHIP_STATUS_SUCCESS;
+    }
+    const bool fuse_colsum = use_ext && g.colsum != nullptr && ch.splitk == 1 && g.tA && !g.tB;
+    // what is left for a pass over C afterwards: sigmoid / tanh always, and addend / ReLU when the kernel is plain
+    const float* addend_after = use_ext ? nullptr : ep.addend;
+    const int act_after = (use_ext && relu_family) ? ACT_NONE : ep.act;
+    Epilogue ep_kernel = ep;
+    if (!use_ext) ep_kernel.addend = nullptr;
+    ep_kernel.act = (use_ext && relu_family) ? ep.act : ACT_NONE;
+
     GemmParams p;
-    p.A = A;
-    p.B = B;
-    p.C = C;
-    p.bias = bias;
+    p.A = g.A;
+    p.B = g.B;
+    p.C = g.C;
+    p.ep = ep_kernel;
+    p.colsum = fuse_colsum ? g.colsum : nullptr;
     p.ws = nullptr;
     p.M = M;
     p.N = N;
     p.K = K;
-    p.lda = lda;
-    p.ldb = ldb;
-    p.ldc = ldc;
-    p.strideA = sA;
-    p.strideB = sB;
-    p.strideC = sC;
+    p.lda = g.lda;
+    p.ldb = g.ldb;
+    p.ldc = g.ldc;
+    p.strideA = g.sA;
+    p.strideB = g.sB;
+    p.strideC = g.sC;
+    p.strideA2 = g.sA2;
+    p.strideB2 = g.sB2;
+    p.strideC2 = g.sC2;
+    p.batch_inner = inner;
     p.tiles_m = ceil_div(M, cfg.BM);
     p.tiles_n = ceil_div(N, cfg.BN);
     p.splitk = ch.splitk;
     p.kchunk = ceil_div(ceil_div(K, ch.splitk), cfg.BK) * cfg.BK;
-    p.alpha = alpha;
-    p.beta = beta;
+    p.alpha = g.alpha;
+    p.beta = g.beta;
     p.group_m = 8;
     p.flags = 0;
     p.counters = nullptr;
     const long long ntiles = (long long)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return SNHIP_STATUS_NOT_SUPPORTED;
-    const bool c_vec = ((uintptr_t)C % 16 == 0) && (ldc % 4 == 0) && (batch == 1 || sC % 4 == 0) &&
-                       (bias == nullptr || (uintptr_t)bias % 16 == 0);
+    const bool c_vec = ((uintptr_t)g.C % 16 == 0) && (g.ldc % 4 == 0) && (!multi || g.sC % 4 == 0) &&
+                       (!two_level || g.sC2 % 4 == 0) && (g.bias == nullptr || (uintptr_t)g.bias % 16 == 0) &&
+                       (ep_kernel.addend == nullptr ||
+                        ((uintptr_t)ep_kernel.addend % 16 == 0 && g.ldd % 4 == 0 && (!multi || g.sD % 4 == 0) &&
+                         (!two_level || g.sD2 % 4 == 0)));
     if (c_vec) p.flags |= GEMM_FLAG_C_VEC;
     bool fused_reduce = false;
     if (ch.splitk > 1) {
@@ -341,21 +453,42 @@ int gemm_rm(Handle* h, bool tA, bool tB, int M, int N, int K, float alpha, const
     h->last_cfg = ch.cfg;
     h->last_splitk = ch.splitk;
 
-    KernelFn fn = cfg.fn[tA ? 1 : 0][tB ? 1 : 0];
+    const KernelFn fn = use_ext ? fn_ext : cfg.fn[g.tA ? 1 : 0][g.tB ? 1 : 0];
     hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)(batch * ch.splitk)), dim3(cfg.NT), cfg.lds_bytes,
                        h->stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return hip_to_status(e);
 
     if (ch.splitk > 1 && !fused_reduce) {
+        // the reduction kernel applies the whole epilogue itself, whatever kind of GEMM kernel produced the partials
+        Epilogue er = ep;
+        er.addend = use_ext ? ep.addend : nullptr;
+        er.act = ep_kernel.act;
         const long long total = (long long)M * N * batch;
         const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, h->stream, h->ws, C, bias, M, N, ldc, sC,
-                           ch.splitk, batch, alpha, beta);
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, h->stream, h->ws, g.C, er, M, N, g.ldc, g.sC,
+                           g.sC2, inner, ch.splitk, batch, g.alpha, g.beta);
         e = hipGetLastError();
         if (e != hipSuccess) return hip_to_status(e);
     }
+    if (addend_after != nullptr || act_after != ACT_NONE) {
+        const int st = after_pass(addend_after, act_after);
+        if (st != SNHIP_STATUS_SUCCESS) return st;
+    }
+    if (g.colsum != nullptr && !fuse_colsum) return standalone_colsum();
     return SNHIP_STATUS_SUCCESS;
+}
+
+// Plain strided-batched product with an optional bias: the shape every entry point that predates the
+// descriptor call reduces to.
+int gemm_rm(Handle* h, bool tA, bool tB, int M, int N, int K, float alpha, const float* A, int lda, long long sA,
+            const float* B, int ldb, long long sB, float beta, float* C, int ldc, long long sC, int batch,
+            const float* bias, int math = -1) {
+    GemmArgs g;
+    g.tA = tA, g.tB = tB, g.M = M, g.N = N, g.K = K, g.alpha = alpha, g.beta = beta;
+    g.A = A, g.lda = lda, g.sA = sA, g.B = B, g.ldb = ldb, g.sB = sB, g.C = C, g.ldc = ldc, g.sC = sC;
+    g.batch = batch, g.bias = bias, g.math = math;
+    return gemm_core(h, g);
 }
 
 inline bool op_is_trans(int op, bool* ok) {
@@ -384,6 +517,13 @@ int snhip_create(void** handle) {
         for (int ta = 0; ta < 2; ++ta)
             for (int tb = 0; tb < 2; ++tb) {
                 e = hipFuncSetAttribute(reinterpret_cast<const void*>(kConfigs[c].fn[ta][tb]),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kConfigs[c].lds_bytes);
+                if (e != hipSuccess) return hip_to_status(e);
+            }
+        for (int ta = 0; ta < 2; ++ta)
+            for (int tb = 0; tb < 2; ++tb) {
+                if (kConfigs[c].fn_ext[ta][tb] == nullptr) continue;
+                e = hipFuncSetAttribute(reinterpret_cast<const void*>(kConfigs[c].fn_ext[ta][tb]),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, kConfigs[c].lds_bytes);
                 if (e != hipSuccess) return hip_to_status(e);
             }
@@ -452,6 +592,63 @@ int snhip_gemm_rm(void* handle, int transposeA, int transposeB, int M, int N, in
                   int ldc, long long strideC, int batch, const float* bias) {
     return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha, A, lda, strideA, B,
                    ldb, strideB, beta, C, ldc, strideC, batch, bias);
+}
+
+int snhip_sizeof_gemm_desc(void) { return (int)sizeof(snhip_gemm_desc); }
+
+int snhip_gemm_ex(void* handle, const snhip_gemm_desc* d) {
+    if (d == nullptr || d->struct_size != (int)sizeof(snhip_gemm_desc)) return SNHIP_STATUS_INVALID_VALUE;
+    GemmArgs g;
+    g.tA = d->transA != 0, g.tB = d->transB != 0;
+    g.M = d->M, g.N = d->N, g.K = d->K;
+    g.alpha = d->alpha, g.beta = d->beta;
+    g.A = d->A, g.lda = d->lda, g.sA = d->strideA, g.sA2 = d->strideA_outer;
+    g.B = d->B, g.ldb = d->ldb, g.sB = d->strideB, g.sB2 = d->strideB_outer;
+    g.C = d->C, g.ldc = d->ldc, g.sC = d->strideC, g.sC2 = d->strideC_outer;
+    g.batch = d->batch, g.batch_inner = d->batch_inner;
+    g.bias = d->bias;
+    g.D = d->D, g.ldd = d->ldd, g.sD = d->strideD, g.sD2 = d->strideD_outer, g.gamma = d->gamma;
+    g.act = d->activation, g.act_param = d->activation_param;
+    g.colsum = d->colsum;
+    g.math = d->math;
+    return gemm_core(static_cast<Handle*>(handle), g);
+}
+
+int snhip_dense_forward(void* handle, float* y, const float* x, const float* weights, const float* bias, int rows,
+                        int in_features, int out_features, int activation, float activation_param) {
+    GemmArgs g;
+    g.tB = true;  // y = x . W^T, W stored (out, in)
+    g.M = rows, g.N = out_features, g.K = in_features;
+    g.A = x, g.lda = in_features, g.B = weights, g.ldb = in_features, g.C = y, g.ldc = out_features;
+    g.bias = bias, g.act = activation, g.act_param = activation_param;
+    return gemm_core(static_cast<Handle*>(handle), g);
+}
+
+int snhip_dense_backward(void* handle, float* dx, float* weight_gradients, float* bias_gradients, const float* x,
+                         const float* dy, const float* weights, int rows, int in_features, int out_features,
+                         float multiplier, float weight_decay_alpha) {
+    Handle* h = static_cast<Handle*>(handle);
+    if (weight_gradients != nullptr || bias_gradients != nullptr) {
+        if (weight_gradients == nullptr) {
+            const int st = snhip_bias_gradient(handle, dy, rows, out_features, bias_gradients);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        } else {
+            GemmArgs g;  // dW = multiplier * dy^T . x (+ weight_decay_alpha * W), db = column sums of dy
+            g.tA = true;
+            g.M = out_features, g.N = in_features, g.K = rows;
+            g.alpha = multiplier;
+            g.A = dy, g.lda = out_features, g.B = x, g.ldb = in_features, g.C = weight_gradients, g.ldc = in_features;
+            g.D = weights, g.ldd = in_features, g.gamma = weight_decay_alpha;
+            g.colsum = bias_gradients;
+            const int st = gemm_core(h, g);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
+    }
+    if (dx == nullptr) return SNHIP_STATUS_SUCCESS;
+    GemmArgs g;  // dx = dy . W
+    g.M = rows, g.N = in_features, g.K = out_features;
+    g.A = dy, g.lda = out_features, g.B = weights, g.ldb = in_features, g.C = dx, g.ldc = in_features;
+    return gemm_core(h, g);
 }
 
 int snhip_dot_bias(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
@@ -530,7 +727,31 @@ int snhip_bias_gradient(void* handle, const float* dy, int rows, int cols, float
     if (cols == 0) return SNHIP_STATUS_SUCCESS;
     if (bias_gradient == nullptr || (rows > 0 && dy == nullptr)) return SNHIP_STATUS_INVALID_VALUE;
     hipLaunchKernelGGL(column_sum_kernel, dim3((cols + 63) / 64), dim3(256), 0, static_cast<Handle*>(handle)->stream, dy,
-                       bias_gradient, rows, cols);
+                       bias_gradient, rows, cols, (long long)cols, 0LL);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_activation_forward(void* handle, int activation, float activation_param, const float* x, float* y,
+                             long long n) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (n < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (activation < ACT_NONE || activation > ACT_TANH) return SNHIP_STATUS_NOT_SUPPORTED;
+    if (n == 0) return SNHIP_STATUS_SUCCESS;
+    if (x == nullptr || y == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(activation_kernel, dim3(grid_for(n)), dim3(256), 0, static_cast<Handle*>(handle)->stream, x, y, n,
+                       activation, activation_param);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_activation_backward(void* handle, int activation, float activation_param, const float* y, const float* dy,
+                              float* dx, long long n) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (n < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (activation < ACT_NONE || activation > ACT_TANH) return SNHIP_STATUS_NOT_SUPPORTED;
+    if (n == 0) return SNHIP_STATUS_SUCCESS;
+    if (y == nullptr || dy == nullptr || dx == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(activation_bwd_kernel, dim3(grid_for(n)), dim3(256), 0, static_cast<Handle*>(handle)->stream, y, dy,
+                       dx, n, activation, activation_param);
     return hip_to_status(hipGetLastError());
 }
 

@@ -307,6 +307,13 @@ class GPUTensor:
                                        bias.Pointer if bias is not None else None)
         check_status(res, "snhip_dot_bias")
 
+    def GemmEx(self, **fields):
+        """snhip_gemm_ex with this tensor as C: keyword arguments are snhip_gemm_desc fields; tensors may be passed
+        for A, B, bias, D and colsum (their device pointers are used)."""
+        fields = {k: (v.Pointer if isinstance(v, GPUTensor) else v) for k, v in fields.items()}
+        desc = hiplib.GemmDesc(C=self.Pointer, **fields)
+        check_status(self._lib.snhip_gemm_ex(self.Wrapper.handle, ctypes.byref(desc)), "snhip_gemm_ex")
+
     # -- lifetime ----------------------------------------------------------------
     def Dispose(self):
         if self._disposed:
@@ -362,8 +369,22 @@ def _add_tensor_methods():
         check_status(self._lib.snhip_set_above_main_diagonal(self.Wrapper.handle, self.Pointer, m, r, c, value),
                      "snhip_set_above_main_diagonal")
 
+    def ActivationForward(self, activationType, activationParameter, y):
+        """y = act(this) for the RELU / LEAKY_RELU / SIGMOID / TANH modes (Tensor.ActivationForward);
+        activationParameter is the leaky slope."""
+        check_status(self._lib.snhip_activation_forward(self.Wrapper.handle, hiplib.activation_code(activationType),
+                                                        float(activationParameter or 0.0), self.Pointer, y.Pointer,
+                                                        self.Count), "snhip_activation_forward")
+
+    def ActivationBackward(self, activationType, activationParameter, dy, dx):
+        """dx = dy * act'(x) with this = y = act(x) (Tensor.ActivationBackward, CPU definitions
+        CpuTensorActivationFunctions.cs:190-244)."""
+        check_status(self._lib.snhip_activation_backward(self.Wrapper.handle, hiplib.activation_code(activationType),
+                                                         float(activationParameter or 0.0), self.Pointer, dy.Pointer,
+                                                         dx.Pointer, self.Count), "snhip_activation_backward")
+
     for f in (Compute_BiasGradient_from_dy, BroadcastAddVectorToOutput, Update_Adding_Alpha_X, SoftmaxLastDimension,
-              SoftmaxLastDimensionBackward, SetAllElementsAboveMainDiagonal):
+              SoftmaxLastDimensionBackward, SetAllElementsAboveMainDiagonal, ActivationForward, ActivationBackward):
         setattr(GPUTensor, f.__name__, f)
 
 

@@ -56,6 +56,47 @@ _ll = ctypes.c_longlong
 _f = ctypes.c_float
 _sz = ctypes.c_size_t
 
+
+
+class GemmDesc(ctypes.Structure):
+    """snhip_gemm_desc of include/sharpnet_hip.h (field for field)."""
+    _fields_ = [
+        ("struct_size", _i), ("transA", _i), ("transB", _i), ("M", _i), ("N", _i), ("K", _i),
+        ("alpha", _f), ("beta", _f), ("A", _vp), ("B", _vp), ("C", _vp), ("lda", _i), ("ldb", _i), ("ldc", _i),
+        ("batch", _i), ("batch_inner", _i), ("strideA", _ll), ("strideB", _ll), ("strideC", _ll),
+        ("strideA_outer", _ll), ("strideB_outer", _ll), ("strideC_outer", _ll), ("bias", _vp), ("D", _vp),
+        ("ldd", _i), ("strideD", _ll), ("strideD_outer", _ll), ("gamma", _f), ("activation", _i),
+        ("activation_param", _f), ("colsum", _vp), ("math", _i),
+    ]
+
+    def __init__(self, **kw):
+        super().__init__()
+        self.struct_size = ctypes.sizeof(GemmDesc)
+        self.alpha, self.batch, self.math = 1.0, 1, -1
+        for k, v in kw.items():
+            if k not in dict(self._fields_):
+                raise TypeError("snhip_gemm_desc has no field %r" % k)
+            setattr(self, k, v)
+
+
+# SNHIP_ACT_* and the reference's cudnnActivationMode_t names for them (Prod/GPU/CudnnWrapper.cs:267-281)
+ACT_NONE, ACT_RELU, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_TANH = range(5)
+ACTIVATIONS = {
+    None: ACT_NONE, "CUDNN_ACTIVATION_IDENTITY": ACT_NONE, "CUDNN_ACTIVATION_RELU": ACT_RELU,
+    "CUDNN_ACTIVATION_LEAKY_RELU": ACT_LEAKY_RELU, "CUDNN_ACTIVATION_SIGMOID": ACT_SIGMOID,
+    "CUDNN_ACTIVATION_TANH": ACT_TANH,
+}
+
+
+def activation_code(mode):
+    """SNHIP_ACT_* for a cudnnActivationMode_t name (or an SNHIP_ACT_* integer, passed through)."""
+    if isinstance(mode, int):
+        return mode
+    if mode not in ACTIVATIONS:
+        raise SharpNetHipError(CublasStatus.CUBLAS_STATUS_NOT_SUPPORTED, "activation %r" % (mode,))
+    return ACTIVATIONS[mode]
+
+
 # name -> argtypes; every function returns int.  Must list every symbol of include/sharpnet_hip.h.
 SIGNATURES = {
     "snhip_create": [_vpp],
@@ -72,6 +113,12 @@ SIGNATURES = {
     "snhip_set_math_mode": [_vp, _i],
     "snhip_dot_bf16": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f, _vp],
     "snhip_bmm_bf16": [_vp, _vp, _i, _i, _i, _ll, _vp, _i, _i, _i, _ll, _vp, _ll, _i, _f, _f],
+    "snhip_gemm_ex": [_vp, ctypes.POINTER(GemmDesc)],
+    "snhip_sizeof_gemm_desc": [],
+    "snhip_dense_forward": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f],
+    "snhip_dense_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f],
+    "snhip_activation_forward": [_vp, _i, _f, _vp, _vp, _ll],
+    "snhip_activation_backward": [_vp, _i, _f, _vp, _vp, _vp, _ll],
     "snhip_bias_gradient": [_vp, _vp, _i, _i, _vp],
     "snhip_broadcast_add_vector": [_vp, _vp, _vp, _i, _i],
     "snhip_axpy": [_vp, _ll, _f, _vp, _vp],

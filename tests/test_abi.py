@@ -62,6 +62,21 @@ def test_argument_errors_without_gpu():
     assert lib.snhip_config_desc(999, d) == 7
 
 
+def test_gemm_descriptor_layout_matches_the_library():
+    """The ctypes mirror of snhip_gemm_desc has the size the compiled library reports, and a descriptor whose
+    struct_size disagrees is rejected before anything else is looked at."""
+    import ctypes
+    from sharpnet_amd import hiplib
+    lib = hiplib.load_library()
+    assert lib.snhip_sizeof_gemm_desc() == ctypes.sizeof(hiplib.GemmDesc)
+    d = hiplib.GemmDesc(M=1, N=1, K=1)
+    d.struct_size -= 4
+    assert lib.snhip_gemm_ex(None, ctypes.byref(d)) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    assert lib.snhip_gemm_ex(None, None) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    d = hiplib.GemmDesc(M=1, N=1, K=1)
+    assert lib.snhip_gemm_ex(None, ctypes.byref(d)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
+
+
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     from sharpnet_amd import hiplib
     with pytest.raises(FileNotFoundError):

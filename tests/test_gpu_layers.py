@@ -30,27 +30,110 @@ def test_dense_layer_forward_backward_config1(oracle, gpu_wrapper):
     for fuse in (True, False):
         gy = GPUTensor([x.shape[0], W.shape[0]], None, gpu_wrapper)
         gy.SetValue(float("nan"))
-        linear.DenseForwardPropagation(gy, gx, gW, gb, False, fuse_bias=fuse)
+        linear.DenseForwardPropagation(gy, gx, gW, gb, False, fused=fuse)
         assert np.max(np.abs(gy.ToNumpy() - ref_y)) <= bound(x.shape[1], x, W, 1e-6)
     gdW, gdb, gdx = GPUTensor(list(W.shape), None, gpu_wrapper), GPUTensor([W.shape[0]], None, gpu_wrapper), \
         GPUTensor(list(x.shape), None, gpu_wrapper)
     for t in (gdW, gdb, gdx):
         t.SetValue(float("nan"))
-    linear.DenseBackwardPropagation(gdx, gdW, gdb, gx, gdy, gW)           # SharpNet mode: multiplier 1/batch
-    rdW, rdb, rdx = oracle.dense_backward(x, dy, W, multiplier=1.0 / x.shape[0])
-    assert np.max(np.abs(gdW.ToNumpy() - rdW)) <= bound(x.shape[0], dy, x) / x.shape[0] + 1e-9
-    assert np.max(np.abs(gdb.ToNumpy() - rdb)) <= 1e-5 * np.sqrt(x.shape[0]) * np.max(np.abs(dy)) + 1e-7
-    assert np.max(np.abs(gdx.ToNumpy() - rdx)) <= bound(W.shape[0], dy, W)
-    # weight decay epilogue (PyTorch mode: dW += batch*wd*W, Linear.cs:168-181) and the input-layer shortcut
-    gdx.SetValue(7.0)
-    linear.DenseBackwardPropagation(gdx, gdW, gdb, gx, gdy, gW, bias_1D=gb, compatibility_mode="PyTorch",
-                                    use_weight_decay_in_backpropagation=True, weight_decay=0.01,
-                                    prevLayerIsInputLayer=True)
-    rdW2, rdb2, _ = oracle.dense_backward(x, dy, W, multiplier=1.0)
-    alpha = 1 * x.shape[0] * 0.01
-    assert np.max(np.abs(gdW.ToNumpy() - (rdW2 + alpha * W))) <= bound(x.shape[0], dy, x) + 1e-5
-    assert np.max(np.abs(gdb.ToNumpy() - (rdb2 + alpha * bias))) <= 1e-4
-    assert np.all(gdx.ToNumpy() == 7.0)                                  # dx untouched when the previous layer is the input
+    for fused in (True, False):
+        for t in (gdW, gdb, gdx):
+            t.SetValue(float("nan"))
+        linear.DenseBackwardPropagation(gdx, gdW, gdb, gx, gdy, gW, fused=fused)   # SharpNet mode: multiplier 1/batch
+        rdW, rdb, rdx = oracle.dense_backward(x, dy, W, multiplier=1.0 / x.shape[0])
+        assert np.max(np.abs(gdW.ToNumpy() - rdW)) <= bound(x.shape[0], dy, x) / x.shape[0] + 1e-9
+        assert np.max(np.abs(gdb.ToNumpy() - rdb)) <= 1e-5 * np.sqrt(x.shape[0]) * np.max(np.abs(dy)) + 1e-7
+        assert np.max(np.abs(gdx.ToNumpy() - rdx)) <= bound(W.shape[0], dy, W)
+        # weight decay (PyTorch mode: dW += batch*wd*W, Linear.cs:168-181) and the input-layer shortcut
+        gdx.SetValue(7.0)
+        linear.DenseBackwardPropagation(gdx, gdW, gdb, gx, gdy, gW, bias_1D=gb, compatibility_mode="PyTorch",
+                                        use_weight_decay_in_backpropagation=True, weight_decay=0.01,
+                                        prevLayerIsInputLayer=True, fused=fused)
+        alpha = 1 * x.shape[0] * 0.01
+        rdW2, rdb2, _ = oracle.dense_backward(x, dy, W, multiplier=1.0, weight_decay_alpha=alpha)
+        assert np.max(np.abs(gdW.ToNumpy() - rdW2)) <= bound(x.shape[0], dy, x) + 1e-5
+        assert np.max(np.abs(gdb.ToNumpy() - (rdb2 + alpha * bias))) <= 1e-4
+        assert np.all(gdx.ToNumpy() == 7.0)                              # dx untouched when the previous layer is the input
+
+
+ACTS = [("relu", "CUDNN_ACTIVATION_RELU", 0.0), ("leaky_relu", "CUDNN_ACTIVATION_LEAKY_RELU", 0.1),
+        ("leaky_relu", "CUDNN_ACTIVATION_LEAKY_RELU", 0.3), ("sigmoid", "CUDNN_ACTIVATION_SIGMOID", 0.0),
+        ("tanh", "CUDNN_ACTIVATION_TANH", 0.0)]
+
+
+@pytest.mark.parametrize("mode,cudnn,slope", ACTS)
+def test_activation_fused_into_forward_and_stand_alone(oracle, gpu_wrapper, mode, cudnn, slope):
+    """Linear + ActivationLayer as one launch (write-out of the GEMM), on direct and split-K paths and on a ragged
+    shape, against the oracle; then ActivationForward / ActivationBackward by themselves."""
+    from sharpnet_amd import GPUTensor, linear
+    rng = np.random.default_rng(11)
+    try:
+        for (rows, fin, fout, tuning) in ((128, 784, 256, (-1, 0)), (77, 301, 130, (-1, 0)), (64, 1024, 96, (6, 4)),
+                                          (300, 200, 515, (3, 1)), (256, 64, 512, (0, 1))):
+            x, W, b = random_tensor(rng, (rows, fin), -1, 1), random_tensor(rng, (fout, fin), -0.2, 0.2), \
+                random_tensor(rng, (fout,), -1, 1)
+            gx, gW, gb = T(gpu_wrapper, x), T(gpu_wrapper, W), T(gpu_wrapper, b)
+            gy = GPUTensor([rows, fout], None, gpu_wrapper)
+            gy.SetValue(float("nan"))
+            gpu_wrapper.set_tuning(*tuning)
+            linear.DenseForwardPropagation(gy, gx, gW, gb, False, activation=cudnn, activation_parameter=slope)
+            want = oracle.activation_forward(oracle.dense_forward(x, W, b), mode, slope)
+            assert np.max(np.abs(gy.ToNumpy() - want)) <= bound(fin, x, W, 1e-6), (rows, fin, fout, tuning)
+            gy2 = GPUTensor([rows, fout], None, gpu_wrapper)
+            linear.DenseForwardPropagation(gy2, gx, gW, gb, False, fused=False, activation=cudnn,
+                                           activation_parameter=slope)
+            assert np.max(np.abs(gy2.ToNumpy() - want)) <= bound(fin, x, W, 1e-6)
+    finally:
+        gpu_wrapper.set_tuning(-1, 0)
+    v = random_tensor(rng, (5, 3, 41), -3, 3)
+    dy = random_tensor(rng, v.shape, -1, 1)
+    gv, gdy = T(gpu_wrapper, v), T(gpu_wrapper, dy)
+    gout, gdx = GPUTensor(list(v.shape), None, gpu_wrapper), GPUTensor(list(v.shape), None, gpu_wrapper)
+    gv.ActivationForward(cudnn, slope, gout)
+    yy = oracle.activation_forward(v, mode, slope)
+    assert np.max(np.abs(gout.ToNumpy() - yy)) <= 2e-6
+    gout.ActivationBackward(cudnn, slope, gdy, gdx)
+    assert np.max(np.abs(gdx.ToNumpy() - oracle.activation_backward(gout.ToNumpy(), dy, mode, slope))) <= 2e-6
+
+
+def test_bias_gradient_rides_along_with_dW_for_every_tile_configuration(oracle, gpu_wrapper):
+    """snhip_gemm_ex colsum (= Compute_BiasGradient_from_dy of the dy the dW product reads) with gamma*D (weight decay),
+    for each fp32 tile configuration, with and without split-K (the split-K case takes the stand-alone kernel),
+    a strided batch, ragged sizes and padded leading dimensions."""
+    from sharpnet_amd import GPUTensor
+    rng = np.random.default_rng(12)
+    w = gpu_wrapper
+    fp32_cfgs = [c["id"] for c in w.configs() if c["kind"] == "fp32"]
+    try:
+        for cfg in fp32_cfgs + [-1]:
+            for splitk in ((1, 2) if cfg >= 0 else (0,)):
+                for (out_f, in_f, rows, batch) in ((333, 190, 517, 1), (64, 64, 32, 3), (700, 130, 96, 2)):
+                    lda, ldb, ldc, ldd = out_f + 3, in_f + 1, in_f + 2, in_f + 5
+                    dy = random_tensor(rng, (batch, rows, lda), -1, 1)
+                    x = random_tensor(rng, (batch, rows, ldb), -1, 1)
+                    Wm = random_tensor(rng, (batch, out_f, ldd), -1, 1)
+                    c0 = random_tensor(rng, (batch, out_f, ldc), -1, 1)
+                    gdy, gx, gWm, gc = T(w, dy), T(w, x), T(w, Wm), T(w, c0)
+                    gcs = GPUTensor([batch, out_f], None, w)
+                    gcs.SetValue(float("nan"))
+                    w.set_tuning(cfg, splitk)
+                    gc.GemmEx(transA=1, M=out_f, N=in_f, K=rows, alpha=0.5, beta=0.25, A=gdy, lda=lda, strideA=rows * lda,
+                              B=gx, ldb=ldb, strideB=rows * ldb, ldc=ldc, strideC=out_f * ldc, batch=batch,
+                              D=gWm, ldd=ldd, strideD=out_f * ldd, gamma=0.75, colsum=gcs)
+                    got, cs = gc.ToNumpy(), gcs.ToNumpy()
+                    for z in range(batch):
+                        a, b = dy[z][:, :out_f], x[z][:, :in_f]
+                        want = oracle.dot(np.ascontiguousarray(a), True, np.ascontiguousarray(b), False, 0.5, 0.25,
+                                          np.ascontiguousarray(c0[z][:, :in_f])) + 0.75 * Wm[z][:, :in_f]
+                        assert np.max(np.abs(got[z][:, :in_f] - want)) <= bound(rows, a, b, 1e-5), (cfg, splitk, out_f)
+                        assert np.array_equal(got[z][:, in_f:], c0[z][:, in_f:])          # padding untouched
+                        ref_cs = a.astype(np.float64).sum(axis=0)
+                        assert np.max(np.abs(cs[z] - ref_cs)) <= 1e-5 * np.sqrt(rows) + 1e-6, (cfg, splitk, out_f)
+    finally:
+        w.set_tuning(-1, 0)
+    # a column sum cannot be asked for without transposeA
+    with pytest.raises(Exception):
+        gc.GemmEx(transA=0, M=4, N=4, K=4, A=gdy, lda=4, B=gx, ldb=4, ldc=4, colsum=gcs)
 
 
 def test_linear_sigmoid_predictions_on_device(golden, gpu_wrapper):
@@ -84,10 +167,10 @@ def test_dense_chain_training_losses_on_device(golden, gpu_wrapper):
     def forward():
         gW1, gb1, gW2, gb2 = (T(w, p) for p in params)
         gh = GPUTensor([2, 3, 4, 3], None, w)
-        linear.DenseForwardPropagation(gh, gX, gW1, gb1, True)            # flatten on last dimension: (24,5).(5,3)
-        h = gh.ToNumpy()
-        r = np.maximum(h, 0)
-        gf = T(w, r.reshape(2, 36))
+        # flatten on last dimension: (24,5).(5,3); the ReLU layer that follows is folded into the product
+        linear.DenseForwardPropagation(gh, gX, gW1, gb1, True, activation="CUDNN_ACTIVATION_RELU")
+        h = r = gh.ToNumpy()
+        gf = gh.Reshape(2, 36)
         gout = GPUTensor([2, 3], None, w)
         linear.DenseForwardPropagation(gout, gf, gW2, gb2, False)
         return h, r, gf, gout.ToNumpy(), (gW1, gW2)
@@ -99,9 +182,10 @@ def test_dense_chain_training_losses_on_device(golden, gpu_wrapper):
         dout = (2.0 * (out - Y) / out.size).astype(np.float32)
         gdW2, gdb2, gdf = GPUTensor([3, 36], None, w), GPUTensor([3], None, w), GPUTensor([2, 36], None, w)
         linear.DenseBackwardPropagation(gdf, gdW2, gdb2, gf, T(w, dout), gW2, compatibility_mode="PyTorch")
-        dh = (gdf.ToNumpy().reshape(r.shape) * (h > 0)).astype(np.float32)
+        gdh = GPUTensor([2, 36], None, w)
+        gf.ActivationBackward("CUDNN_ACTIVATION_RELU", 0.0, gdf, gdh)       # y = relu output, Tensor.ActivationBackward
         gdW1, gdb1 = GPUTensor([3, 5], None, w), GPUTensor([3], None, w)
-        linear.DenseBackwardPropagation(None, gdW1, gdb1, gX, T(w, dh), gW1, compatibility_mode="PyTorch",
+        linear.DenseBackwardPropagation(None, gdW1, gdb1, gX, gdh.Reshape(2, 3, 4, 3), gW1, compatibility_mode="PyTorch",
                                         prevLayerIsInputLayer=True, flattenInputTensorOnLastDimension=True)
         grads = [gdW1.ToNumpy(), gdb1.ToNumpy(), gdW2.ToNumpy(), gdb2.ToNumpy()]
         for i, g in enumerate(grads):

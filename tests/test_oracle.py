@@ -174,7 +174,7 @@ def test_dense_chain_losses(golden, oracle):
 
     def forward():
         h = oracle.dense_forward(X, params[0], params[1], flatten_last=True)    # (24, 3)
-        r = np.maximum(h, 0)
+        r = oracle.activation_forward(h, "relu")
         f = r.reshape(X.shape[0], -1)                                            # Flatten -> (2, 36)
         out = oracle.dense_forward(f, params[2], params[3])
         return h, r, f, out
@@ -189,13 +189,44 @@ def test_dense_chain_losses(golden, oracle):
         dout = (2.0 * (out - Y) / out.size).astype(np.float32)
         dW2, db2, df = oracle.dense_backward(f, dout, params[2])
         dr = df.reshape(r.shape)
-        dh = (dr * (h > 0)).astype(np.float32)
+        dh = oracle.activation_backward(r, dr, "relu")
         dW1, db1, _ = oracle.dense_backward(X, dh, params[0], prev_is_input=True, flatten_last=True)
         for i, g in enumerate([dW1, db1, dW2, db2]):
             vel[i] = (fx["momentum"] * vel[i] + g).astype(np.float32)
             params[i] = (params[i] - fx["lr"] * vel[i]).astype(np.float32)
     loss_after = mse(forward()[3])
     assert abs(loss_after - fx["loss_after"]) < fx["tolerance"]
+
+
+def test_activation_functions(golden, oracle):
+    """sigmoid against the reference's stored predictions, tanh / leaky relu through identities that tie them to the
+    pinned ones, and every gradient (written in terms of the output y) against central differences of the forward."""
+    fx = golden["Linear_1_1_4_4"]
+    y = oracle.dot(np.array(fx["x"], np.float32), False, np.array(fx["w_in_out"], np.float32), False)
+    assert np.max(np.abs(oracle.activation_forward(y, "sigmoid") - np.array(fx["sigmoid_prediction"]))) < 2e-6
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-3, 3, (7, 33)).astype(np.float32)
+    x[np.abs(x) < 1e-2] = 0.5                                   # keep finite differences away from the kinks
+    sig = lambda t: oracle.activation_forward(t, "sigmoid").astype(np.float64)
+    assert np.max(np.abs(oracle.activation_forward(x, "tanh") - (2 * sig(2 * x) - 1))) < 3e-7
+    relu = lambda t: oracle.activation_forward(t, "relu")
+    assert np.array_equal(relu(x), np.where(x > 0, x, 0).astype(np.float32))
+    for a in (0.1, 0.3):                                        # the slopes the reference tests use
+        assert np.allclose(oracle.activation_forward(x, "leaky_relu", a), relu(x) - np.float32(a) * relu(-x), atol=1e-7)
+    dy = rng.uniform(-1, 1, x.shape).astype(np.float32)
+    for mode, a in (("relu", 0.0), ("leaky_relu", 0.1), ("leaky_relu", 0.3), ("sigmoid", 0.0), ("tanh", 0.0)):
+        yy = oracle.activation_forward(x, mode, a)
+        h = 1e-3
+        num = (oracle.activation_forward(x + np.float32(h), mode, a).astype(np.float64) -
+               oracle.activation_forward(x - np.float32(h), mode, a)) / (2 * h) * dy
+        assert np.max(np.abs(oracle.activation_backward(yy, dy, mode, a) - num)) < 2e-3, mode
+    # weight decay enters dW linearly and nowhere else
+    xx, dd, W = rng.uniform(-1, 1, (9, 5)).astype(np.float32), rng.uniform(-1, 1, (9, 4)).astype(np.float32), \
+        rng.uniform(-1, 1, (4, 5)).astype(np.float32)
+    base = oracle.dense_backward(xx, dd, W)
+    wd = oracle.dense_backward(xx, dd, W, weight_decay_alpha=0.5)
+    assert np.allclose(wd[0] - base[0], 0.5 * W, atol=1e-6) and np.array_equal(wd[1], base[1]) and \
+        np.array_equal(wd[2], base[2])
 
 
 def test_attention_chain_losses(golden, oracle):
