@@ -205,6 +205,13 @@ int snhip_softmax_last_dim_backward(void* handle, const float* y, const float* d
  * ScaledDotProductAttentionLayer.cs:73-76; CPU: CpuTensor.cs:3037-3052). */
 int snhip_set_above_main_diagonal(void* handle, float* x, int matrices, int rows, int cols, float value);
 
+/* dst[a][c][b][d] = src[a][b][c][d] for src of shape (d0, d1, d2, d3): Tensor.TransposeSecondAndThirdDimension
+ * (Prod/CPU/CpuTensor.cs:301-322; CUDA kernel Prod/GPU/Kernels/SinglePrecision.cu:1285).  The multi-head attention
+ * layer uses it to split and merge heads (Prod/Layers/MultiheadAttention.cs:207-230); with snhip_gemm_ex's two-level
+ * batch those copies are not needed, this entry point serves callers that keep the reference's sequence. */
+int snhip_transpose_second_and_third_dimension(void* handle, const float* src, float* dst, int d0, int d1, int d2,
+                                               int d3);
+
 /* ---- device memory / stream shims --------------------------------------- */
 /* Replace the nvcuda calls GPUTensor makes: cuMemAlloc_v2 (GpuTensor.cs:41),
  * cuMemFree_v2 (:1634), cuMemsetD32 (:1583), cuMemcpyHtoDAsync (:77),

@@ -34,6 +34,8 @@ sdpa_forward                            Prod/Layers/ScaledDotProductAttention   
                                         Layer.cs:46-91
 softmax_last_dim_backward /             ScaledDotProductAttentionLayer.cs:111-132    central finite differences of sdpa_forward
 sdpa_backward                           (softmax gradient: cuDNN definition)         (tests/test_oracle.py)
+mha_forward / mha_backward              Prod/Layers/MultiheadAttention.cs:178-292    stored losses before / after 10 epochs of
+                                        (head split / merge as explicit transposes)  ParallelRunWithPyTorch.cs:1013-1131, 4 cases
 round_to_bf16                           IEEE-754 round-to-nearest-even to a          closed-form ties/neighbours and torch's CPU
                                         bfloat16 (what v_cvt_pk_bf16_f32 does);      bfloat16 cast (independent implementation)
                                         no reference counterpart (variant is new)
@@ -295,6 +297,52 @@ def sdpa_backward(Q, K, V, dy, weights, use_scale=True):
     dQ = bmm(dS, False, K, False, 1.0, 0.0)                            # :127
     dK = bmm(dS, True, Q, False, 1.0, 0.0)                             # :128
     return dQ, dK, dV
+
+
+def _split_heads(x2d, batch, steps, heads, dim):
+    """(batch*steps, heads*dim) -> (batch*heads, steps, dim): Reshape + TransposeSecondAndThirdDimension
+    (MultiheadAttention.cs:207-211)."""
+    return np.ascontiguousarray(x2d.reshape(batch, steps, heads, dim).transpose(0, 2, 1, 3)).reshape(batch * heads, steps, dim)
+
+
+def _merge_heads(x3d, batch, steps, heads, dim):
+    """(batch*heads, steps, dim) -> (batch, steps, heads*dim) (MultiheadAttention.cs:228-230)."""
+    return np.ascontiguousarray(x3d.reshape(batch, heads, steps, dim).transpose(0, 2, 1, 3)).reshape(batch, steps, heads * dim)
+
+
+def mha_forward(Q, K, V, w_Q, w_K, w_V, w_O, num_heads, key_dim, value_dim, b_Q=None, b_K=None, b_V=None, b_O=None,
+                is_causal=False, use_scale=True):
+    """MultiheadAttention.ForwardPropagation (MultiheadAttention.cs:178-240).  Q, K, V: (batch, steps, embed);
+    weights (out, in).  Returns (y, cache) with cache holding what BackwardPropagation reads."""
+    Q, K, V = (np.asarray(t, dtype=np.float32) for t in (Q, K, V))
+    batch, tq, tkv = K.shape[0], Q.shape[1], V.shape[1]
+    Qh = _split_heads(dense_forward(Q, w_Q, b_Q, flatten_last=True), batch, tq, num_heads, key_dim)
+    Kh = _split_heads(dense_forward(K, w_K, b_K, flatten_last=True), batch, tkv, num_heads, key_dim)
+    Vh = _split_heads(dense_forward(V, w_V, b_V, flatten_last=True), batch, tkv, num_heads, value_dim)
+    heads, weights = sdpa_forward(Qh, Kh, Vh, use_scale=use_scale, is_causal=is_causal)
+    merged = _merge_heads(heads, batch, tkv, num_heads, value_dim)
+    y = dense_forward(merged, w_O, b_O, flatten_last=True).reshape(batch, tkv, -1)
+    return y, dict(Q=Q, K=K, V=V, Qh=Qh, Kh=Kh, Vh=Vh, weights=weights, merged=merged, w=(w_Q, w_K, w_V, w_O),
+                   dims=(batch, tq, tkv, num_heads, key_dim, value_dim), use_scale=use_scale)
+
+
+def mha_backward(dy, cache):
+    """MultiheadAttention.BackwardPropagation (MultiheadAttention.cs:243-292), multiplier 1 (PyTorch / TensorFlow mode).
+    Returns dict with dQ, dK, dV and (dW, db) for each of the four projections."""
+    batch, tq, tkv, H, dk, dv = cache["dims"]
+    w_Q, w_K, w_V, w_O = cache["w"]
+    dWo, dbo, dmerged = dense_backward(cache["merged"], dy, w_O, flatten_last=True)
+    d_heads = _split_heads(dmerged.reshape(batch * tkv, H * dv), batch, tkv, H, dv)
+    dQh, dKh, dVh = sdpa_backward(cache["Qh"], cache["Kh"], cache["Vh"], d_heads, cache["weights"], use_scale=cache["use_scale"])
+    out = {}
+    for name, dh, x, w, steps, dim in (("Q", dQh, cache["Q"], w_Q, tq, dk), ("K", dKh, cache["K"], w_K, tkv, dk),
+                                      ("V", dVh, cache["V"], w_V, tkv, dv)):
+        dpacked = _merge_heads(dh, batch, steps, H, dim)
+        dW, db, dx = dense_backward(x, dpacked, w, flatten_last=True)
+        out["d" + name] = dx.reshape(x.shape)
+        out["dw_" + name], out["db_" + name] = dW, db
+    out["dw_O"], out["db_O"] = dWo, dbo
+    return out
 
 
 # ---------------------------------------------------------------------------

@@ -44,3 +44,154 @@ def ScaledDotProductAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, weight
     dK.BatchMatrixMultiplication(scores_gradients_buffer, True, Q, False, 1.0, 0.0)       # :128
     scores_gradients_buffer.Dispose()
     weights_buffer.Dispose()
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Multi-head attention (Prod/Layers/MultiheadAttention.cs:178-292)
+# ---------------------------------------------------------------------------------------------------------------
+class MultiheadAttentionState:
+    """What ForwardPropagation keeps for BackwardPropagation (MultiheadAttention.cs:53-57)."""
+
+    def __init__(self):
+        self.weights_buffer = None      # (batch*heads, Tq, Tkv) softmax output
+        self.Q_heads = self.K_heads = self.V_heads = None   # projections; packed (batch*T, heads*dim) when heads stay in
+        self.attention_heads_T = None   # place, (batch*heads, T, dim) copies in the reference's sequence
+        self.dims = None
+        self.heads_in_place = True
+
+
+def _heads_gemm(c, a, b, *, transA, transB, M, N, K, alpha, batch, heads, a_packed, b_packed, c_packed,
+                a_steps, b_steps, c_steps, a_dim, b_dim, c_dim):
+    """One product per (batch, head).  A packed operand is a (batch, steps, heads*dim) activation whose head h is the
+    column block [h*dim, (h+1)*dim): leading dimension heads*dim, head stride dim, batch stride steps*heads*dim.
+    An unpacked one is a contiguous (batch*heads, rows, cols) stack."""
+    def strides(packed, steps, dim, rows, cols):
+        if packed:
+            return heads * dim, dim, steps * heads * dim
+        return cols, rows * cols, heads * rows * cols
+    a_rows, a_cols = (K, M) if transA else (M, K)
+    b_rows, b_cols = (N, K) if transB else (K, N)
+    lda, sA, sA2 = strides(a_packed, a_steps, a_dim, a_rows, a_cols)
+    ldb, sB, sB2 = strides(b_packed, b_steps, b_dim, b_rows, b_cols)
+    ldc, sC, sC2 = strides(c_packed, c_steps, c_dim, M, N)
+    c.GemmEx(transA=int(transA), transB=int(transB), M=M, N=N, K=K, alpha=alpha, beta=0.0, A=a, lda=lda, strideA=sA,
+             strideA_outer=sA2, B=b, ldb=ldb, strideB=sB, strideB_outer=sB2, ldc=ldc, strideC=sC, strideC_outer=sC2,
+             batch=batch * heads, batch_inner=heads)
+
+
+def MultiheadAttentionForwardPropagation(Q, K, V, y, w_Q, w_K, w_V, out_proj_weight, num_heads, key_dim, value_dim,
+                                         w_Q_bias=None, w_K_bias=None, w_V_bias=None, out_proj_bias=None,
+                                         isTraining=True, use_scale=True, is_causal=False, heads_in_place=True):
+    """MultiheadAttention.ForwardPropagation.  heads_in_place=True multiplies the heads where the projections left
+    them (two-level strided batch, no TransposeSecondAndThirdDimension copies, the attention output lands directly
+    in the (batch, steps, heads*value_dim) layout the output projection reads); False issues the reference's
+    sequence call by call.  Returns the state BackwardPropagation needs."""
+    from . import linear
+    if V.Shape != K.Shape:
+        raise ValueError("V.Shape and K.Shape must be equal, but are %s and %s" % (V.Shape, K.Shape))
+    if V.Shape != y.Shape:
+        raise ValueError("V.Shape and y.Shape must be equal, but are %s and %s" % (V.Shape, y.Shape))
+    if Q.Shape[2] != V.Shape[2]:
+        raise ValueError("queries.Shape[2] and values.Shape[2] must be equal (same embedding dim)")
+    w = Q.Wrapper
+    batch_size, tq, tkv = K.Shape[0], Q.Shape[1], V.Shape[1]
+    H, dk, dv = num_heads, key_dim, value_dim
+    st = MultiheadAttentionState()
+    st.dims = (batch_size, tq, tkv, H, dk, dv)
+    st.heads_in_place = heads_in_place
+    Q_heads = GPUTensor([batch_size * tq, H * dk], None, w)
+    K_heads = GPUTensor([batch_size * tkv, H * dk], None, w)
+    V_heads = GPUTensor([batch_size * tkv, H * dv], None, w)
+    linear.DenseForwardPropagation(Q_heads, Q, w_Q, w_Q_bias, True)                          # :201-202
+    linear.DenseForwardPropagation(K_heads, K, w_K, w_K_bias, True)                          # :207-208
+    linear.DenseForwardPropagation(V_heads, V, w_V, w_V_bias, True)                          # :213-214
+    scaling = 1.0 / math.sqrt(dk) if use_scale else 1.0
+    if heads_in_place:
+        scores = GPUTensor([batch_size * H, tq, tkv], None, w)
+        _heads_gemm(scores, Q_heads, K_heads, transA=False, transB=True, M=tq, N=tkv, K=dk, alpha=scaling,
+                    batch=batch_size, heads=H, a_packed=True, b_packed=True, c_packed=False, a_steps=tq, b_steps=tkv,
+                    c_steps=0, a_dim=dk, b_dim=dk, c_dim=0)
+        if is_causal:
+            scores.SetAllElementsAboveMainDiagonal(-1e12)
+        weights = GPUTensor(scores.Shape, None, w)
+        scores.SoftmaxLastDimension(weights)
+        scores.Dispose()
+        attention_heads_T = GPUTensor([batch_size, tkv, H * dv], None, w)
+        _heads_gemm(attention_heads_T, weights, V_heads, transA=False, transB=False, M=tq, N=dv, K=tkv, alpha=1.0,
+                    batch=batch_size, heads=H, a_packed=False, b_packed=True, c_packed=True, a_steps=0, b_steps=tkv,
+                    c_steps=tkv, a_dim=0, b_dim=dv, c_dim=dv)
+        st.Q_heads, st.K_heads, st.V_heads = Q_heads, K_heads, V_heads
+    else:
+        def split(packed, steps, dim):                                                      # :203-205
+            t = GPUTensor([batch_size, H, steps, dim], None, w)
+            packed.Reshape(batch_size, steps, H, dim).TransposeSecondAndThirdDimension(t)
+            packed.Dispose()
+            return t.Reshape(batch_size * H, steps, dim)
+        Q_heads_T, K_heads_T, V_heads_T = split(Q_heads, tq, dk), split(K_heads, tkv, dk), split(V_heads, tkv, dv)
+        attention_heads = GPUTensor(V_heads_T.Shape, None, w)
+        weights = ScaledDotProductAttentionForwardPropagation(Q_heads_T, K_heads_T, V_heads_T, attention_heads, True,
+                                                              use_scale, is_causal)           # :221
+        attention_heads_T = GPUTensor([batch_size, tkv, H, dv], None, w)
+        attention_heads.Reshape(batch_size, H, tkv, dv).TransposeSecondAndThirdDimension(attention_heads_T)   # :224
+        attention_heads_T = attention_heads_T.Reshape(batch_size, tkv, H * dv)
+        st.Q_heads, st.K_heads, st.V_heads = Q_heads_T, K_heads_T, V_heads_T
+    linear.DenseForwardPropagation(y, attention_heads_T, out_proj_weight, out_proj_bias, True)   # :226
+    st.weights_buffer, st.attention_heads_T = weights, attention_heads_T
+    return st if isTraining else None
+
+
+def MultiheadAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, st, w_Q, w_K, w_V, out_proj_weight, grads,
+                                          use_scale=True, compatibility_mode="PyTorch"):
+    """MultiheadAttention.BackwardPropagation (:243-292).  ``grads`` maps 'w_Q', 'w_K', 'w_V', 'out_proj_weight' to
+    (weightGradients, biasGradientsOrNone) tensors that are filled in; dQ, dK, dV receive the input gradients."""
+    from . import linear
+    w = Q.Wrapper
+    batch_size, tq, tkv, H, dk, dv = st.dims
+    d_attention_heads_T = GPUTensor(st.attention_heads_T.Shape, None, w)
+    gw, gb = grads["out_proj_weight"]
+    linear.DenseBackwardPropagation(d_attention_heads_T, gw, gb, st.attention_heads_T, dy, out_proj_weight,
+                                    compatibility_mode=compatibility_mode, flattenInputTensorOnLastDimension=True)   # :258
+    # The reference's backward takes the scale from the value dimension (embedding_dim = dV.Shape[2],
+    # ScaledDotProductAttentionLayer.cs:113-121) while its forward uses the key dimension (:60); the two agree
+    # whenever key_dim == value_dim, which is all the reference ever tests.  Mirrored as is.
+    scaling = 1.0 / math.sqrt(dv) if use_scale else 1.0
+    P = st.weights_buffer
+    if st.heads_in_place:
+        dQ_p = GPUTensor([batch_size * tq, H * dk], None, w)
+        dK_p = GPUTensor([batch_size * tkv, H * dk], None, w)
+        dV_p = GPUTensor([batch_size * tkv, H * dv], None, w)
+        common = dict(batch=batch_size, heads=H)
+        # dV = P^T . dO                                                              (ScaledDotProductAttentionLayer.cs:117)
+        _heads_gemm(dV_p, P, d_attention_heads_T, transA=True, transB=False, M=tkv, N=dv, K=tq, alpha=1.0, a_packed=False,
+                    b_packed=True, c_packed=True, a_steps=0, b_steps=tq, c_steps=tkv, a_dim=0, b_dim=dv, c_dim=dv, **common)
+        # dS = scale * dO . V^T, then through the softmax                             (:123-125)
+        dS = GPUTensor(P.Shape, None, w)
+        _heads_gemm(dS, d_attention_heads_T, st.V_heads, transA=False, transB=True, M=tq, N=tkv, K=dv, alpha=scaling,
+                    a_packed=True, b_packed=True, c_packed=False, a_steps=tq, b_steps=tkv, c_steps=0, a_dim=dv, b_dim=dv,
+                    c_dim=0, **common)
+        P.SoftmaxLastDimensionBackward(dS, dS)
+        # dQ = dS . K, dK = dS^T . Q                                                 (:127-128)
+        _heads_gemm(dQ_p, dS, st.K_heads, transA=False, transB=False, M=tq, N=dk, K=tkv, alpha=1.0, a_packed=False,
+                    b_packed=True, c_packed=True, a_steps=0, b_steps=tkv, c_steps=tq, a_dim=0, b_dim=dk, c_dim=dk, **common)
+        _heads_gemm(dK_p, dS, st.Q_heads, transA=True, transB=False, M=tkv, N=dk, K=tq, alpha=1.0, a_packed=False,
+                    b_packed=True, c_packed=True, a_steps=0, b_steps=tq, c_steps=tkv, a_dim=0, b_dim=dk, c_dim=dk, **common)
+        dS.Dispose()
+    else:
+        d_attention_heads = GPUTensor([batch_size, H, tkv, dv], None, w)
+        d_attention_heads_T.Reshape(batch_size, tkv, H, dv).TransposeSecondAndThirdDimension(d_attention_heads)     # :263
+        d_attention_heads = d_attention_heads.Reshape(batch_size * H, tkv, dv)
+        dQ_h, dK_h, dV_h = (GPUTensor(t.Shape, None, w) for t in (st.Q_heads, st.K_heads, st.V_heads))
+        ScaledDotProductAttentionBackwardPropagation(dQ_h, dK_h, dV_h, st.Q_heads, st.K_heads, st.V_heads,
+                                                     d_attention_heads, P, use_scale)                               # :270
+        def merge(t, steps, dim):                                                                                   # :276,279,282
+            out = GPUTensor([batch_size, steps, H, dim], None, w)
+            t.Reshape(batch_size, H, steps, dim).TransposeSecondAndThirdDimension(out)
+            t.Dispose()
+            return out.Reshape(batch_size * steps, H * dim)
+        dQ_p, dK_p, dV_p = merge(dQ_h, tq, dk), merge(dK_h, tkv, dk), merge(dV_h, tkv, dv)
+    for dx, x, dpacked, wt, key in ((dQ, Q, dQ_p, w_Q, "w_Q"), (dK, K, dK_p, w_K, "w_K"), (dV, V, dV_p, w_V, "w_V")):
+        gw, gb = grads[key]
+        linear.DenseBackwardPropagation(dx, gw, gb, x, dpacked, wt, compatibility_mode=compatibility_mode,
+                                        flattenInputTensorOnLastDimension=True)                                      # :277-283
+        dpacked.Dispose()
+    d_attention_heads_T.Dispose()

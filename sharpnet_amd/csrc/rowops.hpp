@@ -130,6 +130,24 @@ __global__ void __launch_bounds__(256) softmax_rows_bwd_kernel(const float* __re
     for (int c = lane; c < cols; c += 64) dxr[c] = yr[c] * (dyr[c] - s);
 }
 
+// dst[a][c][b][d] = src[a][b][c][d]: TransposeSecondAndThirdDimension (Prod/CPU/CpuTensor.cs:301-322, GPU kernel
+// SinglePrecision.cu:1285), the head split / merge copy of MultiheadAttention.cs:207-230.  One thread per element
+// of dst, so writes are contiguous and reads are contiguous over d.
+__global__ void __launch_bounds__(256) transpose_2nd_3rd_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                                int A, int B, int C, int D) {
+    const long long total = (long long)A * B * C * D;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long long)gridDim.x * blockDim.x) {
+        const int d = (int)(i % D);
+        long long t = i / D;
+        const int b = (int)(t % B);
+        t /= B;
+        const int c = (int)(t % C);
+        const int a = (int)(t / C);
+        dst[i] = src[(((long long)a * B + b) * C + c) * D + d];
+    }
+}
+
 // x[b][r][c] = value for c > r
 __global__ void __launch_bounds__(256) set_above_diagonal_kernel(float* x, long long matrices, int rows, int cols,
                                                                  float value) {

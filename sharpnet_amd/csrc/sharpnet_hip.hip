@@ -755,6 +755,18 @@ int snhip_activation_backward(void* handle, int activation, float activation_par
     return hip_to_status(hipGetLastError());
 }
 
+int snhip_transpose_second_and_third_dimension(void* handle, const float* src, float* dst, int d0, int d1, int d2,
+                                               int d3) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (d0 < 0 || d1 < 0 || d2 < 0 || d3 < 0) return SNHIP_STATUS_INVALID_VALUE;
+    const long long total = (long long)d0 * d1 * d2 * d3;
+    if (total == 0) return SNHIP_STATUS_SUCCESS;
+    if (src == nullptr || dst == nullptr || src == dst) return SNHIP_STATUS_INVALID_VALUE;
+    hipLaunchKernelGGL(transpose_2nd_3rd_kernel, dim3(grid_for(total)), dim3(256), 0, static_cast<Handle*>(handle)->stream,
+                       src, dst, d0, d1, d2, d3);
+    return hip_to_status(hipGetLastError());
+}
+
 int snhip_broadcast_add_vector(void* handle, const float* vector, float* y, int rows, int cols) {
     if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     if (rows < 0 || cols < 0) return SNHIP_STATUS_INVALID_VALUE;

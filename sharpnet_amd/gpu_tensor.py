@@ -369,6 +369,16 @@ def _add_tensor_methods():
         check_status(self._lib.snhip_set_above_main_diagonal(self.Wrapper.handle, self.Pointer, m, r, c, value),
                      "snhip_set_above_main_diagonal")
 
+    def TransposeSecondAndThirdDimension(self, target):
+        """target[a][c][b][d] = this[a][b][c][d]; target is reshaped to the swapped shape (CpuTensor.cs:301-322)."""
+        assert len(self.Shape) >= 3 and target.Count == self.Count
+        A, B, C = self.Shape[:3]
+        D = self.Count // max(A * B * C, 1)
+        target.Shape = [A, C, B] + list(self.Shape[3:])
+        check_status(self._lib.snhip_transpose_second_and_third_dimension(self.Wrapper.handle, self.Pointer, target.Pointer,
+                                                                          A, B, C, D),
+                     "snhip_transpose_second_and_third_dimension")
+
     def ActivationForward(self, activationType, activationParameter, y):
         """y = act(this) for the RELU / LEAKY_RELU / SIGMOID / TANH modes (Tensor.ActivationForward);
         activationParameter is the leaky slope."""
@@ -384,7 +394,8 @@ def _add_tensor_methods():
                                                          dx.Pointer, self.Count), "snhip_activation_backward")
 
     for f in (Compute_BiasGradient_from_dy, BroadcastAddVectorToOutput, Update_Adding_Alpha_X, SoftmaxLastDimension,
-              SoftmaxLastDimensionBackward, SetAllElementsAboveMainDiagonal, ActivationForward, ActivationBackward):
+              SoftmaxLastDimensionBackward, SetAllElementsAboveMainDiagonal, TransposeSecondAndThirdDimension,
+              ActivationForward, ActivationBackward):
         setattr(GPUTensor, f.__name__, f)
 
 

@@ -120,6 +120,7 @@ SIGNATURES = {
     "snhip_activation_forward": [_vp, _i, _f, _vp, _vp, _ll],
     "snhip_activation_backward": [_vp, _i, _f, _vp, _vp, _vp, _ll],
     "snhip_bias_gradient": [_vp, _vp, _i, _i, _vp],
+    "snhip_transpose_second_and_third_dimension": [_vp, _vp, _vp, _i, _i, _i, _i],
     "snhip_broadcast_add_vector": [_vp, _vp, _vp, _i, _i],
     "snhip_axpy": [_vp, _ll, _f, _vp, _vp],
     "snhip_softmax_last_dim": [_vp, _vp, _vp, _ll, _i],

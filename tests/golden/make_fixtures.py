@@ -121,6 +121,29 @@ def main():
         "tolerance": 1e-6,
     }
 
+    # ---- same file :1013-1131  multi-head attention chain, without and with bias ----
+    mha = {}
+    for name, lo, hi in (("no_bias", 1013, 1071), ("with_bias", 1073, 1131)):
+        blk = lines(prp, lo, hi)
+        w = numpy_literals(blk)
+        assert len(w) == 6 and len(w[3]) == 18 and len(w[4]) == 6 and len(w[5]) == 3 and len(w[5][0]) == 12, name
+        cases = re.findall(r'\[TestCase\((false|true),\s*([0-9.eE+-]+),\s*([0-9.eE+-]+)\)\]', blk)
+        assert len(cases) == 2
+        mha[name] = {
+            "conv_q": w[0], "conv_k": w[1], "conv_v": w[2], "in_proj_weight": w[3], "out_proj_weight": w[4],
+            "dense_weight_out_in": w[5],
+            "cases": [{"is_causal": c[0] == "true", "loss_before": float(c[1]), "loss_after": float(c[2])} for c in cases],
+        }
+    fx["PyTorch_MultiHeadAttention"] = {
+        "source": "Tests/NonReg/ParallelRunWithPyTorch.cs:1013-1131; X = numpy_array_for_tests(10,2,6) read as (N, C=2, L=6), "
+                  "Y = y_numpy_array_for_tests(10,3); three width-1 Conv1D (with bias, zero at start) feed Q, K, V of a "
+                  "MultiheadAttention(num_heads=3, key_dim=value_dim=2), then Flatten, Linear(3, bias), softmax, categorical "
+                  "cross-entropy; SGD(0.1, momentum 0.9), batch size 2, 10 epochs, no shuffling; all biases start at zero",
+        "x_shape": [10, 2, 6], "y_shape": [10, 3], "num_heads": 3, "key_dim": 2, "value_dim": 2,
+        "lr": 0.1, "momentum": 0.9, "epochs": 10, "batch_size": 2, "tolerance": 1e-6,
+        "no_bias": mha["no_bias"], "with_bias": mha["with_bias"],
+    }
+
     with open(OUT, "w") as f:
         json.dump(fx, f, indent=1)
     print("wrote", OUT, os.path.getsize(OUT), "bytes")

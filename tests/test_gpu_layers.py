@@ -272,3 +272,85 @@ def test_row_helpers_vs_numpy(gpu_wrapper):
     for r in range(5):
         want[:, r, r + 1:] = np.float32(-1e12)
     assert np.array_equal(gm.ToNumpy(), want)
+
+
+def _gpu_mha(gpu_wrapper, heads_in_place):
+    """mha_forward / mha_backward with the oracle's signatures, computed by the device mirror."""
+    from sharpnet_amd import GPUTensor, attention
+    w = gpu_wrapper
+
+    def fwd(Q, K, V, w_Q, w_K, w_V, w_O, H, dk, dv, b_Q=None, b_K=None, b_V=None, b_O=None, is_causal=False,
+            use_scale=True):
+        opt = lambda a: None if a is None else T(w, a)
+        g = dict(Q=T(w, Q), K=T(w, K), V=T(w, V), w_Q=T(w, w_Q), w_K=T(w, w_K), w_V=T(w, w_V), w_O=T(w, w_O),
+                 b=[opt(b_Q), opt(b_K), opt(b_V), opt(b_O)])
+        gy = GPUTensor(list(V.shape), None, w)
+        gy.SetValue(float("nan"))
+        st = attention.MultiheadAttentionForwardPropagation(
+            g["Q"], g["K"], g["V"], gy, g["w_Q"], g["w_K"], g["w_V"], g["w_O"], H, dk, dv, *g["b"], isTraining=True,
+            use_scale=use_scale, is_causal=is_causal, heads_in_place=heads_in_place)
+        g["st"], g["use_scale"] = st, use_scale
+        return gy.ToNumpy(), g
+
+    def bwd(dy, g):
+        has_b = g["b"][0] is not None
+        grads, outs = {}, {}
+        for key, wt in (("w_Q", g["w_Q"]), ("w_K", g["w_K"]), ("w_V", g["w_V"]), ("out_proj_weight", g["w_O"])):
+            gw = GPUTensor(wt.Shape, None, w)
+            gb = GPUTensor([wt.Shape[0]], None, w) if has_b else None
+            for t in (gw, gb):
+                if t is not None:
+                    t.SetValue(float("nan"))
+            grads[key] = (gw, gb)
+        dQ, dK, dV = (GPUTensor(g[k].Shape, None, w) for k in ("Q", "K", "V"))
+        attention.MultiheadAttentionBackwardPropagation(dQ, dK, dV, g["Q"], g["K"], g["V"], T(w, dy), g["st"], g["w_Q"],
+                                                        g["w_K"], g["w_V"], g["w_O"], grads, use_scale=g["use_scale"])
+        outs.update(dQ=dQ.ToNumpy(), dK=dK.ToNumpy(), dV=dV.ToNumpy())
+        for key, short in (("w_Q", "Q"), ("w_K", "K"), ("w_V", "V"), ("out_proj_weight", "O")):
+            outs["dw_" + short] = grads[key][0].ToNumpy()
+            outs["db_" + short] = grads[key][1].ToNumpy() if has_b else None
+        return outs
+    return fwd, bwd
+
+
+@pytest.mark.parametrize("heads_in_place", [True, False])
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_multi_head_attention_forward_backward(oracle, gpu_wrapper, heads_in_place, is_causal):
+    """MultiheadAttention forward and backward (MultiheadAttention.cs:178-292) on the device, with the heads
+    multiplied in place (two-level strided batch) or through the reference's transposition copies, against the
+    oracle; biases on, a batch / step count that leaves ragged tiles (key_dim == value_dim: the reference's attention
+    requires K and V of one shape, ScaledDotProductAttentionLayer.cs:48-51)."""
+    rng = np.random.default_rng(21)
+    B, Tn, H, dk, dv = 3, 37, 4, 16, 16
+    E = H * dv
+    Q, K, V = (random_tensor(rng, (B, Tn, E), -1, 1) for _ in range(3))
+    w_Q, w_K = (random_tensor(rng, (H * dk, E), -0.3, 0.3) for _ in range(2))
+    w_V, w_O = (random_tensor(rng, (H * dv, E), -0.3, 0.3) for _ in range(2))
+    b_Q, b_K = (random_tensor(rng, (H * dk,), -0.5, 0.5) for _ in range(2))
+    b_V, b_O = (random_tensor(rng, (H * dv,), -0.5, 0.5) for _ in range(2))
+    dy = random_tensor(rng, (B, Tn, E), -1, 1)
+    fwd, bwd = _gpu_mha(gpu_wrapper, heads_in_place)
+    y, g = fwd(Q, K, V, w_Q, w_K, w_V, w_O, H, dk, dv, b_Q, b_K, b_V, b_O, is_causal=is_causal)
+    ry, cache = oracle.mha_forward(Q, K, V, w_Q, w_K, w_V, w_O, H, dk, dv, b_Q, b_K, b_V, b_O, is_causal=is_causal)
+    scale = float(np.max(np.abs(ry)))
+    assert np.max(np.abs(y - ry)) <= 2e-4 * scale, np.max(np.abs(y - ry))
+    got = bwd(dy, g)
+    want = oracle.mha_backward(dy, cache)
+    for k, ref in want.items():
+        err = float(np.max(np.abs(got[k] - ref)))
+        assert err <= 3e-4 * max(float(np.max(np.abs(ref))), 1.0), (k, err)
+
+
+@pytest.mark.parametrize("variant,is_causal", [("no_bias", False), ("no_bias", True), ("with_bias", False),
+                                               ("with_bias", True)])
+def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrapper, variant, is_causal):
+    """Tests/NonReg/ParallelRunWithPyTorch.cs:1013-1131: the stored losses before and after 10 epochs with every
+    product of the MultiheadAttention layer (projections, per-head scores and outputs, all gradients) on the device,
+    heads multiplied in place."""
+    from tests.test_oracle import _mha_chain
+    fx = golden["PyTorch_MultiHeadAttention"]
+    case = [c for c in fx[variant]["cases"] if c["is_causal"] == is_causal][0]
+    fwd, bwd = _gpu_mha(gpu_wrapper, True)
+    before, after = _mha_chain(oracle, fx, variant, is_causal, mha_fwd=fwd, mha_bwd=bwd)
+    assert abs(before - case["loss_before"]) < 2e-6, (before, case)
+    assert abs(after - case["loss_after"]) < 5e-6, (after, case)

@@ -302,3 +302,73 @@ def test_sdpa_backward_by_finite_differences(oracle):
             ap[name], am[name] = xp, xm
             num[idx] = (f(ap["Q"], ap["K"], ap["V"]) - f(am["Q"], am["K"], am["V"])) / (2 * eps)
         assert np.max(np.abs(num - dX)) < 2e-4, name
+
+
+def _mha_chain(oracle, fx, variant, is_causal, mha_fwd=None, mha_bwd=None):
+    """The network of Tests/NonReg/ParallelRunWithPyTorch.cs:1013-1131 trained exactly as there; returns
+    (loss_before, loss_after).  mha_fwd / mha_bwd default to the oracle's (the GPU test passes its own)."""
+    mha_fwd = mha_fwd or oracle.mha_forward
+    mha_bwd = mha_bwd or oracle.mha_backward
+    v = fx[variant]
+    use_bias = variant == "with_bias"
+    X = numpy_array_for_tests(*fx["x_shape"])                  # (10, C=2, L=6)
+    Y = y_numpy_array_for_tests(*fx["y_shape"])
+    H, dk, dv = fx["num_heads"], fx["key_dim"], fx["value_dim"]
+    E = H * dk
+    inw = np.array(v["in_proj_weight"], np.float32)
+    P = {"cq": np.array(v["conv_q"], np.float32)[:, :, 0], "ck": np.array(v["conv_k"], np.float32)[:, :, 0],
+         "cv": np.array(v["conv_v"], np.float32)[:, :, 0], "cqb": np.zeros(2, np.float32), "ckb": np.zeros(2, np.float32),
+         "cvb": np.zeros(2, np.float32), "wq": inw[0:E].copy(), "wk": inw[E:2 * E].copy(), "wv": inw[2 * E:3 * E].copy(),
+         "wo": np.array(v["out_proj_weight"], np.float32), "dw": np.array(v["dense_weight_out_in"], np.float32),
+         "db": np.zeros(3, np.float32)}
+    if use_bias:
+        P.update(bq=np.zeros(E, np.float32), bk=np.zeros(E, np.float32), bv=np.zeros(E, np.float32), bo=np.zeros(E, np.float32))
+    vel = {k: np.zeros_like(p) for k, p in P.items()}
+
+    def conv(x, W, b):                                         # width-1 Conv1D over (N, C, L)
+        return np.stack([oracle.dot(W, False, x[n], False) + b[:, None] for n in range(x.shape[0])]).astype(np.float32)
+
+    def forward(x):
+        q, k, vv = conv(x, P["cq"], P["cqb"]), conv(x, P["ck"], P["ckb"]), conv(x, P["cv"], P["cvb"])
+        y, cache = mha_fwd(q, k, vv, P["wq"], P["wk"], P["wv"], P["wo"], H, dk, dv, P.get("bq"), P.get("bk"), P.get("bv"),
+                           P.get("bo"), is_causal=is_causal)
+        flat = y.reshape(x.shape[0], -1)
+        logits = oracle.dense_forward(flat, P["dw"], P["db"])
+        return oracle.softmax_last_dim(logits), (flat, cache)
+
+    def loss():
+        p = forward(X)[0].astype(np.float64)
+        return float(np.mean(-np.sum(Y * np.log(p), axis=1)))
+
+    before = loss()
+    bs = fx["batch_size"]
+    for _ in range(fx["epochs"]):
+        for i in range(0, X.shape[0], bs):
+            x, y = X[i:i + bs], Y[i:i + bs]
+            p, (flat, cache) = forward(x)
+            dlogits = (p - y).astype(np.float32)                # Tensor.cs:1389-1395; the 1/batch sits in the update
+            G = {}
+            G["dw"], G["db"], dflat = oracle.dense_backward(flat, dlogits, P["dw"])
+            g = mha_bwd(dflat.reshape(x.shape[0], 2, E), cache)
+            G["wq"], G["wk"], G["wv"], G["wo"] = g["dw_Q"], g["dw_K"], g["dw_V"], g["dw_O"]
+            if use_bias:
+                G["bq"], G["bk"], G["bv"], G["bo"] = g["db_Q"], g["db_K"], g["db_V"], g["db_O"]
+            for name, d in (("cq", g["dQ"]), ("ck", g["dK"]), ("cv", g["dV"])):
+                G[name] = sum(oracle.dot(d[n], False, x[n], True) for n in range(x.shape[0])).astype(np.float32)
+                G[name + "b"] = d.sum(axis=(0, 2)).astype(np.float32)
+            for k in P:                                         # Sgd.cs / CpuTensor.cs:470-489, lr / batchSize
+                vel[k] = (np.float32(fx["momentum"]) * vel[k] - G[k] * np.float32(fx["lr"] / bs)).astype(np.float32)
+                P[k] = (P[k] + vel[k]).astype(np.float32)
+    return before, loss()
+
+
+@pytest.mark.parametrize("variant", ["no_bias", "with_bias"])
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_multi_head_attention_chain_losses(golden, oracle, variant, is_causal):
+    """Both stored losses of Test_MultiHeadAttention_{no,with}_bias: the first pins mha_forward (projections, head
+    split, scaled scores, causal mask, softmax, head merge), the second - 50 SGD steps later - mha_backward."""
+    fx = golden["PyTorch_MultiHeadAttention"]
+    case = [c for c in fx[variant]["cases"] if c["is_causal"] == is_causal][0]
+    before, after = _mha_chain(oracle, fx, variant, is_causal)
+    assert abs(before - case["loss_before"]) < fx["tolerance"], (before, case)     # the reference's own 1e-6
+    assert abs(after - case["loss_after"]) < fx["tolerance"], (after, case)
