@@ -242,6 +242,7 @@ def main():
             extra["config2_8192_bf16_input_TN"] = hb
         finally:
             w.set_math_mode(w.MATH_FP32)
+        extra["layers_fused_vs_reference_sequence"] = layer_timings(w, wl)
         out["extra"] = extra
         for k, v in extra.items():
             log("[bench]", k, json.dumps(v))
@@ -251,10 +252,90 @@ def main():
     print(json.dumps(out), flush=True)
 
 
+def layer_timings(w, wl):
+    """Linear and multi-head-attention layers as whole calls of the host mirrors: the library's fused forms against
+    the reference's own sequence of calls, both on the device, HIP events around `steps` repetitions (host launch
+    time included: for the small layer that is most of it)."""
+    from sharpnet_amd import GPUTensor, linear, attention
+    rng = np.random.default_rng(7)
+    w.use_memory_pool(True)
+
+    def T(shape, lo=-1.0, hi=1.0):
+        return GPUTensor(list(shape), rng.uniform(lo, hi, shape).astype(np.float32), w)
+
+    def timed(fn, steps, warm):
+        t0 = time.perf_counter()
+        n = 0
+        while n < warm or time.perf_counter() - t0 < 0.06:   # clocks take tens of ms to come up after an idle spell
+            fn()
+            n += 1
+        w.synchronize()
+        e0, e1 = w.new_event(), w.new_event()
+        w.record(e0)
+        for _ in range(steps):
+            fn()
+        w.record(e1)
+        ms = w.elapsed_ms(e0, e1) / steps
+        w.destroy_event(e0)
+        w.destroy_event(e1)
+        return round(ms, 4)
+
+    res = []
+    for (rows, fin, fout, steps) in ((128, 784, 256, 200), (4096, 4096, 4096, 10)):
+        x, W, b, dy = T((rows, fin)), T((fout, fin), -0.05, 0.05), T((fout,)), T((rows, fout))
+        y, dx, dW, db = (GPUTensor(sh, None, w) for sh in ([rows, fout], [rows, fin], [fout, fin], [fout]))
+        for fused in (True, False):
+            f = timed(lambda: linear.DenseForwardPropagation(y, x, W, b, False, fused=fused,
+                                                             activation="CUDNN_ACTIVATION_RELU"), steps, steps // 2)
+            bwd = timed(lambda: linear.DenseBackwardPropagation(dx, dW, db, x, dy, W, bias_1D=b, compatibility_mode="PyTorch",
+                                                                use_weight_decay_in_backpropagation=True, weight_decay=1e-4,
+                                                                fused=fused), steps, steps // 2)
+            res.append({"layer": "Linear %dx%d->%d: forward with bias + ReLU; backward with bias gradient + weight decay"
+                                 % (rows, fin, fout), "form": "fused" if fused else "reference sequence",
+                        "forward_ms": f, "backward_ms": bwd})
+        for t in (x, W, b, dy, y, dx, dW, db):
+            t.Dispose()
+    B, Tn, H, d = 64, 256, 8, 64
+    E = H * d
+    Q, K, V, dy = T((B, Tn, E)), T((B, Tn, E)), T((B, Tn, E)), T((B, Tn, E))
+    wq, wk, wv, wo = (T((E, E), -0.05, 0.05) for _ in range(4))
+    y, dQ, dK, dV = (GPUTensor([B, Tn, E], None, w) for _ in range(4))
+    grads = {k: (GPUTensor([E, E], None, w), None) for k in ("w_Q", "w_K", "w_V", "out_proj_weight")}
+    for in_place in (True, False):
+        state = {}
+
+        def fwd():
+            if state.get("st") is not None:      # a forward without its backward: give the kept buffers back
+                for t in (state["st"].weights_buffer, state["st"].Q_heads, state["st"].K_heads, state["st"].V_heads,
+                          state["st"].attention_heads_T):
+                    t.Dispose()
+            state["st"] = attention.MultiheadAttentionForwardPropagation(Q, K, V, y, wq, wk, wv, wo, H, d, d, is_causal=True,
+                                                                         heads_in_place=in_place)
+
+        def fwd_bwd():
+            fwd()
+            st = state["st"]
+            attention.MultiheadAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, st, wq, wk, wv, wo, grads)
+            for t in (st.weights_buffer, st.Q_heads, st.K_heads, st.V_heads, st.attention_heads_T):
+                t.Dispose()
+            state["st"] = None
+
+        f = timed(fwd, 10, 5)
+        fb = timed(fwd_bwd, 10, 5)
+        res.append({"layer": "MultiheadAttention batch %d, %d steps, %d heads x %d, causal" % (B, Tn, H, d),
+                    "form": "heads in place" if in_place else "reference sequence (transposition copies)",
+                    "forward_ms": f, "backward_ms": round(fb - f, 4)})
+    w.use_memory_pool(False)
+    return res
+
+
 def write_table(path, out):
     """Markdown rendering of the `extra` object (one row per GEMM) plus the headline figures of the same run."""
     rows = []
+    layers = out["extra"].get("layers_fused_vs_reference_sequence", [])
     for name, v in out["extra"].items():
+        if name == "layers_fused_vs_reference_sequence":
+            continue
         items = v if isinstance(v, list) else v.get("gemms") or [x for x in v.values() if isinstance(x, dict)] or [v]
         if isinstance(v, dict) and "gemm" in v:
             items = [v]
@@ -272,6 +353,12 @@ def write_table(path, out):
                 "| configuration | GEMM | ms | TFLOP/s | fraction of roofline | tile config | split-K |\n"
                 "|---|---|---|---|---|---|---|\n" % path)
         f.write("\n".join(rows) + "\n\n")
+        if layers:
+            f.write("Whole layer calls through the host mirrors (HIP events around repeated calls, host launch time included):\n\n"
+                    "| layer | form | forward ms | backward ms |\n|---|---|---|---|\n")
+            for r in layers:
+                f.write("| %s | %s | %.4f | %.4f |\n" % (r["layer"], r["form"], r["forward_ms"], r["backward_ms"]))
+            f.write("\n")
         f.write("Headline line of the same run: %.2f TFLOP/s (%.1f %% of fp32 MFMA peak)" %
                 (out["value"], 100.0 * out["roofline"]["frac"]))
         if cpu:

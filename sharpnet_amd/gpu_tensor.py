@@ -39,6 +39,7 @@ class GPUWrapper:
         check_status(self.lib.snhip_create(ctypes.byref(h)), "snhip_create")
         self.handle = h
         self._disposed = False
+        self._pool = None   # size in bytes -> released device pointers, when the memory pool is in use
 
     @classmethod
     def FromDeviceId(cls, device_id=0):
@@ -93,6 +94,36 @@ class GPUWrapper:
                         "kind": "bf16" if d[5] else "fp32"})
         return out
 
+    # -- device memory -------------------------------------------------------
+    def use_memory_pool(self, enabled=True):
+        """Keep released buffers and hand them out again for requests of the same size, as the reference's
+        TensorMemoryPool does for layer buffers (Prod/Data/TensorMemoryPool.cs:59-64: contents are NOT cleared).
+        Work on one stream stays ordered, so a reused buffer needs no device synchronisation."""
+        if enabled:
+            if self._pool is None:
+                self._pool = {}
+        else:
+            self.empty_memory_pool()
+            self._pool = None
+
+    def empty_memory_pool(self):
+        for ptrs in (self._pool or {}).values():
+            while ptrs:
+                check_status(self.lib.snhip_free(ptrs.pop()), "snhip_free")
+
+    def allocate(self, nbytes):
+        if self._pool is not None and self._pool.get(nbytes):
+            return self._pool[nbytes].pop()
+        p = ctypes.c_void_p()
+        check_status(self.lib.snhip_malloc(ctypes.byref(p), nbytes), "snhip_malloc")
+        return p.value
+
+    def release(self, ptr, nbytes):
+        if self._pool is not None and not self._disposed:
+            self._pool.setdefault(nbytes, []).append(ptr)
+        else:
+            check_status(self.lib.snhip_free(ptr), "snhip_free")
+
     # -- stream / timing ----------------------------------------------------
     def synchronize(self):
         check_status(self.lib.snhip_stream_synchronize(self.handle), "snhip_stream_synchronize")
@@ -115,6 +146,7 @@ class GPUWrapper:
 
     def Dispose(self):
         if not self._disposed:
+            self.empty_memory_pool()
             self._disposed = True
             check_status(self.lib.snhip_destroy(self.handle), "snhip_destroy")
             self.handle = None
@@ -145,10 +177,8 @@ class GPUTensor:
         else:
             self.IsOwnerOfMemory = True
             self._owner = None
-            p = ctypes.c_void_p()
-            nbytes = max(self.Count * 4, 8)  # capacity is at least 8 bytes (GpuTensor.cs:38)
-            check_status(self._lib.snhip_malloc(ctypes.byref(p), nbytes), "snhip_malloc")
-            self.Pointer = p.value
+            self._nbytes = max(self.Count * 4, 8)  # capacity is at least 8 bytes (GpuTensor.cs:38)
+            self.Pointer = self.Wrapper.allocate(self._nbytes)
             if data is not None:
                 self.InitializeFromHostMemory(data)
 
@@ -320,7 +350,7 @@ class GPUTensor:
             return
         self._disposed = True
         if self.IsOwnerOfMemory and self.Pointer:
-            check_status(self._lib.snhip_free(self.Pointer), "snhip_free")  # GpuTensor.cs:1634
+            self.Wrapper.release(self.Pointer, self._nbytes)  # GpuTensor.cs:1634 / TensorMemoryPool.FreeFloatTensor
         self.Pointer = None
 
     def __del__(self):
