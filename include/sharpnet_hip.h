@@ -167,6 +167,34 @@ int snhip_activation_forward(void* handle, int activation, float activation_para
 int snhip_activation_backward(void* handle, int activation, float activation_param, const float* y, const float* dy,
                               float* dx, long long n);
 
+/* ---- scaled-dot-product attention forward in one launch ------------------------ */
+/* O[z] = softmax(scale * Q[z] . K[z]^T, causal mask -1e12 above the diagonal) . V[z] for z in [0, batch): what
+ * ScaledDotProductAttentionLayer.ScaledDotProductAttentionForwardPropagation (Prod/Layers/
+ * ScaledDotProductAttentionLayer.cs:46-91) computes with two BatchMatrixMultiplication calls, a mask and a softmax
+ * pass, here without the (batch, Tq, Tk) scores ever being stored.  `weights` ([batch][Tq][Tk], contiguous) receives the
+ * softmax output the reference keeps for its backward pass (:87-90); NULL skips it (inference).
+ * Q is Tq x dk, K is Tk x dk, V is Tk x dv, O is Tq x dv, each with its own row pitch and two-level batch strides as in
+ * snhip_gemm_desc, so heads can be read from and written to a (batch, steps, heads * dim) activation in place.
+ * Supported: Tk <= 256, dk <= 64, dv <= 64; anything larger returns status 15 (NOT_SUPPORTED) and the caller issues the
+ * reference's sequence of calls instead. */
+typedef struct snhip_attention_desc {
+    int struct_size;
+    int batch, batch_inner; /* matrices; batch_inner as in snhip_gemm_desc (0: single level) */
+    int Tq, Tk, dk, dv;
+    float scale; /* 1/sqrt(dk) with use_scale, else 1 */
+    int causal;  /* 0 / 1 */
+    const float* Q;
+    const float* K;
+    const float* V;
+    float* O;
+    float* weights; /* or NULL */
+    int ldq, ldk, ldv, ldo;
+    long long strideQ, strideK, strideV, strideO;                             /* elements */
+    long long strideQ_outer, strideK_outer, strideV_outer, strideO_outer;     /* used when 0 < batch_inner < batch */
+} snhip_attention_desc;
+int snhip_attention_forward(void* handle, const snhip_attention_desc* desc);
+int snhip_sizeof_attention_desc(void);
+
 /* ---- bf16-input / fp32-accumulate variant (no reference counterpart) ------ */
 /* Operands stay fp32 in device memory; they are rounded to bf16 (nearest even)
  * on their way into LDS and multiplied with v_mfma_f32_32x32x16_bf16, products

@@ -5,12 +5,47 @@ Q, K, V, y are (batch, time, dim) tensors; the (batch, Tq, Tv) score and weight
 buffers are materialised exactly as the reference does.  Forward returns the
 weights buffer (kept for backward when training).
 """
+import ctypes
 import math
 
+from . import hiplib
 from .gpu_tensor import GPUTensor
+from .hiplib import CublasStatus, check_status
+
+FUSED_ATTENTION_MAX_KEYS = 256      # limits of snhip_attention_forward
+FUSED_ATTENTION_MAX_HEAD_DIM = 64
 
 
-def ScaledDotProductAttentionForwardPropagation(Q, K, V, y, isTraining, use_scale, is_causal):
+def fused_attention_forward(Q, K, V, O, weights, *, batch, heads, tq, tkv, dk, dv, scale, is_causal, packed):
+    """snhip_attention_forward.  packed=True: Q, K, V, O are (batch, steps, heads*dim) activations whose heads are
+    addressed in place; False: contiguous (batch*heads, steps, dim) stacks.  Returns False (nothing launched) when
+    the sizes are outside what the kernel handles."""
+    if tkv > FUSED_ATTENTION_MAX_KEYS or max(dk, dv) > FUSED_ATTENTION_MAX_HEAD_DIM:
+        return False
+
+    def strides(steps, dim):
+        if packed:
+            return heads * dim, dim, steps * heads * dim
+        return dim, steps * dim, heads * steps * dim
+    ldq, sq, sq2 = strides(tq, dk)
+    ldk, sk, sk2 = strides(tkv, dk)
+    ldv, sv, sv2 = strides(tkv, dv)
+    ldo, so, so2 = strides(tq, dv)
+    d = hiplib.AttentionDesc(batch=batch * heads, batch_inner=heads, Tq=tq, Tk=tkv, dk=dk, dv=dv, scale=scale,
+                             causal=int(bool(is_causal)), Q=Q.Pointer, K=K.Pointer, V=V.Pointer, O=O.Pointer,
+                             weights=weights.Pointer if weights is not None else None, ldq=ldq, ldk=ldk, ldv=ldv, ldo=ldo,
+                             strideQ=sq, strideK=sk, strideV=sv, strideO=so, strideQ_outer=sq2, strideK_outer=sk2,
+                             strideV_outer=sv2, strideO_outer=so2)
+    st = Q._lib.snhip_attention_forward(Q.Wrapper.handle, ctypes.byref(d))
+    if st == CublasStatus.CUBLAS_STATUS_NOT_SUPPORTED:
+        return False
+    check_status(st, "snhip_attention_forward")
+    return True
+
+
+def ScaledDotProductAttentionForwardPropagation(Q, K, V, y, isTraining, use_scale, is_causal, fused=True):
+    """fused=True runs the whole chain as one launch when the sizes allow it (at most 256 keys, head dimension at
+    most 64); otherwise, or with fused=False, the reference's four calls."""
     if V.Shape != K.Shape:
         raise ValueError("V.Shape and K.Shape must be equal, but are %s and %s" % (V.Shape, K.Shape))
     if V.Shape != y.Shape:
@@ -18,6 +53,15 @@ def ScaledDotProductAttentionForwardPropagation(Q, K, V, y, isTraining, use_scal
     if Q.Shape[2] != V.Shape[2]:
         raise ValueError("queries.Shape[2] and values.Shape[2] must be equal (same embedding dim)")
     batch_size, query_time_steps, value_time_steps, embedding_dim = K.Shape[0], Q.Shape[1], V.Shape[1], K.Shape[2]
+    if fused:
+        weights_buffer = GPUTensor([batch_size, query_time_steps, value_time_steps], None, Q.Wrapper) if isTraining else None
+        if fused_attention_forward(Q, K, V, y, weights_buffer, batch=batch_size, heads=1, tq=query_time_steps,
+                                   tkv=value_time_steps, dk=embedding_dim, dv=V.Shape[2],
+                                   scale=1.0 / math.sqrt(embedding_dim) if use_scale else 1.0, is_causal=is_causal,
+                                   packed=False):
+            return weights_buffer
+        if weights_buffer is not None:
+            weights_buffer.Dispose()
     scores_buffer = GPUTensor([batch_size, query_time_steps, value_time_steps], None, Q.Wrapper)
     scaling = 1.0 / math.sqrt(embedding_dim) if use_scale else 1.0
     scores_buffer.BatchMatrixMultiplication(Q, False, K, True, scaling, 0.0)              # :71
@@ -81,7 +125,8 @@ def _heads_gemm(c, a, b, *, transA, transB, M, N, K, alpha, batch, heads, a_pack
 
 def MultiheadAttentionForwardPropagation(Q, K, V, y, w_Q, w_K, w_V, out_proj_weight, num_heads, key_dim, value_dim,
                                          w_Q_bias=None, w_K_bias=None, w_V_bias=None, out_proj_bias=None,
-                                         isTraining=True, use_scale=True, is_causal=False, heads_in_place=True):
+                                         isTraining=True, use_scale=True, is_causal=False, heads_in_place=True,
+                                         fused_attention=True):
     """MultiheadAttention.ForwardPropagation.  heads_in_place=True multiplies the heads where the projections left
     them (two-level strided batch, no TransposeSecondAndThirdDimension copies, the attention output lands directly
     in the (batch, steps, heads*value_dim) layout the output projection reads); False issues the reference's
@@ -106,7 +151,21 @@ def MultiheadAttentionForwardPropagation(Q, K, V, y, w_Q, w_K, w_V, out_proj_wei
     linear.DenseForwardPropagation(K_heads, K, w_K, w_K_bias, True)                          # :207-208
     linear.DenseForwardPropagation(V_heads, V, w_V, w_V_bias, True)                          # :213-214
     scaling = 1.0 / math.sqrt(dk) if use_scale else 1.0
-    if heads_in_place:
+    fused_done = False
+    if heads_in_place and fused_attention:
+        weights = GPUTensor([batch_size * H, tq, tkv], None, w)
+        attention_heads_T = GPUTensor([batch_size, tkv, H * dv], None, w)
+        fused_done = fused_attention_forward(Q_heads, K_heads, V_heads, attention_heads_T, weights, batch=batch_size,
+                                             heads=H, tq=tq, tkv=tkv, dk=dk, dv=dv, scale=scaling, is_causal=is_causal,
+                                             packed=True)
+        if fused_done:
+            st.Q_heads, st.K_heads, st.V_heads = Q_heads, K_heads, V_heads
+        else:
+            weights.Dispose()
+            attention_heads_T.Dispose()
+    if fused_done:
+        pass
+    elif heads_in_place:
         scores = GPUTensor([batch_size * H, tq, tkv], None, w)
         _heads_gemm(scores, Q_heads, K_heads, transA=False, transB=True, M=tq, N=tkv, K=dk, alpha=scaling,
                     batch=batch_size, heads=H, a_packed=True, b_packed=True, c_packed=False, a_steps=tq, b_steps=tkv,
@@ -130,7 +189,7 @@ def MultiheadAttentionForwardPropagation(Q, K, V, y, w_Q, w_K, w_V, out_proj_wei
         Q_heads_T, K_heads_T, V_heads_T = split(Q_heads, tq, dk), split(K_heads, tkv, dk), split(V_heads, tkv, dv)
         attention_heads = GPUTensor(V_heads_T.Shape, None, w)
         weights = ScaledDotProductAttentionForwardPropagation(Q_heads_T, K_heads_T, V_heads_T, attention_heads, True,
-                                                              use_scale, is_causal)           # :221
+                                                              use_scale, is_causal, fused=False)   # :221
         attention_heads_T = GPUTensor([batch_size, tkv, H, dv], None, w)
         attention_heads.Reshape(batch_size, H, tkv, dv).TransposeSecondAndThirdDimension(attention_heads_T)   # :224
         attention_heads_T = attention_heads_T.Reshape(batch_size, tkv, H * dv)

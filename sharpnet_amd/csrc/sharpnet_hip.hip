@@ -10,6 +10,7 @@
 
 #include <new>
 
+#include "attention_mfma.hpp"
 #include "kernel_list.hpp"
 #include "rowops.hpp"
 
@@ -115,6 +116,19 @@ const ConfigEntry kConfigs[] = {
     make_entry_bf16<BTileCfg<1, 1, 2, 2, 64>>(3, 0.45, 0.60, 1.1),   // 13: 64 x 64, BK 64
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
+
+// Fused attention forward kernels (attention_mfma.hpp)
+struct AttnEntry {
+    int keys, hd, lds_bytes;
+    void (*fn)(const AttnParams);
+};
+template <int NT, int HD>
+constexpr AttnEntry attn_entry() {
+    return AttnEntry{AttnCfg<NT, HD>::KEYS, HD, AttnCfg<NT, HD>::LDS_BYTES, attention_fwd_kernel<NT, HD>};
+}
+// smallest first: the first entry that holds the problem is used
+const AttnEntry kAttn[] = {attn_entry<2, 32>(), attn_entry<4, 32>(), attn_entry<8, 32>(),
+                           attn_entry<2, 64>(), attn_entry<4, 64>(), attn_entry<8, 64>()};
 
 int hip_to_status(hipError_t e) {
     switch (e) {
@@ -528,6 +542,11 @@ int snhip_create(void** handle) {
                 if (e != hipSuccess) return hip_to_status(e);
             }
     }
+    for (const AttnEntry& c : kAttn) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                c.lds_bytes);
+        if (e != hipSuccess) return hip_to_status(e);
+    }
     Handle* h = new (std::nothrow) Handle();
     if (h == nullptr) return SNHIP_STATUS_ALLOC_FAILED;
     h->device = dev;
@@ -592,6 +611,56 @@ int snhip_gemm_rm(void* handle, int transposeA, int transposeB, int M, int N, in
                   int ldc, long long strideC, int batch, const float* bias) {
     return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha, A, lda, strideA, B,
                    ldb, strideB, beta, C, ldc, strideC, batch, bias);
+}
+
+int snhip_sizeof_attention_desc(void) { return (int)sizeof(snhip_attention_desc); }
+
+
+int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
+    Handle* h = static_cast<Handle*>(handle);
+    if (d == nullptr || d->struct_size != (int)sizeof(snhip_attention_desc)) return SNHIP_STATUS_INVALID_VALUE;
+    if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    {
+        int cur = -1;
+        if (hipGetDevice(&cur) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+        if (cur != h->device && hipSetDevice(h->device) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    }
+    if (d->batch < 0 || d->batch_inner < 0 || d->Tq < 0 || d->Tk < 0 || d->dk < 0 || d->dv < 0)
+        return SNHIP_STATUS_INVALID_VALUE;
+    if (d->batch == 0 || d->Tq == 0 || d->dv == 0) return SNHIP_STATUS_SUCCESS;
+    if (d->Tk == 0 || d->dk == 0) return SNHIP_STATUS_NOT_SUPPORTED;  // a softmax over no keys is not defined
+    if (d->Q == nullptr || d->K == nullptr || d->V == nullptr || d->O == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    if (d->ldq < d->dk || d->ldk < d->dk || d->ldv < d->dv || d->ldo < d->dv) return SNHIP_STATUS_INVALID_VALUE;
+    const int inner = d->batch_inner > 0 ? d->batch_inner : d->batch;
+    if (d->batch % inner != 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (d->batch > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
+    const int hd = d->dk > d->dv ? d->dk : d->dv;
+    const AttnEntry* e = nullptr;
+    for (const AttnEntry& c : kAttn)
+        if (d->Tk <= c.keys && hd <= c.hd) {
+            e = &c;
+            break;
+        }
+    if (e == nullptr) return SNHIP_STATUS_NOT_SUPPORTED;
+
+    AttnParams p;
+    p.Q = d->Q, p.K = d->K, p.V = d->V, p.O = d->O, p.P = d->weights;
+    p.Tq = d->Tq, p.Tk = d->Tk, p.dk = d->dk, p.dv = d->dv;
+    p.ldq = d->ldq, p.ldk = d->ldk, p.ldv = d->ldv, p.ldo = d->ldo;
+    p.sQ = d->strideQ, p.sK = d->strideK, p.sV = d->strideV, p.sO = d->strideO;
+    p.sQ2 = d->strideQ_outer, p.sK2 = d->strideK_outer, p.sV2 = d->strideV_outer, p.sO2 = d->strideO_outer;
+    p.batch_inner = inner;
+    p.scale = d->scale;
+    p.causal = d->causal != 0;
+    p.flags = 0;
+    const bool multi = d->batch > 1, two_level = multi && inner < d->batch;
+    if ((uintptr_t)d->O % 16 == 0 && d->ldo % 4 == 0 && (!multi || d->strideO % 4 == 0) &&
+        (!two_level || d->strideO_outer % 4 == 0))
+        p.flags |= 1;
+    if (d->weights != nullptr && (uintptr_t)d->weights % 16 == 0 && d->Tk % 4 == 0) p.flags |= 2;
+    hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(d->Tq, AT_BQ), (unsigned)d->batch), dim3(256), e->lds_bytes,
+                       h->stream, p);
+    return hip_to_status(hipGetLastError());
 }
 
 int snhip_sizeof_gemm_desc(void) { return (int)sizeof(snhip_gemm_desc); }

@@ -75,6 +75,11 @@ def test_gemm_descriptor_layout_matches_the_library():
     assert lib.snhip_gemm_ex(None, None) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
     d = hiplib.GemmDesc(M=1, N=1, K=1)
     assert lib.snhip_gemm_ex(None, ctypes.byref(d)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
+    assert lib.snhip_sizeof_attention_desc() == ctypes.sizeof(hiplib.AttentionDesc)
+    a = hiplib.AttentionDesc(batch=1, Tq=1, Tk=1, dk=1, dv=1)
+    assert lib.snhip_attention_forward(None, ctypes.byref(a)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
+    a.struct_size += 8
+    assert lib.snhip_attention_forward(None, ctypes.byref(a)) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
 
 
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):

@@ -354,3 +354,64 @@ def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrap
     before, after = _mha_chain(oracle, fx, variant, is_causal, mha_fwd=fwd, mha_bwd=bwd)
     assert abs(before - case["loss_before"]) < 2e-6, (before, case)
     assert abs(after - case["loss_after"]) < 5e-6, (after, case)
+
+
+@pytest.mark.parametrize("B,H,Tq,Tk,dk,dv,causal,packed", [
+    (5, 1, 37, 37, 16, 16, False, False), (5, 1, 37, 37, 16, 16, True, False),      # ragged, small tiles
+    (2, 3, 256, 256, 64, 64, True, True), (2, 3, 256, 256, 64, 64, False, False),   # the largest supported size
+    (3, 2, 200, 130, 24, 40, False, True), (3, 2, 129, 65, 33, 7, True, False),     # Tq != Tk, dk != dv, odd sizes
+    (1, 4, 1, 5, 3, 2, False, True),
+])
+def test_fused_attention_forward(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, causal, packed):
+    """snhip_attention_forward (scores, mask, softmax and P.V in one launch) against the oracle's
+    ScaledDotProductAttention, for stacked (batch*heads, steps, dim) operands and for heads addressed in place
+    inside (batch, steps, heads*dim) activations; both the output and the softmax weights kept for backward."""
+    from sharpnet_amd import GPUTensor, attention
+    rng = np.random.default_rng(31)
+    Z = B * H
+    q, k, v = random_tensor(rng, (Z, Tq, dk), -1, 1), random_tensor(rng, (Z, Tk, dk), -1, 1), \
+        random_tensor(rng, (Z, Tk, dv), -1, 1)
+    scale = 1.0 / np.sqrt(dk)
+    s = np.stack([oracle.dot(q[z], False, k[z], True, scale) for z in range(Z)])
+    if causal:
+        s[:, np.triu_indices(Tq, 1, Tk)[0], np.triu_indices(Tq, 1, Tk)[1]] = -1e12
+    wref = oracle.softmax_last_dim(s)
+    oref = oracle.bmm(wref, False, v, False)
+
+    def lay(x, steps, dim):            # (Z, steps, dim) -> what the device sees
+        if not packed:
+            return x
+        return np.ascontiguousarray(x.reshape(B, H, steps, dim).transpose(0, 2, 1, 3)).reshape(B, steps, H * dim)
+    gq, gk, gv = T(gpu_wrapper, lay(q, Tq, dk)), T(gpu_wrapper, lay(k, Tk, dk)), T(gpu_wrapper, lay(v, Tk, dv))
+    go = GPUTensor(list(lay(oref, Tq, dv).shape), None, gpu_wrapper)
+    gw = GPUTensor([Z, Tq, Tk], None, gpu_wrapper)
+    go.SetValue(float("nan"))
+    gw.SetValue(float("nan"))
+    assert attention.fused_attention_forward(gq, gk, gv, go, gw, batch=B, heads=H, tq=Tq, tkv=Tk, dk=dk, dv=dv,
+                                             scale=scale, is_causal=causal, packed=packed)
+    assert np.max(np.abs(gw.ToNumpy() - wref)) <= 2e-6 + 1e-5 * float(np.max(wref))
+    assert np.max(np.abs(go.ToNumpy() - lay(oref, Tq, dv))) <= 1e-5 * max(1.0, float(np.max(np.abs(v))))
+    # inference form: no weights requested, same output
+    go2 = GPUTensor(go.Shape, None, gpu_wrapper)
+    assert attention.fused_attention_forward(gq, gk, gv, go2, None, batch=B, heads=H, tq=Tq, tkv=Tk, dk=dk, dv=dv,
+                                             scale=scale, is_causal=causal, packed=packed)
+    assert np.array_equal(go2.ToNumpy(), go.ToNumpy())
+
+
+def test_fused_attention_limits(gpu_wrapper):
+    """Beyond 256 keys or a head dimension of 64 nothing is launched and the caller is told so."""
+    from sharpnet_amd import GPUTensor, attention
+    w = gpu_wrapper
+    big = GPUTensor([1, 300, 8], None, w)
+    out = GPUTensor([1, 300, 8], None, w)
+    assert attention.fused_attention_forward(big, big, big, out, None, batch=1, heads=1, tq=300, tkv=300, dk=8, dv=8,
+                                             scale=1.0, is_causal=False, packed=False) is False
+    wide = GPUTensor([1, 16, 80], None, w)
+    outw = GPUTensor([1, 16, 80], None, w)
+    assert attention.fused_attention_forward(wide, wide, wide, outw, None, batch=1, heads=1, tq=16, tkv=16, dk=80, dv=80,
+                                             scale=1.0, is_causal=False, packed=False) is False
+    # the layer mirror falls back to the four-call sequence on its own
+    y = GPUTensor([1, 300, 8], None, w)
+    big.SetValue(0.5)
+    wts = attention.ScaledDotProductAttentionForwardPropagation(big, big, big, y, True, True, False)
+    assert abs(float(wts.ToNumpy()[0, 0, 0]) - 1.0 / 300) < 1e-6 and abs(float(y.ToNumpy()[0, 7, 3]) - 0.5) < 1e-6
