@@ -43,6 +43,9 @@ def main():
                     help="also write the per-configuration figures of `extra` as a markdown table to PATH")
     ap.add_argument("--pcie", action="store_true",
                     help="also time the headline GEMM with host->device upload of A, B and device->host download of C")
+    ap.add_argument("--attention-probe", action="store_true",
+                    help="20 launches of the one-launch attention forward of configuration 5 (512 x 256 x 64, weights "
+                         "kept), for profilers")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: 3 plain copies of 1 GiB, then 3 headline GEMMs")
     args = ap.parse_args()
@@ -98,6 +101,18 @@ def main():
             gbias.Dispose()
         return wall_ms, ev_ms, gc
 
+    if args.attention_probe:
+        from sharpnet_amd import attention
+        rng = np.random.default_rng(5)
+        Z, Tn, d = 512, 256, 64
+        q, k, v = (GPUTensor([Z, Tn, d], rng.uniform(-1, 1, (Z, Tn, d)).astype(np.float32), w) for _ in range(3))
+        o, wts = GPUTensor([Z, Tn, d], None, w), GPUTensor([Z, Tn, Tn], None, w)
+        for keep in (wts, None):
+            for _ in range(20):
+                attention.fused_attention_forward(q, k, v, o, keep, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
+                                                  scale=0.125, is_causal=False, packed=False)
+            w.synchronize()
+        return
     if args.probe:
         # known-size launch: copy_f32_kernel reads 2**30 bytes and writes 2**30 bytes
         n = 1 << 28
@@ -295,13 +310,29 @@ def layer_timings(w, wl):
                         "forward_ms": f, "backward_ms": bwd})
         for t in (x, W, b, dy, y, dx, dW, db):
             t.Dispose()
+    # scaled-dot-product attention of benchmark configuration 5: 512 x (256 x 64), fp32
+    Z, Tn, d = 512, 256, 64
+    q, k, v = T((Z, Tn, d)), T((Z, Tn, d)), T((Z, Tn, d))
+    o = GPUTensor([Z, Tn, d], None, w)
+    for fused in (True, False):
+        for causal in (False, True):
+            def sdpa():
+                wts = attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, causal, fused=fused)
+                wts.Dispose()
+            ms = timed(sdpa, 20, 10)
+            res.append({"layer": "ScaledDotProductAttention forward 512 x (256 x 64)%s, weights kept" %
+                                 (", causal" if causal else ""),
+                        "form": "one launch" if fused else "reference sequence (4 calls)", "forward_ms": ms,
+                        "backward_ms": float("nan")})
+    for t in (q, k, v, o):
+        t.Dispose()
     B, Tn, H, d = 64, 256, 8, 64
     E = H * d
     Q, K, V, dy = T((B, Tn, E)), T((B, Tn, E)), T((B, Tn, E)), T((B, Tn, E))
     wq, wk, wv, wo = (T((E, E), -0.05, 0.05) for _ in range(4))
     y, dQ, dK, dV = (GPUTensor([B, Tn, E], None, w) for _ in range(4))
     grads = {k: (GPUTensor([E, E], None, w), None) for k in ("w_Q", "w_K", "w_V", "out_proj_weight")}
-    for in_place in (True, False):
+    for in_place, fused_attn in ((True, True), (True, False), (False, False)):
         state = {}
 
         def fwd():
@@ -310,7 +341,7 @@ def layer_timings(w, wl):
                           state["st"].attention_heads_T):
                     t.Dispose()
             state["st"] = attention.MultiheadAttentionForwardPropagation(Q, K, V, y, wq, wk, wv, wo, H, d, d, is_causal=True,
-                                                                         heads_in_place=in_place)
+                                                                         heads_in_place=in_place, fused_attention=fused_attn)
 
         def fwd_bwd():
             fwd()
@@ -323,7 +354,8 @@ def layer_timings(w, wl):
         f = timed(fwd, 10, 5)
         fb = timed(fwd_bwd, 10, 5)
         res.append({"layer": "MultiheadAttention batch %d, %d steps, %d heads x %d, causal" % (B, Tn, H, d),
-                    "form": "heads in place" if in_place else "reference sequence (transposition copies)",
+                    "form": ("heads in place, attention in one launch" if fused_attn else "heads in place") if in_place
+                    else "reference sequence (transposition copies)",
                     "forward_ms": f, "backward_ms": round(fb - f, 4)})
     w.use_memory_pool(False)
     return res
@@ -357,7 +389,8 @@ def write_table(path, out):
             f.write("Whole layer calls through the host mirrors (HIP events around repeated calls, host launch time included):\n\n"
                     "| layer | form | forward ms | backward ms |\n|---|---|---|---|\n")
             for r in layers:
-                f.write("| %s | %s | %.4f | %.4f |\n" % (r["layer"], r["form"], r["forward_ms"], r["backward_ms"]))
+                f.write("| %s | %s | %.4f | %s |\n" % (r["layer"], r["form"], r["forward_ms"],
+                                                         "" if r["backward_ms"] != r["backward_ms"] else "%.4f" % r["backward_ms"]))
             f.write("\n")
         f.write("Headline line of the same run: %.2f TFLOP/s (%.1f %% of fp32 MFMA peak)" %
                 (out["value"], 100.0 * out["roofline"]["frac"]))

@@ -5,8 +5,8 @@
 // (batch, Tq, Tk) scores travelling through memory three times.  Here they never leave the registers; the softmax
 // output P is written out once if the caller wants it (the reference keeps it for the backward pass, :87-90).
 //
-// Shape of the work.  A workgroup of four wavefronts owns 128 queries of one (batch, head) matrix; each wavefront owns
-// 32 of them and ALL keys (at most 256).  Both products are computed transposed so that the key axis of the scores
+// Shape of the work.  A workgroup of four wavefronts stages K and V of one (batch, head) matrix in LDS once and then
+// walks through its queries 128 at a time; each wavefront owns 32 of those and ALL keys (at most 256).  Both products are computed transposed so that the key axis of the scores
 // lies along a lane's accumulator registers:
 //   S^T[key][query] = K . Q^T   - A operand K from LDS (k-major), B operand Q^T from registers, 8 MFMA tiles of
 //                                 32 keys x 32 queries per wavefront, k = head dimension (at most 64);
@@ -49,10 +49,21 @@ struct AttnParams {
     long long sQ, sK, sV, sO;      // strides between matrices of the inner batch level, elements
     long long sQ2, sK2, sV2, sO2;  // ... of the outer level
     int batch_inner;
+    int q_tiles;  // 128-query tiles one workgroup walks through (K and V stay in LDS across them)
     float scale;
     int causal;
     int flags;  // bit 0: O rows may be written as aligned 16-byte vectors, bit 1: P rows likewise
 };
+
+// Branch-free variant for dimensions that are multiples of 4: the address is clamped into the matrix by the caller,
+// the load is unconditional (so the compiler can keep many of them in flight) and an invalid vector is zeroed
+// afterwards.
+__device__ __forceinline__ f32x4 load4_select(const float* p, bool valid) {
+    f32x4 x;
+    __builtin_memcpy(&x, p, 16);
+    if (!valid) x = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    return x;
+}
 
 __device__ __forceinline__ f32x4 load4_guarded(const float* p, int nvalid) {
     f32x4 x = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -78,49 +89,101 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
     const int z = blockIdx.y;
-    const int q0 = blockIdx.x * AT_BQ;
     const BatchIndex bi = split_batch(z, p.batch_inner);
     const float* Qz = p.Q + batch_offset(bi, p.sQ, p.sQ2);
     const float* Kz = p.K + batch_offset(bi, p.sK, p.sK2);
     const float* Vz = p.V + batch_offset(bi, p.sV, p.sV2);
     float* Oz = p.O + batch_offset(bi, p.sO, p.sO2);
 
-    // ---- K -> Ks[d][key]: consecutive threads take consecutive keys, so the transposing LDS stores of one
-    //      instruction hit consecutive addresses; a thread walks along d ----
+    const bool vec4 = (p.dk % 4 == 0) && (p.dv % 4 == 0);  // uniform: whole 16-byte vectors are inside or outside
+
+    // this lane's query row as the B operand of the score product: qf[s] = Q[row][2 s + lane / 32]
+    auto load_q = [&](float (&dst)[AT_D / 2], int qrow_index) {
+        const bool ok = qrow_index < p.Tq;
+        const float* qrow = Qz + (long long)(ok ? qrow_index : p.Tq - 1) * p.ldq;
+        if (vec4) {
 #pragma unroll
-    for (int it = 0; it < (AT_TK * AT_D / 4) / 256; ++it) {
-        const int idx = it * 256 + tid;
-        const int key = idx % AT_TK, v = idx / AT_TK;
-        const int nvalid = (key < p.Tk) ? (p.dk - 4 * v) : 0;
-        const f32x4 x = load4_guarded(Kz + (long long)key * p.ldk + 4 * v, nvalid);
-        Ks[(4 * v + 0) * AT_KP + key] = x.x;
-        Ks[(4 * v + 1) * AT_KP + key] = x.y;
-        Ks[(4 * v + 2) * AT_KP + key] = x.z;
-        Ks[(4 * v + 3) * AT_KP + key] = x.w;
-    }
-    // ---- V -> Vs[key][dv]: 16 consecutive threads read one 256-byte row ----
-#pragma unroll
-    for (int it = 0; it < (AT_TK * AT_D / 4) / 256; ++it) {
-        const int idx = it * 256 + tid;
-        const int key = idx / (AT_D / 4), v = idx % (AT_D / 4);
-        const int nvalid = (key < p.Tk) ? (p.dv - 4 * v) : 0;
-        const f32x4 x = load4_guarded(Vz + (long long)key * p.ldv + 4 * v, nvalid);
-        *reinterpret_cast<f32x4*>(Vs + key * AT_VP + 4 * v) = x;
-    }
-    // ---- this lane's query row as the B operand of the score product: qf[s] = Q[row][2 s + lane / 32] ----
-    const int row = q0 + wave * 32 + l32;
-    const bool row_ok = row < p.Tq;
+            for (int j = 0; j < AT_D / 4; ++j) {
+                const f32x4 x = load4_select(qrow + (4 * j < p.dk ? 4 * j : 0), ok && 4 * j < p.dk);
+                dst[2 * j] = lhi ? x.y : x.x;
+                dst[2 * j + 1] = lhi ? x.w : x.z;
+            }
+        } else {
+            for (int j = 0; j < AT_D / 4; ++j) {
+                const f32x4 x = load4_guarded(qrow + 4 * j, ok ? (p.dk - 4 * j) : 0);
+                dst[2 * j] = lhi ? x.y : x.x;
+                dst[2 * j + 1] = lhi ? x.w : x.z;
+            }
+        }
+    };
+    // the first tile's queries are asked for before K and V: loads return in order, and step 0 needs them
+    const int qt0 = blockIdx.x * p.q_tiles;
     float qf[AT_D / 2];
-    {
-        const float* qrow = Qz + (long long)row * p.ldq;
+    load_q(qf, qt0 * AT_BQ + wave * 32 + l32);
+
+
+    // ---- K -> Ks[d][key]: consecutive threads take consecutive keys, so the transposing LDS stores of one
+    //      instruction hit consecutive addresses; a thread walks along d.
+    //      V -> Vs[key][dv]: 16 consecutive threads read one 256-byte row.
+    //      All loads are issued before the first LDS store, so they are in flight together; V is not needed until
+    //      the second product, so it stays in registers while the first score product runs. ----
+    constexpr int KIT = (AT_TK * AT_D / 4) / 256;
+    f32x4 kx[KIT], vx[KIT];  // fast path: K and V on their way to LDS; V stays in registers while the first
+                             // score product runs and is stored after it
+    if (vec4) {
 #pragma unroll
-        for (int j = 0; j < AT_D / 4; ++j) {
-            const f32x4 x = load4_guarded(qrow + 4 * j, row_ok ? (p.dk - 4 * j) : 0);
-            qf[2 * j] = lhi ? x.y : x.x;
-            qf[2 * j + 1] = lhi ? x.w : x.z;
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = idx % AT_TK, v = idx / AT_TK;
+            const bool ok = key < p.Tk && 4 * v < p.dk;
+            kx[it] = load4_select(Kz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldk + (4 * v < p.dk ? 4 * v : 0), ok);
+        }
+    } else {
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = idx % AT_TK, v = idx / AT_TK;
+            const f32x4 x = load4_guarded(Kz + (long long)key * p.ldk + 4 * v, (key < p.Tk) ? (p.dk - 4 * v) : 0);
+            Ks[(4 * v + 0) * AT_KP + key] = x.x;
+            Ks[(4 * v + 1) * AT_KP + key] = x.y;
+            Ks[(4 * v + 2) * AT_KP + key] = x.z;
+            Ks[(4 * v + 3) * AT_KP + key] = x.w;
+        }
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = idx / (AT_D / 4), v = idx % (AT_D / 4);
+            const f32x4 x = load4_guarded(Vz + (long long)key * p.ldv + 4 * v, (key < p.Tk) ? (p.dv - 4 * v) : 0);
+            *reinterpret_cast<f32x4*>(Vs + key * AT_VP + 4 * v) = x;
         }
     }
+    auto load_v = [&]() {
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = idx / (AT_D / 4), v = idx % (AT_D / 4);
+            const bool ok = key < p.Tk && 4 * v < p.dv;
+            vx[it] = load4_select(Vz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldv + (4 * v < p.dv ? 4 * v : 0), ok);
+        }
+    };
+    if (vec4) {
+        load_v();
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = idx % AT_TK, v = idx / AT_TK;
+            Ks[(4 * v + 0) * AT_KP + key] = kx[it].x;
+            Ks[(4 * v + 1) * AT_KP + key] = kx[it].y;
+            Ks[(4 * v + 2) * AT_KP + key] = kx[it].z;
+            Ks[(4 * v + 3) * AT_KP + key] = kx[it].w;
+        }
+    }
+
     __syncthreads();
+
+    for (int qt = qt0; qt < qt0 + p.q_tiles; ++qt) {
+    const int q0 = qt * AT_BQ;
+    if (q0 >= p.Tq) break;
+    const int row = q0 + wave * 32 + l32;
+    const bool row_ok = row < p.Tq;
 
     // ---- S^T = K . Q^T: 8 tiles of 32 keys x 32 queries ----
     f32x16 sacc[AT_TK / 32];
@@ -128,28 +191,69 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
     for (int t = 0; t < AT_TK / 32; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[t][r] = 0.0f;
+    // A operands are read from LDS one k step ahead of the MFMAs that use them (the fences keep the scheduler
+    // from sinking the reads back next to their use).
+    {
+        constexpr int NTILE = AT_TK / 32;
+        const float* kbase = Ks + lhi * AT_KP + l32;
+        float ka[2][NTILE];
 #pragma unroll
-    for (int s = 0; s < AT_D / 2; ++s) {
-        const float* kr = Ks + (2 * s + lhi) * AT_KP + l32;
+        for (int t = 0; t < NTILE; ++t) ka[0][t] = kbase[t * 32];
 #pragma unroll
-        for (int t = 0; t < AT_TK / 32; ++t)
-            sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[t * 32], qf[s], sacc[t], 0, 0, 0);
+        for (int s = 0; s < AT_D / 2; ++s) {
+            if (s + 1 < AT_D / 2) {
+#pragma unroll
+                for (int t = 0; t < NTILE; ++t) ka[(s + 1) & 1][t] = kbase[(2 * (s + 1)) * AT_KP + t * 32];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < NTILE; ++t)
+                sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s & 1][t], qf[s], sacc[t], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (vec4 && qt == qt0) {
+        // V reaches LDS now (uniform branch: the barrier is taken by every wavefront)
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = idx / (AT_D / 4), v = idx % (AT_D / 4);
+            *reinterpret_cast<f32x4*>(Vs + key * AT_VP + 4 * v) = vx[it];
+        }
+        __syncthreads();
     }
 
-    // ---- scale, mask, softmax over the keys of this lane's query ----
-    // sacc[t][r] is key  t*32 + 8*(r/4) + 4*lhi + r%4  of query  l32.
-    constexpr float kNegInf = -3.402823466e+38f;
-    float m = kNegInf;
+    // Scores are kept as log2-domain values s * scale * log2(e), so that exp(s - max) is one v_exp_f32.
+    // A masked score (above the diagonal: the reference's -1e12, ScaledDotProductAttentionLayer.cs:73-76; or a key
+    // past Tk) becomes a value so negative that its exponential is exactly zero.  Key index of register (t, r) is
+    // t*32 + 8*(r/4) + r%4 + 4*lhi: "key > limit" is one compare against a per-lane constant.
+    constexpr float kLog2e = 1.44269504088896340736f;
+    constexpr float kMasked = -1e12f * kLog2e;
+    const float sl = p.scale * kLog2e;
+    float m = -3.402823466e+38f;
+    if (p.causal || p.Tk < AT_TK) {  // uniform
+        int lim = p.Tk - 1;
+        if (p.causal && row < lim) lim = row;
+        lim -= 4 * lhi;
 #pragma unroll
-    for (int t = 0; t < AT_TK / 32; ++t) {
+        for (int t = 0; t < AT_TK / 32; ++t) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int key = t * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-            float v = p.scale * sacc[t][r];
-            if (p.causal && key > row) v = -1e12f;  // SetAllElementsAboveMainDiagonal(-1e12), :73-76
-            if (key >= p.Tk) v = kNegInf;
-            sacc[t][r] = v;
-            m = fmaxf(m, v);
+            for (int r = 0; r < 16; ++r) {
+                float v = sl * sacc[t][r];
+                v = (t * 32 + 8 * (r / 4) + (r % 4) > lim) ? kMasked : v;
+                sacc[t][r] = v;
+                m = fmaxf(m, v);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < AT_TK / 32; ++t) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float v = sl * sacc[t][r];
+                sacc[t][r] = v;
+                m = fmaxf(m, v);
+            }
         }
     }
     m = fmaxf(m, __shfl_xor(m, 32, 64));
@@ -158,8 +262,7 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
     for (int t = 0; t < AT_TK / 32; ++t) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int key = t * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-            const float e = (key < p.Tk) ? __expf(sacc[t][r] - m) : 0.0f;
+            const float e = __builtin_amdgcn_exp2f(sacc[t][r] - m);
             sacc[t][r] = e;
             sum += e;
         }
@@ -192,22 +295,46 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
         }
     }
 
-    // ---- O^T = V^T . P^T: the probabilities are already where the B operand wants them ----
+    // the next tile's queries travel while this tile's second product runs
+    float qf_next[AT_D / 2];
+    load_q(qf_next, (qt + 1 < qt0 + p.q_tiles) ? (q0 + AT_BQ + wave * 32 + l32) : p.Tq);
+
+    // ---- O^T = V^T . P^T: the probabilities are already where the B operand wants them.  Even and odd k steps
+    //      accumulate separately, so an MFMA never waits for the result of the one issued just before it. ----
     f32x16 oacc[AT_D / 32];
+    {
+        constexpr int NSTEP = (AT_TK / 32) * 16;  // k steps: one per accumulator register of the score tiles
+        constexpr int MT = AT_D / 32;
+        constexpr int LOOK = 2;                   // steps of look-ahead for the LDS reads of V
+        f32x16 part[2][MT];
 #pragma unroll
-    for (int mt = 0; mt < AT_D / 32; ++mt)
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[mt][r] = 0.0f;
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int t = 0; t < AT_TK / 32; ++t) {
+                for (int r = 0; r < 16; ++r) part[h][mt][r] = 0.0f;
+        const float* vbase = Vs + (4 * lhi) * AT_VP + l32;
+        float va[4][MT];
+        auto v_off = [](int i) { return ((i / 16) * 32 + 8 * ((i % 16) / 4) + (i % 4)) * AT_VP; };
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int key = t * 32 + 8 * (r / 4) + 4 * lhi + (r % 4);
-            const float* vr = Vs + key * AT_VP + l32;
+        for (int i = 0; i < LOOK; ++i)
 #pragma unroll
-            for (int mt = 0; mt < AT_D / 32; ++mt)
-                oacc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[mt * 32], sacc[t][r], oacc[mt], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt) va[i][mt] = vbase[v_off(i) + mt * 32];
+#pragma unroll
+        for (int i = 0; i < NSTEP; ++i) {
+            if (i + LOOK < NSTEP) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) va[(i + LOOK) % 4][mt] = vbase[v_off(i + LOOK) + mt * 32];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                part[i & 1][mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[i % 4][mt], sacc[i / 16][i % 16], part[i & 1][mt],
+                                                                       0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) oacc[mt] = part[0][mt] + part[1][mt];
     }
     // oacc[mt][r] is O[row][mt*32 + 8*(r/4) + 4*lhi + r%4]
     if (row_ok) {
@@ -229,6 +356,9 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
             }
         }
     }
+#pragma unroll
+    for (int j = 0; j < AT_D / 2; ++j) qf[j] = qf_next[j];
+    }  // query tiles
 }
 
 }  // namespace snhip

@@ -658,7 +658,13 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
         (!two_level || d->strideO_outer % 4 == 0))
         p.flags |= 1;
     if (d->weights != nullptr && (uintptr_t)d->weights % 16 == 0 && d->Tk % 4 == 0) p.flags |= 2;
-    hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(d->Tq, AT_BQ), (unsigned)d->batch), dim3(256), e->lds_bytes,
+    // K and V are staged once per workgroup: let one workgroup walk through all query tiles of its matrix unless
+    // that would leave compute units without work
+    const int tiles = ceil_div(d->Tq, AT_BQ);
+    int groups = 1;
+    while (groups < tiles && (long long)d->batch * groups < 2LL * h->num_cu) ++groups;
+    p.q_tiles = ceil_div(tiles, groups);
+    hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256), e->lds_bytes,
                        h->stream, p);
     return hip_to_status(hipGetLastError());
 }
