@@ -97,6 +97,21 @@ int snhip_gemm_rm(void* handle, int transposeA, int transposeB, int M, int N, in
                   int lda, long long strideA, const float* B, int ldb, long long strideB, float beta, float* C,
                   int ldc, long long strideC, int batch, const float* bias);
 
+/* ---- the other two cuBLAS entry points the reference binds -------------------- */
+/* Column-major C (m x n) = alpha * op(A) + beta * op(B): argument for argument cublasSgeam
+ * (Prod/GPU/CublasWrapper.cs:250), which the reference calls with transa = T, beta = 0, B = NULL as its 2-D transpose
+ * (Prod/GPU/GpuTensor.cs:1256-1291).  An operand whose scalar is zero is not read and may be NULL.  In-place
+ * transposition (C == A with transa) is not supported (status 15). */
+int snhip_sgeam(void* handle, int transa, int transb, int m, int n, const float* alpha, const float* A, int lda,
+                const float* beta, const float* B, int ldb, float* C, int ldc);
+/* Column-major C (m x n) = A * diag(x) (mode = SNHIP_SIDE_RIGHT, x has n entries) or diag(x) * A (SNHIP_SIDE_LEFT, m
+ * entries): cublasSdgmm (CublasWrapper.cs:246) with cublasSideMode_t's numbering, the reference's Tensor.MultiplyTensor
+ * (GpuTensor.cs:1380-1395).  C may be A. */
+#define SNHIP_SIDE_LEFT 0
+#define SNHIP_SIDE_RIGHT 1
+int snhip_sdgmm(void* handle, int mode, int m, int n, const float* A, int lda, const float* x, int incx, float* C,
+                int ldc);
+
 /* ---- fused Linear-layer forms ---------------------------------------------- */
 /* Element-wise functions the GEMM epilogue can apply; the reference runs them as the ActivationLayer that follows
  * a Linear layer (cudnnActivationMode_t RELU / LEAKY_RELU / SIGMOID / TANH, Prod/GPU/CudnnWrapper.cs:267-281;

@@ -36,6 +36,9 @@ softmax_last_dim_backward /             ScaledDotProductAttentionLayer.cs:111-13
 sdpa_backward                           (softmax gradient: cuDNN definition)         (tests/test_oracle.py)
 mha_forward / mha_backward              Prod/Layers/MultiheadAttention.cs:178-292    stored losses before / after 10 epochs of
                                         (head split / merge as explicit transposes)  ParallelRunWithPyTorch.cs:1013-1131, 4 cases
+sgeam_colmajor / sdgmm_colmajor /       cuBLAS Sgeam / Sdgmm as called at            reference's known transposes TestCpuTensor.cs:82-100,
+transpose / multiply_tensor             Prod/GPU/GpuTensor.cs:1256-1291,1380-1395;   closed form of TestCpuTensor.cs:216-241
+                                        Prod/CPU/CpuTensor.cs:1060-1094              (expected[i] = a[i] * x[i / 49])
 round_to_bf16                           IEEE-754 round-to-nearest-even to a          closed-form ties/neighbours and torch's CPU
                                         bfloat16 (what v_cvt_pk_bf16_f32 does);      bfloat16 cast (independent implementation)
                                         no reference counterpart (variant is new)
@@ -159,6 +162,57 @@ def sgemm_colmajor(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc)
     _lib().oracle_sgemm_colmajor(int(transa), int(transb), m, n, k, float(alpha), _p(A), lda, _p(B), ldb, float(beta),
                                  _p(out), ldc)
     return out
+
+
+def sgeam_colmajor(transa, transb, m, n, alpha, A, lda, beta, B, ldb, C, ldc):
+    """Column-major C (m x n) = alpha * op(A) + beta * op(B) on flat float32 buffers (cublasSgeam); returns the
+    updated copy of C.  An operand whose scalar is zero is not read."""
+    out = np.array(C, dtype=np.float32).copy()
+
+    def op(buf, ld, trans):
+        buf = np.asarray(buf, dtype=np.float32)
+        if trans:       # stored n x m column-major: element (i, j) of op at j + i * ld
+            return np.array([[buf[j + i * ld] for j in range(n)] for i in range(m)], dtype=np.float64).reshape(m, n)
+        return np.array([[buf[i + j * ld] for j in range(n)] for i in range(m)], dtype=np.float64).reshape(m, n)
+    acc = np.zeros((m, n), dtype=np.float64)
+    if alpha != 0:
+        acc += np.float32(alpha) * op(A, lda, transa)
+    if beta != 0:
+        acc += np.float32(beta) * op(B, ldb, transb)
+    for j in range(n):
+        for i in range(m):
+            out[i + j * ldc] = np.float32(acc[i, j])
+    return out
+
+
+def sdgmm_colmajor(right, m, n, A, lda, x, incx, C, ldc):
+    """Column-major C (m x n) = A . diag(x) (right) or diag(x) . A (left) (cublasSdgmm); returns the updated copy of C."""
+    A = np.asarray(A, dtype=np.float32)
+    x = np.asarray(x, dtype=np.float32)
+    out = np.array(C, dtype=np.float32).copy()
+    for j in range(n):
+        for i in range(m):
+            out[i + j * ldc] = np.float32(A[i + j * lda] * x[(j if right else i) * incx])
+    return out
+
+
+def transpose(a2d):
+    """Tensor.Transpose as the GPU path performs it (GpuTensor.cs:1256-1291): Sgeam(T, N, M, N, 1, this, lda = N, 0, -,
+    ldb = M, transposed, ldc = M) on the row-major buffers."""
+    a2d = np.asarray(a2d, dtype=np.float32)
+    M, N = a2d.shape
+    out = sgeam_colmajor(True, False, M, N, 1.0, a2d.reshape(-1), N, 0.0, None, M, np.zeros(M * N, np.float32), M)
+    return out.reshape(N, M)
+
+
+def multiply_tensor(a, diagonal):
+    """Tensor.MultiplyTensor as the GPU path performs it (GpuTensor.cs:1380-1395): Sdgmm(RIGHT, m = Count / n,
+    n = diagonal.Count, a, lda = m, diagonal, 1, c, ldc = m)."""
+    a = np.asarray(a, dtype=np.float32)
+    d = np.asarray(diagonal, dtype=np.float32).reshape(-1)
+    n = d.size
+    m = a.size // n
+    return sdgmm_colmajor(True, m, n, a.reshape(-1), m, d, 1, np.zeros(a.size, np.float32), m).reshape(a.shape)
 
 
 def round_to_bf16(x):

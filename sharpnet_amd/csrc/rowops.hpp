@@ -148,6 +148,53 @@ __global__ void __launch_bounds__(256) transpose_2nd_3rd_kernel(const float* __r
     }
 }
 
+// Column-major C (m x n, ldc) = alpha * op(A) + beta * op(B): cublasSgeam, which the reference uses with
+// transa = T, beta = 0 as its matrix transpose (Prod/GPU/GpuTensor.cs:1256-1291).  A workgroup of 32 x 8 threads owns
+// a 32 x 32 tile of C; a transposed operand goes through a padded LDS tile so that both its reads and the writes
+// of C are contiguous.  B is not touched when beta == 0.
+__global__ void __launch_bounds__(256) geam_kernel(int ta, int tb, int m, int n, float alpha, const float* __restrict__ A,
+                                                   long long lda, float beta, const float* __restrict__ B, long long ldb,
+                                                   float* C, long long ldc) {
+    __shared__ float tA[32][33], tB[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int i0 = blockIdx.x * 32, j0 = blockIdx.y * 32;
+    const bool use_b = (beta != 0.0f);
+    if (ta || (tb && use_b)) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int r = ty + 8 * k;  // index along i inside the tile; tx runs along j: contiguous in a transposed operand
+            if (i0 + r < m && j0 + tx < n) {
+                if (ta) tA[r][tx] = A[(long long)(i0 + r) * lda + (j0 + tx)];
+                if (tb && use_b) tB[r][tx] = B[(long long)(i0 + r) * ldb + (j0 + tx)];
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int c = ty + 8 * k;  // index along j inside the tile; tx runs along i: contiguous in C
+        const int i = i0 + tx, j = j0 + c;
+        if (i < m && j < n) {
+            float v = alpha * (ta ? tA[tx][c] : A[(long long)j * lda + i]);
+            if (use_b) v += beta * (tb ? tB[tx][c] : B[(long long)j * ldb + i]);
+            C[(long long)j * ldc + i] = v;
+        }
+    }
+}
+
+// Column-major C (m x n, ldc) = A . diag(x) (right, x has n entries) or diag(x) . A (left, m entries): cublasSdgmm,
+// the reference's MultiplyTensor (Prod/GPU/GpuTensor.cs:1380-1395).  C may be A.
+__global__ void __launch_bounds__(256) dgmm_kernel(int right, int m, int n, const float* A, long long lda,
+                                                   const float* __restrict__ x, long long incx, float* C, long long ldc) {
+    const long long total = (long long)m * n;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long long)gridDim.x * blockDim.x) {
+        const int i = (int)(idx % m), j = (int)(idx / m);
+        const float s = x[(long long)(right ? j : i) * incx];
+        C[(long long)j * ldc + i] = A[(long long)j * lda + i] * s;
+    }
+}
+
 // x[b][r][c] = value for c > r
 __global__ void __launch_bounds__(256) set_above_diagonal_kernel(float* x, long long matrices, int rows, int cols,
                                                                  float value) {

@@ -842,6 +842,41 @@ int snhip_transpose_second_and_third_dimension(void* handle, const float* src, f
     return hip_to_status(hipGetLastError());
 }
 
+int snhip_sgeam(void* handle, int transa, int transb, int m, int n, const float* alpha, const float* A, int lda,
+                const float* beta, const float* B, int ldb, float* C, int ldc) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    bool oka = false, okb = false;
+    const bool ta = op_is_trans(transa, &oka), tb = op_is_trans(transb, &okb);
+    if (!oka || !okb || m < 0 || n < 0 || alpha == nullptr || beta == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    if (m == 0 || n == 0) return SNHIP_STATUS_SUCCESS;
+    const bool use_a = (*alpha != 0.0f), use_b = (*beta != 0.0f);
+    if (C == nullptr || ldc < m) return SNHIP_STATUS_INVALID_VALUE;
+    if (use_a && (A == nullptr || lda < (ta ? n : m))) return SNHIP_STATUS_INVALID_VALUE;
+    if (use_b && (B == nullptr || ldb < (tb ? n : m))) return SNHIP_STATUS_INVALID_VALUE;
+    if ((use_a && A == C && ta) || (use_b && B == C && tb)) return SNHIP_STATUS_NOT_SUPPORTED;  // in-place transpose
+    // alpha == 0 must not read A (it may be NULL): hand the kernel B's data under both names then
+    const float* a_eff = use_a ? A : (use_b ? B : C);
+    const int lda_eff = use_a ? lda : (use_b ? ldb : ldc);
+    const int ta_eff = use_a ? ta : (use_b ? tb : 0);
+    if ((long long)ceil_div(n, 32) > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
+    hipLaunchKernelGGL(geam_kernel, dim3((unsigned)ceil_div(m, 32), (unsigned)ceil_div(n, 32)), dim3(256), 0,
+                       static_cast<Handle*>(handle)->stream, (int)ta_eff, (int)tb, m, n, *alpha, a_eff, (long long)lda_eff,
+                       *beta, B, (long long)ldb, C, (long long)ldc);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_sdgmm(void* handle, int mode, int m, int n, const float* A, int lda, const float* x, int incx, float* C,
+                int ldc) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if ((mode != SNHIP_SIDE_LEFT && mode != SNHIP_SIDE_RIGHT) || m < 0 || n < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (m == 0 || n == 0) return SNHIP_STATUS_SUCCESS;
+    if (A == nullptr || x == nullptr || C == nullptr || lda < m || ldc < m || incx == 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (incx < 0) return SNHIP_STATUS_NOT_SUPPORTED;
+    hipLaunchKernelGGL(dgmm_kernel, dim3(grid_for((long long)m * n)), dim3(256), 0, static_cast<Handle*>(handle)->stream,
+                       (int)(mode == SNHIP_SIDE_RIGHT), m, n, A, (long long)lda, x, (long long)incx, C, (long long)ldc);
+    return hip_to_status(hipGetLastError());
+}
+
 int snhip_broadcast_add_vector(void* handle, const float* vector, float* y, int rows, int cols) {
     if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     if (rows < 0 || cols < 0) return SNHIP_STATUS_INVALID_VALUE;

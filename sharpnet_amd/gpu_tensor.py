@@ -399,6 +399,26 @@ def _add_tensor_methods():
         check_status(self._lib.snhip_set_above_main_diagonal(self.Wrapper.handle, self.Pointer, m, r, c, value),
                      "snhip_set_above_main_diagonal")
 
+    def Transpose(self, transposed):
+        """transposed = this^T for a 2-D tensor, through the Sgeam-shaped entry point with the reference's own
+        arguments (GpuTensor.cs:1256-1291)."""
+        assert self.Dimension == 2 and transposed.Count >= self.Count
+        transposed.Shape = [self.Shape[1], self.Shape[0]]
+        M, N = self.Shape
+        alpha, beta = ctypes.c_float(1.0), ctypes.c_float(0.0)
+        check_status(self._lib.snhip_sgeam(self.Wrapper.handle, CUBLAS_OP_T, CUBLAS_OP_N, M, N, ctypes.byref(alpha),
+                                           self.Pointer, N, ctypes.byref(beta), None, M, transposed.Pointer, M), "snhip_sgeam")
+
+    def MultiplyTensor(self, a, diagonalMatrix):
+        """this = a * diagonalMatrix, element-wise when both have the same size, else every run of
+        a.Count / diagonalMatrix.Count consecutive elements scaled by one entry (CpuTensor.cs:1060-1094), through the
+        Sdgmm-shaped entry point as the reference calls it (GpuTensor.cs:1380-1395)."""
+        assert a.Count == self.Count and self.Count % diagonalMatrix.Count == 0
+        n = diagonalMatrix.Count
+        m = self.Count // n
+        check_status(self._lib.snhip_sdgmm(self.Wrapper.handle, 1, m, n, a.Pointer, m, diagonalMatrix.Pointer, 1,
+                                           self.Pointer, m), "snhip_sdgmm")
+
     def TransposeSecondAndThirdDimension(self, target):
         """target[a][c][b][d] = this[a][b][c][d]; target is reshaped to the swapped shape (CpuTensor.cs:301-322)."""
         assert len(self.Shape) >= 3 and target.Count == self.Count
@@ -424,7 +444,8 @@ def _add_tensor_methods():
                                                          dx.Pointer, self.Count), "snhip_activation_backward")
 
     for f in (Compute_BiasGradient_from_dy, BroadcastAddVectorToOutput, Update_Adding_Alpha_X, SoftmaxLastDimension,
-              SoftmaxLastDimensionBackward, SetAllElementsAboveMainDiagonal, TransposeSecondAndThirdDimension,
+              SoftmaxLastDimensionBackward, SetAllElementsAboveMainDiagonal, Transpose, MultiplyTensor,
+              TransposeSecondAndThirdDimension,
               ActivationForward, ActivationBackward):
         setattr(GPUTensor, f.__name__, f)
 

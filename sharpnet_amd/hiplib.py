@@ -140,6 +140,8 @@ SIGNATURES = {
     "snhip_dense_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f],
     "snhip_activation_forward": [_vp, _i, _f, _vp, _vp, _ll],
     "snhip_activation_backward": [_vp, _i, _f, _vp, _vp, _vp, _ll],
+    "snhip_sgeam": [_vp, _i, _i, _i, _i, _c_float_p, _vp, _i, _c_float_p, _vp, _i, _vp, _i],
+    "snhip_sdgmm": [_vp, _i, _i, _i, _vp, _i, _vp, _i, _vp, _i],
     "snhip_bias_gradient": [_vp, _vp, _i, _i, _vp],
     "snhip_transpose_second_and_third_dimension": [_vp, _vp, _vp, _i, _i, _i, _i],
     "snhip_broadcast_add_vector": [_vp, _vp, _vp, _i, _i],

@@ -422,3 +422,49 @@ def test_random_shapes_offsets_and_pitches(oracle, gpu_wrapper):
         assert np.array_equal(got, want), (case, "padding overwritten")
         for t in (gA, gB, gC):
             t.Dispose()
+
+
+def test_sgeam_transpose_and_sdgmm(oracle, gpu_wrapper):
+    """Tensor.Transpose (cublasSgeam with the reference's arguments, Tests/TestParallelRunCpuVersusGpu.cs:522-533 sizes and
+    larger ones that span several tiles), the general Sgeam form, and Tensor.MultiplyTensor (cublasSdgmm, same file
+    :511-519,583-590) against the oracle; bit-exact, these are copies and single products."""
+    import ctypes
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    rng = np.random.default_rng(8)
+    for h in (1, 2, 5, 10, 33, 257):
+        for wd in (1, 2, 5, 10, 64, 100):
+            a = random_tensor(rng, (h, wd), -1.5, 1.5)
+            ga, gt = GPUTensor([h, wd], a, w), GPUTensor([wd, h], None, w)
+            gt.SetValue(float("nan"))
+            ga.Transpose(gt)
+            assert gt.Shape == [wd, h] and np.array_equal(gt.ToNumpy(), oracle.transpose(a)) and \
+                np.array_equal(gt.ToNumpy(), a.T)
+    # general form: alpha * A^T + beta * B^T into a padded C
+    m, n = 45, 70
+    A, B, C0 = random_tensor(rng, ((n + 2) * (m + 3),), -1, 1), random_tensor(rng, ((n + 5) * m,), -1, 1), \
+        random_tensor(rng, ((m + 4) * n,), -1, 1)
+    gA, gB, gC = GPUTensor([A.size], A, w), GPUTensor([B.size], B, w), GPUTensor([C0.size], C0, w)
+    al, be = ctypes.c_float(0.5), ctypes.c_float(-2.0)
+    st = w.lib.snhip_sgeam(w.handle, 1, 1, m, n, ctypes.byref(al), gA.Pointer, n + 2, ctypes.byref(be), gB.Pointer, n + 5,
+                           gC.Pointer, m + 4)
+    assert st == 0
+    want = oracle.sgeam_colmajor(True, True, m, n, 0.5, A, n + 2, -2.0, B, n + 5, C0, m + 4)
+    assert np.max(np.abs(gC.ToNumpy() - want)) <= 1e-6
+    assert np.array_equal(gC.ToNumpy().reshape(n, m + 4)[:, m:], C0.reshape(n, m + 4)[:, m:])
+    # argument errors follow cuBLAS: bad op, short leading dimension, in-place transpose
+    assert w.lib.snhip_sgeam(w.handle, 7, 0, m, n, ctypes.byref(al), gA.Pointer, n + 2, ctypes.byref(be), gB.Pointer, n + 5,
+                             gC.Pointer, m + 4) == 7
+    assert w.lib.snhip_sgeam(w.handle, 1, 1, m, n, ctypes.byref(al), gA.Pointer, n - 1, ctypes.byref(be), gB.Pointer, n + 5,
+                             gC.Pointer, m + 4) == 7
+    # MultiplyTensor: same shape, and one factor per (batch, channel)
+    shape = (4, 9, 7, 7)
+    a, x_same, x_bc = random_tensor(rng, shape, -10, 10), random_tensor(rng, shape, -10, 10), \
+        random_tensor(rng, (4, 9, 1, 1), -10, 10)
+    ga, gc = GPUTensor(list(shape), a, w), GPUTensor(list(shape), None, w)
+    gc.MultiplyTensor(ga, GPUTensor(list(shape), x_same, w))
+    assert np.array_equal(gc.ToNumpy(), oracle.multiply_tensor(a, x_same))
+    gc.MultiplyTensor(ga, GPUTensor([4, 9, 1, 1], x_bc, w))
+    assert np.array_equal(gc.ToNumpy(), oracle.multiply_tensor(a, x_bc))
+    ga.MultiplyTensor(ga, GPUTensor([4, 9, 1, 1], x_bc, w))             # in place
+    assert np.array_equal(ga.ToNumpy(), oracle.multiply_tensor(a, x_bc))

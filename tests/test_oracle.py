@@ -372,3 +372,34 @@ def test_multi_head_attention_chain_losses(golden, oracle, variant, is_causal):
     before, after = _mha_chain(oracle, fx, variant, is_causal)
     assert abs(before - case["loss_before"]) < fx["tolerance"], (before, case)     # the reference's own 1e-6
     assert abs(after - case["loss_after"]) < fx["tolerance"], (after, case)
+
+
+def test_transpose_and_multiply_tensor(oracle):
+    """The Sgeam / Sdgmm restatements against the reference's known transposes (Tests/CPU/TestCpuTensor.cs:82-100) and
+    the closed form its MultiplyTensor test asserts (:216-241: expected[i] = a[i] * x[i] and a[i] * x[i / (7*7)])."""
+    assert np.array_equal(oracle.transpose(np.array([[1.0]], np.float32)), [[1.0]])
+    assert np.array_equal(oracle.transpose(np.arange(6, dtype=np.float32).reshape(1, 6)), np.arange(6).reshape(6, 1))
+    assert np.array_equal(oracle.transpose(np.arange(6, dtype=np.float32).reshape(2, 3)).reshape(-1), [0, 3, 1, 4, 2, 5])
+    rng = np.random.default_rng(0)
+    a = rng.uniform(-10, 10, (4, 9, 7, 7)).astype(np.float32)
+    x_same = rng.uniform(-10, 10, a.shape).astype(np.float32)
+    assert np.array_equal(oracle.multiply_tensor(a, x_same), a * x_same)
+    x = rng.uniform(-10, 10, (4, 9, 1, 1)).astype(np.float32)
+    want = (a.reshape(-1) * x.reshape(-1)[np.arange(a.size) // 49]).reshape(a.shape)
+    assert np.array_equal(oracle.multiply_tensor(a, x), want)
+    # general geam: both operands, both transposes, padded leading dimensions, against numpy
+    m, n = 5, 7
+    A = rng.uniform(-1, 1, (n + 2) * (m + 3)).astype(np.float32)      # op(A) = A^T: A stored n x m, lda = n + 2
+    B = rng.uniform(-1, 1, (m + 1) * n).astype(np.float32)            # B stored m x n, ldb = m + 1
+    C0 = rng.uniform(-1, 1, (m + 4) * n).astype(np.float32)
+    got = oracle.sgeam_colmajor(True, False, m, n, 0.5, A, n + 2, -2.0, B, m + 1, C0, m + 4)
+    Am = np.array([[A[j + i * (n + 2)] for j in range(n)] for i in range(m)])
+    Bm = np.array([[B[i + j * (m + 1)] for j in range(n)] for i in range(m)])
+    want = C0.copy()
+    for j in range(n):
+        for i in range(m):
+            want[i + j * (m + 4)] = np.float32(0.5 * Am[i, j] - 2.0 * Bm[i, j])
+    assert np.allclose(got, want, atol=1e-6) and np.array_equal(got.reshape(n, m + 4)[:, m:], C0.reshape(n, m + 4)[:, m:])
+    left = oracle.sdgmm_colmajor(False, 3, 2, np.arange(6, dtype=np.float32), 3, np.array([2, 3, 4], np.float32), 1,
+                                 np.zeros(6, np.float32), 3)
+    assert np.array_equal(left, [0, 3, 8, 6, 12, 20])
