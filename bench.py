@@ -46,6 +46,9 @@ def main():
     ap.add_argument("--attention-probe", action="store_true",
                     help="20 launches of the one-launch attention forward of configuration 5 (512 x 256 x 64, weights "
                          "kept), for profilers")
+    ap.add_argument("--shapes-probe", action="store_true",
+                    help="30 launches each of the skinny, small-M and batched shapes (and the bf16-input headline), in "
+                         "the order printed, for profilers")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: 3 plain copies of 1 GiB, then 3 headline GEMMs")
     args = ap.parse_args()
@@ -112,6 +115,24 @@ def main():
                 attention.fused_attention_forward(q, k, v, o, keep, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
                                                   scale=0.125, is_causal=False, packed=False)
             w.synchronize()
+        return
+    if args.shapes_probe:
+        shapes = [("skinny 8192x64x8192 NN", wl.Gemm(8192, 64, 8192), 0), ("skinny 8192x64x8192 TN", wl.Gemm(8192, 64, 8192, True, False), 0)]
+        shapes += [("dense " + gm.name, gm, 0) for gm in wl.dense_layer_gemms()]
+        proj, rec, _ = wl.lstm_gemms()
+        shapes += [("lstm input projection", proj, 0), ("lstm recurrent step (beta=1)", rec, 0)]
+        shapes += [("attention " + gm.name, gm, 0) for gm in wl.attention_gemms()]
+        shapes += [("bf16-input 8192^3 TN", wl.Gemm(8192, 8192, 8192, True, False), 1),
+                   ("bf16-input 4096^3 NN", wl.Gemm(4096, 4096, 4096), 1)]
+        for name, gm, math_mode in shapes:
+            w.set_math_mode(math_mode)
+            aa, bb, cc = wl.uniform_operands(gm, 2)
+            _, ms, gcx = time_gemm(gm, aa, bb, cc, 20, 10)
+            gcx.Dispose()
+            print(json.dumps({"shape": name, "M": gm.M, "N": gm.N, "K": gm.K, "batch": gm.batch, "launches": 30,
+                              "flops": gm.flops, "bytes": gm.bytes, "event_ms": round(ms, 5),
+                              "tile_config": w.last_tuning()[0], "splitk": w.last_tuning()[1]}), flush=True)
+        w.set_math_mode(0)
         return
     if args.probe:
         # known-size launch: copy_f32_kernel reads 2**30 bytes and writes 2**30 bytes
