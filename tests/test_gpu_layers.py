@@ -415,3 +415,29 @@ def test_fused_attention_limits(gpu_wrapper):
     big.SetValue(0.5)
     wts = attention.ScaledDotProductAttentionForwardPropagation(big, big, big, y, True, True, False)
     assert abs(float(wts.ToNumpy()[0, 0, 0]) - 1.0 / 300) < 1e-6 and abs(float(y.ToNumpy()[0, 7, 3]) - 0.5) < 1e-6
+
+
+def test_fused_attention_on_views_at_odd_element_offsets(oracle, gpu_wrapper):
+    """Operands that are views starting 1, 2 and 3 floats into their buffers (4-byte alignment only, as tensor
+    slices are, GpuTensor.cs:616): the vector loads and stores of the attention kernel must not assume more."""
+    from sharpnet_amd import GPUTensor, attention
+    rng = np.random.default_rng(41)
+    Z, Tn, d = 3, 40, 8
+    q, k, v = (random_tensor(rng, (Z, Tn, d), -1, 1) for _ in range(3))
+    ref, wref = oracle.sdpa_forward(q, k, v, use_scale=True, is_causal=True)
+    bufs = []
+    for off, x in zip((1, 2, 3), (q, k, v)):
+        flat = np.concatenate([np.full(off, 7.0, np.float32), x.reshape(-1)])
+        g = GPUTensor([flat.size], flat, gpu_wrapper)
+        bufs.append((g, g.Slice(off, [Z, Tn, d])))
+    obuf = GPUTensor([Z * Tn * d + 5], None, gpu_wrapper)
+    obuf.SetValue(-3.0)
+    wbuf = GPUTensor([Z * Tn * Tn + 2], None, gpu_wrapper)
+    wbuf.SetValue(-3.0)
+    assert attention.fused_attention_forward(bufs[0][1], bufs[1][1], bufs[2][1], obuf.Slice(1, [Z, Tn, d]),
+                                             wbuf.Slice(1, [Z, Tn, Tn]), batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
+                                             scale=1.0 / np.sqrt(d), is_causal=True, packed=False)
+    o, wt = obuf.ToNumpy(), wbuf.ToNumpy()
+    assert np.max(np.abs(o[1:1 + Z * Tn * d].reshape(Z, Tn, d) - ref)) <= 1e-5
+    assert np.max(np.abs(wt[1:1 + Z * Tn * Tn].reshape(Z, Tn, Tn) - wref)) <= 1e-5
+    assert o[0] == -3.0 and np.all(o[1 + Z * Tn * d:] == -3.0) and wt[0] == -3.0 and wt[-1] == -3.0
