@@ -321,9 +321,25 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     if (M == 0 || N == 0 || batch == 0) return SNHIP_STATUS_SUCCESS;
     if (g.C == nullptr || g.ldc < N) return SNHIP_STATUS_INVALID_VALUE;
     if (g.D != nullptr && g.ldd < N) return SNHIP_STATUS_INVALID_VALUE;
-    if (batch > 65535) return SNHIP_STATUS_NOT_SUPPORTED;  // grid.y carries batch * splitk
     const int inner = (g.batch_inner > 0) ? g.batch_inner : batch;
     if (batch % inner != 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (batch > 65535) {
+        // grid.y carries batch * splitk: a longer single-level batch goes out in slices (cuBLAS takes any batchCount)
+        if (inner < batch) return SNHIP_STATUS_NOT_SUPPORTED;
+        GemmArgs part = g;
+        part.batch_inner = 0;
+        for (int z0 = 0; z0 < batch; z0 += 65535) {
+            part.batch = (batch - z0 < 65535) ? (batch - z0) : 65535;
+            part.A = (g.A != nullptr) ? g.A + (long long)z0 * g.sA : nullptr;
+            part.B = (g.B != nullptr) ? g.B + (long long)z0 * g.sB : nullptr;
+            part.C = g.C + (long long)z0 * g.sC;
+            part.D = (g.D != nullptr) ? g.D + (long long)z0 * g.sD : nullptr;
+            part.colsum = (g.colsum != nullptr) ? g.colsum + (long long)z0 * M : nullptr;
+            const int st = gemm_core(h, part);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
+        return SNHIP_STATUS_SUCCESS;
+    }
     const bool multi = batch > 1;
     const bool two_level = multi && inner < batch;
 

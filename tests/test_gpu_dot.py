@@ -343,18 +343,24 @@ def test_splitk_modes_batched_and_bias(oracle, gpu_wrapper):
 
 
 def test_limits_and_user_stream(oracle, gpu_wrapper):
-    """Batch counts beyond the grid limit are refused with a status; a caller-supplied stream is honoured."""
+    """Batch counts beyond the grid limit go out in slices; a caller-supplied stream is honoured."""
     from sharpnet_amd import GPUTensor
     from sharpnet_amd.hiplib import check_status
     lib, h = gpu_wrapper.lib, gpu_wrapper.handle
     rng = np.random.default_rng(10)
     tiny = GPUTensor([70000, 1, 1], np.ones(70000, np.float32), gpu_wrapper)
     out = GPUTensor([70000, 1, 1], None, gpu_wrapper)
-    # 70000 matrices > 65535: status 15 (NOT_SUPPORTED), nothing launched
-    assert lib.snhip_bmm(h, tiny.Pointer, 1, 1, 0, 1, tiny.Pointer, 1, 1, 0, 1, out.Pointer, 1, 70000, 1.0, 0.0) == 15
-    # the largest supported batch works
-    assert lib.snhip_bmm(h, tiny.Pointer, 1, 1, 0, 1, tiny.Pointer, 1, 1, 0, 1, out.Pointer, 1, 65535, 2.0, 0.0) == 0
-    assert np.all(out.ToNumpy().reshape(-1)[:65535] == 2.0)
+    # 70000 matrices > 65535 (the grid limit): sliced inside the library, every matrix computed
+    vals = np.arange(70000, dtype=np.float32) % 97
+    tiny2 = GPUTensor([70000, 1, 1], vals, gpu_wrapper)
+    assert lib.snhip_bmm(h, tiny.Pointer, 1, 1, 0, 1, tiny2.Pointer, 1, 1, 0, 1, out.Pointer, 1, 70000, 2.0, 0.0) == 0
+    assert np.array_equal(out.ToNumpy().reshape(-1), 2.0 * vals)
+    # a two-level batch that long is refused (status 15)
+    from sharpnet_amd import hiplib
+    import ctypes
+    d = hiplib.GemmDesc(M=1, N=1, K=1, A=tiny.Pointer, lda=1, strideA=1, strideA_outer=2, B=tiny2.Pointer, ldb=1, strideB=1,
+                        strideB_outer=2, C=out.Pointer, ldc=1, strideC=1, strideC_outer=2, batch=70000, batch_inner=2)
+    assert lib.snhip_gemm_ex(h, ctypes.byref(d)) == 15
     # K == 0 on a batch: C = beta * C
     c0 = random_tensor(rng, (4, 3, 5))
     gc = GPUTensor([4, 3, 5], c0, gpu_wrapper)
