@@ -250,6 +250,29 @@ def main():
 
         extra["config1_dense_layer"] = [run(gm, 1, 50, 10, bias=np.zeros(gm.N, np.float32) if gm.bias else None)
                                         for gm in wl.dense_layer_gemms()]
+        if not args.no_cpu:
+            # the same three products (and the bias add) on the host: the reference's CPU route through MKL
+            d = wl.dense_layer_inputs(seed=1)
+            x, wt, dyv = d["x"], d["w_out_in"], d["dy"]
+            y, dwv, dxv = (np.empty(sh, np.float32) for sh in ((x.shape[0], wt.shape[0]), wt.shape, x.shape))
+            bias0 = np.zeros((1, wt.shape[0]), np.float32)
+
+            def cpu_layer():
+                dot_oracle.mkl_dot(x, False, wt, True, y)
+                np.add(y, bias0, out=y)
+                dot_oracle.mkl_dot(dyv, True, x, False, dwv)
+                dot_oracle.mkl_dot(dyv, False, wt, False, dxv)
+            for _ in range(20):
+                cpu_layer()
+            t0 = time.perf_counter()
+            for _ in range(200):
+                cpu_layer()
+            cpu_ms = (time.perf_counter() - t0) * 1e3 / 200
+            gpu_ms = sum(r["ms"] for r in extra["config1_dense_layer"])
+            extra["config1_dense_layer_fwd_bwd"] = {
+                "gpu_ms": round(gpu_ms, 4), "cpu_mkl_ms": round(cpu_ms, 4), "cpu_cores": dot_oracle.mkl_threads(),
+                "note": "forward + dW + dx of the 128 x 784 -> 256 layer; GPU = sum of the three launches above, "
+                        "CPU = cblas_sgemm x 3 + bias add, 200 repetitions"}
         sweep = []
         for (M, N, K) in wl.SWEEP_SIZES:
             for tA in (False, True):
@@ -387,7 +410,7 @@ def write_table(path, out):
     rows = []
     layers = out["extra"].get("layers_fused_vs_reference_sequence", [])
     for name, v in out["extra"].items():
-        if name == "layers_fused_vs_reference_sequence":
+        if name in ("layers_fused_vs_reference_sequence", "config1_dense_layer_fwd_bwd"):
             continue
         items = v if isinstance(v, list) else v.get("gemms") or [x for x in v.values() if isinstance(x, dict)] or [v]
         if isinstance(v, dict) and "gemm" in v:
@@ -406,6 +429,10 @@ def write_table(path, out):
                 "| configuration | GEMM | ms | TFLOP/s | fraction of roofline | tile config | split-K |\n"
                 "|---|---|---|---|---|---|---|\n" % path)
         f.write("\n".join(rows) + "\n\n")
+        fb = out["extra"].get("config1_dense_layer_fwd_bwd")
+        if fb:
+            f.write("Dense layer forward + backward (configuration 1): %.4f ms on the GPU (three launches) against %.4f ms "
+                    "through MKL on %d host threads.\n\n" % (fb["gpu_ms"], fb["cpu_mkl_ms"], fb["cpu_cores"]))
         if layers:
             f.write("Whole layer calls through the host mirrors (HIP events around repeated calls, host launch time included):\n\n"
                     "| layer | form | forward ms | backward ms |\n|---|---|---|---|\n")
