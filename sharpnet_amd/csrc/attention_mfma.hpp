@@ -274,8 +274,10 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[t][r] *= inv;
 
-    // ---- P out (four consecutive keys per register group) ----
-    if (p.P != nullptr && row_ok) {
+    // ---- P out (four consecutive keys per register group).  With all keys present and aligned rows the stores
+    //      are spread over the second product's MFMAs instead (below); this is the general form. ----
+    const bool p_inline = p.P != nullptr && (p.flags & 2) && p.Tk == AT_TK;  // uniform
+    if (p.P != nullptr && !p_inline && row_ok) {
         float* prow = p.P + ((long long)z * p.Tq + row) * p.Tk;
 #pragma unroll
         for (int t = 0; t < AT_TK / 32; ++t) {
@@ -302,7 +304,8 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
     // ---- O^T = V^T . P^T: the probabilities are already where the B operand wants them.  Even and odd k steps
     //      accumulate separately, so an MFMA never waits for the result of the one issued just before it. ----
     f32x16 oacc[AT_D / 32];
-    {
+    auto second_product = [&](auto store_tag) {
+        constexpr bool STORE_P = decltype(store_tag)::value;
         constexpr int NSTEP = (AT_TK / 32) * 16;  // k steps: one per accumulator register of the score tiles
         constexpr int MT = AT_D / 32;
         constexpr int LOOK = 2;                   // steps of look-ahead for the LDS reads of V
@@ -314,6 +317,7 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 #pragma unroll
                 for (int r = 0; r < 16; ++r) part[h][mt][r] = 0.0f;
         const float* vbase = Vs + (4 * lhi) * AT_VP + l32;
+        float* const prow = STORE_P ? p.P + ((long long)z * p.Tq + (row_ok ? row : 0)) * p.Tk + 4 * lhi : nullptr;
         float va[4][MT];
         auto v_off = [](int i) { return ((i / 16) * 32 + 8 * ((i % 16) / 4) + (i % 4)) * AT_VP; };
 #pragma unroll
@@ -326,6 +330,13 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) va[(i + LOOK) % 4][mt] = vbase[v_off(i + LOOK) + mt * 32];
             }
+            if (STORE_P && i % 4 == 0) {
+                // one 16-byte store of P every four k steps: the write-out rides in the MFMAs' shadow
+                const int t = i / 16, g = (i % 16) / 4;
+                if (row_ok)
+                    *reinterpret_cast<f32x4*>(prow + t * 32 + 8 * g) =
+                        f32x4{sacc[t][4 * g], sacc[t][4 * g + 1], sacc[t][4 * g + 2], sacc[t][4 * g + 3]};
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
@@ -335,7 +346,11 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
         }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) oacc[mt] = part[0][mt] + part[1][mt];
-    }
+    };
+    if (p_inline)
+        second_product(std::true_type{});
+    else
+        second_product(std::false_type{});
     // oacc[mt][r] is O[row][mt*32 + 8*(r/4) + 4*lhi + r%4]
     if (row_ok) {
         float* orow = Oz + (long long)row * p.ldo;
