@@ -47,6 +47,13 @@ __global__ void __launch_bounds__(256) column_sum_kernel(const float* __restrict
         out[(long long)blockIdx.y * cols + c] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
 }
 
+// dst[i] = value for count 32-bit words (a kernel rather than a memset node, so that a caller may record it into a
+// HIP graph like any other launch of this library).
+__global__ void __launch_bounds__(256) fill32_kernel(unsigned int* dst, unsigned int value, long long count) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (long long)gridDim.x * blockDim.x)
+        dst[i] = value;
+}
+
 // y = act(x) element-wise (x and y may be the same buffer); `act` as in the GEMM epilogue.
 __global__ void __launch_bounds__(256) activation_kernel(const float* x, float* y, long long n, int act, float a) {
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)

@@ -966,7 +966,9 @@ int snhip_memset32(void* handle, void* dptr, unsigned int value, size_t count) {
     if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     if (count == 0) return SNHIP_STATUS_SUCCESS;
     if (dptr == nullptr) return SNHIP_STATUS_INVALID_VALUE;
-    return hip_to_status(hipMemsetD32Async((hipDeviceptr_t)dptr, (int)value, count, static_cast<Handle*>(handle)->stream));
+    hipLaunchKernelGGL(fill32_kernel, dim3(grid_for((long long)count)), dim3(256), 0, static_cast<Handle*>(handle)->stream,
+                       static_cast<unsigned int*>(dptr), value, (long long)count);
+    return hip_to_status(hipGetLastError());
 }
 
 int snhip_memcpy_htod_async(void* handle, void* dst, const void* src, size_t bytes) {

@@ -148,3 +148,74 @@ def test_config5_attention_batched(oracle, gpu_wrapper, bf16):
             assert np.max(np.abs(o[sel] - ref32)) / np.max(np.abs(ref32)) <= 1e-2
     finally:
         w.set_math_mode(w.MATH_FP32)
+
+
+def test_calls_can_be_recorded_into_a_hip_graph_and_replayed(oracle, gpu_wrapper):
+    """A Dense forward (fused bias + ReLU), a split-K product, a fill and the one-launch attention, recorded into a HIP
+    graph on a capturing stream and replayed three times with eager work and synchronisations in between: every
+    replay must reproduce the eager results (the calls launch kernels only: no allocation once the split-K workspace
+    exists, no memset nodes)."""
+    import ctypes
+    from sharpnet_amd import GPUTensor, linear, attention
+    from sharpnet_amd.hiplib import check_status
+    from tests.helpers import random_tensor
+    w = gpu_wrapper
+    rng = np.random.default_rng(77)
+    x, W, b = random_tensor(rng, (96, 300), -1, 1), random_tensor(rng, (130, 300), -0.2, 0.2), random_tensor(rng, (130,), -1, 1)
+    a2, b2 = random_tensor(rng, (64, 4096), -1, 1), random_tensor(rng, (4096, 48), -1, 1)      # long K: split-K path
+    q = random_tensor(rng, (6, 50, 16), -1, 1)
+    gx, gW, gb, ga2, gb2, gq = (GPUTensor(list(t.shape), t, w) for t in (x, W, b, a2, b2, q))
+    gy, gc2, go, gfill = GPUTensor([96, 130], None, w), GPUTensor([64, 48], None, w), GPUTensor([6, 50, 16], None, w), \
+        GPUTensor([1000], None, w)
+
+    def work():
+        linear.DenseForwardPropagation(gy, gx, gW, gb, False, activation="CUDNN_ACTIVATION_RELU")
+        gc2.Dot(ga2, False, gb2, False, 1.0, 0.0)
+        gfill.SetValue(3.5)
+        assert attention.fused_attention_forward(gq, gq, gq, go, None, batch=6, heads=1, tq=50, tkv=50, dk=16, dv=16,
+                                                 scale=0.25, is_causal=True, packed=False)
+
+    def results():
+        return [t.ToNumpy().copy() for t in (gy, gc2, go, gfill)]
+
+    work()                                   # eager: also sizes the split-K workspace
+    w.synchronize()
+    assert w.last_tuning() is not None
+    eager = results()
+    assert np.max(np.abs(eager[0] - oracle.activation_forward(oracle.dense_forward(x, W, b), "relu"))) < 1e-3
+    assert np.all(eager[3] == 3.5)
+
+    # the HIP runtime the library itself is linked against (same shared object, found by soname)
+    hip = ctypes.CDLL("libamdhip64.so")
+    vp = ctypes.c_void_p
+    for name, args in (("hipStreamBeginCapture", [vp, ctypes.c_int]), ("hipStreamEndCapture", [vp, ctypes.POINTER(vp)]),
+                       ("hipGraphInstantiate", [ctypes.POINTER(vp), vp, vp, vp, ctypes.c_size_t]),
+                       ("hipGraphLaunch", [vp, vp]), ("hipGraphExecDestroy", [vp]), ("hipGraphDestroy", [vp])):
+        getattr(hip, name).argtypes = args
+        getattr(hip, name).restype = ctypes.c_int
+    stream = vp()
+    check_status(w.lib.snhip_stream_create(ctypes.byref(stream)), "snhip_stream_create")
+    check_status(w.lib.snhip_set_stream(w.handle, stream), "snhip_set_stream")
+    graph, graph_exec = vp(), vp()
+    try:
+        assert hip.hipStreamBeginCapture(stream, 0) == 0          # hipStreamCaptureModeGlobal
+        try:
+            work()
+        finally:
+            assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+        assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, 0) == 0
+        for rep in range(3):
+            for t in (gy, gc2, go, gfill):   # eager work between replays: wipe the outputs on the same stream
+                t.SetValue(float("nan"))
+            w.synchronize()
+            assert hip.hipGraphLaunch(graph_exec, stream) == 0
+            w.synchronize()
+            for got, want in zip(results(), eager):
+                assert np.array_equal(got, want), rep
+    finally:
+        check_status(w.lib.snhip_set_stream(w.handle, None), "snhip_set_stream")
+        if graph_exec:
+            hip.hipGraphExecDestroy(graph_exec)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        check_status(w.lib.snhip_stream_destroy(stream), "snhip_stream_destroy")
