@@ -441,3 +441,51 @@ def test_fused_attention_on_views_at_odd_element_offsets(oracle, gpu_wrapper):
     assert np.max(np.abs(o[1:1 + Z * Tn * d].reshape(Z, Tn, d) - ref)) <= 1e-5
     assert np.max(np.abs(wt[1:1 + Z * Tn * Tn].reshape(Z, Tn, Tn) - wref)) <= 1e-5
     assert o[0] == -3.0 and np.all(o[1 + Z * Tn * d:] == -3.0) and wt[0] == -3.0 and wt[-1] == -3.0
+
+
+def test_gemm_ex_degenerate_products_keep_the_rest_of_the_epilogue(oracle, gpu_wrapper):
+    """alpha == 0 or K == 0: A and B are not read (BLAS rule) but bias, beta * C, gamma * D and the activation still apply,
+    and a requested column sum is still produced (zeros for K == 0)."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    rng = np.random.default_rng(51)
+    M, N, K = 37, 29, 11
+    a, b = random_tensor(rng, (K, M), -1, 1), random_tensor(rng, (K, N), -1, 1)
+    c0, d, bias = random_tensor(rng, (M, N), -1, 1), random_tensor(rng, (M, N), -1, 1), random_tensor(rng, (N,), -1, 1)
+    want = np.maximum(0.5 * c0 + bias[None, :] + 0.25 * d, 0)
+    for alpha, k in ((0.0, K), (1.0, 0)):
+        gc, gcs = T(w, c0), GPUTensor([M], None, w)
+        gcs.SetValue(float("nan"))
+        gc.GemmEx(transA=1, M=M, N=N, K=k, alpha=alpha, beta=0.5, A=T(w, a), lda=M, B=T(w, b), ldb=N, ldc=N, bias=T(w, bias),
+                  D=T(w, d), ldd=N, gamma=0.25, activation=1, colsum=gcs)
+        assert np.max(np.abs(gc.ToNumpy() - want)) <= 1e-6
+        ref_cs = a.astype(np.float64).sum(axis=0) if k else np.zeros(M)
+        assert np.max(np.abs(gcs.ToNumpy() - ref_cs)) <= 1e-5
+
+
+def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
+    """The bf16-input kernels have no extended instantiations: addend, ReLU, column sum and the two-level batch are
+    then applied by extra passes / one launch per outer step, with the same results (checked against the oracle on
+    bf16-rounded operands, fp32 bound)."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    rng = np.random.default_rng(52)
+    Bo, Bi, M, N, K = 2, 3, 70, 90, 130
+    a = random_tensor(rng, (Bo, Bi, K, M), -1, 1)      # transposed A: stored K x M
+    b = random_tensor(rng, (Bo, Bi, K, N), -1, 1)
+    d = random_tensor(rng, (Bo, Bi, M, N), -1, 1)
+    bias = random_tensor(rng, (N,), -1, 1)
+    gc, gcs = GPUTensor([Bo, Bi, M, N], None, w), GPUTensor([Bo * Bi, M], None, w)
+    gc.SetValue(float("nan"))
+    gc.GemmEx(transA=1, M=M, N=N, K=K, alpha=0.5, A=T(w, a), lda=M, strideA=K * M, strideA_outer=Bi * K * M, B=T(w, b), ldb=N,
+              strideB=K * N, strideB_outer=Bi * K * N, ldc=N, strideC=M * N, strideC_outer=Bi * M * N, batch=Bo * Bi,
+              batch_inner=Bi, bias=T(w, bias), D=T(w, d), ldd=N, strideD=M * N, strideD_outer=Bi * M * N, gamma=-0.75,
+              activation=2, activation_param=0.1, colsum=gcs, math=1)
+    got, cs = gc.ToNumpy(), gcs.ToNumpy().reshape(Bo, Bi, M)
+    ar, br = oracle.round_to_bf16(a), oracle.round_to_bf16(b)
+    for o in range(Bo):
+        for i in range(Bi):
+            pre = oracle.dot(ar[o, i], True, br[o, i], False, 0.5) + bias[None, :] - 0.75 * d[o, i]
+            want = np.where(pre >= 0, pre, 0.1 * pre)
+            assert np.max(np.abs(got[o, i] - want)) <= bound(K, a, b, 1e-5), (o, i)
+            assert np.max(np.abs(cs[o, i] - a[o, i].astype(np.float64).sum(axis=0))) <= 1e-5 * np.sqrt(K) + 1e-6
