@@ -31,6 +31,8 @@ HIPCC_FLAGS = [
     # packed fp32 VALU forms are switched off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # some fully unrolled staging loops of the bf16-input kernel keep a rolled remainder; that is fine, not worth a warning
+    "-Wno-pass-failed",
 ]
 
 
