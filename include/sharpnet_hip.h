@@ -210,6 +210,35 @@ typedef struct snhip_attention_desc {
 int snhip_attention_forward(void* handle, const snhip_attention_desc* desc);
 int snhip_sizeof_attention_desc(void);
 
+/* Backward of the above: ScaledDotProductAttentionLayer.ScaledDotProductAttentionBackwardPropagation
+ * (Prod/Layers/ScaledDotProductAttentionLayer.cs:111-132) as one call:
+ *     dV = P^T . dO;   dS = softmax-gradient(P, scale * dO . V^T);   dQ = dS . K;   dK = dS^T . Q
+ * `weights` is the softmax output the forward pass kept, `scores_gradients` ([batch][Tq][Tk], contiguous) is the buffer
+ * the reference takes from its memory pool for dS (:121) and must be supplied.  Q / dQ, K / dK and V / dV share their
+ * row pitch and batch strides; dO has its own.  `scale` is the factor the reference applies here (1/sqrt(dV.Shape[2])
+ * with use_scale, :113-119).  Three launches when Tk <= 256 and both dimensions <= 64 (dS and dQ come from one
+ * kernel); otherwise five, the reference's own sequence. */
+typedef struct snhip_attention_bwd_desc {
+    int struct_size;
+    int batch, batch_inner;
+    int Tq, Tk, dk, dv;
+    float scale;
+    const float* Q;
+    const float* K;
+    const float* V;
+    const float* dO;
+    const float* weights;
+    float* scores_gradients;
+    float* dQ;
+    float* dK;
+    float* dV;
+    int ldq, ldk, ldv, ldo;
+    long long strideQ, strideK, strideV, strideO;
+    long long strideQ_outer, strideK_outer, strideV_outer, strideO_outer;
+} snhip_attention_bwd_desc;
+int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* desc);
+int snhip_sizeof_attention_bwd_desc(void);
+
 /* ---- bf16-input / fp32-accumulate variant (no reference counterpart) ------ */
 /* Operands stay fp32 in device memory; they are rounded to bf16 (nearest even)
  * on their way into LDS and multiplied with v_mfma_f32_32x32x16_bf16, products

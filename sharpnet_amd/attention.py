@@ -43,6 +43,26 @@ def fused_attention_forward(Q, K, V, O, weights, *, batch, heads, tq, tkv, dk, d
     return True
 
 
+def attention_backward(dQ, dK, dV, Q, K, V, dO, weights, scores_gradients, *, batch, heads, tq, tkv, dk, dv, scale, packed):
+    """snhip_attention_backward: dV, dS (into scores_gradients), dQ, dK in three launches (five beyond the one-kernel
+    limits).  Layout conventions as in fused_attention_forward; weights and scores_gradients are contiguous
+    (batch*heads, tq, tkv) stacks."""
+    def strides(steps, dim):
+        if packed:
+            return heads * dim, dim, steps * heads * dim
+        return dim, steps * dim, heads * steps * dim
+    ldq, sq, sq2 = strides(tq, dk)
+    ldk, sk, sk2 = strides(tkv, dk)
+    ldv, sv, sv2 = strides(tkv, dv)
+    ldo, so, so2 = strides(tq, dv)
+    d = hiplib.AttentionBwdDesc(batch=batch * heads, batch_inner=heads, Tq=tq, Tk=tkv, dk=dk, dv=dv, scale=scale,
+                                Q=Q.Pointer, K=K.Pointer, V=V.Pointer, dO=dO.Pointer, weights=weights.Pointer,
+                                scores_gradients=scores_gradients.Pointer, dQ=dQ.Pointer, dK=dK.Pointer, dV=dV.Pointer,
+                                ldq=ldq, ldk=ldk, ldv=ldv, ldo=ldo, strideQ=sq, strideK=sk, strideV=sv, strideO=so,
+                                strideQ_outer=sq2, strideK_outer=sk2, strideV_outer=sv2, strideO_outer=so2)
+    check_status(Q._lib.snhip_attention_backward(Q.Wrapper.handle, ctypes.byref(d)), "snhip_attention_backward")
+
+
 def ScaledDotProductAttentionForwardPropagation(Q, K, V, y, isTraining, use_scale, is_causal, fused=True):
     """fused=True runs the whole chain as one launch when the sizes allow it (at most 256 keys, head dimension at
     most 64); otherwise, or with fused=False, the reference's four calls."""
@@ -77,8 +97,18 @@ def ScaledDotProductAttentionForwardPropagation(Q, K, V, y, isTraining, use_scal
     return weights_buffer
 
 
-def ScaledDotProductAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, weights_buffer, use_scale):
+def ScaledDotProductAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, weights_buffer, use_scale, fused=True):
+    """fused=True: one library call (the score gradient and dQ come out of one kernel when the sizes allow it);
+    False: the reference's five calls one by one."""
     embedding_dim = dV.Shape[2]
+    if fused:
+        scaling = 1.0 / math.sqrt(embedding_dim) if use_scale else 1.0
+        scores_gradients_buffer = GPUTensor(weights_buffer.Shape, None, Q.Wrapper)
+        attention_backward(dQ, dK, dV, Q, K, V, dy, weights_buffer, scores_gradients_buffer, batch=K.Shape[0], heads=1,
+                           tq=Q.Shape[1], tkv=V.Shape[1], dk=K.Shape[2], dv=V.Shape[2], scale=scaling, packed=False)
+        scores_gradients_buffer.Dispose()
+        weights_buffer.Dispose()
+        return
     dV.BatchMatrixMultiplication(weights_buffer, True, dy, False, 1.0, 0.0)                # :117
     scaling = 1.0 / math.sqrt(embedding_dim) if use_scale else 1.0
     scores_gradients_buffer = GPUTensor(weights_buffer.Shape, None, Q.Wrapper)
@@ -200,7 +230,7 @@ def MultiheadAttentionForwardPropagation(Q, K, V, y, w_Q, w_K, w_V, out_proj_wei
 
 
 def MultiheadAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, st, w_Q, w_K, w_V, out_proj_weight, grads,
-                                          use_scale=True, compatibility_mode="PyTorch"):
+                                          use_scale=True, compatibility_mode="PyTorch", fused_attention=True):
     """MultiheadAttention.BackwardPropagation (:243-292).  ``grads`` maps 'w_Q', 'w_K', 'w_V', 'out_proj_weight' to
     (weightGradients, biasGradientsOrNone) tensors that are filled in; dQ, dK, dV receive the input gradients."""
     from . import linear
@@ -219,21 +249,28 @@ def MultiheadAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, st, w_Q, w_K,
         dQ_p = GPUTensor([batch_size * tq, H * dk], None, w)
         dK_p = GPUTensor([batch_size * tkv, H * dk], None, w)
         dV_p = GPUTensor([batch_size * tkv, H * dv], None, w)
-        common = dict(batch=batch_size, heads=H)
-        # dV = P^T . dO                                                              (ScaledDotProductAttentionLayer.cs:117)
-        _heads_gemm(dV_p, P, d_attention_heads_T, transA=True, transB=False, M=tkv, N=dv, K=tq, alpha=1.0, a_packed=False,
-                    b_packed=True, c_packed=True, a_steps=0, b_steps=tq, c_steps=tkv, a_dim=0, b_dim=dv, c_dim=dv, **common)
-        # dS = scale * dO . V^T, then through the softmax                             (:123-125)
         dS = GPUTensor(P.Shape, None, w)
-        _heads_gemm(dS, d_attention_heads_T, st.V_heads, transA=False, transB=True, M=tq, N=tkv, K=dv, alpha=scaling,
-                    a_packed=True, b_packed=True, c_packed=False, a_steps=tq, b_steps=tkv, c_steps=0, a_dim=dv, b_dim=dv,
-                    c_dim=0, **common)
-        P.SoftmaxLastDimensionBackward(dS, dS)
-        # dQ = dS . K, dK = dS^T . Q                                                 (:127-128)
-        _heads_gemm(dQ_p, dS, st.K_heads, transA=False, transB=False, M=tq, N=dk, K=tkv, alpha=1.0, a_packed=False,
-                    b_packed=True, c_packed=True, a_steps=0, b_steps=tkv, c_steps=tq, a_dim=0, b_dim=dk, c_dim=dk, **common)
-        _heads_gemm(dK_p, dS, st.Q_heads, transA=True, transB=False, M=tkv, N=dk, K=tq, alpha=1.0, a_packed=False,
-                    b_packed=True, c_packed=True, a_steps=0, b_steps=tq, c_steps=tkv, a_dim=0, b_dim=dk, c_dim=dk, **common)
+        if fused_attention:
+            attention_backward(dQ_p, dK_p, dV_p, st.Q_heads, st.K_heads, st.V_heads, d_attention_heads_T, P, dS,
+                               batch=batch_size, heads=H, tq=tq, tkv=tkv, dk=dk, dv=dv, scale=scaling, packed=True)
+        else:
+            common = dict(batch=batch_size, heads=H)
+            # dV = P^T . dO                                                          (ScaledDotProductAttentionLayer.cs:117)
+            _heads_gemm(dV_p, P, d_attention_heads_T, transA=True, transB=False, M=tkv, N=dv, K=tq, alpha=1.0,
+                        a_packed=False, b_packed=True, c_packed=True, a_steps=0, b_steps=tq, c_steps=tkv, a_dim=0, b_dim=dv,
+                        c_dim=dv, **common)
+            # dS = scale * dO . V^T, then through the softmax                         (:123-125)
+            _heads_gemm(dS, d_attention_heads_T, st.V_heads, transA=False, transB=True, M=tq, N=tkv, K=dv, alpha=scaling,
+                        a_packed=True, b_packed=True, c_packed=False, a_steps=tq, b_steps=tkv, c_steps=0, a_dim=dv,
+                        b_dim=dv, c_dim=0, **common)
+            P.SoftmaxLastDimensionBackward(dS, dS)
+            # dQ = dS . K, dK = dS^T . Q                                             (:127-128)
+            _heads_gemm(dQ_p, dS, st.K_heads, transA=False, transB=False, M=tq, N=dk, K=tkv, alpha=1.0, a_packed=False,
+                        b_packed=True, c_packed=True, a_steps=0, b_steps=tkv, c_steps=tq, a_dim=0, b_dim=dk, c_dim=dk,
+                        **common)
+            _heads_gemm(dK_p, dS, st.Q_heads, transA=True, transB=False, M=tkv, N=dk, K=tq, alpha=1.0, a_packed=False,
+                        b_packed=True, c_packed=True, a_steps=0, b_steps=tq, c_steps=tkv, a_dim=0, b_dim=dk, c_dim=dk,
+                        **common)
         dS.Dispose()
     else:
         d_attention_heads = GPUTensor([batch_size, H, tkv, dv], None, w)
@@ -241,7 +278,7 @@ def MultiheadAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, st, w_Q, w_K,
         d_attention_heads = d_attention_heads.Reshape(batch_size * H, tkv, dv)
         dQ_h, dK_h, dV_h = (GPUTensor(t.Shape, None, w) for t in (st.Q_heads, st.K_heads, st.V_heads))
         ScaledDotProductAttentionBackwardPropagation(dQ_h, dK_h, dV_h, st.Q_heads, st.K_heads, st.V_heads,
-                                                     d_attention_heads, P, use_scale)                               # :270
+                                                     d_attention_heads, P, use_scale, fused=False)                  # :270
         def merge(t, steps, dim):                                                                                   # :276,279,282
             out = GPUTensor([batch_size, steps, H, dim], None, w)
             t.Reshape(batch_size, H, steps, dim).TransposeSecondAndThirdDimension(out)

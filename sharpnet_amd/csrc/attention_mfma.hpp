@@ -20,6 +20,13 @@
 // NT = 2, 4, 8 key tiles (up to 64, 128, 256 keys) and a head dimension of up to 32 or 64; keys and dimensions short of
 // the instantiated size are zero-filled and masked.  Sizes beyond 256 keys or a head dimension beyond 64 are not
 // handled here (the caller runs the four-call sequence instead).
+//
+// The same kernel, instantiated with BWD, is the first half of the backward pass
+// (ScaledDotProductAttentionBackwardPropagation, same file :111-132): with the roles Q <- dO, K <- V, V <- K it
+// computes dP^T = V . dO^T in place of the scores, turns it into the score gradient with the stored softmax output
+// (dS = scale * P * (dP - sum_k dP * P), the softmax gradient of :125 applied in registers; P is read twice, row sum
+// first), writes dS, and its second product is dQ = dS . K.  dV = P^T . dO and dK = dS^T . Q contract over the queries,
+// which lie along the lanes here, and stay batched GEMMs.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -43,7 +50,8 @@ struct AttnParams {
     const float* K;
     const float* V;
     float* O;
-    float* P;  // softmax output [z][Tq][Tk] (contiguous), or nullptr
+    float* P;  // forward: softmax output [z][Tq][Tk] (contiguous), or nullptr; backward: the score gradient dS (out)
+    const float* Pin;  // backward: the stored softmax output [z][Tq][Tk]
     int Tq, Tk, dk, dv;
     int ldq, ldk, ldv, ldo;
     long long sQ, sK, sV, sO;      // strides between matrices of the inner batch level, elements
@@ -77,7 +85,7 @@ __device__ __forceinline__ f32x4 load4_guarded(const float* p, int nvalid) {
     return x;
 }
 
-template <int NT, int HD>
+template <int NT, int HD, bool BWD = false>
 __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) {
     using CFG = AttnCfg<NT, HD>;
     constexpr int AT_TK = CFG::KEYS, AT_D = HD, AT_KP = CFG::KP, AT_VP = CFG::VP;
@@ -223,6 +231,44 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
         __syncthreads();
     }
 
+    if constexpr (BWD) {
+        // sacc holds dP^T (key t*32 + 8*(r/4) + r%4 + 4*lhi of query l32).  Score gradient through the softmax:
+        // dS = scale * P * (dP - sum_k dP_k P_k).  P comes from memory in the accumulator layout (four consecutive keys
+        // per 16-byte load), once for the row sum and once more (from cache) for the product.
+        const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + 4 * lhi;
+        const bool p_vec = (p.flags & 4) != 0;  // uniform: rows of P are 16-byte aligned
+        auto load_p = [&](int t, int g) {
+            const int key0 = t * 32 + 8 * g;    // + 4 * lhi, already in prow
+            const int nvalid = p.Tk - key0 - 4 * lhi;
+            if (p_vec && p.Tk == AT_TK) {
+                f32x4 x;
+                __builtin_memcpy(&x, prow + key0, 16);
+                return x;
+            }
+            return load4_guarded(prow + key0, nvalid);
+        };
+        float rs = 0.0f;
+#pragma unroll
+        for (int t = 0; t < AT_TK / 32; ++t) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 pv = load_p(t, g);
+                rs += sacc[t][4 * g] * pv.x + sacc[t][4 * g + 1] * pv.y + sacc[t][4 * g + 2] * pv.z + sacc[t][4 * g + 3] * pv.w;
+            }
+        }
+        rs += __shfl_xor(rs, 32, 64);
+#pragma unroll
+        for (int t = 0; t < AT_TK / 32; ++t) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 pv = load_p(t, g);
+                sacc[t][4 * g] = p.scale * pv.x * (sacc[t][4 * g] - rs);
+                sacc[t][4 * g + 1] = p.scale * pv.y * (sacc[t][4 * g + 1] - rs);
+                sacc[t][4 * g + 2] = p.scale * pv.z * (sacc[t][4 * g + 2] - rs);
+                sacc[t][4 * g + 3] = p.scale * pv.w * (sacc[t][4 * g + 3] - rs);
+            }
+        }
+    } else {
     // Scores are kept as log2-domain values s * scale * log2(e), so that exp(s - max) is one v_exp_f32.
     // A masked score (above the diagonal: the reference's -1e12, ScaledDotProductAttentionLayer.cs:73-76; or a key
     // past Tk) becomes a value so negative that its exponential is exactly zero.  Key index of register (t, r) is
@@ -273,6 +319,8 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
     for (int t = 0; t < AT_TK / 32; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[t][r] *= inv;
+
+    }
 
     // ---- P out (four consecutive keys per register group).  With all keys present and aligned rows the stores
     //      are spread over the second product's MFMAs instead (below); this is the general form. ----

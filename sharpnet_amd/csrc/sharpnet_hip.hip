@@ -129,6 +129,12 @@ constexpr AttnEntry attn_entry() {
 // smallest first: the first entry that holds the problem is used
 const AttnEntry kAttn[] = {attn_entry<2, 32>(), attn_entry<4, 32>(), attn_entry<8, 32>(),
                            attn_entry<2, 64>(), attn_entry<4, 64>(), attn_entry<8, 64>()};
+template <int NT, int HD>
+constexpr AttnEntry attn_bwd_entry() {
+    return AttnEntry{AttnCfg<NT, HD>::KEYS, HD, AttnCfg<NT, HD>::LDS_BYTES, attention_fwd_kernel<NT, HD, true>};
+}
+const AttnEntry kAttnBwd[] = {attn_bwd_entry<2, 32>(), attn_bwd_entry<4, 32>(), attn_bwd_entry<8, 32>(),
+                              attn_bwd_entry<2, 64>(), attn_bwd_entry<4, 64>(), attn_bwd_entry<8, 64>()};
 
 int hip_to_status(hipError_t e) {
     switch (e) {
@@ -563,6 +569,11 @@ int snhip_create(void** handle) {
                                 c.lds_bytes);
         if (e != hipSuccess) return hip_to_status(e);
     }
+    for (const AttnEntry& c : kAttnBwd) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                c.lds_bytes);
+        if (e != hipSuccess) return hip_to_status(e);
+    }
     Handle* h = new (std::nothrow) Handle();
     if (h == nullptr) return SNHIP_STATUS_ALLOC_FAILED;
     h->device = dev;
@@ -683,6 +694,102 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
     hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256), e->lds_bytes,
                        h->stream, p);
     return hip_to_status(hipGetLastError());
+}
+
+int snhip_sizeof_attention_bwd_desc(void) { return (int)sizeof(snhip_attention_bwd_desc); }
+
+int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
+    Handle* h = static_cast<Handle*>(handle);
+    if (d == nullptr || d->struct_size != (int)sizeof(snhip_attention_bwd_desc)) return SNHIP_STATUS_INVALID_VALUE;
+    if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (d->batch < 0 || d->batch_inner < 0 || d->Tq < 0 || d->Tk < 0 || d->dk < 0 || d->dv < 0)
+        return SNHIP_STATUS_INVALID_VALUE;
+    if (d->batch == 0 || d->Tq == 0 || d->Tk == 0) return SNHIP_STATUS_SUCCESS;
+    if (d->Q == nullptr || d->K == nullptr || d->V == nullptr || d->dO == nullptr || d->weights == nullptr ||
+        d->scores_gradients == nullptr || d->dQ == nullptr || d->dK == nullptr || d->dV == nullptr)
+        return SNHIP_STATUS_INVALID_VALUE;
+    if (d->ldq < d->dk || d->ldk < d->dk || d->ldv < d->dv || d->ldo < d->dv) return SNHIP_STATUS_INVALID_VALUE;
+    const int inner = d->batch_inner > 0 ? d->batch_inner : d->batch;
+    if (d->batch % inner != 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (d->batch > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
+    const long long tt = (long long)d->Tq * d->Tk;  // P and dS are contiguous stacks
+
+    // dV = P^T . dO                                                         (ScaledDotProductAttentionLayer.cs:117)
+    GemmArgs g;
+    g.tA = true;
+    g.M = d->Tk, g.N = d->dv, g.K = d->Tq;
+    g.A = d->weights, g.lda = d->Tk, g.sA = tt, g.sA2 = tt * inner;
+    g.B = d->dO, g.ldb = d->ldo, g.sB = d->strideO, g.sB2 = d->strideO_outer;
+    g.C = d->dV, g.ldc = d->ldv, g.sC = d->strideV, g.sC2 = d->strideV_outer;
+    g.batch = d->batch, g.batch_inner = d->batch_inner;
+    int st = gemm_core(h, g);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+
+    // dS and dQ: one kernel when it fits, else dS = scale * dO . V^T, softmax gradient, dQ = dS . K   (:123-127)
+    const int hd = d->dk > d->dv ? d->dk : d->dv;
+    const AttnEntry* e = nullptr;
+    for (const AttnEntry& c : kAttnBwd)
+        if (d->Tk <= c.keys && hd <= c.hd) {
+            e = &c;
+            break;
+        }
+    if (e != nullptr && d->dk > 0 && d->dv > 0) {
+        AttnParams p;
+        p.Q = d->dO, p.K = d->V, p.V = d->K, p.O = d->dQ, p.P = d->scores_gradients, p.Pin = d->weights;
+        p.Tq = d->Tq, p.Tk = d->Tk, p.dk = d->dv, p.dv = d->dk;  // first product contracts over dv, second produces dk
+        p.ldq = d->ldo, p.ldk = d->ldv, p.ldv = d->ldk, p.ldo = d->ldq;
+        p.sQ = d->strideO, p.sK = d->strideV, p.sV = d->strideK, p.sO = d->strideQ;
+        p.sQ2 = d->strideO_outer, p.sK2 = d->strideV_outer, p.sV2 = d->strideK_outer, p.sO2 = d->strideQ_outer;
+        p.batch_inner = inner;
+        p.scale = d->scale;
+        p.causal = 0;
+        p.flags = 0;
+        const bool multi = d->batch > 1, two_level = multi && inner < d->batch;
+        if ((uintptr_t)d->dQ % 16 == 0 && d->ldq % 4 == 0 && (!multi || d->strideQ % 4 == 0) &&
+            (!two_level || d->strideQ_outer % 4 == 0))
+            p.flags |= 1;
+        if ((uintptr_t)d->scores_gradients % 16 == 0 && d->Tk % 4 == 0) p.flags |= 2;
+        if ((uintptr_t)d->weights % 16 == 0 && d->Tk % 4 == 0) p.flags |= 4;
+        const int tiles = ceil_div(d->Tq, AT_BQ);
+        int groups = 1;
+        while (groups < tiles && (long long)d->batch * groups < 2LL * h->num_cu) ++groups;
+        p.q_tiles = ceil_div(tiles, groups);
+        hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256), e->lds_bytes,
+                           h->stream, p);
+        st = hip_to_status(hipGetLastError());
+        if (st != SNHIP_STATUS_SUCCESS) return st;
+    } else {
+        GemmArgs s1;
+        s1.tB = true;
+        s1.M = d->Tq, s1.N = d->Tk, s1.K = d->dv, s1.alpha = d->scale;
+        s1.A = d->dO, s1.lda = d->ldo, s1.sA = d->strideO, s1.sA2 = d->strideO_outer;
+        s1.B = d->V, s1.ldb = d->ldv, s1.sB = d->strideV, s1.sB2 = d->strideV_outer;
+        s1.C = d->scores_gradients, s1.ldc = d->Tk, s1.sC = tt, s1.sC2 = tt * inner;
+        s1.batch = d->batch, s1.batch_inner = d->batch_inner;
+        st = gemm_core(h, s1);
+        if (st != SNHIP_STATUS_SUCCESS) return st;
+        st = snhip_softmax_last_dim_backward(handle, d->weights, d->scores_gradients, d->scores_gradients,
+                                             (long long)d->batch * d->Tq, d->Tk);
+        if (st != SNHIP_STATUS_SUCCESS) return st;
+        GemmArgs s2;
+        s2.M = d->Tq, s2.N = d->dk, s2.K = d->Tk;
+        s2.A = d->scores_gradients, s2.lda = d->Tk, s2.sA = tt, s2.sA2 = tt * inner;
+        s2.B = d->K, s2.ldb = d->ldk, s2.sB = d->strideK, s2.sB2 = d->strideK_outer;
+        s2.C = d->dQ, s2.ldc = d->ldq, s2.sC = d->strideQ, s2.sC2 = d->strideQ_outer;
+        s2.batch = d->batch, s2.batch_inner = d->batch_inner;
+        st = gemm_core(h, s2);
+        if (st != SNHIP_STATUS_SUCCESS) return st;
+    }
+
+    // dK = dS^T . Q                                                                                    (:128)
+    GemmArgs k;
+    k.tA = true;
+    k.M = d->Tk, k.N = d->dk, k.K = d->Tq;
+    k.A = d->scores_gradients, k.lda = d->Tk, k.sA = tt, k.sA2 = tt * inner;
+    k.B = d->Q, k.ldb = d->ldq, k.sB = d->strideQ, k.sB2 = d->strideQ_outer;
+    k.C = d->dK, k.ldc = d->ldk, k.sC = d->strideK, k.sC2 = d->strideK_outer;
+    k.batch = d->batch, k.batch_inner = d->batch_inner;
+    return gemm_core(h, k);
 }
 
 int snhip_sizeof_gemm_desc(void) { return (int)sizeof(snhip_gemm_desc); }

@@ -98,6 +98,26 @@ class AttentionDesc(ctypes.Structure):
             setattr(self, k, v)
 
 
+class AttentionBwdDesc(ctypes.Structure):
+    """snhip_attention_bwd_desc of include/sharpnet_hip.h (field for field)."""
+    _fields_ = [
+        ("struct_size", _i), ("batch", _i), ("batch_inner", _i), ("Tq", _i), ("Tk", _i), ("dk", _i), ("dv", _i),
+        ("scale", _f), ("Q", _vp), ("K", _vp), ("V", _vp), ("dO", _vp), ("weights", _vp), ("scores_gradients", _vp),
+        ("dQ", _vp), ("dK", _vp), ("dV", _vp), ("ldq", _i), ("ldk", _i), ("ldv", _i), ("ldo", _i),
+        ("strideQ", _ll), ("strideK", _ll), ("strideV", _ll), ("strideO", _ll), ("strideQ_outer", _ll),
+        ("strideK_outer", _ll), ("strideV_outer", _ll), ("strideO_outer", _ll),
+    ]
+
+    def __init__(self, **kw):
+        super().__init__()
+        self.struct_size = ctypes.sizeof(AttentionBwdDesc)
+        self.scale = 1.0
+        for k, v in kw.items():
+            if k not in dict(self._fields_):
+                raise TypeError("snhip_attention_bwd_desc has no field %r" % k)
+            setattr(self, k, v)
+
+
 # SNHIP_ACT_* and the reference's cudnnActivationMode_t names for them (Prod/GPU/CudnnWrapper.cs:267-281)
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_TANH = range(5)
 ACTIVATIONS = {
@@ -136,6 +156,8 @@ SIGNATURES = {
     "snhip_sizeof_gemm_desc": [],
     "snhip_attention_forward": [_vp, ctypes.POINTER(AttentionDesc)],
     "snhip_sizeof_attention_desc": [],
+    "snhip_attention_backward": [_vp, ctypes.POINTER(AttentionBwdDesc)],
+    "snhip_sizeof_attention_bwd_desc": [],
     "snhip_dense_forward": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f],
     "snhip_dense_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f],
     "snhip_activation_forward": [_vp, _i, _f, _vp, _vp, _ll],

@@ -489,3 +489,44 @@ def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
             want = np.where(pre >= 0, pre, 0.1 * pre)
             assert np.max(np.abs(got[o, i] - want)) <= bound(K, a, b, 1e-5), (o, i)
             assert np.max(np.abs(cs[o, i] - a[o, i].astype(np.float64).sum(axis=0))) <= 1e-5 * np.sqrt(K) + 1e-6
+
+
+@pytest.mark.parametrize("B,H,Tq,Tk,dk,dv,packed", [
+    (5, 1, 37, 37, 16, 16, False), (2, 3, 256, 256, 64, 64, True), (2, 3, 256, 256, 64, 64, False),
+    (3, 2, 200, 130, 24, 40, True), (3, 2, 129, 65, 33, 7, False), (1, 4, 1, 5, 3, 2, True),
+    (1, 2, 40, 300, 8, 8, False),                                  # beyond 256 keys: the five-launch sequence
+])
+def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, packed):
+    """snhip_attention_backward (dV, score gradient through the softmax, dQ, dK; the middle two from one kernel when
+    the sizes allow it) against the oracle's ScaledDotProductAttentionBackwardPropagation, stacked and in-place-head
+    layouts, including the score-gradient buffer itself."""
+    from sharpnet_amd import GPUTensor, attention
+    rng = np.random.default_rng(61)
+    Z = B * H
+    q, k = random_tensor(rng, (Z, Tq, dk), -1, 1), random_tensor(rng, (Z, Tk, dk), -1, 1)
+    v, do = random_tensor(rng, (Z, Tk, dv), -1, 1), random_tensor(rng, (Z, Tq, dv), -1, 1)
+    wts = oracle.softmax_last_dim(random_tensor(rng, (Z, Tq, Tk), -3, 3))
+    scale = 0.37
+    # reference sequence, ScaledDotProductAttentionLayer.cs:117-128
+    dv_ref = oracle.bmm(wts, True, do, False)
+    ds_ref = oracle.softmax_last_dim_backward(wts, oracle.bmm(do, False, v, True, scale))
+    dq_ref = oracle.bmm(ds_ref, False, k, False)
+    dk_ref = oracle.bmm(ds_ref, True, q, False)
+
+    def lay(x, steps, dim):
+        if not packed:
+            return x
+        return np.ascontiguousarray(x.reshape(B, H, steps, dim).transpose(0, 2, 1, 3)).reshape(B, steps, H * dim)
+    w = gpu_wrapper
+    gq, gk, gv, gdo = T(w, lay(q, Tq, dk)), T(w, lay(k, Tk, dk)), T(w, lay(v, Tk, dv)), T(w, lay(do, Tq, dv))
+    gw, gds = T(w, wts), GPUTensor([Z, Tq, Tk], None, w)
+    gdq, gdk, gdv = (GPUTensor(t.Shape, None, w) for t in (gq, gk, gv))
+    for t in (gds, gdq, gdk, gdv):
+        t.SetValue(float("nan"))
+    attention.attention_backward(gdq, gdk, gdv, gq, gk, gv, gdo, gw, gds, batch=B, heads=H, tq=Tq, tkv=Tk, dk=dk, dv=dv,
+                                 scale=scale, packed=packed)
+    tol = 2e-5 * np.sqrt(max(Tq, Tk, dk, dv))
+    assert np.max(np.abs(gds.ToNumpy() - ds_ref)) <= tol
+    assert np.max(np.abs(gdv.ToNumpy() - lay(dv_ref, Tk, dv))) <= tol
+    assert np.max(np.abs(gdq.ToNumpy() - lay(dq_ref, Tq, dk))) <= tol
+    assert np.max(np.abs(gdk.ToNumpy() - lay(dk_ref, Tk, dk))) <= tol
