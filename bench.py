@@ -368,7 +368,21 @@ def layer_timings(w, wl):
                                  (", causal" if causal else ""),
                         "form": "one launch" if fused else "reference sequence (4 calls)", "forward_ms": ms,
                         "backward_ms": float("nan")})
-    for t in (q, k, v, o):
+    dq, dk_, dv_, do = (GPUTensor([Z, Tn, d], None, w) for _ in range(4))
+    do.SetValue(0.01)
+    for fused in (True, False):
+        def sdpa_fb():
+            wts = attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, True, fused=fused)
+            attention.ScaledDotProductAttentionBackwardPropagation(dq, dk_, dv_, q, k, v, do, wts, True, fused=fused)
+
+        def sdpa_f():
+            attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, True, fused=fused).Dispose()
+        f = timed(sdpa_f, 20, 10)
+        fb = timed(sdpa_fb, 20, 10)
+        res.append({"layer": "ScaledDotProductAttention forward + backward 512 x (256 x 64), causal",
+                    "form": "one launch forward, three backward" if fused else "reference sequence (4 + 5 calls)",
+                    "forward_ms": f, "backward_ms": round(fb - f, 4)})
+    for t in (q, k, v, o, dq, dk_, dv_, do):
         t.Dispose()
     B, Tn, H, d = 64, 256, 8, 64
     E = H * d
@@ -390,7 +404,8 @@ def layer_timings(w, wl):
         def fwd_bwd():
             fwd()
             st = state["st"]
-            attention.MultiheadAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, st, wq, wk, wv, wo, grads)
+            attention.MultiheadAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, st, wq, wk, wv, wo, grads,
+                                                            fused_attention=fused_attn)
             for t in (st.weights_buffer, st.Q_heads, st.K_heads, st.V_heads, st.attention_heads_T):
                 t.Dispose()
             state["st"] = None
@@ -398,7 +413,7 @@ def layer_timings(w, wl):
         f = timed(fwd, 10, 5)
         fb = timed(fwd_bwd, 10, 5)
         res.append({"layer": "MultiheadAttention batch %d, %d steps, %d heads x %d, causal" % (B, Tn, H, d),
-                    "form": ("heads in place, attention in one launch" if fused_attn else "heads in place") if in_place
+                    "form": ("heads in place, attention kernels" if fused_attn else "heads in place") if in_place
                     else "reference sequence (transposition copies)",
                     "forward_ms": f, "backward_ms": round(fb - f, 4)})
     w.use_memory_pool(False)

@@ -80,6 +80,12 @@ def test_gemm_descriptor_layout_matches_the_library():
     assert lib.snhip_attention_forward(None, ctypes.byref(a)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
     a.struct_size += 8
     assert lib.snhip_attention_forward(None, ctypes.byref(a)) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    assert lib.snhip_sizeof_attention_bwd_desc() == ctypes.sizeof(hiplib.AttentionBwdDesc)
+    g = hiplib.AttentionBwdDesc(batch=1, Tq=1, Tk=1, dk=1, dv=1)
+    assert lib.snhip_attention_backward(None, ctypes.byref(g)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
+    g.struct_size -= 8
+    assert lib.snhip_attention_backward(None, ctypes.byref(g)) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    assert lib.snhip_attention_backward(None, None) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
 
 
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
