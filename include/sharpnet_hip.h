@@ -239,6 +239,59 @@ typedef struct snhip_attention_bwd_desc {
 int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* desc);
 int snhip_sizeof_attention_bwd_desc(void);
 
+/* ---- recurrent layers on the GEMM ------------------------------------------ */
+/* Replace the cuDNN calls of Prod/Layers/RecurrentLayer.cs: cudnnGetRNNWeightSpaceSize (:138), cudnnGetRNNWeightParams
+ * (:176), cudnnGetRNNTempSpaceSizes (:335), cudnnRNNForward (:353), cudnnRNNBackwardData_v8 (:456) and
+ * cudnnRNNBackwardWeights_v8 (:485); bindings at Prod/GPU/CudnnWrapper.cs:1038-1125.  Same cell formulas as cuDNN's
+ * CUDNN_RNN_ALGO_STANDARD with linear input, data batch-major and unpacked ((batch, steps, features),
+ * Prod/GPU/GPUWrapper.cs:538), every sequence of full length.  x is (batch, steps, input_size), y and dy are
+ * (batch, steps, dirs * hidden_size) with the reverse direction in the second half of a row; hx, hy, cx, cy and their
+ * gradients are (dirs * num_layers, batch, hidden_size), any of them may be NULL (zeros in, nothing out).
+ * Each time step is one GEMM with the recurrent matrix plus one element-wise kernel; the input projections of all
+ * steps, dx and both weight gradients are one GEMM each per layer and direction.  Dropout between stacked layers is
+ * not implemented (the descriptor has no such field; the caller stacks single layers if it needs it). */
+#define SNHIP_RNN_RELU 0 /* cudnnRNNMode_t, Prod/GPU/CudnnWrapper.cs:313-327 */
+#define SNHIP_RNN_TANH 1
+#define SNHIP_RNN_LSTM 2
+#define SNHIP_RNN_GRU 3
+#define SNHIP_RNN_NO_BIAS 0 /* cudnnRNNBiasMode_t, :396-410 */
+#define SNHIP_RNN_SINGLE_INP_BIAS 1
+#define SNHIP_RNN_DOUBLE_BIAS 2
+#define SNHIP_RNN_SINGLE_REC_BIAS 3
+typedef struct snhip_rnn_desc { /* the fields of Prod/Layers/RNNDescriptor.cs this path uses */
+    int struct_size;            /* sizeof(snhip_rnn_desc) */
+    int cell_mode, bias_mode;
+    int bidirectional;          /* 0 / 1 */
+    int num_layers;
+    int input_size, hidden_size;
+} snhip_rnn_desc;
+int snhip_sizeof_rnn_desc(void);
+/* Bytes of the weight space.  Layout: all matrices (pseudo-layer by pseudo-layer = layer * dirs + direction: the
+ * input matrices of the gates i,f,g,o / r,z,n, then the recurrent ones, each hidden_size x inputs, row-major), then
+ * the bias vectors in the same order.  The reference never assumes a layout: it asks for addresses (:176). */
+int snhip_rnn_weight_space_size(const snhip_rnn_desc* desc, size_t* bytes);
+/* Offsets in floats from the start of the weight space of matrix and bias `lin_layer_id` (0 .. gates-1: input side,
+ * gates .. 2*gates-1: recurrent side) of `pseudo_layer`; *bias_offset = -1 when the bias mode has no such vector. */
+int snhip_rnn_weight_params(const snhip_rnn_desc* desc, int pseudo_layer, int lin_layer_id, long long* matrix_offset,
+                            int* rows, int* cols, long long* bias_offset);
+/* Sizes of the two buffers the calls below take.  reserve (training only) carries the forward pass's gates, cell
+ * states and layer outputs to the two backward calls; workspace is scratch for one call. */
+int snhip_rnn_temp_space_sizes(const snhip_rnn_desc* desc, int training, int batch, int steps,
+                               size_t* workspace_bytes, size_t* reserve_bytes);
+int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, int batch, int steps, const float* x,
+                      float* y, const float* hx, float* hy, const float* cx, float* cy, const float* weights,
+                      void* workspace, size_t workspace_bytes, void* reserve, size_t reserve_bytes);
+/* dx may be NULL (first layer of a network).  Leaves the gate gradients in reserve for snhip_rnn_backward_weights. */
+int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch, int steps, const float* y,
+                            const float* dy, float* dx, const float* hx, const float* dhy, float* dhx,
+                            const float* cx, const float* dcy, float* dcx, const float* weights, void* workspace,
+                            size_t workspace_bytes, void* reserve, size_t reserve_bytes);
+/* Adds to weight_gradients (CUDNN_WGRAD_MODE_ADD, RecurrentLayer.cs:488: the caller zeroes them first), same layout
+ * as the weight space.  Must follow snhip_rnn_backward_data on the same reserve buffer. */
+int snhip_rnn_backward_weights(void* handle, const snhip_rnn_desc* desc, int batch, int steps, const float* x,
+                               const float* hx, const float* y, float* weight_gradients, void* workspace,
+                               size_t workspace_bytes, void* reserve, size_t reserve_bytes);
+
 /* ---- bf16-input / fp32-accumulate variant (no reference counterpart) ------ */
 /* Operands stay fp32 in device memory; they are rounded to bf16 (nearest even)
  * on their way into LDS and multiplied with v_mfma_f32_32x32x16_bf16, products

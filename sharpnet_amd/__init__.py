@@ -6,5 +6,5 @@ mirrors the reference's ``GPUWrapper`` / ``GPUTensor<float>`` for that path.
 """
 from .hiplib import CublasStatus, SharpNetHipError, load_library, library_path  # noqa: F401
 from .gpu_tensor import GPUWrapper, GPUTensor  # noqa: F401
-from . import linear, attention  # noqa: F401
+from . import linear, attention, recurrent  # noqa: F401
 

@@ -19,8 +19,10 @@ MAIN_SOURCE = os.path.join(CSRC, "sharpnet_hip.hip")       # C ABI, dispatch, sm
 KERNEL_SOURCE = os.path.join(CSRC, "gemm_kernels.hip")     # GEMM kernels, compiled once per group of kernel_list.hpp
 KERNEL_GROUPS = 8                                          # SNHIP_NUM_KERNEL_GROUPS
 SOURCES = [MAIN_SOURCE, KERNEL_SOURCE]
-HEADERS = [os.path.join(CSRC, n) for n in ("sgemm_mfma.hpp", "bgemm_mfma.hpp", "rowops.hpp", "kernel_list.hpp", "attention_mfma.hpp")] + \
+HEADERS = [os.path.join(CSRC, n) for n in ("sgemm_mfma.hpp", "bgemm_mfma.hpp", "rowops.hpp", "kernel_list.hpp", "attention_mfma.hpp", "rnn_cells.hpp", "rnn_layers.hpp")] + \
           [os.path.join(REPO, "include", "sharpnet_hip.h")]
+# what gemm_kernels.hip includes; the other headers belong to the translation unit with the C ABI
+KERNEL_HEADERS = [os.path.join(CSRC, n) for n in ("sgemm_mfma.hpp", "bgemm_mfma.hpp", "kernel_list.hpp")]
 OBJ_DIR = os.path.join(HERE, "_obj")
 
 HIPCC_FLAGS = [
@@ -81,10 +83,11 @@ def build_library(force=False, verbose=True, jobs=None):
     jobs = jobs or max(1, min(8, os.cpu_count() or 1))
     objs = [u[-1] for u in units]
     if not force:
-        # rebuild only the objects that are older than their own source or any header
+        # rebuild only the objects that are older than their own source or a header they include
         def fresh(unit):
             obj, src = unit[-1], unit[-3]
-            return os.path.exists(obj) and all(os.path.getmtime(p) <= os.path.getmtime(obj) for p in [src] + HEADERS)
+            deps = HEADERS if src == MAIN_SOURCE else KERNEL_HEADERS
+            return os.path.exists(obj) and all(os.path.getmtime(p) <= os.path.getmtime(obj) for p in [src] + deps)
         units = [u for u in units if not fresh(u)]
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         outs = list(pool.map(lambda c: _run(c, verbose), units))

@@ -1,0 +1,420 @@
+// Recurrent layers (RELU / TANH / LSTM / GRU cells, stacked, one or two directions) as sequences of GEMM launches
+// and the element-wise kernels of rnn_cells.hpp.  Included at the end of sharpnet_hip.hip and nowhere else: it uses
+// that file's Handle, GemmArgs and gemm_core.  Entry points are declared in include/sharpnet_hip.h.
+//
+// Work of one layer and direction (n = batch * steps rows, G gates, H hidden units, I inputs):
+//   forward    gates (n x G*H) = X (n x I) . W^T + bW                                  one GEMM over all steps
+//              per step: gates[:, t] += h[t-1] . R^T (GRU: into a buffer of its own)   GEMM batch x G*H x H
+//                        cell kernel -> h[t] into y and into the slot the next step reads
+//   backward   per step, last to first: cell kernel -> d(gates)[:, t]; dh = d(gates)[:, t] . R   GEMM batch x H x G*H
+//              dX (n x I) = d(gates) . W                                               one GEMM
+//   weights    dW += d(gates)^T . X, dR += d(gates_h)^T . Hprev, bias gradients = column sums     two GEMMs
+// Hprev (n x H) holds, for every (sample, step), the state that entered the step, so the recurrent weight gradient
+// is a single product over all steps.
+#pragma once
+#include "rnn_cells.hpp"
+
+namespace {
+
+struct RnnDims {
+    int cell, G, H, I, K, L, P;      // P = K * L pseudo-layers
+    bool bias_w, bias_r;
+    int batch, steps;
+    long long n;                      // batch * steps
+    long long per_p;                  // floats of one pseudo-layer's region
+    long long gates_off, hprev_off, cells_off, gh_off;   // inside a pseudo-layer's region
+    long long out_off;                // start of the stacked layers' outputs, after all regions
+    long long total;                  // floats carried from forward to backward
+    long long bwd_ws;                 // floats of scratch the backward calls need
+};
+
+int rnn_gates(int cell) { return cell == RNN_LSTM ? 4 : (cell == RNN_GRU ? 3 : 1); }
+
+int rnn_check_desc(const snhip_rnn_desc* d) {
+    if (d == nullptr || d->struct_size != (int)sizeof(snhip_rnn_desc)) return SNHIP_STATUS_INVALID_VALUE;
+    if (d->cell_mode < SNHIP_RNN_RELU || d->cell_mode > SNHIP_RNN_GRU) return SNHIP_STATUS_INVALID_VALUE;
+    if (d->bias_mode < SNHIP_RNN_NO_BIAS || d->bias_mode > SNHIP_RNN_SINGLE_REC_BIAS) return SNHIP_STATUS_INVALID_VALUE;
+    if (d->bidirectional != 0 && d->bidirectional != 1) return SNHIP_STATUS_INVALID_VALUE;
+    if (d->num_layers < 1 || d->input_size < 1 || d->hidden_size < 1) return SNHIP_STATUS_INVALID_VALUE;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+RnnDims rnn_dims(const snhip_rnn_desc* d, int batch, int steps) {
+    RnnDims r;
+    r.cell = d->cell_mode;
+    r.G = rnn_gates(d->cell_mode);
+    r.H = d->hidden_size;
+    r.I = d->input_size;
+    r.K = d->bidirectional ? 2 : 1;
+    r.L = d->num_layers;
+    r.P = r.K * r.L;
+    r.bias_w = d->bias_mode == SNHIP_RNN_DOUBLE_BIAS || d->bias_mode == SNHIP_RNN_SINGLE_INP_BIAS;
+    r.bias_r = d->bias_mode == SNHIP_RNN_DOUBLE_BIAS || d->bias_mode == SNHIP_RNN_SINGLE_REC_BIAS;
+    r.batch = batch;
+    r.steps = steps;
+    r.n = (long long)batch * steps;
+    r.gates_off = 0;
+    r.hprev_off = r.n * r.G * r.H;
+    r.cells_off = r.hprev_off + r.n * r.H;
+    r.gh_off = r.cells_off + (r.cell == RNN_LSTM ? r.n * r.H : 0);
+    r.per_p = r.gh_off + (r.cell == RNN_GRU ? r.n * 3 * r.H : 0);
+    r.out_off = r.per_p * r.P;
+    r.total = r.out_off + (long long)(r.L - 1) * r.n * r.K * r.H;
+    // dh, dc, one bias gradient, and two buffers for the gradients that travel between stacked layers
+    r.bwd_ws = 2LL * batch * r.H + (long long)r.G * r.H + (r.L > 1 ? 2 * r.n * r.K * r.H : 0);
+    return r;
+}
+
+long long rnn_layer_inputs(const RnnDims& r, int layer) { return layer == 0 ? r.I : (long long)r.K * r.H; }
+long long rnn_matrix_floats(const RnnDims& r, int p) {
+    return (long long)r.G * r.H * (rnn_layer_inputs(r, p / r.K) + r.H);
+}
+long long rnn_bias_floats(const RnnDims& r) { return (long long)r.G * r.H * ((r.bias_w ? 1 : 0) + (r.bias_r ? 1 : 0)); }
+long long rnn_all_matrices(const RnnDims& r) {
+    long long s = 0;
+    for (int p = 0; p < r.P; ++p) s += rnn_matrix_floats(r, p);
+    return s;
+}
+
+// Where the stacked matrices and bias vectors of one pseudo-layer sit in a weight space, in floats (-1: absent).
+struct RnnOffsets {
+    long long W, R, bW, bR;
+};
+RnnOffsets rnn_offsets(const RnnDims& r, int p) {
+    RnnOffsets o;
+    o.W = 0;
+    for (int q = 0; q < p; ++q) o.W += rnn_matrix_floats(r, q);
+    o.R = o.W + (long long)r.G * r.H * rnn_layer_inputs(r, p / r.K);
+    const long long b = rnn_all_matrices(r) + (long long)p * rnn_bias_floats(r);
+    o.bW = r.bias_w ? b : -1;
+    o.bR = r.bias_r ? b + (r.bias_w ? (long long)r.G * r.H : 0) : -1;
+    return o;
+}
+struct RnnWeights {
+    float* W;    // (G*H, inputs)
+    float* R;    // (G*H, H)
+    float* bW;   // (G*H) or nullptr
+    float* bR;
+};
+RnnWeights rnn_weights(const RnnDims& r, float* space, int p) {
+    const RnnOffsets o = rnn_offsets(r, p);
+    return RnnWeights{space + o.W, space + o.R, o.bW >= 0 ? space + o.bW : nullptr, o.bR >= 0 ? space + o.bR : nullptr};
+}
+
+int rnn_set_rows(Handle* h, float* dst, long long ld_dst, const float* src, long long ld_src, int rows, int cols) {
+    const long long total = (long long)rows * cols;
+    hipLaunchKernelGGL(set_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, h->stream, dst, ld_dst, src,
+                       ld_src, rows, cols);
+    return hip_to_status(hipGetLastError());
+}
+
+int rnn_common_checks(Handle* h, const snhip_rnn_desc* desc, int batch, int steps) {
+    const int st = rnn_check_desc(desc);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (batch < 0 || steps < 0) return SNHIP_STATUS_INVALID_VALUE;
+    // row counts and row pitches travel as 32-bit integers through the GEMM arguments
+    const long long widest = (long long)rnn_gates(desc->cell_mode) * desc->hidden_size;
+    const long long in_max = desc->input_size > 2LL * desc->hidden_size ? desc->input_size : 2LL * desc->hidden_size;
+    if ((long long)batch * steps > 0x7fffffffLL || (long long)steps * (widest > in_max ? widest : in_max) > 0x7fffffffLL ||
+        (long long)batch * desc->hidden_size > 0x7fffffffLL)
+        return SNHIP_STATUS_NOT_SUPPORTED;
+    // the handle belongs to one device; a caller thread on another one is switched over, as in the GEMM calls
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (cur != h->device && hipSetDevice(h->device) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" {
+
+int snhip_sizeof_rnn_desc(void) { return (int)sizeof(snhip_rnn_desc); }
+
+int snhip_rnn_weight_space_size(const snhip_rnn_desc* desc, size_t* bytes) {
+    const int st = rnn_check_desc(desc);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    if (bytes == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    const RnnDims r = rnn_dims(desc, 0, 0);
+    *bytes = (size_t)(rnn_all_matrices(r) + (long long)r.P * rnn_bias_floats(r)) * sizeof(float);
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_rnn_weight_params(const snhip_rnn_desc* desc, int pseudo_layer, int lin_layer_id, long long* matrix_offset,
+                            int* rows, int* cols, long long* bias_offset) {
+    const int st = rnn_check_desc(desc);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    const RnnDims r = rnn_dims(desc, 0, 0);
+    if (pseudo_layer < 0 || pseudo_layer >= r.P || lin_layer_id < 0 || lin_layer_id >= 2 * r.G)
+        return SNHIP_STATUS_INVALID_VALUE;
+    const bool recurrent = lin_layer_id >= r.G;
+    const int gate = recurrent ? lin_layer_id - r.G : lin_layer_id;
+    const long long inputs = recurrent ? r.H : rnn_layer_inputs(r, pseudo_layer / r.K);
+    const RnnOffsets o = rnn_offsets(r, pseudo_layer);
+    const long long b = recurrent ? o.bR : o.bW;
+    if (matrix_offset != nullptr) *matrix_offset = (recurrent ? o.R : o.W) + (long long)gate * r.H * inputs;
+    if (rows != nullptr) *rows = r.H;
+    if (cols != nullptr) *cols = (int)inputs;
+    if (bias_offset != nullptr) *bias_offset = b >= 0 ? b + (long long)gate * r.H : -1;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_rnn_temp_space_sizes(const snhip_rnn_desc* desc, int training, int batch, int steps, size_t* workspace_bytes,
+                               size_t* reserve_bytes) {
+    const int st = rnn_check_desc(desc);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    if (batch < 0 || steps < 0 || workspace_bytes == nullptr || reserve_bytes == nullptr)
+        return SNHIP_STATUS_INVALID_VALUE;
+    const RnnDims r = rnn_dims(desc, batch, steps);
+    // inference keeps the gates in the workspace; training keeps them in reserve and its backward calls use the
+    // workspace (the reference sizes it once, in the forward call, and reuses that size: RecurrentLayer.cs:335-345,461)
+    const long long ws = training ? r.bwd_ws : (r.total > r.bwd_ws ? r.total : r.bwd_ws);
+    *workspace_bytes = (size_t)(ws > 4 ? ws : 4) * sizeof(float);
+    *reserve_bytes = training ? (size_t)(r.total > 4 ? r.total : 4) * sizeof(float) : 0;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, int batch, int steps, const float* x,
+                      float* y, const float* hx, float* hy, const float* cx, float* cy, const float* weights,
+                      void* workspace, size_t workspace_bytes, void* reserve, size_t reserve_bytes) {
+    Handle* h = static_cast<Handle*>(handle);
+    int st = rnn_common_checks(h, desc, batch, steps);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    if (batch == 0 || steps == 0) return SNHIP_STATUS_SUCCESS;
+    if (x == nullptr || y == nullptr || weights == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    const RnnDims r = rnn_dims(desc, batch, steps);
+    float* keep = static_cast<float*>(training ? reserve : workspace);
+    const size_t keep_bytes = training ? reserve_bytes : workspace_bytes;
+    if (keep == nullptr || keep_bytes < (size_t)r.total * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
+    const int B = batch, T = steps, H = r.H, G = r.G, K = r.K;
+    const long long GH = (long long)G * H;
+
+    for (int layer = 0; layer < r.L; ++layer) {
+        const float* inp = layer == 0 ? x : keep + r.out_off + (long long)(layer - 1) * r.n * K * H;
+        float* out = layer == r.L - 1 ? y : keep + r.out_off + (long long)layer * r.n * K * H;
+        const long long I = rnn_layer_inputs(r, layer);
+        for (int d = 0; d < K; ++d) {
+            const int p = layer * K + d;
+            const RnnWeights w = rnn_weights(r, const_cast<float*>(weights), p);
+            float* region = keep + (long long)p * r.per_p;
+            float* gates = region + r.gates_off;
+            float* hprev = region + r.hprev_off;
+            float* cells = region + r.cells_off;
+            float* gh = region + r.gh_off;
+            const float* hx_p = hx ? hx + (long long)p * B * H : nullptr;
+            const float* cx_p = cx ? cx + (long long)p * B * H : nullptr;
+
+            GemmArgs g;  // input projections of every step at once
+            g.tB = true;
+            g.M = (int)r.n, g.N = (int)GH, g.K = (int)I;
+            g.A = inp, g.lda = (int)I, g.B = w.W, g.ldb = (int)I, g.C = gates, g.ldc = (int)GH;
+            g.bias = w.bW;
+            st = gemm_core(h, g);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+
+            const int first = d == 0 ? 0 : T - 1, dir = d == 0 ? 1 : -1;
+            st = rnn_set_rows(h, hprev + (long long)first * H, (long long)T * H, hx_p, H, B, H);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+            for (int k = 0; k < T; ++k) {
+                const int t = first + dir * k;
+                const bool last = k == T - 1;
+                const bool zero_state = k == 0 && hx_p == nullptr;
+                if (r.cell == RNN_GRU || !zero_state) {
+                    GemmArgs s;  // h[t-1] . R^T
+                    s.tB = true;
+                    s.M = B, s.N = (int)GH, s.K = H;
+                    s.A = hprev + (long long)t * H, s.lda = T * H;
+                    s.B = w.R, s.ldb = H;
+                    if (r.cell == RNN_GRU) {
+                        s.C = gh + (long long)t * 3 * H, s.ldc = T * 3 * H;
+                    } else {
+                        s.C = gates + (long long)t * GH, s.ldc = (int)(T * GH), s.beta = 1.0f;
+                    }
+                    st = gemm_core(h, s);
+                    if (st != SNHIP_STATUS_SUCCESS) return st;
+                }
+                RnnStepFwd c;
+                c.gates = gates + (long long)t * GH, c.ld_gates = T * GH;
+                c.gh = gh + (long long)t * 3 * H, c.ld_gh = (long long)T * 3 * H;
+                c.bias_r = w.bR;
+                c.h_prev = hprev + (long long)t * H, c.ld_hprev = (long long)T * H;
+                if (k == 0) {
+                    c.c_prev = cx_p, c.ld_cprev = H;
+                } else {
+                    c.c_prev = cells + (long long)(t - dir) * H, c.ld_cprev = (long long)T * H;
+                }
+                c.c_out = cells + (long long)t * H, c.ld_c = (long long)T * H;
+                c.y = out + (long long)t * K * H + (long long)d * H, c.ld_y = (long long)T * K * H;
+                c.h_next = last ? nullptr : hprev + (long long)(t + dir) * H, c.ld_hnext = (long long)T * H;
+                c.hy = (last && hy) ? hy + (long long)p * B * H : nullptr;
+                c.cy = (last && cy && r.cell == RNN_LSTM) ? cy + (long long)p * B * H : nullptr;
+                c.batch = B, c.hidden = H, c.cell = r.cell;
+                hipLaunchKernelGGL(rnn_cell_fwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
+                                   h->stream, c);
+                st = hip_to_status(hipGetLastError());
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+        }
+    }
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch, int steps, const float* y,
+                            const float* dy, float* dx, const float* hx, const float* dhy, float* dhx,
+                            const float* cx, const float* dcy, float* dcx, const float* weights, void* workspace,
+                            size_t workspace_bytes, void* reserve, size_t reserve_bytes) {
+    Handle* h = static_cast<Handle*>(handle);
+    int st = rnn_common_checks(h, desc, batch, steps);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    if (batch == 0 || steps == 0) return SNHIP_STATUS_SUCCESS;
+    (void)hx;  // the states that entered every step are in reserve
+    if (y == nullptr || dy == nullptr || weights == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    const RnnDims r = rnn_dims(desc, batch, steps);
+    float* keep = static_cast<float*>(reserve);
+    float* ws = static_cast<float*>(workspace);
+    if (keep == nullptr || reserve_bytes < (size_t)r.total * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
+    if (ws == nullptr || workspace_bytes < (size_t)r.bwd_ws * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
+    const int B = batch, T = steps, H = r.H, G = r.G, K = r.K;
+    const long long GH = (long long)G * H;
+    float* dh = ws;
+    float* dc = ws + (long long)B * H;
+    float* between[2] = {ws + 2LL * B * H + GH, ws + 2LL * B * H + GH + r.n * K * H};
+
+    for (int layer = r.L - 1; layer >= 0; --layer) {
+        const float* out = layer == r.L - 1 ? y : keep + r.out_off + (long long)layer * r.n * K * H;
+        const float* dout = layer == r.L - 1 ? dy : between[layer & 1];
+        float* dinp = layer == 0 ? dx : between[(layer - 1) & 1];
+        const long long I = rnn_layer_inputs(r, layer);
+        for (int d = 0; d < K; ++d) {
+            const int p = layer * K + d;
+            const RnnWeights w = rnn_weights(r, const_cast<float*>(weights), p);
+            float* region = keep + (long long)p * r.per_p;
+            float* gates = region + r.gates_off;
+            float* hprev = region + r.hprev_off;
+            float* cells = region + r.cells_off;
+            float* gh = region + r.gh_off;
+            const float* cx_p = cx ? cx + (long long)p * B * H : nullptr;
+            st = rnn_set_rows(h, dh, H, dhy ? dhy + (long long)p * B * H : nullptr, H, B, H);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+            if (r.cell == RNN_LSTM) {
+                st = rnn_set_rows(h, dc, H, dcy ? dcy + (long long)p * B * H : nullptr, H, B, H);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+            const int first = d == 0 ? 0 : T - 1, dir = d == 0 ? 1 : -1;
+            for (int k = T - 1; k >= 0; --k) {
+                const int t = first + dir * k;
+                RnnStepBwd c;
+                c.gates = gates + (long long)t * GH, c.ld_gates = T * GH;
+                c.gh = gh + (long long)t * 3 * H, c.ld_gh = (long long)T * 3 * H;
+                c.h_prev = hprev + (long long)t * H, c.ld_hprev = (long long)T * H;
+                c.y = out + (long long)t * K * H + (long long)d * H, c.ld_y = (long long)T * K * H;
+                if (k == 0) {
+                    c.c_prev = cx_p, c.ld_cprev = H;
+                } else {
+                    c.c_prev = cells + (long long)(t - dir) * H, c.ld_cprev = (long long)T * H;
+                }
+                c.c = cells + (long long)t * H, c.ld_c = (long long)T * H;
+                c.dy = dout + (long long)t * K * H + (long long)d * H, c.ld_dy = (long long)T * K * H;
+                c.dh = dh, c.dc = dc;
+                c.batch = B, c.hidden = H, c.cell = r.cell;
+                hipLaunchKernelGGL(rnn_cell_bwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
+                                   h->stream, c);
+                st = hip_to_status(hipGetLastError());
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+                if (k == 0 && dhx == nullptr) break;  // nobody asks for the gradient of the initial state
+                GemmArgs s;  // dh = d(R h)[:, t] . R  (GRU: added to dh * z)
+                s.M = B, s.N = H, s.K = (int)GH;
+                s.A = (r.cell == RNN_GRU) ? gh + (long long)t * 3 * H : gates + (long long)t * GH;
+                s.lda = (int)(T * GH);
+                s.B = w.R, s.ldb = H;
+                s.C = dh, s.ldc = H;
+                s.beta = (r.cell == RNN_GRU) ? 1.0f : 0.0f;
+                st = gemm_core(h, s);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+            if (dhx != nullptr) {
+                st = rnn_set_rows(h, dhx + (long long)p * B * H, H, dh, H, B, H);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+            if (dcx != nullptr && r.cell == RNN_LSTM) {
+                st = rnn_set_rows(h, dcx + (long long)p * B * H, H, dc, H, B, H);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+            if (dinp != nullptr) {
+                GemmArgs g;  // gradient of the layer's input: both directions add up
+                g.M = (int)r.n, g.N = (int)I, g.K = (int)GH;
+                g.A = gates, g.lda = (int)GH, g.B = w.W, g.ldb = (int)I, g.C = dinp, g.ldc = (int)I;
+                g.beta = d == 0 ? 0.0f : 1.0f;
+                st = gemm_core(h, g);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+        }
+    }
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_rnn_backward_weights(void* handle, const snhip_rnn_desc* desc, int batch, int steps, const float* x,
+                               const float* hx, const float* y, float* weight_gradients, void* workspace,
+                               size_t workspace_bytes, void* reserve, size_t reserve_bytes) {
+    Handle* h = static_cast<Handle*>(handle);
+    int st = rnn_common_checks(h, desc, batch, steps);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    if (batch == 0 || steps == 0) return SNHIP_STATUS_SUCCESS;
+    (void)hx, (void)y;  // both are in reserve, arranged per step
+    if (x == nullptr || weight_gradients == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    const RnnDims r = rnn_dims(desc, batch, steps);
+    float* keep = static_cast<float*>(reserve);
+    float* ws = static_cast<float*>(workspace);
+    if (keep == nullptr || reserve_bytes < (size_t)r.total * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
+    if (ws == nullptr || workspace_bytes < (size_t)r.bwd_ws * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
+    const int H = r.H, G = r.G, K = r.K;
+    const long long GH = (long long)G * H;
+    float* colsum = ws + 2LL * batch * H;
+
+    for (int layer = 0; layer < r.L; ++layer) {
+        const float* inp = layer == 0 ? x : keep + r.out_off + (long long)(layer - 1) * r.n * K * H;
+        const long long I = rnn_layer_inputs(r, layer);
+        for (int d = 0; d < K; ++d) {
+            const int p = layer * K + d;
+            const RnnWeights dw = rnn_weights(r, weight_gradients, p);
+            float* region = keep + (long long)p * r.per_p;
+            const float* dgates = region + r.gates_off;
+            const float* hprev = region + r.hprev_off;
+            const float* dgh = (r.cell == RNN_GRU) ? region + r.gh_off : dgates;
+
+            GemmArgs g;  // dW += d(gates)^T . X, column sums of d(gates) on the side
+            g.tA = true;
+            g.M = (int)GH, g.N = (int)I, g.K = (int)r.n;
+            g.A = dgates, g.lda = (int)GH, g.B = inp, g.ldb = (int)I, g.C = dw.W, g.ldc = (int)I;
+            g.beta = 1.0f;
+            g.colsum = (dw.bW != nullptr || (dw.bR != nullptr && r.cell != RNN_GRU)) ? colsum : nullptr;
+            st = gemm_core(h, g);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+            if (dw.bW != nullptr) {
+                st = snhip_axpy(handle, GH, 1.0f, colsum, dw.bW);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+            if (dw.bR != nullptr && r.cell != RNN_GRU) {
+                st = snhip_axpy(handle, GH, 1.0f, colsum, dw.bR);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+
+            GemmArgs q;  // dR += d(R h + bR)^T . Hprev
+            q.tA = true;
+            q.M = (int)GH, q.N = H, q.K = (int)r.n;
+            q.A = dgh, q.lda = (int)GH, q.B = hprev, q.ldb = H, q.C = dw.R, q.ldc = H;
+            q.beta = 1.0f;
+            q.colsum = (dw.bR != nullptr && r.cell == RNN_GRU) ? colsum : nullptr;
+            st = gemm_core(h, q);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+            if (q.colsum != nullptr) {
+                st = snhip_axpy(handle, GH, 1.0f, colsum, dw.bR);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
+        }
+    }
+    return SNHIP_STATUS_SUCCESS;
+}
+
+}  // extern "C"

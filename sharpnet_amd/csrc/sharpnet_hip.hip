@@ -1232,3 +1232,5 @@ int snhip_config_desc(int config, int desc[6]) {
 }
 
 }  // extern "C"
+
+#include "rnn_layers.hpp"

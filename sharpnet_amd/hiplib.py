@@ -118,6 +118,21 @@ class AttentionBwdDesc(ctypes.Structure):
             setattr(self, k, v)
 
 
+class RnnDesc(ctypes.Structure):
+    """snhip_rnn_desc of include/sharpnet_hip.h (field for field)."""
+    _fields_ = [("struct_size", _i), ("cell_mode", _i), ("bias_mode", _i), ("bidirectional", _i), ("num_layers", _i),
+                ("input_size", _i), ("hidden_size", _i)]
+
+    def __init__(self, **kw):
+        super().__init__()
+        self.struct_size = ctypes.sizeof(RnnDesc)
+        self.num_layers = 1
+        for k, v in kw.items():
+            if k not in dict(self._fields_):
+                raise TypeError("snhip_rnn_desc has no field %r" % k)
+            setattr(self, k, int(v))
+
+
 # SNHIP_ACT_* and the reference's cudnnActivationMode_t names for them (Prod/GPU/CudnnWrapper.cs:267-281)
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_TANH = range(5)
 ACTIVATIONS = {
@@ -158,6 +173,15 @@ SIGNATURES = {
     "snhip_sizeof_attention_desc": [],
     "snhip_attention_backward": [_vp, ctypes.POINTER(AttentionBwdDesc)],
     "snhip_sizeof_attention_bwd_desc": [],
+    "snhip_sizeof_rnn_desc": [],
+    "snhip_rnn_weight_space_size": [ctypes.POINTER(RnnDesc), ctypes.POINTER(_sz)],
+    "snhip_rnn_weight_params": [ctypes.POINTER(RnnDesc), _i, _i, ctypes.POINTER(_ll), _c_int_p, _c_int_p,
+                                ctypes.POINTER(_ll)],
+    "snhip_rnn_temp_space_sizes": [ctypes.POINTER(RnnDesc), _i, _i, _i, ctypes.POINTER(_sz), ctypes.POINTER(_sz)],
+    "snhip_rnn_forward": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz],
+    "snhip_rnn_backward_data": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                _vp, _sz, _vp, _sz],
+    "snhip_rnn_backward_weights": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz],
     "snhip_dense_forward": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f],
     "snhip_dense_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f],
     "snhip_activation_forward": [_vp, _i, _f, _vp, _vp, _ll],

@@ -32,6 +32,10 @@ def numpy_literals(block):
     return out
 
 
+def np_shape(v):
+    return (len(v), len(v[0])) if isinstance(v, list) and isinstance(v[0], list) else len(v)
+
+
 def const_literal(text, name):
     m = re.search(r'const string ' + re.escape(name) + r'\s*=\s*@?"([^"]*)"', text)
     body = m.group(1)
@@ -142,6 +146,22 @@ def main():
         "x_shape": [10, 2, 6], "y_shape": [10, 3], "num_heads": 3, "key_dim": 2, "value_dim": 2,
         "lr": 0.1, "momentum": 0.9, "epochs": 10, "batch_size": 2, "tolerance": 1e-6,
         "no_bias": mha["no_bias"], "with_bias": mha["with_bias"],
+    }
+
+    # ---- same file :896-953  two stacked SimpleRNN layers (cuDNN tanh cells) ----
+    blk = lines(prp, 896, 953)
+    w = numpy_literals(blk)
+    assert len(w) == 10 and len(w[2][0]) == 4 and len(w[8][0]) == 4, [np_shape(v) for v in w]
+    losses = [float(v) for v in re.findall(r'Assert\.AreEqual\(([0-9.eE+-]+), loss_', blk)]
+    fx["PyTorch_SimpleRNN"] = {
+        "source": "Tests/NonReg/ParallelRunWithPyTorch.cs:896-953; X = numpy_array_for_tests(4,2,1), Y = y_numpy_array_for_tests(4,2); "
+                  "SimpleRNN(hidden 2, return sequences, bidirectional, 2 layers) then SimpleRNN(hidden 2, last step only); tanh "
+                  "cells with two zero-initialised bias vectors (PyTorch compatibility mode); MSE; SGD(0.01, momentum 0.9), "
+                  "batch size 2, 10 epochs, no shuffling",
+        "x_shape": [4, 2, 1], "y_shape": [4, 2],
+        "layer1_weight_ih": w[0:4], "layer1_weight_hh": w[4:8], "layer2_weight_ih": [w[8]], "layer2_weight_hh": [w[9]],
+        "lr": 0.01, "momentum": 0.9, "epochs": 10, "batch_size": 2,
+        "loss_before": losses[0], "loss_after": losses[1], "tolerance": 1e-6,
     }
 
     with open(OUT, "w") as f:

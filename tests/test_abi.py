@@ -86,6 +86,17 @@ def test_gemm_descriptor_layout_matches_the_library():
     g.struct_size -= 8
     assert lib.snhip_attention_backward(None, ctypes.byref(g)) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
     assert lib.snhip_attention_backward(None, None) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    assert lib.snhip_sizeof_rnn_desc() == ctypes.sizeof(hiplib.RnnDesc)
+    r = hiplib.RnnDesc(cell_mode=2, bias_mode=1, bidirectional=1, num_layers=2, input_size=3, hidden_size=5)
+    nbytes = ctypes.c_size_t()
+    assert lib.snhip_rnn_weight_space_size(ctypes.byref(r), ctypes.byref(nbytes)) == 0
+    # two directions, four gates: layer 0 reads 3 inputs, layer 1 reads 2 * 5; input-side biases only
+    assert nbytes.value == 4 * (2 * 4 * 5 * (3 + 5) + 2 * 4 * 5 * (10 + 5) + 4 * 4 * 5)
+    assert lib.snhip_rnn_forward(None, ctypes.byref(r), 0, 1, 1, None, None, None, None, None, None, None, None, 0, None,
+                                 0) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
+    r.struct_size += 4
+    assert lib.snhip_rnn_weight_space_size(ctypes.byref(r), ctypes.byref(nbytes)) == \
+        hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
 
 
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):

@@ -1,0 +1,209 @@
+"""GPU tests of the recurrent layers (snhip_rnn_*): the raw entry points against oracle/rnn_oracle.py for every
+cell, direction, depth and bias mode, with and without initial states; the RecurrentLayer mirror through the
+reference's stored SimpleRNN losses."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import rnn_oracle as ro
+from tests.rnn_chain import simple_rnn_chain
+
+pytestmark = pytest.mark.gpu
+
+
+def T(w, a):
+    from sharpnet_amd import GPUTensor
+    a = np.asarray(a, np.float32)
+    return GPUTensor(list(a.shape), a, w)
+
+
+def lib_desc(desc):
+    from sharpnet_amd.hiplib import RnnDesc
+    return RnnDesc(cell_mode=desc.cell, bias_mode=desc.bias_mode, bidirectional=desc.bidirectional,
+                   num_layers=desc.num_layers, input_size=desc.input_size, hidden_size=desc.hidden_size)
+
+
+def check(st, what):
+    from sharpnet_amd.hiplib import check_status
+    check_status(st, what)
+
+
+def run_gpu(w, desc, x, weights, dy, hx=None, cx=None, dhy=None, dcy=None, training=True):
+    """Forward (+ backward when training) through the C ABI; returns dict of numpy arrays."""
+    from sharpnet_amd import GPUTensor
+    lib, d = w.lib, lib_desc(desc)
+    B, Tn, _ = x.shape
+    H, K, P = desc.hidden_size, desc.dirs, desc.pseudo_layers
+    ws, rs = ctypes.c_size_t(), ctypes.c_size_t()
+    check(lib.snhip_rnn_temp_space_sizes(ctypes.byref(d), int(training), B, Tn, ctypes.byref(ws), ctypes.byref(rs)), "sizes")
+    gws = GPUTensor([ws.value // 4], None, w)
+    grs = GPUTensor([max(rs.value // 4, 2)], None, w)
+    gws.SetValue(float("nan"))
+    grs.SetValue(float("nan"))
+    gx, gw = T(w, x), T(w, weights)
+    gy = GPUTensor([B, Tn, K * H], None, w)
+    ghy, gcy = GPUTensor([P, B, H], None, w), GPUTensor([P, B, H], None, w)
+    for t in (gy, ghy, gcy):
+        t.SetValue(float("nan"))
+    ghx = T(w, hx) if hx is not None else None
+    gcx = T(w, cx) if cx is not None else None
+    ptr = lambda t: t.Pointer if t is not None else None
+    check(lib.snhip_rnn_forward(w.handle, ctypes.byref(d), int(training), B, Tn, gx.Pointer, gy.Pointer, ptr(ghx), ghy.Pointer,
+                                ptr(gcx), gcy.Pointer, gw.Pointer, gws.Pointer, ws.value, grs.Pointer if training else None,
+                                rs.value), "snhip_rnn_forward")
+    out = {"y": gy.ToNumpy(), "hy": ghy.ToNumpy(), "cy": gcy.ToNumpy()}
+    if not training:
+        return out
+    gdy = T(w, dy)
+    gdx = GPUTensor(list(x.shape), None, w)
+    gdhx, gdcx = GPUTensor([P, B, H], None, w), GPUTensor([P, B, H], None, w)
+    for t in (gdx, gdhx, gdcx):
+        t.SetValue(float("nan"))
+    gdhy = T(w, dhy) if dhy is not None else None
+    gdcy = T(w, dcy) if dcy is not None else None
+    check(lib.snhip_rnn_backward_data(w.handle, ctypes.byref(d), B, Tn, gy.Pointer, gdy.Pointer, gdx.Pointer, ptr(ghx),
+                                      ptr(gdhy), gdhx.Pointer, ptr(gcx), ptr(gdcy), gdcx.Pointer, gw.Pointer, gws.Pointer,
+                                      ws.value, grs.Pointer, rs.value), "snhip_rnn_backward_data")
+    gdw = GPUTensor([weights.size], None, w)
+    gdw.ZeroMemory()
+    check(lib.snhip_rnn_backward_weights(w.handle, ctypes.byref(d), B, Tn, gx.Pointer, ptr(ghx), gy.Pointer, gdw.Pointer,
+                                         gws.Pointer, ws.value, grs.Pointer, rs.value), "snhip_rnn_backward_weights")
+    out.update(dx=gdx.ToNumpy(), dw=gdw.ToNumpy(), dhx=gdhx.ToNumpy(), dcx=gdcx.ToNumpy())
+    return out
+
+
+def compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, tol):
+    y, hy, cy, cache = ro.rnn_forward(desc, x, weights, hx, cx)
+    assert np.max(np.abs(got["y"] - y)) <= tol, "y"
+    assert np.max(np.abs(got["hy"] - hy)) <= tol, "hy"
+    if desc.cell == ro.LSTM:
+        assert np.max(np.abs(got["cy"] - cy)) <= tol, "cy"
+    if "dx" not in got:
+        return
+    dx, dw, dhx, dcx = ro.rnn_backward(desc, dy, cache, dhy, dcy if desc.cell == ro.LSTM else None)
+    scale = max(1.0, float(np.max(np.abs(dw))))
+    assert np.max(np.abs(got["dx"] - dx)) <= tol * max(1.0, float(np.max(np.abs(dx)))), "dx"
+    assert np.max(np.abs(got["dw"] - dw)) <= tol * scale, "dw"
+    assert np.max(np.abs(got["dhx"] - dhx)) <= tol * max(1.0, float(np.max(np.abs(dhx)))), "dhx"
+    if desc.cell == ro.LSTM:
+        assert np.max(np.abs(got["dcx"] - dcx)) <= tol * max(1.0, float(np.max(np.abs(dcx)))), "dcx"
+
+
+@pytest.mark.parametrize("cell", [ro.RELU, ro.TANH, ro.LSTM, ro.GRU])
+@pytest.mark.parametrize("bidirectional,layers", [(False, 1), (True, 1), (False, 2), (True, 2)])
+@pytest.mark.parametrize("bias_mode", [ro.DOUBLE_BIAS, ro.SINGLE_INP_BIAS, ro.SINGLE_REC_BIAS, ro.NO_BIAS])
+def test_cells_small(gpu_wrapper, cell, bidirectional, layers, bias_mode):
+    if bias_mode != ro.DOUBLE_BIAS and (layers, bidirectional) != (2, True):
+        pytest.skip("bias modes are checked on the largest arrangement only")
+    rng = np.random.default_rng(1000 + cell * 100 + layers * 10 + int(bidirectional) + bias_mode)
+    desc = ro.RnnDesc(cell, input_size=5, hidden_size=3, num_layers=layers, bidirectional=bidirectional, bias_mode=bias_mode)
+    B, Tn = 4, 6
+    weights = rng.uniform(-0.6, 0.6, ro.weight_space_size(desc)).astype(np.float32)
+    x = rng.uniform(-1, 1, (B, Tn, 5)).astype(np.float32)
+    dy = rng.uniform(-1, 1, (B, Tn, desc.dirs * 3)).astype(np.float32)
+    st = lambda: rng.uniform(-1, 1, (desc.pseudo_layers, B, 3)).astype(np.float32)
+    hx, cx, dhy, dcy = st(), st(), st(), st()
+    if cell != ro.LSTM:
+        cx = dcy = None
+    got = run_gpu(gpu_wrapper, desc, x, weights, dy)
+    compare(desc, got, x, weights, dy, None, None, None, None, 2e-5)
+    got = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy)
+    compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, 2e-5)
+
+
+@pytest.mark.parametrize("cell", [ro.TANH, ro.LSTM, ro.GRU])
+def test_cells_wider(gpu_wrapper, cell):
+    """Sizes at which the GEMMs use full tiles, split-K and the fused column sums; odd batch and widths."""
+    rng = np.random.default_rng(50 + cell)
+    desc = ro.RnnDesc(cell, input_size=45, hidden_size=68, num_layers=2, bidirectional=True, bias_mode=ro.DOUBLE_BIAS)
+    B, Tn = 33, 17
+    weights = rng.uniform(-0.12, 0.12, ro.weight_space_size(desc)).astype(np.float32)
+    x = rng.uniform(-1, 1, (B, Tn, 45)).astype(np.float32)
+    dy = rng.uniform(-1, 1, (B, Tn, 2 * 68)).astype(np.float32)
+    got = run_gpu(gpu_wrapper, desc, x, weights, dy)
+    compare(desc, got, x, weights, dy, None, None, None, None, 1e-4)
+
+
+@pytest.mark.parametrize("cell", [ro.RELU, ro.LSTM, ro.GRU])
+def test_inference_equals_training_forward(gpu_wrapper, cell):
+    rng = np.random.default_rng(7 + cell)
+    desc = ro.RnnDesc(cell, input_size=9, hidden_size=16, num_layers=2, bidirectional=True, bias_mode=ro.SINGLE_INP_BIAS)
+    weights = rng.uniform(-0.3, 0.3, ro.weight_space_size(desc)).astype(np.float32)
+    x = rng.uniform(-1, 1, (6, 5, 9)).astype(np.float32)
+    a = run_gpu(gpu_wrapper, desc, x, weights, None, training=False)
+    b = run_gpu(gpu_wrapper, desc, x, weights, np.zeros((6, 5, 32), np.float32), training=True)
+    assert np.array_equal(a["y"], b["y"]) and np.array_equal(a["hy"], b["hy"])
+
+
+def test_weight_params_match_oracle_layout(gpu_wrapper):
+    lib = gpu_wrapper.lib
+    for cell in (ro.RELU, ro.TANH, ro.LSTM, ro.GRU):
+        for mode in (ro.NO_BIAS, ro.SINGLE_INP_BIAS, ro.DOUBLE_BIAS, ro.SINGLE_REC_BIAS):
+            desc = ro.RnnDesc(cell, 7, 5, num_layers=3, bidirectional=True, bias_mode=mode)
+            d = lib_desc(desc)
+            nbytes = ctypes.c_size_t()
+            check(lib.snhip_rnn_weight_space_size(ctypes.byref(d), ctypes.byref(nbytes)), "size")
+            assert nbytes.value == 4 * ro.weight_space_size(desc)
+            for p in range(desc.pseudo_layers):
+                for lin in range(desc.lin_layer_ids):
+                    off, rows, cols, boff = ctypes.c_longlong(), ctypes.c_int(), ctypes.c_int(), ctypes.c_longlong()
+                    check(lib.snhip_rnn_weight_params(ctypes.byref(d), p, lin, ctypes.byref(off), ctypes.byref(rows),
+                                                      ctypes.byref(cols), ctypes.byref(boff)), "params")
+                    o, (r, c), b = ro.weight_params(desc, p, lin)
+                    assert (off.value, rows.value, cols.value, boff.value) == (o, r, c, -1 if b is None else b)
+
+
+def test_simple_rnn_training_losses_on_device(golden, gpu_wrapper):
+    """Tests/NonReg/ParallelRunWithPyTorch.cs:896-953 with both layers run by the RecurrentLayer mirror: the stored
+    losses before and after 10 epochs (the reference's tolerance 1e-6 is for cuDNN against PyTorch; 2e-6 here)."""
+    from sharpnet_amd import GPUTensor, recurrent
+    fx = golden["PyTorch_SimpleRNN"]
+    layers = {}
+
+    def layer_for(desc, return_sequences):
+        key = (desc.input_size, desc.num_layers, return_sequences)
+        if key not in layers:
+            layers[key] = recurrent.RecurrentLayer(gpu_wrapper, desc.input_size, desc.hidden_size, desc.cell, desc.bias_mode,
+                                                   return_sequences, desc.bidirectional, desc.num_layers)
+        return layers[key]
+
+    def forward(desc, x, weights, return_sequences):
+        layer = layer_for(desc, return_sequences)
+        layer._weightsAndBiases.InitializeFromHostMemory(weights)
+        gx = T(gpu_wrapper, x)
+        gy = GPUTensor(layer.OutputShape(x.shape[0], x.shape[1]), None, gpu_wrapper)
+        layer.ForwardPropagation(gx, gy, True)
+        return gy.ToNumpy(), (layer, gx, gy)
+
+    def backward(desc, dy, cache):
+        layer, gx, gy = cache
+        gdx = GPUTensor(gx.Shape, None, gpu_wrapper)
+        layer.BackwardPropagation(gx, gy, T(gpu_wrapper, dy), gdx)
+        return gdx.ToNumpy(), layer._weightsAndBiasesGradients.ToNumpy()
+
+    before, after = simple_rnn_chain(fx, forward, backward)
+    assert abs(before - fx["loss_before"]) < 2e-6, (before, fx["loss_before"])
+    assert abs(after - fx["loss_after"]) < 2e-6, (after, fx["loss_after"])
+
+
+def test_rnn_argument_checks(gpu_wrapper):
+    from sharpnet_amd.hiplib import CublasStatus, RnnDesc
+    lib = gpu_wrapper.lib
+    d = RnnDesc(cell_mode=2, bias_mode=2, bidirectional=0, num_layers=1, input_size=4, hidden_size=4)
+    ws, rs = ctypes.c_size_t(), ctypes.c_size_t()
+    check(lib.snhip_rnn_temp_space_sizes(ctypes.byref(d), 1, 2, 3, ctypes.byref(ws), ctypes.byref(rs)), "sizes")
+    x = T(gpu_wrapper, np.zeros((2, 3, 4)))
+    y = T(gpu_wrapper, np.zeros((2, 3, 4)))
+    wt = T(gpu_wrapper, np.zeros(4 * 4 * 8 + 32))
+    buf = T(gpu_wrapper, np.zeros(max(ws.value, rs.value) // 4))
+    # a reserve buffer that is too small is refused before anything is launched
+    st = lib.snhip_rnn_forward(gpu_wrapper.handle, ctypes.byref(d), 1, 2, 3, x.Pointer, y.Pointer, None, None, None, None,
+                               wt.Pointer, buf.Pointer, ws.value, buf.Pointer, rs.value - 4)
+    assert st == CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    bad = RnnDesc(cell_mode=4, bias_mode=2, bidirectional=0, num_layers=1, input_size=4, hidden_size=4)
+    assert lib.snhip_rnn_temp_space_sizes(ctypes.byref(bad), 1, 2, 3, ctypes.byref(ws), ctypes.byref(rs)) == \
+        CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    # empty problems are no-ops
+    check(lib.snhip_rnn_forward(gpu_wrapper.handle, ctypes.byref(d), 1, 0, 3, None, None, None, None, None, None, None,
+                                None, 0, None, 0), "empty batch")
