@@ -416,6 +416,36 @@ def layer_timings(w, wl):
                     "form": ("heads in place, attention kernels" if fused_attn else "heads in place") if in_place
                     else "reference sequence (transposition copies)",
                     "forward_ms": f, "backward_ms": round(fb - f, 4)})
+    for t in (Q, K, V, dy, wq, wk, wv, wo, y, dQ, dK, dV) + tuple(g[0] for g in grads.values()):
+        t.Dispose()
+    # recurrent layers at the shape of benchmark configuration 4: batch 256, 128 steps, 256 inputs, 512 hidden units
+    from sharpnet_amd import recurrent
+    B, Tn, I, H = 256, 128, 256, 512
+    x, dyr = T((B, Tn, I)), T((B, Tn, H), -0.01, 0.01)
+    yr, dxr = GPUTensor([B, Tn, H], None, w), GPUTensor([B, Tn, I], None, w)
+    for name, cell, bias in (("LSTM", recurrent.CUDNN_LSTM, recurrent.CUDNN_RNN_SINGLE_INP_BIAS),
+                             ("GRU", recurrent.CUDNN_GRU, recurrent.CUDNN_RNN_DOUBLE_BIAS)):
+        layer = recurrent.RecurrentLayer(w, I, H, cell, bias, True, False, 1)
+        layer._weightsAndBiases.InitializeFromHostMemory(
+            rng.uniform(-0.04, 0.04, layer._weightsAndBiases.Count).astype(np.float32))
+
+        def rnn_f():
+            layer.ForwardPropagation(x, yr, True)
+            layer._reserveSpace.Dispose()
+
+        def rnn_fb():
+            layer.ForwardPropagation(x, yr, True)
+            layer.BackwardPropagation(x, yr, dyr, dxr)
+        f = timed(rnn_f, 3, 1)
+        fb = timed(rnn_fb, 3, 1)
+        gates = 4 if name == "LSTM" else 3
+        flop = 2.0 * B * Tn * gates * H * (I + H)
+        res.append({"layer": "%s batch %d, %d steps, %d -> %d (forward %.1f GFLOP: %d sequential steps of %dx%dx%d)" %
+                             (name, B, Tn, I, H, flop / 1e9, Tn, B, gates * H, H),
+                    "form": "one GEMM + one cell kernel per step", "forward_ms": f, "backward_ms": round(fb - f, 4)})
+        layer.Dispose()
+    for t in (x, dyr, yr, dxr):
+        t.Dispose()
     w.use_memory_pool(False)
     return res
 

@@ -29,22 +29,47 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// out[z][c] = sum over rows of x[z][r][c] (row pitch ld, matrix z at x + z * stride; blockIdx.y = z).  A workgroup
-// of 4 wavefronts owns 64 columns; wavefront w adds rows w, w+4, ... (lanes along columns, 256-byte coalesced
-// reads), the four partial sums meet in LDS in a fixed order.
+// out[z][k][c] = sum of x[z][r][c] over the rows r of chunk k (row pitch ld, matrix z at x + z * stride;
+// blockIdx.y = z, blockIdx.z = k, chunks of rows_per_chunk rows).  A workgroup of 4 wavefronts owns 64 columns of
+// one chunk; wavefront w adds rows w, w+4, ... of it (lanes along columns, 256-byte coalesced reads, four rows in
+// flight per wavefront), the four partial sums meet in LDS in a fixed order.  With one chunk this is the whole
+// column sum; a tall matrix is cut into chunks so that the launch fills the chip, and column_sum_finish_kernel
+// adds the chunks in index order (deterministic, no float atomics).
 __global__ void __launch_bounds__(256) column_sum_kernel(const float* __restrict__ x, float* __restrict__ out, int rows,
-                                                         int cols, long long ld, long long stride) {
+                                                         int cols, long long ld, long long stride, int rows_per_chunk) {
     __shared__ float part[4][64];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int c = blockIdx.x * 64 + lane;
     const float* xz = x + (long long)blockIdx.y * stride;
-    float s = 0.0f;
-    if (c < cols)
-        for (int r = w; r < rows; r += 4) s += xz[(long long)r * ld + c];
-    part[w][lane] = s;
+    const int r0 = blockIdx.z * rows_per_chunk;
+    const int r1 = (r0 + rows_per_chunk < rows) ? r0 + rows_per_chunk : rows;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    if (c < cols) {
+        int r = r0 + w;
+        for (; r + 12 < r1; r += 16) {
+            s0 += xz[(long long)r * ld + c];
+            s1 += xz[(long long)(r + 4) * ld + c];
+            s2 += xz[(long long)(r + 8) * ld + c];
+            s3 += xz[(long long)(r + 12) * ld + c];
+        }
+        for (; r < r1; r += 4) s0 += xz[(long long)r * ld + c];
+    }
+    part[w][lane] = (s0 + s1) + (s2 + s3);
     __syncthreads();
     if (w == 0 && c < cols)
-        out[(long long)blockIdx.y * cols + c] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+        out[((long long)blockIdx.y * gridDim.z + blockIdx.z) * cols + c] =
+            (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+}
+
+// out[z][c] = partial[z][0][c] + partial[z][1][c] + ... in index order.
+__global__ void __launch_bounds__(256) column_sum_finish_kernel(const float* __restrict__ partial, float* __restrict__ out,
+                                                                int chunks, int cols, int nz) {
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long long)nz * cols) return;
+    const int z = (int)(idx / cols), c = (int)(idx % cols);
+    float s = 0.0f;
+    for (int k = 0; k < chunks; ++k) s += partial[((long long)z * chunks + k) * cols + c];
+    out[idx] = s;
 }
 
 // dst[i] = value for count 32-bit words (a kernel rather than a memset node, so that a caller may record it into a

@@ -254,6 +254,35 @@ int ensure_workspace(Handle* h, size_t bytes) {
     return SNHIP_STATUS_SUCCESS;
 }
 
+// out[z][c] = sum_r x[z][r][c] for nz matrices of rows x cols (row pitch ld, `stride` floats apart).  A matrix too
+// tall for cols / 64 workgroups to fill the chip is summed in row chunks through the handle's workspace.
+int launch_column_sum(Handle* h, const float* x, float* out, int rows, int cols, long long ld, long long stride, int nz) {
+    const int col_blocks = (cols + 63) / 64;
+    const long long base = (long long)col_blocks * nz;
+    int chunks = 1;
+    if (rows >= 512 && base < 2LL * h->num_cu) {
+        chunks = (int)((4LL * h->num_cu + base - 1) / base);
+        if (chunks > rows / 128) chunks = rows / 128;  // at least 128 rows per chunk
+        if (chunks > 4096) chunks = 4096;
+    }
+    const int rows_per_chunk = chunks > 1 ? ceil_div(rows, chunks) : (rows > 0 ? rows : 1);
+    chunks = rows > 0 ? ceil_div(rows, rows_per_chunk) : 1;
+    float* dst = out;
+    if (chunks > 1) {
+        const int st = ensure_workspace(h, (size_t)chunks * nz * cols * sizeof(float));
+        if (st != SNHIP_STATUS_SUCCESS) return st;
+        dst = h->ws;
+    }
+    hipLaunchKernelGGL(column_sum_kernel, dim3(col_blocks, nz, chunks), dim3(256), 0, h->stream, x, dst, rows, cols, ld,
+                       stride, rows_per_chunk);
+    if (chunks > 1) {
+        const long long total = (long long)nz * cols;
+        hipLaunchKernelGGL(column_sum_finish_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, h->stream,
+                           (const float*)h->ws, out, chunks, cols, nz);
+    }
+    return hip_to_status(hipGetLastError());
+}
+
 // The last-arriving workgroup can add the split-K partial sums itself (splitk_mode 2), which saves the
 // second launch.  Measured on MI355X it is slower than the second kernel for every shape tried
 // (8192x64x8192 split 4: 171 us against 87 us; 128x256x784 split 4: 21.7 us against 12.9 us): each
@@ -377,11 +406,11 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     auto standalone_colsum = [&]() -> int {
         if (K > 0 && g.A == nullptr) return SNHIP_STATUS_INVALID_VALUE;
         for (int zo = 0; zo < batch / inner; ++zo) {
-            hipLaunchKernelGGL(column_sum_kernel, dim3((M + 63) / 64, inner), dim3(256), 0, h->stream,
-                               g.A + (long long)zo * g.sA2, g.colsum + (long long)zo * inner * M, K, M,
-                               (long long)g.lda, g.sA);
+            const int st = launch_column_sum(h, g.A + (long long)zo * g.sA2, g.colsum + (long long)zo * inner * M, K, M,
+                                             (long long)g.lda, g.sA, inner);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
         }
-        return hip_to_status(hipGetLastError());
+        return SNHIP_STATUS_SUCCESS;
     };
     if (K == 0 || g.alpha == 0.0f) {
         // BLAS semantics: A and B are not referenced by the product, C = beta * C (then the rest of the epilogue).
@@ -924,9 +953,7 @@ int snhip_bias_gradient(void* handle, const float* dy, int rows, int cols, float
     if (rows < 0 || cols < 0) return SNHIP_STATUS_INVALID_VALUE;
     if (cols == 0) return SNHIP_STATUS_SUCCESS;
     if (bias_gradient == nullptr || (rows > 0 && dy == nullptr)) return SNHIP_STATUS_INVALID_VALUE;
-    hipLaunchKernelGGL(column_sum_kernel, dim3((cols + 63) / 64), dim3(256), 0, static_cast<Handle*>(handle)->stream, dy,
-                       bias_gradient, rows, cols, (long long)cols, 0LL);
-    return hip_to_status(hipGetLastError());
+    return launch_column_sum(static_cast<Handle*>(handle), dy, bias_gradient, rows, cols, (long long)cols, 0LL, 1);
 }
 
 int snhip_activation_forward(void* handle, int activation, float activation_param, const float* x, float* y,

@@ -530,3 +530,16 @@ def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, pack
     assert np.max(np.abs(gdv.ToNumpy() - lay(dv_ref, Tk, dv))) <= tol
     assert np.max(np.abs(gdq.ToNumpy() - lay(dq_ref, Tq, dk))) <= tol
     assert np.max(np.abs(gdk.ToNumpy() - lay(dk_ref, Tk, dk))) <= tol
+
+
+@pytest.mark.parametrize("rows,cols", [(33333, 130), (512, 64), (511, 3), (100000, 1), (4096, 4096)])
+def test_bias_gradient_tall_matrices(gpu_wrapper, rows, cols):
+    """Column sums of matrices much taller than wide are cut into row chunks (two kernels); same result as one pass."""
+    from sharpnet_amd import GPUTensor
+    rng = np.random.default_rng(rows + cols)
+    dy = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
+    g = GPUTensor([cols], None, gpu_wrapper)
+    g.SetValue(float("nan"))
+    T(gpu_wrapper, dy).Compute_BiasGradient_from_dy(g)
+    ref = dy.astype(np.float64).sum(axis=0)
+    assert np.max(np.abs(g.ToNumpy() - ref)) <= 1e-5 * np.sqrt(rows) + 1e-6 * rows ** 0.5
