@@ -436,13 +436,17 @@ def layer_timings(w, wl):
         def rnn_fb():
             layer.ForwardPropagation(x, yr, True)
             layer.BackwardPropagation(x, yr, dyr, dxr)
-        f = timed(rnn_f, 3, 1)
-        fb = timed(rnn_fb, 3, 1)
         gates = 4 if name == "LSTM" else 3
         flop = 2.0 * B * Tn * gates * H * (I + H)
-        res.append({"layer": "%s batch %d, %d steps, %d -> %d (forward %.1f GFLOP: %d sequential steps of %dx%dx%d)" %
-                             (name, B, Tn, I, H, flop / 1e9, Tn, B, gates * H, H),
-                    "form": "one GEMM + one cell kernel per step", "forward_ms": f, "backward_ms": round(fb - f, 4)})
+        for form, cfg in (("forward: one launch per step (product + cell)", -1),
+                          ("forward: GEMM + cell kernel per step", 6)):
+            w.set_tuning(cfg, 1 if cfg >= 0 else 0)     # a forced GEMM configuration selects the two-launch form
+            f = timed(rnn_f, 3, 1)
+            fb = timed(rnn_fb, 3, 1)
+            w.set_tuning(-1, 0)
+            res.append({"layer": "%s batch %d, %d steps, %d -> %d (forward %.1f GFLOP: %d sequential steps of %dx%dx%d)" %
+                                 (name, B, Tn, I, H, flop / 1e9, Tn, B, gates * H, H),
+                        "form": form, "forward_ms": f, "backward_ms": round(fb - f, 4)})
         layer.Dispose()
     for t in (x, dyr, yr, dxr):
         t.Dispose()

@@ -15,6 +15,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include "sgemm_mfma.hpp"
+
 namespace snhip {
 
 enum : int { RNN_RELU = 0, RNN_TANH = 1, RNN_LSTM = 2, RNN_GRU = 3 };
@@ -71,6 +73,206 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd_kernel(const RnnStepFwd s) {
     s.y[b * s.ld_y + j] = h;
     if (s.h_next) s.h_next[b * s.ld_hnext + j] = h;
     if (s.hy) s.hy[(long long)b * H + j] = h;
+}
+
+// One forward time step in one launch: the product h[t-1] . R^T and the cell arithmetic.
+//
+// The step's GEMM (batch x G*H x H, e.g. 256 x 2048 x 512) is far too small to fill the chip with 64 x 64 tiles -
+// it is bound by the length of one wavefront's chain of MFMAs, not by the MFMA rate.  This kernel cuts it so that
+// every SIMD of the chip gets one short chain: a workgroup owns 32 samples x U hidden units x all G gates
+// (U = 16; 32 for the single-gate cells), i.e. one or two 32 x 32 MFMA tiles whose 32 columns are gathered from
+// the gates' row blocks of R, and splits K (the hidden dimension) over its wavefronts: four wavefronts =
+// (tiles) x (K slices).  Each wavefront is on its own in the main loop: per group of 32 k values it reads its
+// 32 x 32 pieces of h[t-1] and R with whole-line loads (a lane takes 16 bytes, eight lanes one 128-byte row piece),
+// DEPTH groups in flight in registers, passes a group through a private LDS patch to turn it into MFMA operand
+// layout (row = lane % 32, sixteen consecutive k per half-wave), and multiplies - no workgroup barrier until the
+// partial tiles meet in LDS, where each thread picks up all gates of its (sample, unit) pairs, adds W x + bW from
+// the gates buffer and finishes the cell exactly as rnn_cell_fwd_kernel does.
+// Requires H % 32 == 0 and 16-byte aligned rows; the caller falls back to GEMM + cell kernel otherwise.
+template <int G>
+struct RnnFusedCfg {
+    static constexpr int U = (G == 1) ? 32 : 16;       // hidden units per workgroup
+    static constexpr int COLS = G * U;                 // columns of the workgroup's tile: [gate][unit]
+    static constexpr int NT = (COLS + 31) / 32;        // 32-column MFMA tiles
+    static constexpr int KS = 4 / NT;                  // K slices
+    static constexpr int DEPTH = 4;                    // groups of 32 k values in flight per wavefront
+    static constexpr int PITCH = 36;                   // floats per row of an LDS patch (32 + 4: conflict-free b128)
+};
+
+template <int G>
+__global__ void __launch_bounds__(256) rnn_step_fused_kernel(const RnnStepFwd s, const float* __restrict__ R) {
+    using C = RnnFusedCfg<G>;
+    constexpr int U = C::U, NT = C::NT, KS = C::KS, D = C::DEPTH, P = C::PITCH;
+    __shared__ float part[KS][NT][32][33];
+    __shared__ __attribute__((aligned(16))) float patch[4][2][32 * P];   // per wavefront: h rows, R rows
+    const int H = s.hidden;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int nt = wave % NT, kg = wave / NT;
+    // unit blocks along x: workgroups are dealt to the eight XCDs by their linear index, so the (few) workgroups that
+    // share a slice of R land on one XCD and find it in that XCD's L2
+    const int row0 = blockIdx.y * 32, u0 = blockIdx.x * U;
+
+    // global side: instruction i of a group fetches rows 8 i + lane / 8, floats 4 (lane % 8) .. + 3
+    const int lrow = lane >> 3, lcol = (lane & 7) * 4;
+    const float* ap[4];
+    const float* bp[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ar = (row0 + 8 * i + lrow < s.batch) ? row0 + 8 * i + lrow : s.batch - 1;
+        ap[i] = s.h_prev + (long long)ar * s.ld_hprev + lcol;
+        const int col = nt * 32 + 8 * i + lrow;                 // column of the workgroup's tile -> row of R
+        const int gate = col / U, unit = u0 + col % U;
+        bp[i] = R + (long long)((col < C::COLS && unit < H) ? gate * H + unit : 0) * H + lcol;
+    }
+    float* pa = &patch[wave][0][0];
+    float* pb = &patch[wave][1][0];
+
+    const int groups = H / 32;                                   // groups of 32 k values
+    const int per = (groups + KS - 1) / KS;
+    const int mbeg = kg * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
+
+    // what the cell arithmetic at the end reads from global memory is fetched now, behind the main loop:
+    // thread -> pairs p = threadIdx.x + 256 q of the tile's 32 x U (sample, unit) pairs
+    constexpr int Q = 32 * U / 256;
+    float gxv[Q][G], brv[Q][G], cpv[Q], hpv[Q];
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+        const int p = threadIdx.x + 256 * q;
+        const int b = row0 + p / U, j = u0 + p % U;
+        const bool ok = b < s.batch && j < H;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            gxv[q][g] = ok ? s.gates[b * s.ld_gates + g * H + j] : 0.0f;
+            brv[q][g] = (ok && s.bias_r) ? s.bias_r[g * H + j] : 0.0f;
+        }
+        cpv[q] = (G == 4 && ok && s.c_prev) ? s.c_prev[b * s.ld_cprev + j] : 0.0f;
+        hpv[q] = (G == 3 && ok) ? s.h_prev[b * s.ld_hprev + j] : 0.0f;
+    }
+
+    f32x4 ra[D][4], rb[D][4];
+    f32x16 acc[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[e][r] = 0.0f;
+
+    auto load = [&](int slot, int m) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            ra[slot][i] = *reinterpret_cast<const f32x4*>(ap[i] + m * 32);
+            rb[slot][i] = *reinterpret_cast<const f32x4*>(bp[i] + m * 32);
+        }
+    };
+    // stage(slot, f): a group goes from the registers it was loaded into, through the wavefront's LDS patch, into
+    // operand layout in fragment buffer f.  The wavefront's lanes exchange data through the patch: the fences keep
+    // the compiler from moving LDS accesses across these points (the hardware runs one wavefront's LDS
+    // instructions in order, so a patch can be rewritten as soon as the reads of the previous group are issued).
+    f32x4 fa[2][4], fb[2][4];
+    auto stage = [&](int slot, int f) {
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<f32x4*>(pa + (8 * i + lrow) * P + lcol) = ra[slot][i];
+            *reinterpret_cast<f32x4*>(pb + (8 * i + lrow) * P + lcol) = rb[slot][i];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            fa[f][j] = *reinterpret_cast<const f32x4*>(pa + l32 * P + 16 * lhi + 4 * j);
+            fb[f][j] = *reinterpret_cast<const f32x4*>(pb + l32 * P + 16 * lhi + 4 * j);
+        }
+    };
+    auto multiply = [&](int f) {
+        // element e of vector j is k = 32 m + 16 lhi + 4 j + e for both operands; four independent chains
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                acc[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[f][j][e], fb[f][j][e], acc[e], 0, 0, 0);
+    };
+
+    // Whole blocks of D groups run without a branch between a load and its use, so that the compiler can wait for
+    // exactly the group it needs (s_waitcnt vmcnt(N)) while the later ones are still in flight; the LDS round trip
+    // of group i + 1 is issued before the MFMAs of group i (D is even: fragment buffer = slot % 2).
+    const int cnt = mend > mbeg ? mend - mbeg : 0;
+    const int mmain = mbeg + (cnt / D) * D;
+    int m = mbeg;
+    if (m < mmain) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) load(d, m + d);
+        stage(0, 0);
+        for (; m + D < mmain; m += D) {
+            load(0, m + D);
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                stage((d + 1) % D, (d + 1) % 2);       // d == D - 1: slot 0 already holds group m + D
+                if (d + 1 < D) load(d + 1, m + d + 1 + D);
+                multiply(d % 2);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if (d + 1 < D) stage(d + 1, (d + 1) % 2);
+            multiply(d % 2);
+        }
+    }
+    // fewer than D groups left: all loads first, then the products
+#pragma unroll
+    for (int d = 0; d < D - 1; ++d)
+        if (mmain + d < mend) load(d, mmain + d);
+#pragma unroll
+    for (int d = 0; d < D - 1; ++d)
+        if (mmain + d < mend) {
+            stage(d, 0);
+            multiply(0);
+        }
+    // accumulator register r holds row 8 (r / 4) + 4 lhi + r % 4, column l32 of the 32 x 32 tile
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        part[kg][nt][8 * (r / 4) + 4 * lhi + (r % 4)][l32] = (acc[0][r] + acc[1][r]) + (acc[2][r] + acc[3][r]);
+    __syncthreads();
+
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+        const int p = threadIdx.x + 256 * q;
+        const int lr = p / U, b = row0 + lr, j = u0 + p % U;
+        if (b >= s.batch || j >= H) continue;
+        float gh[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int c = g * U + p % U;
+            float v = 0.0f;
+#pragma unroll
+            for (int k = 0; k < KS; ++k) v += part[k][c / 32][lr][c % 32];
+            gh[g] = v + brv[q][g];
+        }
+        float* gx = s.gates + b * s.ld_gates;
+        float h;
+        if constexpr (G == 1) {
+            const float pre = gxv[q][0] + gh[0];
+            h = (s.cell == RNN_RELU) ? (pre < 0.0f ? 0.0f : pre) : tanhf(pre);
+        } else if constexpr (G == 4) {
+            const float i = sigmoidf_(gxv[q][0] + gh[0]), f = sigmoidf_(gxv[q][1] + gh[1]);
+            const float gg = tanhf(gxv[q][2] + gh[2]), o = sigmoidf_(gxv[q][3] + gh[3]);
+            const float c = f * cpv[q] + i * gg;
+            gx[j] = i, gx[H + j] = f, gx[2 * H + j] = gg, gx[3 * H + j] = o;
+            s.c_out[b * s.ld_c + j] = c;
+            if (s.cy) s.cy[(long long)b * H + j] = c;
+            h = o * tanhf(c);
+        } else {
+            const float r = sigmoidf_(gxv[q][0] + gh[0]), z = sigmoidf_(gxv[q][1] + gh[1]);
+            const float qn = gh[2];
+            const float n = tanhf(gxv[q][2] + r * qn);
+            gx[j] = r, gx[H + j] = z, gx[2 * H + j] = n;
+            s.gh[b * s.ld_gh + 2 * H + j] = qn;
+            h = (1.0f - z) * n + z * hpv[q];
+        }
+        s.y[b * s.ld_y + j] = h;
+        if (s.h_next) s.h_next[b * s.ld_hnext + j] = h;
+        if (s.hy) s.hy[(long long)b * H + j] = h;
+    }
 }
 
 struct RnnStepBwd {

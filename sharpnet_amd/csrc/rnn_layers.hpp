@@ -11,6 +11,10 @@
 //   weights    dW += d(gates)^T . X, dR += d(gates_h)^T . Hprev, bias gradients = column sums     two GEMMs
 // Hprev (n x H) holds, for every (sample, step), the state that entered the step, so the recurrent weight gradient
 // is a single product over all steps.
+// Everything the library keeps between the calls is stored step-major ((steps, batch, width)): the rows of one
+// time step are contiguous, whereas in the caller's batch-major tensors they lie steps * width floats apart - a
+// power-of-two pitch of hundreds of KB that sends every row of a step to the same memory channel.  x is copied
+// into that order once per forward call; y, dy and dx are read and written in place through their row pitch.
 #pragma once
 #include "rnn_cells.hpp"
 
@@ -24,6 +28,7 @@ struct RnnDims {
     long long per_p;                  // floats of one pseudo-layer's region
     long long gates_off, hprev_off, cells_off, gh_off;   // inside a pseudo-layer's region
     long long out_off;                // start of the stacked layers' outputs, after all regions
+    long long xt_off;                 // step-major copy of x
     long long total;                  // floats carried from forward to backward
     long long bwd_ws;                 // floats of scratch the backward calls need
 };
@@ -59,7 +64,8 @@ RnnDims rnn_dims(const snhip_rnn_desc* d, int batch, int steps) {
     r.gh_off = r.cells_off + (r.cell == RNN_LSTM ? r.n * r.H : 0);
     r.per_p = r.gh_off + (r.cell == RNN_GRU ? r.n * 3 * r.H : 0);
     r.out_off = r.per_p * r.P;
-    r.total = r.out_off + (long long)(r.L - 1) * r.n * r.K * r.H;
+    r.xt_off = r.out_off + (long long)(r.L - 1) * r.n * r.K * r.H;
+    r.total = r.xt_off + r.n * r.I;
     // dh, dc, one bias gradient, and two buffers for the gradients that travel between stacked layers
     r.bwd_ws = 2LL * batch * r.H + (long long)r.G * r.H + (r.L > 1 ? 2 * r.n * r.K * r.H : 0);
     return r;
@@ -188,11 +194,18 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
     const size_t keep_bytes = training ? reserve_bytes : workspace_bytes;
     if (keep == nullptr || keep_bytes < (size_t)r.total * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
     const int B = batch, T = steps, H = r.H, G = r.G, K = r.K;
-    const long long GH = (long long)G * H;
+    const long long GH = (long long)G * H, KH = (long long)K * H;
+
+    // (batch, steps, inputs) -> (steps, batch, inputs)
+    st = snhip_transpose_second_and_third_dimension(handle, x, keep + r.xt_off, 1, B, T, r.I);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
 
     for (int layer = 0; layer < r.L; ++layer) {
-        const float* inp = layer == 0 ? x : keep + r.out_off + (long long)(layer - 1) * r.n * K * H;
-        float* out = layer == r.L - 1 ? y : keep + r.out_off + (long long)layer * r.n * K * H;
+        const float* inp = layer == 0 ? keep + r.xt_off : keep + r.out_off + (long long)(layer - 1) * r.n * KH;
+        const bool top = layer == r.L - 1;
+        float* out = top ? y : keep + r.out_off + (long long)layer * r.n * KH;
+        // rows of step t: the caller's y is batch-major, the stacked layers' outputs are step-major
+        const long long out_step = top ? KH : (long long)B * KH, out_ld = top ? (long long)T * KH : KH;
         const long long I = rnn_layer_inputs(r, layer);
         for (int d = 0; d < K; ++d) {
             const int p = layer * K + d;
@@ -214,44 +227,54 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
             if (st != SNHIP_STATUS_SUCCESS) return st;
 
             const int first = d == 0 ? 0 : T - 1, dir = d == 0 ? 1 : -1;
-            st = rnn_set_rows(h, hprev + (long long)first * H, (long long)T * H, hx_p, H, B, H);
+            st = rnn_set_rows(h, hprev + (long long)first * B * H, H, hx_p, H, B, H);
             if (st != SNHIP_STATUS_SUCCESS) return st;
+            // product and cell in one launch per step when the rows can be read in 16-byte pieces; a forced GEMM
+            // configuration (tuning hook) selects the two-launch form
+            const bool fused = H % 32 == 0 && (uintptr_t)hprev % 16 == 0 && (uintptr_t)w.R % 16 == 0 && h->force_cfg < 0;
             for (int k = 0; k < T; ++k) {
                 const int t = first + dir * k;
                 const bool last = k == T - 1;
                 const bool zero_state = k == 0 && hx_p == nullptr;
-                if (r.cell == RNN_GRU || !zero_state) {
+                if (!fused && (r.cell == RNN_GRU || !zero_state)) {
                     GemmArgs s;  // h[t-1] . R^T
                     s.tB = true;
                     s.M = B, s.N = (int)GH, s.K = H;
-                    s.A = hprev + (long long)t * H, s.lda = T * H;
+                    s.A = hprev + (long long)t * B * H, s.lda = H;
                     s.B = w.R, s.ldb = H;
                     if (r.cell == RNN_GRU) {
-                        s.C = gh + (long long)t * 3 * H, s.ldc = T * 3 * H;
+                        s.C = gh + (long long)t * B * 3 * H, s.ldc = 3 * H;
                     } else {
-                        s.C = gates + (long long)t * GH, s.ldc = (int)(T * GH), s.beta = 1.0f;
+                        s.C = gates + (long long)t * B * GH, s.ldc = (int)GH, s.beta = 1.0f;
                     }
                     st = gemm_core(h, s);
                     if (st != SNHIP_STATUS_SUCCESS) return st;
                 }
                 RnnStepFwd c;
-                c.gates = gates + (long long)t * GH, c.ld_gates = T * GH;
-                c.gh = gh + (long long)t * 3 * H, c.ld_gh = (long long)T * 3 * H;
+                c.gates = gates + (long long)t * B * GH, c.ld_gates = GH;
+                c.gh = gh + (long long)t * B * 3 * H, c.ld_gh = 3LL * H;
                 c.bias_r = w.bR;
-                c.h_prev = hprev + (long long)t * H, c.ld_hprev = (long long)T * H;
-                if (k == 0) {
-                    c.c_prev = cx_p, c.ld_cprev = H;
-                } else {
-                    c.c_prev = cells + (long long)(t - dir) * H, c.ld_cprev = (long long)T * H;
-                }
-                c.c_out = cells + (long long)t * H, c.ld_c = (long long)T * H;
-                c.y = out + (long long)t * K * H + (long long)d * H, c.ld_y = (long long)T * K * H;
-                c.h_next = last ? nullptr : hprev + (long long)(t + dir) * H, c.ld_hnext = (long long)T * H;
+                c.h_prev = hprev + (long long)t * B * H, c.ld_hprev = H;
+                c.c_prev = k == 0 ? cx_p : cells + (long long)(t - dir) * B * H, c.ld_cprev = H;
+                c.c_out = cells + (long long)t * B * H, c.ld_c = H;
+                c.y = out + (long long)t * out_step + (long long)d * H, c.ld_y = out_ld;
+                c.h_next = last ? nullptr : hprev + (long long)(t + dir) * B * H, c.ld_hnext = H;
                 c.hy = (last && hy) ? hy + (long long)p * B * H : nullptr;
                 c.cy = (last && cy && r.cell == RNN_LSTM) ? cy + (long long)p * B * H : nullptr;
                 c.batch = B, c.hidden = H, c.cell = r.cell;
-                hipLaunchKernelGGL(rnn_cell_fwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
-                                   h->stream, c);
+                if (fused) {
+                    const int U = G == 1 ? 32 : 16;
+                    const dim3 grid((unsigned)((H + U - 1) / U), (unsigned)((B + 31) / 32));
+                    if (G == 4)
+                        hipLaunchKernelGGL(rnn_step_fused_kernel<4>, grid, dim3(256), 0, h->stream, c, (const float*)w.R);
+                    else if (G == 3)
+                        hipLaunchKernelGGL(rnn_step_fused_kernel<3>, grid, dim3(256), 0, h->stream, c, (const float*)w.R);
+                    else
+                        hipLaunchKernelGGL(rnn_step_fused_kernel<1>, grid, dim3(256), 0, h->stream, c, (const float*)w.R);
+                } else {
+                    hipLaunchKernelGGL(rnn_cell_fwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
+                                       h->stream, c);
+                }
                 st = hip_to_status(hipGetLastError());
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
@@ -276,14 +299,16 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
     if (keep == nullptr || reserve_bytes < (size_t)r.total * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
     if (ws == nullptr || workspace_bytes < (size_t)r.bwd_ws * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
     const int B = batch, T = steps, H = r.H, G = r.G, K = r.K;
-    const long long GH = (long long)G * H;
+    const long long GH = (long long)G * H, KH = (long long)K * H;
     float* dh = ws;
     float* dc = ws + (long long)B * H;
-    float* between[2] = {ws + 2LL * B * H + GH, ws + 2LL * B * H + GH + r.n * K * H};
+    float* between[2] = {ws + 2LL * B * H + GH, ws + 2LL * B * H + GH + r.n * KH};
 
     for (int layer = r.L - 1; layer >= 0; --layer) {
-        const float* out = layer == r.L - 1 ? y : keep + r.out_off + (long long)layer * r.n * K * H;
-        const float* dout = layer == r.L - 1 ? dy : between[layer & 1];
+        const bool top = layer == r.L - 1;
+        const float* out = top ? y : keep + r.out_off + (long long)layer * r.n * KH;
+        const float* dout = top ? dy : between[layer & 1];
+        const long long out_step = top ? KH : (long long)B * KH, out_ld = top ? (long long)T * KH : KH;
         float* dinp = layer == 0 ? dx : between[(layer - 1) & 1];
         const long long I = rnn_layer_inputs(r, layer);
         for (int d = 0; d < K; ++d) {
@@ -305,17 +330,13 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
             for (int k = T - 1; k >= 0; --k) {
                 const int t = first + dir * k;
                 RnnStepBwd c;
-                c.gates = gates + (long long)t * GH, c.ld_gates = T * GH;
-                c.gh = gh + (long long)t * 3 * H, c.ld_gh = (long long)T * 3 * H;
-                c.h_prev = hprev + (long long)t * H, c.ld_hprev = (long long)T * H;
-                c.y = out + (long long)t * K * H + (long long)d * H, c.ld_y = (long long)T * K * H;
-                if (k == 0) {
-                    c.c_prev = cx_p, c.ld_cprev = H;
-                } else {
-                    c.c_prev = cells + (long long)(t - dir) * H, c.ld_cprev = (long long)T * H;
-                }
-                c.c = cells + (long long)t * H, c.ld_c = (long long)T * H;
-                c.dy = dout + (long long)t * K * H + (long long)d * H, c.ld_dy = (long long)T * K * H;
+                c.gates = gates + (long long)t * B * GH, c.ld_gates = GH;
+                c.gh = gh + (long long)t * B * 3 * H, c.ld_gh = 3LL * H;
+                c.h_prev = hprev + (long long)t * B * H, c.ld_hprev = H;
+                c.y = out + (long long)t * out_step + (long long)d * H, c.ld_y = out_ld;
+                c.c_prev = k == 0 ? cx_p : cells + (long long)(t - dir) * B * H, c.ld_cprev = H;
+                c.c = cells + (long long)t * B * H, c.ld_c = H;
+                c.dy = dout + (long long)t * out_step + (long long)d * H, c.ld_dy = out_ld;
                 c.dh = dh, c.dc = dc;
                 c.batch = B, c.hidden = H, c.cell = r.cell;
                 hipLaunchKernelGGL(rnn_cell_bwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
@@ -325,8 +346,8 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
                 if (k == 0 && dhx == nullptr) break;  // nobody asks for the gradient of the initial state
                 GemmArgs s;  // dh = d(R h)[:, t] . R  (GRU: added to dh * z)
                 s.M = B, s.N = H, s.K = (int)GH;
-                s.A = (r.cell == RNN_GRU) ? gh + (long long)t * 3 * H : gates + (long long)t * GH;
-                s.lda = (int)(T * GH);
+                s.A = (r.cell == RNN_GRU) ? gh + (long long)t * B * 3 * H : gates + (long long)t * B * GH;
+                s.lda = (int)GH;
                 s.B = w.R, s.ldb = H;
                 s.C = dh, s.ldc = H;
                 s.beta = (r.cell == RNN_GRU) ? 1.0f : 0.0f;
@@ -341,14 +362,20 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
                 st = rnn_set_rows(h, dcx + (long long)p * B * H, H, dc, H, B, H);
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
-            if (dinp != nullptr) {
-                GemmArgs g;  // gradient of the layer's input: both directions add up
-                g.M = (int)r.n, g.N = (int)I, g.K = (int)GH;
-                g.A = gates, g.lda = (int)GH, g.B = w.W, g.ldb = (int)I, g.C = dinp, g.ldc = (int)I;
-                g.beta = d == 0 ? 0.0f : 1.0f;
-                st = gemm_core(h, g);
-                if (st != SNHIP_STATUS_SUCCESS) return st;
+            if (dinp == nullptr) continue;
+            GemmArgs g;  // gradient of the layer's input: both directions add up
+            g.K = (int)GH, g.N = (int)I;
+            g.A = gates, g.lda = (int)GH, g.B = w.W, g.ldb = (int)I, g.C = dinp;
+            g.beta = d == 0 ? 0.0f : 1.0f;
+            if (layer == 0) {
+                // one product per step: step-major rows in, the caller's batch-major dx out
+                g.M = B, g.batch = T;
+                g.sA = (long long)B * GH, g.sB = 0, g.sC = I, g.ldc = (int)(T * I);
+            } else {
+                g.M = (int)r.n, g.ldc = (int)I;
             }
+            st = gemm_core(h, g);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
         }
     }
     return SNHIP_STATUS_SUCCESS;
@@ -361,7 +388,7 @@ int snhip_rnn_backward_weights(void* handle, const snhip_rnn_desc* desc, int bat
     int st = rnn_common_checks(h, desc, batch, steps);
     if (st != SNHIP_STATUS_SUCCESS) return st;
     if (batch == 0 || steps == 0) return SNHIP_STATUS_SUCCESS;
-    (void)hx, (void)y;  // both are in reserve, arranged per step
+    (void)hx, (void)y;  // both are in reserve, arranged per step, and so is a step-major copy of x
     if (x == nullptr || weight_gradients == nullptr) return SNHIP_STATUS_INVALID_VALUE;
     const RnnDims r = rnn_dims(desc, batch, steps);
     float* keep = static_cast<float*>(reserve);
@@ -373,7 +400,7 @@ int snhip_rnn_backward_weights(void* handle, const snhip_rnn_desc* desc, int bat
     float* colsum = ws + 2LL * batch * H;
 
     for (int layer = 0; layer < r.L; ++layer) {
-        const float* inp = layer == 0 ? x : keep + r.out_off + (long long)(layer - 1) * r.n * K * H;
+        const float* inp = layer == 0 ? keep + r.xt_off : keep + r.out_off + (long long)(layer - 1) * r.n * K * H;
         const long long I = rnn_layer_inputs(r, layer);
         for (int d = 0; d < K; ++d) {
             const int p = layer * K + d;

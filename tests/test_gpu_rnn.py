@@ -125,6 +125,33 @@ def test_cells_wider(gpu_wrapper, cell):
     compare(desc, got, x, weights, dy, None, None, None, None, 1e-4)
 
 
+@pytest.mark.parametrize("cell", [ro.RELU, ro.TANH, ro.LSTM, ro.GRU])
+@pytest.mark.parametrize("hidden,batch", [(32, 5), (64, 33), (96, 70), (160, 32)])
+def test_cells_one_launch_per_step(gpu_wrapper, cell, hidden, batch):
+    """Hidden sizes that are multiples of 32 take the kernel that computes h . R^T and the cell in one launch
+    (K split over the wavefronts of a workgroup); checked against the oracle and against the GEMM + cell-kernel form selected through the
+    tuning hook (different summation orders: 2e-5)."""
+    rng = np.random.default_rng(hidden * 10 + batch + cell)
+    desc = ro.RnnDesc(cell, input_size=20, hidden_size=hidden, num_layers=2, bidirectional=True, bias_mode=ro.DOUBLE_BIAS)
+    Tn = 7
+    weights = rng.uniform(-0.15, 0.15, ro.weight_space_size(desc)).astype(np.float32)
+    x = rng.uniform(-1, 1, (batch, Tn, 20)).astype(np.float32)
+    dy = rng.uniform(-1, 1, (batch, Tn, 2 * hidden)).astype(np.float32)
+    st = lambda: rng.uniform(-1, 1, (desc.pseudo_layers, batch, hidden)).astype(np.float32)
+    hx, cx, dhy, dcy = st(), st(), st(), st()
+    if cell != ro.LSTM:
+        cx = dcy = None
+    got = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy)
+    compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, 5e-5)
+    gpu_wrapper.set_tuning(6, 1)
+    try:
+        two = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy)
+    finally:
+        gpu_wrapper.set_tuning(-1, 0)
+    compare(desc, two, x, weights, dy, hx, cx, dhy, dcy, 5e-5)
+    assert np.max(np.abs(two["y"] - got["y"])) <= 2e-5
+
+
 @pytest.mark.parametrize("cell", [ro.RELU, ro.LSTM, ro.GRU])
 def test_inference_equals_training_forward(gpu_wrapper, cell):
     rng = np.random.default_rng(7 + cell)
