@@ -46,6 +46,9 @@ def main():
     ap.add_argument("--attention-probe", action="store_true",
                     help="20 launches of the one-launch attention forward of configuration 5 (512 x 256 x 64, weights "
                          "kept), for profilers")
+    ap.add_argument("--rnn-probe", choices=["lstm", "gru"], default=None,
+                    help="3 forward + backward passes of a recurrent layer at configuration 4's shape (batch 256, 128 "
+                         "steps, 256 -> 512), for profilers")
     ap.add_argument("--shapes-probe", action="store_true",
                     help="30 launches each of the skinny, small-M and batched shapes (and the bf16-input headline), in "
                          "the order printed, for profilers")
@@ -115,6 +118,24 @@ def main():
                 attention.fused_attention_forward(q, k, v, o, keep, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
                                                   scale=0.125, is_causal=False, packed=False)
             w.synchronize()
+        return
+    if args.rnn_probe:
+        from sharpnet_amd import recurrent
+        rng = np.random.default_rng(4)
+        w.use_memory_pool(True)
+        B, Tn, I, H = 256, 128, 256, 512
+        x = GPUTensor([B, Tn, I], rng.uniform(-1, 1, (B, Tn, I)).astype(np.float32), w)
+        dy = GPUTensor([B, Tn, H], rng.uniform(-0.01, 0.01, (B, Tn, H)).astype(np.float32), w)
+        y, dx = GPUTensor([B, Tn, H], None, w), GPUTensor([B, Tn, I], None, w)
+        cell, bias = ((recurrent.CUDNN_LSTM, recurrent.CUDNN_RNN_SINGLE_INP_BIAS) if args.rnn_probe == "lstm" else
+                      (recurrent.CUDNN_GRU, recurrent.CUDNN_RNN_DOUBLE_BIAS))
+        layer = recurrent.RecurrentLayer(w, I, H, cell, bias, True, False, 1)
+        layer._weightsAndBiases.InitializeFromHostMemory(
+            rng.uniform(-0.04, 0.04, layer._weightsAndBiases.Count).astype(np.float32))
+        for _ in range(3):
+            layer.ForwardPropagation(x, y, True)
+            layer.BackwardPropagation(x, y, dy, dx)
+        w.synchronize()
         return
     if args.shapes_probe:
         shapes = [("skinny 8192x64x8192 NN", wl.Gemm(8192, 64, 8192), 0), ("skinny 8192x64x8192 TN", wl.Gemm(8192, 64, 8192, True, False), 0)]
@@ -438,12 +459,12 @@ def layer_timings(w, wl):
             layer.BackwardPropagation(x, yr, dyr, dxr)
         gates = 4 if name == "LSTM" else 3
         flop = 2.0 * B * Tn * gates * H * (I + H)
-        for form, cfg in (("forward: one launch per step (product + cell)", -1),
-                          ("forward: GEMM + cell kernel per step", 6)):
-            w.set_tuning(cfg, 1 if cfg >= 0 else 0)     # a forced GEMM configuration selects the two-launch form
+        for form, mode in (("forward: one launch per step (product + cell)", 0),
+                           ("forward: GEMM + cell kernel per step", 1)):
+            w.lib.snhip_rnn_set_step_mode(w.handle, mode)
             f = timed(rnn_f, 3, 1)
             fb = timed(rnn_fb, 3, 1)
-            w.set_tuning(-1, 0)
+            w.lib.snhip_rnn_set_step_mode(w.handle, 0)
             res.append({"layer": "%s batch %d, %d steps, %d -> %d (forward %.1f GFLOP: %d sequential steps of %dx%dx%d)" %
                                  (name, B, Tn, I, H, flop / 1e9, Tn, B, gates * H, H),
                         "form": form, "forward_ms": f, "backward_ms": round(fb - f, 4)})

@@ -181,6 +181,13 @@ int snhip_rnn_temp_space_sizes(const snhip_rnn_desc* desc, int training, int bat
     return SNHIP_STATUS_SUCCESS;
 }
 
+int snhip_rnn_set_step_mode(void* handle, int mode) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (mode < 0 || mode > 1) return SNHIP_STATUS_INVALID_VALUE;
+    static_cast<Handle*>(handle)->rnn_step_mode = mode;
+    return SNHIP_STATUS_SUCCESS;
+}
+
 int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, int batch, int steps, const float* x,
                       float* y, const float* hx, float* hy, const float* cx, float* cy, const float* weights,
                       void* workspace, size_t workspace_bytes, void* reserve, size_t reserve_bytes) {
@@ -229,9 +236,8 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
             const int first = d == 0 ? 0 : T - 1, dir = d == 0 ? 1 : -1;
             st = rnn_set_rows(h, hprev + (long long)first * B * H, H, hx_p, H, B, H);
             if (st != SNHIP_STATUS_SUCCESS) return st;
-            // product and cell in one launch per step when the rows can be read in 16-byte pieces; a forced GEMM
-            // configuration (tuning hook) selects the two-launch form
-            const bool fused = H % 32 == 0 && (uintptr_t)hprev % 16 == 0 && (uintptr_t)w.R % 16 == 0 && h->force_cfg < 0;
+            // product and cell in one launch per step when the rows can be read in 16-byte pieces
+            const bool fused = H % 32 == 0 && (uintptr_t)hprev % 16 == 0 && (uintptr_t)w.R % 16 == 0 && h->rnn_step_mode == 0;
             for (int k = 0; k < T; ++k) {
                 const int t = first + dir * k;
                 const bool last = k == T - 1;

@@ -37,6 +37,7 @@ struct Handle {
     int force_splitk = 0;
     int last_cfg = -1;
     int last_splitk = 0;
+    int rnn_step_mode = 0;  // 0: recurrent forward steps as one launch when the shape allows, 1: always GEMM + cell kernel
 };
 
 // Upper bound for the split-K workspace; larger requests fall back to fewer splits.

@@ -179,6 +179,7 @@ SIGNATURES = {
                                 ctypes.POINTER(_ll)],
     "snhip_rnn_temp_space_sizes": [ctypes.POINTER(RnnDesc), _i, _i, _i, ctypes.POINTER(_sz), ctypes.POINTER(_sz)],
     "snhip_rnn_forward": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz],
+    "snhip_rnn_set_step_mode": [_vp, _i],
     "snhip_rnn_backward_data": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                 _vp, _sz, _vp, _sz],
     "snhip_rnn_backward_weights": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz],

@@ -129,8 +129,8 @@ def test_cells_wider(gpu_wrapper, cell):
 @pytest.mark.parametrize("hidden,batch", [(32, 5), (64, 33), (96, 70), (160, 32)])
 def test_cells_one_launch_per_step(gpu_wrapper, cell, hidden, batch):
     """Hidden sizes that are multiples of 32 take the kernel that computes h . R^T and the cell in one launch
-    (K split over the wavefronts of a workgroup); checked against the oracle and against the GEMM + cell-kernel form selected through the
-    tuning hook (different summation orders: 2e-5)."""
+    (K split over the wavefronts of a workgroup); checked against the oracle and against the GEMM + cell-kernel form selected through
+    snhip_rnn_set_step_mode (different summation orders: 2e-5)."""
     rng = np.random.default_rng(hidden * 10 + batch + cell)
     desc = ro.RnnDesc(cell, input_size=20, hidden_size=hidden, num_layers=2, bidirectional=True, bias_mode=ro.DOUBLE_BIAS)
     Tn = 7
@@ -143,11 +143,11 @@ def test_cells_one_launch_per_step(gpu_wrapper, cell, hidden, batch):
         cx = dcy = None
     got = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy)
     compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, 5e-5)
-    gpu_wrapper.set_tuning(6, 1)
+    check(gpu_wrapper.lib.snhip_rnn_set_step_mode(gpu_wrapper.handle, 1), "step mode")
     try:
         two = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy)
     finally:
-        gpu_wrapper.set_tuning(-1, 0)
+        check(gpu_wrapper.lib.snhip_rnn_set_step_mode(gpu_wrapper.handle, 0), "step mode")
     compare(desc, two, x, weights, dy, hx, cx, dhy, dcy, 5e-5)
     assert np.max(np.abs(two["y"] - got["y"])) <= 2e-5
 
