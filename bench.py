@@ -459,8 +459,8 @@ def layer_timings(w, wl):
             layer.BackwardPropagation(x, yr, dyr, dxr)
         gates = 4 if name == "LSTM" else 3
         flop = 2.0 * B * Tn * gates * H * (I + H)
-        for form, mode in (("forward: one launch per step (product + cell)", 0),
-                           ("forward: GEMM + cell kernel per step", 1)):
+        for form, mode in (("one launch per step (product with R + cell arithmetic)", 0),
+                           ("GEMM + cell kernel per step (+ split-K reduction on the way back)", 1)):
             w.lib.snhip_rnn_set_step_mode(w.handle, mode)
             f = timed(rnn_f, 3, 1)
             fb = timed(rnn_fb, 3, 1)

@@ -75,82 +75,16 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd_kernel(const RnnStepFwd s) {
     if (s.hy) s.hy[(long long)b * H + j] = h;
 }
 
-// One forward time step in one launch: the product h[t-1] . R^T and the cell arithmetic.
-//
-// The step's GEMM (batch x G*H x H, e.g. 256 x 2048 x 512) is far too small to fill the chip with 64 x 64 tiles -
-// it is bound by the length of one wavefront's chain of MFMAs, not by the MFMA rate.  This kernel cuts it so that
-// every SIMD of the chip gets one short chain: a workgroup owns 32 samples x U hidden units x all G gates
-// (U = 16; 32 for the single-gate cells), i.e. one or two 32 x 32 MFMA tiles whose 32 columns are gathered from
-// the gates' row blocks of R, and splits K (the hidden dimension) over its wavefronts: four wavefronts =
-// (tiles) x (K slices).  Each wavefront is on its own in the main loop: per group of 32 k values it reads its
-// 32 x 32 pieces of h[t-1] and R with whole-line loads (a lane takes 16 bytes, eight lanes one 128-byte row piece),
-// DEPTH groups in flight in registers, passes a group through a private LDS patch to turn it into MFMA operand
-// layout (row = lane % 32, sixteen consecutive k per half-wave), and multiplies - no workgroup barrier until the
-// partial tiles meet in LDS, where each thread picks up all gates of its (sample, unit) pairs, adds W x + bW from
-// the gates buffer and finishes the cell exactly as rnn_cell_fwd_kernel does.
-// Requires H % 32 == 0 and 16-byte aligned rows; the caller falls back to GEMM + cell kernel otherwise.
-template <int G>
-struct RnnFusedCfg {
-    static constexpr int U = (G == 1) ? 32 : 16;       // hidden units per workgroup
-    static constexpr int COLS = G * U;                 // columns of the workgroup's tile: [gate][unit]
-    static constexpr int NT = (COLS + 31) / 32;        // 32-column MFMA tiles
-    static constexpr int KS = 4 / NT;                  // K slices
-    static constexpr int DEPTH = 4;                    // groups of 32 k values in flight per wavefront
-    static constexpr int PITCH = 36;                   // floats per row of an LDS patch (32 + 4: conflict-free b128)
-};
-
-template <int G>
-__global__ void __launch_bounds__(256) rnn_step_fused_kernel(const RnnStepFwd s, const float* __restrict__ R) {
-    using C = RnnFusedCfg<G>;
-    constexpr int U = C::U, NT = C::NT, KS = C::KS, D = C::DEPTH, P = C::PITCH;
-    __shared__ float part[KS][NT][32][33];
-    __shared__ __attribute__((aligned(16))) float patch[4][2][32 * P];   // per wavefront: h rows, R rows
-    const int H = s.hidden;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
-    const int nt = wave % NT, kg = wave / NT;
-    // unit blocks along x: workgroups are dealt to the eight XCDs by their linear index, so the (few) workgroups that
-    // share a slice of R land on one XCD and find it in that XCD's L2
-    const int row0 = blockIdx.y * 32, u0 = blockIdx.x * U;
-
-    // global side: instruction i of a group fetches rows 8 i + lane / 8, floats 4 (lane % 8) .. + 3
-    const int lrow = lane >> 3, lcol = (lane & 7) * 4;
-    const float* ap[4];
-    const float* bp[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ar = (row0 + 8 * i + lrow < s.batch) ? row0 + 8 * i + lrow : s.batch - 1;
-        ap[i] = s.h_prev + (long long)ar * s.ld_hprev + lcol;
-        const int col = nt * 32 + 8 * i + lrow;                 // column of the workgroup's tile -> row of R
-        const int gate = col / U, unit = u0 + col % U;
-        bp[i] = R + (long long)((col < C::COLS && unit < H) ? gate * H + unit : 0) * H + lcol;
-    }
-    float* pa = &patch[wave][0][0];
-    float* pb = &patch[wave][1][0];
-
-    const int groups = H / 32;                                   // groups of 32 k values
-    const int per = (groups + KS - 1) / KS;
-    const int mbeg = kg * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
-
-    // what the cell arithmetic at the end reads from global memory is fetched now, behind the main loop:
-    // thread -> pairs p = threadIdx.x + 256 q of the tile's 32 x U (sample, unit) pairs
-    constexpr int Q = 32 * U / 256;
-    float gxv[Q][G], brv[Q][G], cpv[Q], hpv[Q];
-#pragma unroll
-    for (int q = 0; q < Q; ++q) {
-        const int p = threadIdx.x + 256 * q;
-        const int b = row0 + p / U, j = u0 + p % U;
-        const bool ok = b < s.batch && j < H;
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            gxv[q][g] = ok ? s.gates[b * s.ld_gates + g * H + j] : 0.0f;
-            brv[q][g] = (ok && s.bias_r) ? s.bias_r[g * H + j] : 0.0f;
-        }
-        cpv[q] = (G == 4 && ok && s.c_prev) ? s.c_prev[b * s.ld_cprev + j] : 0.0f;
-        hpv[q] = (G == 3 && ok) ? s.h_prev[b * s.ld_hprev + j] : 0.0f;
-    }
-
+// acc[0..3] (to be added up by the caller) = A . B^T for one wavefront: 32 rows of A (lane l fetches from ap[i] the row
+// 8 i + l / 8, floats 4 (l % 8) .. + 3 of a group), 32 rows of B (bp[i] likewise), over the groups of 32 k values
+// mbeg .. mend - 1.  Whole-line global loads, DEPTH groups in flight in registers; a group passes through the
+// wavefront's private LDS patches pa / pb (32 rows x PITCH floats each) to reach MFMA operand layout (row = l % 32,
+// sixteen consecutive k per half-wave).  No workgroup barrier inside.
+template <int D, int P>
+__device__ __forceinline__ void wave_product_32x32(const float* const (&ap)[4], const float* const (&bp)[4], int mbeg,
+                                                   int mend, float* pa, float* pb, int lane, f32x16 (&acc)[4]) {
+    const int l32 = lane & 31, lhi = lane >> 5, lrow = lane >> 3, lcol = (lane & 7) * 4;
     f32x4 ra[D][4], rb[D][4];
-    f32x16 acc[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
@@ -228,6 +162,84 @@ __global__ void __launch_bounds__(256) rnn_step_fused_kernel(const RnnStepFwd s,
             stage(d, 0);
             multiply(0);
         }
+}
+
+// One forward time step in one launch: the product h[t-1] . R^T and the cell arithmetic.
+//
+// The step's GEMM (batch x G*H x H, e.g. 256 x 2048 x 512) is far too small to fill the chip with 64 x 64 tiles -
+// it is bound by the length of one wavefront's chain of MFMAs, not by the MFMA rate.  This kernel cuts it so that
+// every SIMD of the chip gets one short chain: a workgroup owns 32 samples x U hidden units x all G gates
+// (U = 16; 32 for the single-gate cells), i.e. one or two 32 x 32 MFMA tiles whose 32 columns are gathered from
+// the gates' row blocks of R, and splits K (the hidden dimension) over its wavefronts: four wavefronts =
+// (tiles) x (K slices).  Each wavefront is on its own in the main loop: per group of 32 k values it reads its
+// 32 x 32 pieces of h[t-1] and R with whole-line loads (a lane takes 16 bytes, eight lanes one 128-byte row piece),
+// DEPTH groups in flight in registers, passes a group through a private LDS patch to turn it into MFMA operand
+// layout (row = lane % 32, sixteen consecutive k per half-wave), and multiplies - no workgroup barrier until the
+// partial tiles meet in LDS, where each thread picks up all gates of its (sample, unit) pairs, adds W x + bW from
+// the gates buffer and finishes the cell exactly as rnn_cell_fwd_kernel does.
+// Requires H % 32 == 0 and 16-byte aligned rows; the caller falls back to GEMM + cell kernel otherwise.
+template <int G>
+struct RnnFusedCfg {
+    static constexpr int U = (G == 1) ? 32 : 16;       // hidden units per workgroup
+    static constexpr int COLS = G * U;                 // columns of the workgroup's tile: [gate][unit]
+    static constexpr int NT = (COLS + 31) / 32;        // 32-column MFMA tiles
+    static constexpr int KS = 4 / NT;                  // K slices
+    static constexpr int DEPTH = 4;                    // groups of 32 k values in flight per wavefront
+    static constexpr int PITCH = 36;                   // floats per row of an LDS patch (32 + 4: conflict-free b128)
+};
+
+template <int G>
+__global__ void __launch_bounds__(256) rnn_step_fused_kernel(const RnnStepFwd s, const float* __restrict__ R) {
+    using C = RnnFusedCfg<G>;
+    constexpr int U = C::U, NT = C::NT, KS = C::KS, D = C::DEPTH, P = C::PITCH;
+    __shared__ float part[KS][NT][32][33];
+    __shared__ __attribute__((aligned(16))) float patch[4][2][32 * P];   // per wavefront: h rows, R rows
+    const int H = s.hidden;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int nt = wave % NT, kg = wave / NT;
+    // unit blocks along x: workgroups are dealt to the eight XCDs by their linear index, so the (few) workgroups that
+    // share a slice of R land on one XCD and find it in that XCD's L2
+    const int row0 = blockIdx.y * 32, u0 = blockIdx.x * U;
+
+    // global side: instruction i of a group fetches rows 8 i + lane / 8, floats 4 (lane % 8) .. + 3
+    const int lrow = lane >> 3, lcol = (lane & 7) * 4;
+    const float* ap[4];
+    const float* bp[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ar = (row0 + 8 * i + lrow < s.batch) ? row0 + 8 * i + lrow : s.batch - 1;
+        ap[i] = s.h_prev + (long long)ar * s.ld_hprev + lcol;
+        const int col = nt * 32 + 8 * i + lrow;                 // column of the workgroup's tile -> row of R
+        const int gate = col / U, unit = u0 + col % U;
+        bp[i] = R + (long long)((col < C::COLS && unit < H) ? gate * H + unit : 0) * H + lcol;
+    }
+    float* pa = &patch[wave][0][0];
+    float* pb = &patch[wave][1][0];
+
+    const int groups = H / 32;                                   // groups of 32 k values
+    const int per = (groups + KS - 1) / KS;
+    const int mbeg = kg * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
+
+    // what the cell arithmetic at the end reads from global memory is fetched now, behind the main loop:
+    // thread -> pairs p = threadIdx.x + 256 q of the tile's 32 x U (sample, unit) pairs
+    constexpr int Q = 32 * U / 256;
+    float gxv[Q][G], brv[Q][G], cpv[Q], hpv[Q];
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+        const int p = threadIdx.x + 256 * q;
+        const int b = row0 + p / U, j = u0 + p % U;
+        const bool ok = b < s.batch && j < H;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            gxv[q][g] = ok ? s.gates[b * s.ld_gates + g * H + j] : 0.0f;
+            brv[q][g] = (ok && s.bias_r) ? s.bias_r[g * H + j] : 0.0f;
+        }
+        cpv[q] = (G == 4 && ok && s.c_prev) ? s.c_prev[b * s.ld_cprev + j] : 0.0f;
+        hpv[q] = (G == 3 && ok) ? s.h_prev[b * s.ld_hprev + j] : 0.0f;
+    }
+
+    f32x16 acc[4];
+    wave_product_32x32<D, P>(ap, bp, mbeg, mend, pa, pb, lane, acc);
     // accumulator register r holds row 8 (r / 4) + 4 lhi + r % 4, column l32 of the 32 x 32 tile
 #pragma unroll
     for (int r = 0; r < 16; ++r)
@@ -320,6 +332,118 @@ __global__ void __launch_bounds__(256) rnn_cell_bwd_kernel(const RnnStepBwd s) {
         g[j] = dr, g[H + j] = dz, g[2 * H + j] = dn;
         gh[j] = dr, gh[H + j] = dz, gh[2 * H + j] = dn * r;
         s.dh[idx] = dh * z;
+    }
+}
+
+// One backward time step in one launch: dh = d(R h + bR)[step after] . R, then the cell gradient of this step.
+//
+// The product is batch x H x G*H (256 x 512 x 2048): 128 tiles of 32 x 32 with a long K.  A workgroup of eight
+// wavefronts owns one tile (32 samples x 32 hidden units) and gives each wavefront an eighth of K
+// (wave_product_32x32 on rows of d(gates) and rows of R^T, which the caller lays out once per call), so the chip
+// holds 1024 chains of 128 MFMAs as in the forward kernel.  The partial tiles meet in LDS; each thread then owns two
+// (sample, unit) pairs, adds the gradient arriving from the layer above (and, for the GRU, dh * z carried over
+// from the step after) and does what rnn_cell_bwd_kernel does, with its inputs fetched before the main loop.
+// `dg_next` is the d(R h + bR) the step after (in time order of this direction) left behind.
+struct RnnBwdFusedCfg {
+    static constexpr int KS = 8;
+    static constexpr int DEPTH = 2;   // two wavefronts per SIMD: 256 registers each
+    static constexpr int PITCH = 36;
+    static constexpr int LDS_BYTES = (KS * 2 * 32 * PITCH + KS * 32 * 33) * 4;
+};
+
+template <int G>
+__global__ void __launch_bounds__(512) rnn_step_bwd_fused_kernel(const RnnStepBwd s, const float* __restrict__ dg_next,
+                                                                 long long ld_dg, const float* __restrict__ Rt) {
+    using C = RnnBwdFusedCfg;
+    constexpr int KS = C::KS, D = C::DEPTH, P = C::PITCH;
+    extern __shared__ __attribute__((aligned(16))) float lds_bwd[];
+    float* patch = lds_bwd;                                   // [KS][2][32 * P]
+    float(*part)[32][33] = reinterpret_cast<float(*)[32][33]>(lds_bwd + KS * 2 * 32 * P);   // [KS][32][33]
+    const int H = s.hidden, GH = G * H;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int row0 = blockIdx.y * 32, u0 = blockIdx.x * 32;
+
+    const int lrow = lane >> 3, lcol = (lane & 7) * 4;
+    const float* ap[4];
+    const float* bp[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ar = (row0 + 8 * i + lrow < s.batch) ? row0 + 8 * i + lrow : s.batch - 1;
+        ap[i] = dg_next + (long long)ar * ld_dg + lcol;
+        const int unit = (u0 + 8 * i + lrow < H) ? u0 + 8 * i + lrow : H - 1;
+        bp[i] = Rt + (long long)unit * GH + lcol;
+    }
+    const int groups = GH / 32;
+    const int per = (groups + KS - 1) / KS;
+    const int mbeg = wave * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
+
+    // inputs of the cell gradient: thread -> pairs p = threadIdx.x + 512 q of the tile's 32 x 32 (sample, unit) pairs
+    constexpr int Q = 2;
+    float gv[Q][G], dyv[Q], dhv[Q], av[Q], bv[Q], cv[Q];
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+        const int p = threadIdx.x + 512 * q;
+        const int b = row0 + p / 32, j = u0 + p % 32;
+        const bool ok = b < s.batch && j < H;
+        const long long idx = (long long)b * H + j;
+#pragma unroll
+        for (int g = 0; g < G; ++g) gv[q][g] = ok ? s.gates[b * s.ld_gates + g * H + j] : 0.0f;
+        dyv[q] = ok ? s.dy[b * s.ld_dy + j] : 0.0f;
+        dhv[q] = (G == 3 && ok) ? s.dh[idx] : 0.0f;                       // GRU: dh * z of the step after
+        if constexpr (G == 1) {
+            av[q] = ok ? s.y[b * s.ld_y + j] : 0.0f;                     // h'
+            bv[q] = cv[q] = 0.0f;
+        } else if constexpr (G == 4) {
+            av[q] = ok ? s.c[b * s.ld_c + j] : 0.0f;                     // c'
+            bv[q] = (ok && s.c_prev) ? s.c_prev[b * s.ld_cprev + j] : 0.0f;
+            cv[q] = ok ? s.dc[idx] : 0.0f;
+        } else {
+            av[q] = ok ? s.gh[b * s.ld_gh + 2 * H + j] : 0.0f;           // Rn h + bRn
+            bv[q] = ok ? s.h_prev[b * s.ld_hprev + j] : 0.0f;
+            cv[q] = 0.0f;
+        }
+    }
+
+    f32x16 acc[4];
+    wave_product_32x32<D, P>(ap, bp, mbeg, mend, patch + (wave * 2) * 32 * P, patch + (wave * 2 + 1) * 32 * P, lane, acc);
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        part[wave][8 * (r / 4) + 4 * lhi + (r % 4)][l32] = (acc[0][r] + acc[1][r]) + (acc[2][r] + acc[3][r]);
+    __syncthreads();
+
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+        const int p = threadIdx.x + 512 * q;
+        const int lr = p / 32, b = row0 + lr, j = u0 + p % 32;
+        if (b >= s.batch || j >= H) continue;
+        const long long idx = (long long)b * H + j;
+        float rec = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KS; ++k) rec += part[k][lr][p % 32];
+        const float dh = rec + dhv[q] + dyv[q];
+        float* g = s.gates + b * s.ld_gates;
+        if constexpr (G == 1) {
+            const float h = av[q];
+            g[j] = (s.cell == RNN_RELU) ? (h > 0.0f ? dh : 0.0f) : dh * (1.0f - h * h);
+        } else if constexpr (G == 4) {
+            const float i = gv[q][0], f = gv[q][1], gg = gv[q][2], o = gv[q][3];
+            const float tc = tanhf(av[q]);
+            const float dc = cv[q] + dh * o * (1.0f - tc * tc);
+            g[j] = dc * gg * i * (1.0f - i);
+            g[H + j] = dc * bv[q] * f * (1.0f - f);
+            g[2 * H + j] = dc * i * (1.0f - gg * gg);
+            g[3 * H + j] = dh * tc * o * (1.0f - o);
+            s.dc[idx] = dc * f;
+        } else {
+            const float r = gv[q][0], z = gv[q][1], n = gv[q][2], qn = av[q], hp = bv[q];
+            const float dn = dh * (1.0f - z) * (1.0f - n * n);
+            const float dz = dh * (hp - n) * z * (1.0f - z);
+            const float dr = dn * qn * r * (1.0f - r);
+            float* gh = s.gh + b * s.ld_gh;
+            g[j] = dr, g[H + j] = dz, g[2 * H + j] = dn;
+            gh[j] = dr, gh[H + j] = dz, gh[2 * H + j] = dn * r;
+            s.dh[idx] = dh * z;
+        }
     }
 }
 

@@ -30,6 +30,7 @@ struct RnnDims {
     long long out_off;                // start of the stacked layers' outputs, after all regions
     long long xt_off;                 // step-major copy of x
     long long total;                  // floats carried from forward to backward
+    long long rt_off;                 // inside the backward scratch: the transposed recurrent matrix of one direction
     long long bwd_ws;                 // floats of scratch the backward calls need
 };
 
@@ -66,8 +67,9 @@ RnnDims rnn_dims(const snhip_rnn_desc* d, int batch, int steps) {
     r.out_off = r.per_p * r.P;
     r.xt_off = r.out_off + (long long)(r.L - 1) * r.n * r.K * r.H;
     r.total = r.xt_off + r.n * r.I;
-    // dh, dc, one bias gradient, and two buffers for the gradients that travel between stacked layers
-    r.bwd_ws = 2LL * batch * r.H + (long long)r.G * r.H + (r.L > 1 ? 2 * r.n * r.K * r.H : 0);
+    // dh, dc, one bias gradient, two buffers for the gradients that travel between stacked layers, and R^T
+    r.rt_off = 2LL * batch * r.H + (long long)r.G * r.H + (r.L > 1 ? 2 * r.n * r.K * r.H : 0);
+    r.bwd_ws = r.rt_off + (long long)r.G * r.H * r.H;
     return r;
 }
 
@@ -112,6 +114,18 @@ int rnn_set_rows(Handle* h, float* dst, long long ld_dst, const float* src, long
     hipLaunchKernelGGL(set_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, h->stream, dst, ld_dst, src,
                        ld_src, rows, cols);
     return hip_to_status(hipGetLastError());
+}
+
+// The backward step kernel stages more than the 64 KiB of LDS a kernel gets without asking.
+hipError_t rnn_prepare_kernels() {
+    const void* fns[3] = {reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<1>),
+                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<3>),
+                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<4>)};
+    for (const void* f : fns) {
+        const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, RnnBwdFusedCfg::LDS_BYTES);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 int rnn_common_checks(Handle* h, const snhip_rnn_desc* desc, int batch, int steps) {
@@ -333,6 +347,15 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
             const int first = d == 0 ? 0 : T - 1, dir = d == 0 ? 1 : -1;
+            // every step but the first one processed runs as one launch (product with R, then the cell gradient) when
+            // rows can be read in 16-byte pieces; that kernel wants the rows of R^T
+            float* Rt = ws + r.rt_off;
+            const bool fused = H % 32 == 0 && T > 1 && (uintptr_t)gates % 16 == 0 && (uintptr_t)Rt % 16 == 0 &&
+                               h->rnn_step_mode == 0;
+            if (fused) {
+                st = snhip_transpose_second_and_third_dimension(handle, w.R, Rt, 1, (int)GH, H, 1);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+            }
             for (int k = T - 1; k >= 0; --k) {
                 const int t = first + dir * k;
                 RnnStepBwd c;
@@ -345,11 +368,26 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
                 c.dy = dout + (long long)t * out_step + (long long)d * H, c.ld_dy = out_ld;
                 c.dh = dh, c.dc = dc;
                 c.batch = B, c.hidden = H, c.cell = r.cell;
-                hipLaunchKernelGGL(rnn_cell_bwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
-                                   h->stream, c);
+                if (fused && k < T - 1) {
+                    const float* dg_next = ((r.cell == RNN_GRU) ? gh : gates) + (long long)(t + dir) * B * GH;
+                    const dim3 grid((unsigned)((H + 31) / 32), (unsigned)((B + 31) / 32));
+                    if (G == 4)
+                        hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<4>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
+                                           c, dg_next, GH, (const float*)Rt);
+                    else if (G == 3)
+                        hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<3>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
+                                           c, dg_next, GH, (const float*)Rt);
+                    else
+                        hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<1>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
+                                           c, dg_next, GH, (const float*)Rt);
+                } else {
+                    hipLaunchKernelGGL(rnn_cell_bwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
+                                       h->stream, c);
+                }
                 st = hip_to_status(hipGetLastError());
                 if (st != SNHIP_STATUS_SUCCESS) return st;
                 if (k == 0 && dhx == nullptr) break;  // nobody asks for the gradient of the initial state
+                if (fused && k > 0) continue;         // the next launch multiplies by R itself
                 GemmArgs s;  // dh = d(R h)[:, t] . R  (GRU: added to dh * z)
                 s.M = B, s.N = H, s.K = (int)GH;
                 s.A = (r.cell == RNN_GRU) ? gh + (long long)t * B * 3 * H : gates + (long long)t * B * GH;

@@ -156,6 +156,8 @@ int hip_to_status(hipError_t e) {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+hipError_t rnn_prepare_kernels();  // rnn_layers.hpp: LDS opt-in of the recurrent step kernels
+
 struct Choice {
     int cfg;
     int splitk;
@@ -604,6 +606,8 @@ int snhip_create(void** handle) {
                                 c.lds_bytes);
         if (e != hipSuccess) return hip_to_status(e);
     }
+    e = rnn_prepare_kernels();
+    if (e != hipSuccess) return hip_to_status(e);
     Handle* h = new (std::nothrow) Handle();
     if (h == nullptr) return SNHIP_STATUS_ALLOC_FAILED;
     h->device = dev;
