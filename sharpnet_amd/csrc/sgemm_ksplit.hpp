@@ -1,0 +1,203 @@
+// fp32 GEMM for products with few output tiles and a K of up to about a thousand (a Dense layer on a small batch:
+// 128 x 256 x 784, 256 x 784 x 128; 512 x 512 x 512).  The tiled kernels of sgemm_mfma.hpp give
+// such a product a handful of workgroups, each walking a long k loop behind LDS barriers: 8-16 us for 3 us of
+// MFMA work, or a split-K launch plus a reduction launch.  Here a workgroup owns a 32 x 32 tile of C and splits K
+// over its four wavefronts instead; a wavefront works alone - whole-line global loads of its 32 x 32 operand
+// pieces, several groups of 32 k values in flight in registers, a private LDS patch to bring a group into MFMA
+// operand layout, v_mfma_f32_32x32x2_f32 on four independent accumulators - and the four partial tiles meet in
+// LDS once, where alpha, beta, the bias, the addend and the (leaky) ReLU are applied.  One launch, no workspace,
+// deterministic.
+//
+// Operands: op(A) is M x K, op(B) is K x N, row-major storage with row pitch lda / ldb.  An operand whose storage
+// is contiguous along k (A not transposed, B transposed) is fetched 16 bytes per lane along k; one that is
+// contiguous along its rows (A transposed, B not transposed) is fetched 16 bytes per lane along the rows and
+// transposed on its way into the patch.  Both need 16-byte aligned rows (the dispatcher checks pointers, pitches
+// and the contiguous extent); M, N are arbitrary, K is a multiple of 4.
+// Must be included by exactly one translation unit.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "sgemm_mfma.hpp"
+
+namespace snhip {
+
+struct KsplitCfg {
+    static constexpr int KS = 4;       // wavefronts = K slices
+    static constexpr int DEPTH = 4;    // groups of 32 k values in flight per wavefront
+    static constexpr int PITCH = 36;   // floats per patch row
+};
+
+// One operand of one wavefront: 32 rows (m or n) x the k range.
+//   KMAJOR = false: storage [row][k]; instruction i of a group reads row 8 i + lane / 8, k 4 (lane % 8) .. + 3.
+//   KMAJOR = true:  storage [k][row]; instruction i reads k 8 i + lane / 8, rows 4 (lane % 8) .. + 3.
+template <bool KMAJOR>
+struct KsplitOperand {
+    const float* ptr[4];   // address of the lane's vector of group 0, per instruction
+    long long step;        // floats between consecutive groups
+    bool row_ok[4];        // KMAJOR: the lane's four rows exist; else unused (rows are clamped instead)
+    int k_first[4];        // k of the lane's vector (element 0) within a group
+
+    __device__ __forceinline__ void init(const float* base, long long ld, int row0, int rows, int lane) {
+        const int lrow = lane >> 3, lcol = (lane & 7) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (KMAJOR) {
+                row_ok[i] = row0 + lcol < rows;                       // rows % 4 == 0: all four or none
+                k_first[i] = 8 * i + lrow;
+                ptr[i] = base + (long long)k_first[i] * ld + (row_ok[i] ? row0 + lcol : 0);
+            } else {
+                const int r = (row0 + 8 * i + lrow < rows) ? row0 + 8 * i + lrow : rows - 1;
+                row_ok[i] = true;
+                k_first[i] = lcol;
+                ptr[i] = base + (long long)r * ld + lcol;
+            }
+        }
+        step = KMAJOR ? 32 * ld : 32;
+    }
+    // the vector of group m; beyond K the address falls back to group 0 (always inside the matrix) and the value
+    // is discarded in `keep`
+    __device__ __forceinline__ f32x4 load(int i, int m, int K) const {
+        const bool ok = 32 * m + k_first[i] < K;
+        return *reinterpret_cast<const f32x4*>(ptr[i] + (ok ? (long long)m * step : 0));
+    }
+    __device__ __forceinline__ f32x4 keep(f32x4 v, int i, int m, int K) const {
+        const bool ok = (32 * m + k_first[i] < K) && row_ok[i];
+        f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
+        return ok ? v : z;
+    }
+    // registers -> patch[row][k]
+    __device__ __forceinline__ void to_patch(float* patch, int P, int i, int lane, f32x4 v) const {
+        const int lrow = lane >> 3, lcol = (lane & 7) * 4;
+        if constexpr (KMAJOR) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) patch[(lcol + e) * P + 8 * i + lrow] = v[e];
+        } else {
+            *reinterpret_cast<f32x4*>(patch + (8 * i + lrow) * P + lcol) = v;
+        }
+    }
+};
+
+template <bool TA, bool TB>
+__global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
+    using C = KsplitCfg;
+    constexpr int KS = C::KS, D = C::DEPTH, P = C::PITCH;
+    __shared__ float part[KS][32][33];
+    __shared__ __attribute__((aligned(16))) float patch[KS][2][32 * P];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
+    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+    const int m0 = tile_m * 32, n0 = tile_n * 32;
+    const int z = blockIdx.y;
+    const float* Ab = p.A + (long long)z * p.strideA;
+    const float* Bb = p.B + (long long)z * p.strideB;
+    float* Cb = p.C + (long long)z * p.strideC;
+
+    KsplitOperand<TA> oa;     // A transposed: stored K x M, contiguous along m
+    KsplitOperand<!TB> ob;    // B not transposed: stored K x N, contiguous along n
+    oa.init(Ab, p.lda, m0, p.M, lane);
+    ob.init(Bb, p.ldb, n0, p.N, lane);
+    float* pa = &patch[wave][0][0];
+    float* pb = &patch[wave][1][0];
+
+    const int K = p.K;
+    const int groups = (K + 31) / 32;
+    const int per = (groups + KS - 1) / KS;
+    const int mbeg = wave * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
+
+    f32x4 ra[D][4], rb[D][4], fa[2][4], fb[2][4];
+    f32x16 acc[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[e][r] = 0.0f;
+
+    auto load = [&](int slot, int m) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            ra[slot][i] = oa.load(i, m, K);
+            rb[slot][i] = ob.load(i, m, K);
+        }
+    };
+    // a group goes from its registers through the wavefront's LDS patch into operand layout (fragment buffer f);
+    // the fences keep the compiler from moving LDS accesses across the points where lanes exchange data
+    auto stage = [&](int slot, int m, int f) {
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            oa.to_patch(pa, P, i, lane, oa.keep(ra[slot][i], i, m, K));
+            ob.to_patch(pb, P, i, lane, ob.keep(rb[slot][i], i, m, K));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            fa[f][j] = *reinterpret_cast<const f32x4*>(pa + l32 * P + 16 * lhi + 4 * j);
+            fb[f][j] = *reinterpret_cast<const f32x4*>(pb + l32 * P + 16 * lhi + 4 * j);
+        }
+    };
+    auto multiply = [&](int f) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                acc[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[f][j][e], fb[f][j][e], acc[e], 0, 0, 0);
+    };
+
+    // blocks of D groups without a branch between a load and its use (exact s_waitcnt vmcnt(N)); the LDS round
+    // trip of group i + 1 is issued before the MFMAs of group i
+    const int cnt = mend > mbeg ? mend - mbeg : 0;
+    const int mmain = mbeg + (cnt / D) * D;
+    int m = mbeg;
+    if (m < mmain) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) load(d, m + d);
+        stage(0, m, 0);
+        for (; m + D < mmain; m += D) {
+            load(0, m + D);
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                stage((d + 1) % D, m + d + 1, (d + 1) % 2);
+                if (d + 1 < D) load(d + 1, m + d + 1 + D);
+                multiply(d % 2);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if (d + 1 < D) stage(d + 1, m + d + 1, (d + 1) % 2);
+            multiply(d % 2);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < D - 1; ++d)
+        if (mmain + d < mend) load(d, mmain + d);
+#pragma unroll
+    for (int d = 0; d < D - 1; ++d)
+        if (mmain + d < mend) {
+            stage(d, mmain + d, 0);
+            multiply(0);
+        }
+
+    // accumulator register r holds row 8 (r / 4) + 4 lhi + r % 4, column l32 of the tile
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        part[wave][8 * (r / 4) + 4 * lhi + (r % 4)][l32] = (acc[0][r] + acc[1][r]) + (acc[2][r] + acc[3][r]);
+    __syncthreads();
+
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int e = threadIdx.x + 256 * q;
+        const int lr = e >> 5, lc = e & 31;
+        const int row = m0 + lr, col = n0 + lc;
+        if (row >= p.M || col >= p.N) continue;
+        float v = (part[0][lr][lc] + part[1][lr][lc]) + (part[2][lr][lc] + part[3][lr][lc]);
+        v *= p.alpha;
+        if (p.ep.bias != nullptr) v += p.ep.bias[col];
+        float* c = Cb + (long long)row * p.ldc + col;
+        if (p.beta != 0.0f) v += p.beta * *c;
+        if (p.ep.addend != nullptr) v += p.ep.gamma * p.ep.addend[(long long)z * p.ep.strideD + (long long)row * p.ep.ldd + col];
+        if (p.ep.act == ACT_RELU || p.ep.act == ACT_LEAKY_RELU) v = leaky_relu(v, p.ep.act_param);
+        *c = v;
+    }
+}
+
+}  // namespace snhip

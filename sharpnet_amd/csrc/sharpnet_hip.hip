@@ -13,6 +13,7 @@
 #include "attention_mfma.hpp"
 #include "kernel_list.hpp"
 #include "rowops.hpp"
+#include "sgemm_ksplit.hpp"
 
 // The GEMM kernels are compiled in gemm_kernels.hip; here they are only declared.
 SNHIP_ALL_KERNEL_GROUPS(SNHIP_DECLARE_KERNELS)
@@ -115,8 +116,18 @@ const ConfigEntry kConfigs[] = {
     make_entry_bf16<BTileCfg<2, 2, 2, 2, 32>>(2, 0.60, 0.75, 1.3),   // 11: 128 x 128, BK 32
     make_entry_bf16<BTileCfg<2, 1, 2, 2, 64>>(2, 0.45, 0.60, 1.15),  // 12: 128 x 64, BK 64
     make_entry_bf16<BTileCfg<1, 1, 2, 2, 64>>(3, 0.45, 0.60, 1.1),   // 13: 64 x 64, BK 64
+    // K split over the wavefronts of a workgroup (sgemm_ksplit.hpp): not part of the cost model's search, see
+    // prefer_ksplit()
+    ConfigEntry{32, 32, 32, 256, 0, 1, 2,
+                {{sgemm_ksplit_kernel<false, false>, sgemm_ksplit_kernel<false, true>},
+                 {sgemm_ksplit_kernel<true, false>, sgemm_ksplit_kernel<true, true>}},
+                // the same kernels serve as the extended form: they always apply the addend and the (leaky) ReLU
+                {{sgemm_ksplit_kernel<false, false>, sgemm_ksplit_kernel<false, true>},
+                 {sgemm_ksplit_kernel<true, false>, sgemm_ksplit_kernel<true, true>}},
+                6, 0.5, 0.5, 1.0},  // 14: 32 x 32, four K slices
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
+constexpr int kKsplitConfig = kNumConfigs - 1;
 
 // Fused attention forward kernels (attention_mfma.hpp)
 struct AttnEntry {
@@ -211,7 +222,7 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
 }
 
 Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
-    Choice best{kind == 0 ? 6 : kNumConfigs - 1, 1};
+    Choice best{kind == 0 ? 6 : kKsplitConfig - 1, 1};
     double best_cost = 1e300;
     const bool forced = h->force_cfg >= 0 && kConfigs[h->force_cfg].kind == kind;
     for (int c = 0; c < kNumConfigs; ++c) {
@@ -341,6 +352,28 @@ struct GemmArgs {
     int math = -1;  // -1: the handle's math mode
 };
 
+// Whether the product goes to sgemm_ksplit_kernel (32 x 32 tiles, K split inside the workgroup) instead of the
+// configuration the cost model chose.  It needs 16-byte pieces along each operand's contiguous direction, and it
+// pays when the tiled kernels cannot fill the chip: few 32 x 32 tiles and a K of at least a few groups of 32.
+bool prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level, const Choice& chosen) {
+    if (math != SNHIP_MATH_FP32 || two_level || g.K < 32 || g.K % 4 != 0) return false;
+    if (h->force_cfg >= 0 && h->force_cfg != kKsplitConfig) return false;
+    const bool multi = g.batch > 1;
+    auto aligned = [&](const float* ptr, int ld, long long stride, bool rows_contiguous, int rows) {
+        return (uintptr_t)ptr % 16 == 0 && ld % 4 == 0 && (!multi || stride % 4 == 0) && (!rows_contiguous || rows % 4 == 0);
+    };
+    if (!aligned(g.A, g.lda, g.sA, g.tA, g.M) || !aligned(g.B, g.ldb, g.sB, !g.tB, g.N)) return false;
+    if (h->force_cfg == kKsplitConfig) return true;
+    if (h->force_splitk > 0) return false;
+    // Measured on MI355X: 128 x 256 x 784 8.8 us against 12.8 (64 x 64 tiles, split-K 4 + reduction), 128 x 784 x 256
+    // 5.5 against 10.5, 512^3 6.8 against 12.9; no gain once every compute unit has a tile of its own anyway
+    // (256 x 2048 x 512: 16.3 against 15.5) and a loss when a wavefront's share of K gets long (256 x 256 x 4096:
+    // 30.5 against 17.2 with split-K 16).
+    const long long tiles = (long long)ceil_div(g.M, 32) * ceil_div(g.N, 32) * g.batch;
+    (void)chosen;
+    return tiles <= (long long)h->num_cu && g.K <= 1024;
+}
+
 int gemm_core(Handle* h, const GemmArgs& g) {
     if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     const int math = (g.math < 0) ? h->math_mode : g.math;
@@ -433,6 +466,7 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     if (g.lda < (g.tA ? M : K) || g.ldb < (g.tB ? K : N)) return SNHIP_STATUS_INVALID_VALUE;
 
     Choice ch = choose(h, M, N, K, batch, math);
+    if (prefer_ksplit(h, g, math, two_level, ch)) ch = Choice{kKsplitConfig, 1};
     const ConfigEntry& cfg = kConfigs[ch.cfg];
     if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
 
@@ -459,7 +493,7 @@ int gemm_core(Handle* h, const GemmArgs& g) {
         }
         return SNHIP_STATUS_SUCCESS;
     }
-    const bool fuse_colsum = use_ext && g.colsum != nullptr && ch.splitk == 1 && g.tA && !g.tB;
+    const bool fuse_colsum = use_ext && g.colsum != nullptr && ch.splitk == 1 && g.tA && !g.tB && ch.cfg != kKsplitConfig;
     // what is left for a pass over C afterwards: sigmoid / tanh always, and addend / ReLU when the kernel is plain
     const float* addend_after = use_ext ? nullptr : ep.addend;
     const int act_after = (use_ext && relu_family) ? ACT_NONE : ep.act;

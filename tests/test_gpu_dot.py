@@ -474,3 +474,56 @@ def test_sgeam_transpose_and_sdgmm(oracle, gpu_wrapper):
     assert np.array_equal(gc.ToNumpy(), oracle.multiply_tensor(a, x_bc))
     ga.MultiplyTensor(ga, GPUTensor([4, 9, 1, 1], x_bc, w))             # in place
     assert np.array_equal(ga.ToNumpy(), oracle.multiply_tensor(a, x_bc))
+
+
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
+    """The kernel for products with few output tiles (32 x 32 tiles, K split over a workgroup's wavefronts): ragged
+    M and N, K tails that are not multiples of 32, alpha / beta, the fused bias, a strided batch; forced through the
+    tuning hook and picked automatically for a Dense layer on a small batch."""
+    from sharpnet_amd import GPUTensor
+    ks = [c["id"] for c in gpu_wrapper.configs() if c["kind"] == "fp32-ksplit"][0]
+    rng = np.random.default_rng(400 + 2 * tA + tB)
+    try:
+        for (M, N, K) in [(100, 36, 72), (36, 100, 264), (128, 256, 784), (260, 2048, 512), (4, 8, 36), (32, 32, 32),
+                          (64, 132, 1000)]:
+            a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
+            b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
+            c = random_tensor(rng, (M, N), -1, 1)
+            gpu_wrapper.set_tuning(ks, 1)
+            for alpha, beta in [(1.0, 0.0), (-0.5, 1.0), (0.25, -2.0)]:
+                ref = oracle.dot(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
+                got = gpu_dot(gpu_wrapper, a, tA, b, tB, alpha, beta, c=c) if beta != 0 else \
+                    gpu_dot(gpu_wrapper, a, tA, b, tB, alpha, beta, c_shape=[M, N], prefill=float("nan"))
+                assert gpu_wrapper.last_tuning() == (ks, 1), (M, N, K)
+                assert np.max(np.abs(got - ref)) <= tol(K, a, b, alpha, beta, c), (M, N, K, alpha, beta)
+        # strided batch + bias through the row-major entry point
+        batch, M, N, K = 3, 40, 52, 96
+        a = random_tensor(rng, (batch, K, M) if tA else (batch, M, K), -1, 1)
+        b = random_tensor(rng, (batch, N, K) if tB else (batch, K, N), -1, 1)
+        ga, gb = GPUTensor(a.shape, a, gpu_wrapper), GPUTensor(b.shape, b, gpu_wrapper)
+        gc = GPUTensor([batch, M, N], None, gpu_wrapper)
+        gc.SetValue(float("nan"))
+        gc.BatchMatrixMultiplication(ga, tA, gb, tB, 0.5, 0.0)
+        assert gpu_wrapper.last_tuning() == (ks, 1)
+        assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, tA, b, tB, 0.5))) <= tol(K, a, b, 0.5)
+        gpu_wrapper.set_tuning(-1, 0)
+        # automatic choice: the Dense layer of benchmark configuration 1 and a square product of one tile per CU
+        for (M, N, K) in [(128, 256, 784), (512, 512, 512)]:
+            a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
+            b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
+            got = gpu_dot(gpu_wrapper, a, tA, b, tB, 1.0, 0.0, c_shape=[M, N], prefill=float("nan"))
+            assert gpu_wrapper.last_tuning() == (ks, 1)
+            assert np.max(np.abs(got - oracle.dot(a, tA, b, tB))) <= tol(K, a, b)
+        # an operand view at an odd element offset cannot be read in 16-byte pieces: another kernel takes over
+        big = GPUTensor([128 * 784 + 1], None, gpu_wrapper)
+        big.ZeroMemory()
+        view = big.Slice(1, [128, 784])
+        w_ = random_tensor(rng, (256, 784), -1, 1)
+        gw = GPUTensor(w_.shape, w_, gpu_wrapper)
+        gy = GPUTensor([128, 256], None, gpu_wrapper)
+        gy.Dot(view, False, gw, True, 1.0, 0.0)
+        assert gpu_wrapper.last_tuning()[0] != ks
+        assert np.all(gy.ToNumpy() == 0.0)
+    finally:
+        gpu_wrapper.set_tuning(-1, 0)
