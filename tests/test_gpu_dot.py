@@ -527,3 +527,63 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
         assert np.all(gy.ToNumpy() == 0.0)
     finally:
         gpu_wrapper.set_tuning(-1, 0)
+
+
+def test_k_split_kernel_padded_pitches_fuzz(oracle, gpu_wrapper):
+    """Random small products through the descriptor call with padded row pitches, padded batch strides, bias, addend
+    and ReLU, forced onto the K-split kernel; operands sit in NaN-filled buffers so that any read outside a matrix
+    shows up in the result."""
+    from sharpnet_amd import GPUTensor
+    ks = [c["id"] for c in gpu_wrapper.configs() if c["kind"] == "fp32-ksplit"][0]
+    rng = np.random.default_rng(77)
+    used = 0
+    try:
+        gpu_wrapper.set_tuning(ks, 1)
+        for it in range(60):
+            tA, tB = bool(rng.integers(2)), bool(rng.integers(2))
+            M, N = int(rng.integers(1, 90)), int(rng.integers(1, 90))
+            if tA:
+                M = 4 * ((M + 3) // 4)
+            if not tB:
+                N = 4 * ((N + 3) // 4)
+            K = 4 * int(rng.integers(8, 80))
+            batch = int(rng.integers(1, 4))
+            ar, ac = (K, M) if tA else (M, K)
+            br, bc = (N, K) if tB else (K, N)
+            lda, ldb, ldc, ldd = ac + 4 * int(rng.integers(0, 3)), bc + 4 * int(rng.integers(0, 3)), N + int(rng.integers(0, 5)), \
+                N + int(rng.integers(0, 5))
+            sA, sB, sC, sD = ar * lda + 4 * int(rng.integers(0, 3)), br * ldb + 4 * int(rng.integers(0, 3)), M * ldc + 3, M * ldd + 1
+
+            def padded(rows, cols, ld, stride, lo=-1.0, hi=1.0):
+                buf = np.full(batch * stride + 8, np.nan, np.float32)
+                mats = rng.uniform(lo, hi, (batch, rows, cols)).astype(np.float32)
+                for z in range(batch):
+                    for r in range(rows):
+                        buf[z * stride + r * ld: z * stride + r * ld + cols] = mats[z, r]
+                return buf, mats
+            abuf, a = padded(ar, ac, lda, sA)
+            bbuf, b = padded(br, bc, ldb, sB)
+            cbuf, c = padded(M, N, ldc, sC)
+            dbuf, dmat = padded(M, N, ldd, sD)
+            bias = rng.uniform(-1, 1, N).astype(np.float32)
+            alpha, beta, gamma = float(rng.uniform(-1, 1)), float(rng.choice([0.0, 1.0, -0.5])), float(rng.choice([0.0, 0.75]))
+            relu = bool(rng.integers(2))
+            ga, gb, gc, gd, gbias = (GPUTensor([t.size], t, gpu_wrapper) for t in (abuf, bbuf, cbuf, dbuf, bias))
+            gc.GemmEx(transA=int(tA), transB=int(tB), M=M, N=N, K=K, alpha=alpha, beta=beta, A=ga, lda=lda, strideA=sA, B=gb,
+                      ldb=ldb, strideB=sB, ldc=ldc, strideC=sC, batch=batch, bias=gbias, D=gd, ldd=ldd, strideD=sD, gamma=gamma,
+                      activation=1 if relu else 0)
+            used += gpu_wrapper.last_tuning()[0] == ks
+            out = gc.ToNumpy()
+            for z in range(batch):
+                ref = oracle.dot_f64(a[z], tA, b[z], tB, alpha, 0.0) + bias[None, :] + beta * c[z] + gamma * dmat[z]
+                if relu:
+                    ref = np.maximum(ref, 0.0)
+                got = np.stack([out[z * sC + r * ldc: z * sC + r * ldc + N] for r in range(M)])
+                assert np.all(np.isfinite(got)), (it, tA, tB, M, N, K)
+                assert np.max(np.abs(got - ref)) <= tol(K, a, b, alpha) + 1e-5, (it, tA, tB, M, N, K, batch)
+                # the gaps between rows stay untouched
+                if ldc > N:
+                    assert np.all(np.isnan(out[z * sC + N: z * sC + ldc]))
+        assert used >= 50, used
+    finally:
+        gpu_wrapper.set_tuning(-1, 0)
