@@ -380,14 +380,18 @@ int snhip_device_info(void* handle, int info[6]);
 int snhip_set_tuning(void* handle, int config, int splitk);
 int snhip_get_last_tuning(void* handle, int* config, int* splitk);
 /* What the automatic choice would be for a row-major M x N x K product of `batch` matrices (no launch, no
- * device access).  handle may be NULL: the model then assumes an MI355X (256 CUs) and no overrides. */
+ * device access).  handle may be NULL: the model then assumes an MI355X (256 CUs) and no overrides.  The answer is
+ * the tiled kernels' cost model; whether the K-split kernel (kind 2) takes a small product over also depends on the
+ * operands' alignment, which this call does not see. */
 int snhip_query_tuning(void* handle, int m, int n, int k, int batch, int math_mode, int* config, int* splitk);
 /* How split-K partial sums are added: 0 = automatic (currently always a second kernel, the faster
  * choice on MI355X), 1 = a second kernel, 2 = in the GEMM kernel by the last workgroup to arrive for
  * its tile.  The order of summation is fixed in both, so results are run-to-run identical either way. */
 int snhip_set_splitk_mode(void* handle, int mode);
 int snhip_config_count(void);
-/* desc[0..5] = BM, BN, BK, threads, LDS bytes, kind (0 fp32 kernel, 1 bf16-input kernel) */
+/* desc[0..5] = BM, BN, BK, threads, dynamic LDS bytes, kind (0 fp32 tiled kernel, 1 bf16-input kernel, 2 fp32 kernel
+ * with 32 x 32 tiles and K split over the wavefronts of a workgroup: chosen by itself for products with few output
+ * tiles, never part of a split-K launch, used only when the operands can be read in 16-byte pieces) */
 int snhip_config_desc(int config, int desc[6]);
 
 #ifdef __cplusplus
