@@ -337,39 +337,50 @@ __global__ void __launch_bounds__(256) rnn_cell_bwd_kernel(const RnnStepBwd s) {
 
 // One backward time step in one launch: dh = d(R h + bR)[step after] . R, then the cell gradient of this step.
 //
-// The product is batch x H x G*H (256 x 512 x 2048): 128 tiles of 32 x 32 with a long K.  A workgroup of eight
-// wavefronts owns one tile (32 samples x 32 hidden units) and gives each wavefront an eighth of K
-// (wave_product_32x32 on rows of d(gates) and rows of R^T, which the caller lays out once per call), so the chip
-// holds 1024 chains of 128 MFMAs as in the forward kernel.  The partial tiles meet in LDS; each thread then owns two
-// (sample, unit) pairs, adds the gradient arriving from the layer above (and, for the GRU, dh * z carried over
-// from the step after) and does what rnn_cell_bwd_kernel does, with its inputs fetched before the main loop.
-// `dg_next` is the d(R h + bR) the step after (in time order of this direction) left behind.
+// The product is batch x H x G*H (256 x 512 x 2048): few output elements, a long K.  A workgroup of eight
+// wavefronts owns 32 samples x 16 hidden units and gives each wavefront an eighth of K, so that the chip holds 256
+// workgroups (one per compute unit, two wavefronts per SIMD).  With 16 columns the tile is built from
+// v_mfma_f32_16x16x4_f32: per group of 32 k values a wavefront loads 32 rows of d(gates) and 16 rows of R^T (which
+// the caller lays out once per call) with whole-line loads, passes them through its private LDS patches, and issues
+// 16 MFMAs (two 16 x 16 tiles x 8 k steps) on four independent accumulators.  The partial tiles meet in LDS; each
+// thread then owns one (sample, unit) pair, adds the gradient arriving from the layer above (and, for the GRU,
+// dh * z carried over from the step after) and does what rnn_cell_bwd_kernel does, with its inputs fetched before
+// the main loop.  `dg_next` is the d(R h + bR) the step after (in time order of this direction) left behind.
 struct RnnBwdFusedCfg {
     static constexpr int KS = 8;
-    static constexpr int DEPTH = 2;   // two wavefronts per SIMD: 256 registers each
+    static constexpr int DEPTH = 4;
     static constexpr int PITCH = 36;
-    static constexpr int LDS_BYTES = (KS * 2 * 32 * PITCH + KS * 32 * 33) * 4;
+    static constexpr int U = 16;                                       // hidden units per workgroup
+    static constexpr int PATCH = (32 + U) * PITCH;                     // floats per wavefront: d(gates) rows, R^T rows
+    static constexpr int LDS_BYTES = (KS * PATCH + KS * 32 * (U + 1)) * 4;
 };
+
+typedef float f32x4_acc __attribute__((ext_vector_type(4)));
 
 template <int G>
 __global__ void __launch_bounds__(512) rnn_step_bwd_fused_kernel(const RnnStepBwd s, const float* __restrict__ dg_next,
                                                                  long long ld_dg, const float* __restrict__ Rt) {
     using C = RnnBwdFusedCfg;
-    constexpr int KS = C::KS, D = C::DEPTH, P = C::PITCH;
+    constexpr int KS = C::KS, D = C::DEPTH, P = C::PITCH, U = C::U;
     extern __shared__ __attribute__((aligned(16))) float lds_bwd[];
-    float* patch = lds_bwd;                                   // [KS][2][32 * P]
-    float(*part)[32][33] = reinterpret_cast<float(*)[32][33]>(lds_bwd + KS * 2 * 32 * P);   // [KS][32][33]
+    float(*part)[32][U + 1] = reinterpret_cast<float(*)[32][U + 1]>(lds_bwd + KS * C::PATCH);   // [KS][32][U + 1]
     const int H = s.hidden, GH = G * H;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
-    const int row0 = blockIdx.y * 32, u0 = blockIdx.x * 32;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l16 = lane & 15, lq = lane >> 4;
+    const int row0 = blockIdx.y * 32, u0 = blockIdx.x * U;
+    float* pa = lds_bwd + wave * C::PATCH;      // 32 rows of d(gates)
+    float* pb = pa + 32 * P;                    // U rows of R^T
 
+    // global side: instruction i of a group fetches row 8 i + lane / 8, floats 4 (lane % 8) .. + 3
     const int lrow = lane >> 3, lcol = (lane & 7) * 4;
     const float* ap[4];
-    const float* bp[4];
+    const float* bp[2];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int ar = (row0 + 8 * i + lrow < s.batch) ? row0 + 8 * i + lrow : s.batch - 1;
         ap[i] = dg_next + (long long)ar * ld_dg + lcol;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
         const int unit = (u0 + 8 * i + lrow < H) ? u0 + 8 * i + lrow : H - 1;
         bp[i] = Rt + (long long)unit * GH + lcol;
     }
@@ -377,13 +388,13 @@ __global__ void __launch_bounds__(512) rnn_step_bwd_fused_kernel(const RnnStepBw
     const int per = (groups + KS - 1) / KS;
     const int mbeg = wave * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
 
-    // inputs of the cell gradient: thread -> pairs p = threadIdx.x + 512 q of the tile's 32 x 32 (sample, unit) pairs
-    constexpr int Q = 2;
+    // inputs of the cell gradient: thread -> pair p = threadIdx.x of the tile's 32 x 16 (sample, unit) pairs
+    constexpr int Q = 1;
     float gv[Q][G], dyv[Q], dhv[Q], av[Q], bv[Q], cv[Q];
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
         const int p = threadIdx.x + 512 * q;
-        const int b = row0 + p / 32, j = u0 + p % 32;
+        const int b = row0 + p / U, j = u0 + p % U;
         const bool ok = b < s.batch && j < H;
         const long long idx = (long long)b * H + j;
 #pragma unroll
@@ -404,22 +415,96 @@ __global__ void __launch_bounds__(512) rnn_step_bwd_fused_kernel(const RnnStepBw
         }
     }
 
-    f32x16 acc[4];
-    wave_product_32x32<D, P>(ap, bp, mbeg, mend, patch + (wave * 2) * 32 * P, patch + (wave * 2 + 1) * 32 * P, lane, acc);
+    // main loop: as wave_product_32x32, with 16 x 16 x 4 MFMAs.  A lane reads from the patches the four consecutive
+    // k values 16 j + 4 (lane / 16) .. + 3 of its row; element e of that vector feeds the MFMA whose four k are
+    // 16 j + e, + 4, + 8, + 12 (lane / 16 picks one of them) - the same for both operands.
+    f32x4 ra[D][4], rb[D][2], fa[2][2][2], fb[2][2];
+    f32x4_acc acc[2][2];
 #pragma unroll
-    for (int r = 0; r < 16; ++r)
-        part[wave][8 * (r / 4) + 4 * lhi + (r % 4)][l32] = (acc[0][r] + acc[1][r]) + (acc[2][r] + acc[3][r]);
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) acc[hh][c] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+    auto load = [&](int slot, int m) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ra[slot][i] = *reinterpret_cast<const f32x4*>(ap[i] + m * 32);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) rb[slot][i] = *reinterpret_cast<const f32x4*>(bp[i] + m * 32);
+    };
+    auto stage = [&](int slot, int f) {
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4*>(pa + (8 * i + lrow) * P + lcol) = ra[slot][i];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<f32x4*>(pb + (8 * i + lrow) * P + lcol) = rb[slot][i];
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh)
+                fa[f][hh][j] = *reinterpret_cast<const f32x4*>(pa + (16 * hh + l16) * P + 16 * j + 4 * lq);
+            fb[f][j] = *reinterpret_cast<const f32x4*>(pb + l16 * P + 16 * j + 4 * lq);
+        }
+    };
+    auto multiply = [&](int f) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh)
+                    acc[hh][e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[f][hh][j][e], fb[f][j][e], acc[hh][e & 1], 0, 0, 0);
+    };
+    {
+        const int cnt = mend > mbeg ? mend - mbeg : 0;
+        const int mmain = mbeg + (cnt / D) * D;
+        int m = mbeg;
+        if (m < mmain) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) load(d, m + d);
+            stage(0, 0);
+            for (; m + D < mmain; m += D) {
+                load(0, m + D);
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    stage((d + 1) % D, (d + 1) % 2);
+                    if (d + 1 < D) load(d + 1, m + d + 1 + D);
+                    multiply(d % 2);
+                }
+            }
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                if (d + 1 < D) stage(d + 1, (d + 1) % 2);
+                multiply(d % 2);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D - 1; ++d)
+            if (mmain + d < mend) load(d, mmain + d);
+#pragma unroll
+        for (int d = 0; d < D - 1; ++d)
+            if (mmain + d < mend) {
+                stage(d, 0);
+                multiply(0);
+            }
+    }
+    // accumulator register r of a 16 x 16 tile holds row 4 (lane / 16) + r, column lane % 16
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) part[wave][16 * hh + 4 * lq + r][l16] = acc[hh][0][r] + acc[hh][1][r];
     __syncthreads();
 
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
         const int p = threadIdx.x + 512 * q;
-        const int lr = p / 32, b = row0 + lr, j = u0 + p % 32;
+        const int lr = p / U, b = row0 + lr, j = u0 + p % U;
         if (b >= s.batch || j >= H) continue;
         const long long idx = (long long)b * H + j;
         float rec = 0.0f;
 #pragma unroll
-        for (int k = 0; k < KS; ++k) rec += part[k][lr][p % 32];
+        for (int k = 0; k < KS; ++k) rec += part[k][lr][p % U];
         const float dh = rec + dhv[q] + dyv[q];
         float* g = s.gates + b * s.ld_gates;
         if constexpr (G == 1) {

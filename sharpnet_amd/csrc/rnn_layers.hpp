@@ -370,7 +370,7 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
                 c.batch = B, c.hidden = H, c.cell = r.cell;
                 if (fused && k < T - 1) {
                     const float* dg_next = ((r.cell == RNN_GRU) ? gh : gates) + (long long)(t + dir) * B * GH;
-                    const dim3 grid((unsigned)((H + 31) / 32), (unsigned)((B + 31) / 32));
+                    const dim3 grid((unsigned)((H + RnnBwdFusedCfg::U - 1) / RnnBwdFusedCfg::U), (unsigned)((B + 31) / 32));
                     if (G == 4)
                         hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<4>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
                                            c, dg_next, GH, (const float*)Rt);
