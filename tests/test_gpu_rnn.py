@@ -234,3 +234,30 @@ def test_rnn_argument_checks(gpu_wrapper):
     # empty problems are no-ops
     check(lib.snhip_rnn_forward(gpu_wrapper.handle, ctypes.byref(d), 1, 0, 3, None, None, None, None, None, None, None,
                                 None, 0, None, 0), "empty batch")
+
+
+@pytest.mark.parametrize("cell", [ro.LSTM, ro.GRU])
+def test_full_size_layer_properties(gpu_wrapper, cell):
+    """Benchmark configuration 4's shape (batch 256, 128 steps, 256 -> 512), too large for the oracle: the two forms
+    of the time step (one launch / separate launches) agree on values and on every gradient, the final state equals
+    the last step of y, and a second run reproduces the first bit for bit."""
+    rng = np.random.default_rng(40 + cell)
+    B, Tn, I, H = 256, 128, 256, 512
+    desc = ro.RnnDesc(cell, input_size=I, hidden_size=H, num_layers=1, bidirectional=False, bias_mode=ro.DOUBLE_BIAS)
+    weights = rng.uniform(-0.04, 0.04, ro.weight_space_size(desc)).astype(np.float32)
+    x = rng.uniform(-1, 1, (B, Tn, I)).astype(np.float32)
+    dy = rng.uniform(-0.01, 0.01, (B, Tn, H)).astype(np.float32)
+    one = run_gpu(gpu_wrapper, desc, x, weights, dy)
+    again = run_gpu(gpu_wrapper, desc, x, weights, dy)
+    for key in ("y", "hy", "dx", "dw"):
+        assert np.array_equal(one[key], again[key]), key
+    assert np.array_equal(one["hy"][0], one["y"][:, -1, :])
+    check(gpu_wrapper.lib.snhip_rnn_set_step_mode(gpu_wrapper.handle, 1), "step mode")
+    try:
+        two = run_gpu(gpu_wrapper, desc, x, weights, dy)
+    finally:
+        check(gpu_wrapper.lib.snhip_rnn_set_step_mode(gpu_wrapper.handle, 0), "step mode")
+    assert np.max(np.abs(one["y"] - two["y"])) <= 1e-4
+    for key in ("dx", "dw", "dhx"):
+        scale = max(1.0, float(np.max(np.abs(two[key]))))
+        assert np.max(np.abs(one[key] - two[key])) <= 2e-4 * scale, key
