@@ -151,8 +151,8 @@ def test_config5_attention_batched(oracle, gpu_wrapper, bf16):
 
 
 def test_calls_can_be_recorded_into_a_hip_graph_and_replayed(oracle, gpu_wrapper):
-    """A Dense forward (fused bias + ReLU), a split-K product, a fill and the one-launch attention, recorded into a HIP
-    graph on a capturing stream and replayed three times with eager work and synchronisations in between: every
+    """An LSTM forward + backward, a Dense forward (fused bias + ReLU), a split-K product, a fill and the one-launch
+    attention, recorded into a HIP graph on a capturing stream and replayed three times with eager work and synchronisations in between: every
     replay must reproduce the eager results (the calls launch kernels only: no allocation once the split-K workspace
     exists, no memset nodes)."""
     import ctypes
@@ -168,7 +168,27 @@ def test_calls_can_be_recorded_into_a_hip_graph_and_replayed(oracle, gpu_wrapper
     gy, gc2, go, gfill = GPUTensor([96, 130], None, w), GPUTensor([64, 48], None, w), GPUTensor([6, 50, 16], None, w), \
         GPUTensor([1000], None, w)
 
+    # a small LSTM (hidden size 32: the one-launch step kernels) with caller-owned workspace and reserve buffers
+    from sharpnet_amd.hiplib import RnnDesc
+    rd = RnnDesc(cell_mode=2, bias_mode=2, bidirectional=1, num_layers=1, input_size=12, hidden_size=32)
+    nb, wsb, rsb = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    check_status(w.lib.snhip_rnn_weight_space_size(ctypes.byref(rd), ctypes.byref(nb)), "rnn weight space")
+    check_status(w.lib.snhip_rnn_temp_space_sizes(ctypes.byref(rd), 1, 9, 5, ctypes.byref(wsb), ctypes.byref(rsb)), "rnn sizes")
+    rx, rw, rdy = random_tensor(rng, (9, 5, 12), -1, 1), random_tensor(rng, (nb.value // 4,), -0.3, 0.3), \
+        random_tensor(rng, (9, 5, 64), -1, 1)
+    grx, grw, grdy = (GPUTensor(list(t.shape), t, w) for t in (rx, rw, rdy))
+    gry, grdx, grws, grrs = GPUTensor([9, 5, 64], None, w), GPUTensor([9, 5, 12], None, w), \
+        GPUTensor([wsb.value // 4], None, w), GPUTensor([rsb.value // 4], None, w)
+
+    def rnn():
+        check_status(w.lib.snhip_rnn_forward(w.handle, ctypes.byref(rd), 1, 9, 5, grx.Pointer, gry.Pointer, None, None, None,
+                                             None, grw.Pointer, grws.Pointer, wsb.value, grrs.Pointer, rsb.value), "rnn forward")
+        check_status(w.lib.snhip_rnn_backward_data(w.handle, ctypes.byref(rd), 9, 5, gry.Pointer, grdy.Pointer, grdx.Pointer,
+                                                   None, None, None, None, None, None, grw.Pointer, grws.Pointer, wsb.value,
+                                                   grrs.Pointer, rsb.value), "rnn backward")
+
     def work():
+        rnn()
         linear.DenseForwardPropagation(gy, gx, gW, gb, False, activation="CUDNN_ACTIVATION_RELU")
         gc2.Dot(ga2, False, gb2, False, 1.0, 0.0)
         gfill.SetValue(3.5)
@@ -176,7 +196,7 @@ def test_calls_can_be_recorded_into_a_hip_graph_and_replayed(oracle, gpu_wrapper
                                                  scale=0.25, is_causal=True, packed=False)
 
     def results():
-        return [t.ToNumpy().copy() for t in (gy, gc2, go, gfill)]
+        return [t.ToNumpy().copy() for t in (gy, gc2, go, gfill, gry, grdx)]
 
     work()                                   # eager: also sizes the split-K workspace
     w.synchronize()
@@ -205,7 +225,7 @@ def test_calls_can_be_recorded_into_a_hip_graph_and_replayed(oracle, gpu_wrapper
             assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
         assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, 0) == 0
         for rep in range(3):
-            for t in (gy, gc2, go, gfill):   # eager work between replays: wipe the outputs on the same stream
+            for t in (gy, gc2, go, gfill, gry, grdx):   # eager work between replays: wipe the outputs on the same stream
                 t.SetValue(float("nan"))
             w.synchronize()
             assert hip.hipGraphLaunch(graph_exec, stream) == 0
