@@ -29,7 +29,7 @@ def check(st, what):
     check_status(st, what)
 
 
-def run_gpu(w, desc, x, weights, dy, hx=None, cx=None, dhy=None, dcy=None, training=True):
+def run_gpu(w, desc, x, weights, dy, hx=None, cx=None, dhy=None, dcy=None, training=True, want_dstate=True):
     """Forward (+ backward when training) through the C ABI; returns dict of numpy arrays."""
     from sharpnet_amd import GPUTensor
     lib, d = w.lib, lib_desc(desc)
@@ -63,7 +63,8 @@ def run_gpu(w, desc, x, weights, dy, hx=None, cx=None, dhy=None, dcy=None, train
     gdhy = T(w, dhy) if dhy is not None else None
     gdcy = T(w, dcy) if dcy is not None else None
     check(lib.snhip_rnn_backward_data(w.handle, ctypes.byref(d), B, Tn, gy.Pointer, gdy.Pointer, gdx.Pointer, ptr(ghx),
-                                      ptr(gdhy), gdhx.Pointer, ptr(gcx), ptr(gdcy), gdcx.Pointer, gw.Pointer, gws.Pointer,
+                                      ptr(gdhy), gdhx.Pointer if want_dstate else None, ptr(gcx), ptr(gdcy),
+                                      gdcx.Pointer if want_dstate else None, gw.Pointer, gws.Pointer,
                                       ws.value, grs.Pointer, rs.value), "snhip_rnn_backward_data")
     gdw = GPUTensor([weights.size], None, w)
     gdw.ZeroMemory()
@@ -143,6 +144,9 @@ def test_cells_one_launch_per_step(gpu_wrapper, cell, hidden, batch):
         cx = dcy = None
     got = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy)
     compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, 5e-5)
+    # without the gradients of the initial states (what a layer inside a network asks for): same dx and dw
+    plain = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy, want_dstate=False)
+    assert np.array_equal(plain["dx"], got["dx"]) and np.array_equal(plain["dw"], got["dw"])
     check(gpu_wrapper.lib.snhip_rnn_set_step_mode(gpu_wrapper.handle, 1), "step mode")
     try:
         two = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy)
