@@ -10,8 +10,8 @@
 //
 // Operands: op(A) is M x K, op(B) is K x N, row-major storage with row pitch lda / ldb.  An operand whose storage
 // is contiguous along k (A not transposed, B transposed) is fetched 16 bytes per lane along k; one that is
-// contiguous along its rows (A transposed, B not transposed) is fetched 16 bytes per lane along the rows and
-// transposed on its way into the patch.  Both need 16-byte aligned rows (the dispatcher checks pointers, pitches
+// contiguous along its rows (A transposed, B not transposed) is fetched 16 bytes per lane along the rows, kept in
+// that orientation in the patch and transposed by the reads.  Both need 16-byte aligned rows (the dispatcher checks pointers, pitches
 // and the contiguous extent); M, N are arbitrary, K is a multiple of 4.
 // Must be included by exactly one translation unit.
 #pragma once
@@ -21,10 +21,17 @@
 
 namespace snhip {
 
+// GemmParams::flags bit of this kernel (next to GEMM_FLAG_C_VEC / GEMM_FLAG_WS_VEC of the tiled kernels): the
+// column-tile index runs fastest in blockIdx.x
+constexpr int GEMM_FLAG_TILE_N_FASTEST = 4;
+
+// NT: 32-column tiles per workgroup (1 or 2); the four wavefronts are NT tiles x 4 / NT slices of K.
+template <int NT_>
 struct KsplitCfg {
-    static constexpr int KS = 4;       // wavefronts = K slices
-    static constexpr int DEPTH = 4;    // groups of 32 k values in flight per wavefront
-    static constexpr int PITCH = 36;   // floats per patch row
+    static constexpr int NT = NT_;
+    static constexpr int KS = 4 / NT_;  // K slices
+    static constexpr int DEPTH = 4;     // groups of 32 k values in flight per wavefront
+    static constexpr int PITCH = 36;    // floats per patch row
 };
 
 // One operand of one wavefront: 32 rows (m or n) x the k range.
@@ -65,27 +72,42 @@ struct KsplitOperand {
         f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
         return ok ? v : z;
     }
-    // registers -> patch[row][k]
+    // registers -> patch, in the orientation of the storage: patch[row][k], or patch[k][row] for KMAJOR (either way
+    // one 16-byte store per vector, eight lanes per 128-byte line)
     __device__ __forceinline__ void to_patch(float* patch, int P, int i, int lane, f32x4 v) const {
         const int lrow = lane >> 3, lcol = (lane & 7) * 4;
+        *reinterpret_cast<f32x4*>(patch + (8 * i + lrow) * P + lcol) = v;
+    }
+    // MFMA operand piece of a lane: row lane % 32, k = 16 (lane / 32) + 4 j .. + 3.  One 16-byte read from
+    // patch[row][k]; four 4-byte reads from patch[k][row] (consecutive lanes on consecutive banks).
+    __device__ __forceinline__ f32x4 fragment(const float* patch, int P, int lane, int j) const {
+        const int l32 = lane & 31, lhi = lane >> 5;
         if constexpr (KMAJOR) {
+            f32x4 v;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) patch[(lcol + e) * P + 8 * i + lrow] = v[e];
+            for (int e = 0; e < 4; ++e) v[e] = patch[(16 * lhi + 4 * j + e) * P + l32];
+            return v;
         } else {
-            *reinterpret_cast<f32x4*>(patch + (8 * i + lrow) * P + lcol) = v;
+            return *reinterpret_cast<const f32x4*>(patch + l32 * P + 16 * lhi + 4 * j);
         }
     }
 };
 
-template <bool TA, bool TB>
+template <bool TA, bool TB, int NT = 1>
 __global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
-    using C = KsplitCfg;
+    using C = KsplitCfg<NT>;
     constexpr int KS = C::KS, D = C::DEPTH, P = C::PITCH;
-    __shared__ float part[KS][32][33];
-    __shared__ __attribute__((aligned(16))) float patch[KS][2][32 * P];
+    __shared__ float part[KS][NT][32][33];
+    __shared__ __attribute__((aligned(16))) float patch[4][2][32 * P];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
-    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
-    const int m0 = tile_m * 32, n0 = tile_n * 32;
+    const int nt = wave % NT, kg = wave / NT;
+    // Workgroups go to the eight XCDs round-robin by their linear index.  The index that runs fastest spreads over
+    // the XCDs, the other one stays put (when the fast count is a multiple of 8): the dispatcher lets the tiles of
+    // the smaller operand run fastest, so that each XCD's L2 fetches its own part of the larger operand only once.
+    const bool n_fastest = (p.flags & GEMM_FLAG_TILE_N_FASTEST) != 0;
+    const int tile_m = n_fastest ? blockIdx.x / p.tiles_n : blockIdx.x % p.tiles_m;
+    const int tile_n = n_fastest ? blockIdx.x % p.tiles_n : blockIdx.x / p.tiles_m;
+    const int m0 = tile_m * 32, n0 = tile_n * (32 * NT) + 32 * nt;
     const int z = blockIdx.y;
     const float* Ab = p.A + (long long)z * p.strideA;
     const float* Bb = p.B + (long long)z * p.strideB;
@@ -101,7 +123,7 @@ __global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
     const int K = p.K;
     const int groups = (K + 31) / 32;
     const int per = (groups + KS - 1) / KS;
-    const int mbeg = wave * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
+    const int mbeg = kg * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
 
     f32x4 ra[D][4], rb[D][4], fa[2][4], fb[2][4];
     f32x16 acc[4];
@@ -131,8 +153,8 @@ __global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            fa[f][j] = *reinterpret_cast<const f32x4*>(pa + l32 * P + 16 * lhi + 4 * j);
-            fb[f][j] = *reinterpret_cast<const f32x4*>(pb + l32 * P + 16 * lhi + 4 * j);
+            fa[f][j] = oa.fragment(pa, P, lane, j);
+            fb[f][j] = ob.fragment(pb, P, lane, j);
         }
     };
     auto multiply = [&](int f) {
@@ -180,16 +202,19 @@ __global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
     // accumulator register r holds row 8 (r / 4) + 4 lhi + r % 4, column l32 of the tile
 #pragma unroll
     for (int r = 0; r < 16; ++r)
-        part[wave][8 * (r / 4) + 4 * lhi + (r % 4)][l32] = (acc[0][r] + acc[1][r]) + (acc[2][r] + acc[3][r]);
+        part[kg][nt][8 * (r / 4) + 4 * lhi + (r % 4)][l32] = (acc[0][r] + acc[1][r]) + (acc[2][r] + acc[3][r]);
     __syncthreads();
 
+    const int nbase = tile_n * (32 * NT);
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < 4 * NT; ++q) {
         const int e = threadIdx.x + 256 * q;
-        const int lr = e >> 5, lc = e & 31;
-        const int row = m0 + lr, col = n0 + lc;
+        const int lr = e / (32 * NT), lc = e % (32 * NT);
+        const int row = m0 + lr, col = nbase + lc;
         if (row >= p.M || col >= p.N) continue;
-        float v = (part[0][lr][lc] + part[1][lr][lc]) + (part[2][lr][lc] + part[3][lr][lc]);
+        float v = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KS; ++k) v += part[k][lc / 32][lr][lc % 32];
         v *= p.alpha;
         if (p.ep.bias != nullptr) v += p.ep.bias[col];
         float* c = Cb + (long long)row * p.ldc + col;

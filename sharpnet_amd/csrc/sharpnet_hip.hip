@@ -125,9 +125,15 @@ const ConfigEntry kConfigs[] = {
                 {{sgemm_ksplit_kernel<false, false>, sgemm_ksplit_kernel<false, true>},
                  {sgemm_ksplit_kernel<true, false>, sgemm_ksplit_kernel<true, true>}},
                 6, 0.5, 0.5, 1.0},  // 14: 32 x 32, four K slices
+    ConfigEntry{32, 64, 32, 256, 0, 1, 2,
+                {{sgemm_ksplit_kernel<false, false, 2>, sgemm_ksplit_kernel<false, true, 2>},
+                 {sgemm_ksplit_kernel<true, false, 2>, sgemm_ksplit_kernel<true, true, 2>}},
+                {{sgemm_ksplit_kernel<false, false, 2>, sgemm_ksplit_kernel<false, true, 2>},
+                 {sgemm_ksplit_kernel<true, false, 2>, sgemm_ksplit_kernel<true, true, 2>}},
+                6, 0.5, 0.5, 1.0},  // 15: 32 x 64 (two column tiles), two K slices
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
-constexpr int kKsplitConfig = kNumConfigs - 1;
+constexpr int kKsplitConfig = kNumConfigs - 2;   // and kKsplitConfig + 1
 
 // Fused attention forward kernels (attention_mfma.hpp)
 struct AttnEntry {
@@ -355,23 +361,25 @@ struct GemmArgs {
 // Whether the product goes to sgemm_ksplit_kernel (32 x 32 tiles, K split inside the workgroup) instead of the
 // configuration the cost model chose.  It needs 16-byte pieces along each operand's contiguous direction, and it
 // pays when the tiled kernels cannot fill the chip: few 32 x 32 tiles and a K of at least a few groups of 32.
-bool prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level, const Choice& chosen) {
-    if (math != SNHIP_MATH_FP32 || two_level || g.K < 32 || g.K % 4 != 0) return false;
-    if (h->force_cfg >= 0 && h->force_cfg != kKsplitConfig) return false;
+int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) {
+    if (math != SNHIP_MATH_FP32 || two_level || g.K < 32 || g.K % 4 != 0) return -1;
+    const bool forced = h->force_cfg == kKsplitConfig || h->force_cfg == kKsplitConfig + 1;
+    if (h->force_cfg >= 0 && !forced) return -1;
     const bool multi = g.batch > 1;
     auto aligned = [&](const float* ptr, int ld, long long stride, bool rows_contiguous, int rows) {
         return (uintptr_t)ptr % 16 == 0 && ld % 4 == 0 && (!multi || stride % 4 == 0) && (!rows_contiguous || rows % 4 == 0);
     };
-    if (!aligned(g.A, g.lda, g.sA, g.tA, g.M) || !aligned(g.B, g.ldb, g.sB, !g.tB, g.N)) return false;
-    if (h->force_cfg == kKsplitConfig) return true;
-    if (h->force_splitk > 0) return false;
+    if (!aligned(g.A, g.lda, g.sA, g.tA, g.M) || !aligned(g.B, g.ldb, g.sB, !g.tB, g.N)) return -1;
+    if (forced) return h->force_cfg;
+    if (h->force_splitk > 0 || g.K > 1024) return -1;
     // Measured on MI355X: 128 x 256 x 784 8.8 us against 12.8 (64 x 64 tiles, split-K 4 + reduction), 128 x 784 x 256
-    // 5.5 against 10.5, 512^3 6.8 against 12.9; no gain once every compute unit has a tile of its own anyway
-    // (256 x 2048 x 512: 16.3 against 15.5) and a loss when a wavefront's share of K gets long (256 x 256 x 4096:
-    // 30.5 against 17.2 with split-K 16).
-    const long long tiles = (long long)ceil_div(g.M, 32) * ceil_div(g.N, 32) * g.batch;
-    (void)chosen;
-    return tiles <= (long long)h->num_cu && g.K <= 1024;
+    // 5.5 against 10.5, 512^3 6.8 against 12.9; a loss when a wavefront's share of K gets long (256 x 256 x 4096:
+    // 30.5 against 17.2 with split-K 16).  Up to one 32 x 32 tile per compute unit: four K slices; up to one
+    // 32 x 64 tile per compute unit: two.
+    const long long rows32 = (long long)ceil_div(g.M, 32) * g.batch;
+    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu) return kKsplitConfig;
+    if (rows32 * ceil_div(g.N, 64) <= (long long)h->num_cu) return kKsplitConfig + 1;
+    return -1;
 }
 
 int gemm_core(Handle* h, const GemmArgs& g) {
@@ -466,7 +474,8 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     if (g.lda < (g.tA ? M : K) || g.ldb < (g.tB ? K : N)) return SNHIP_STATUS_INVALID_VALUE;
 
     Choice ch = choose(h, M, N, K, batch, math);
-    if (prefer_ksplit(h, g, math, two_level, ch)) ch = Choice{kKsplitConfig, 1};
+    const int ks_cfg = prefer_ksplit(h, g, math, two_level);
+    if (ks_cfg >= 0) ch = Choice{ks_cfg, 1};
     const ConfigEntry& cfg = kConfigs[ch.cfg];
     if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
 
@@ -493,7 +502,7 @@ int gemm_core(Handle* h, const GemmArgs& g) {
         }
         return SNHIP_STATUS_SUCCESS;
     }
-    const bool fuse_colsum = use_ext && g.colsum != nullptr && ch.splitk == 1 && g.tA && !g.tB && ch.cfg != kKsplitConfig;
+    const bool fuse_colsum = use_ext && g.colsum != nullptr && ch.splitk == 1 && g.tA && !g.tB && kConfigs[ch.cfg].kind != 2;
     // what is left for a pass over C afterwards: sigmoid / tanh always, and addend / ReLU when the kernel is plain
     const float* addend_after = use_ext ? nullptr : ep.addend;
     const int act_after = (use_ext && relu_family) ? ACT_NONE : ep.act;
@@ -538,6 +547,7 @@ int gemm_core(Handle* h, const GemmArgs& g) {
                         ((uintptr_t)ep_kernel.addend % 16 == 0 && g.ldd % 4 == 0 && (!multi || g.sD % 4 == 0) &&
                          (!two_level || g.sD2 % 4 == 0)));
     if (c_vec) p.flags |= GEMM_FLAG_C_VEC;
+    if (cfg.kind == 2 && M <= N) p.flags |= GEMM_FLAG_TILE_N_FASTEST;  // the K-split kernel keeps B's column blocks per XCD
     bool fused_reduce = false;
     if (ch.splitk > 1) {
         const size_t need = (size_t)M * N * batch * ch.splitk * sizeof(float);

@@ -482,7 +482,8 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
     M and N, K tails that are not multiples of 32, alpha / beta, the fused bias, a strided batch; forced through the
     tuning hook and picked automatically for a Dense layer on a small batch."""
     from sharpnet_amd import GPUTensor
-    ks = [c["id"] for c in gpu_wrapper.configs() if c["kind"] == "fp32-ksplit"][0]
+    ks_all = [c["id"] for c in gpu_wrapper.configs() if c["kind"] == "fp32-ksplit"]
+    ks = ks_all[0]
     rng = np.random.default_rng(400 + 2 * tA + tB)
     try:
         for (M, N, K) in [(100, 36, 72), (36, 100, 264), (128, 256, 784), (260, 2048, 512), (4, 8, 36), (32, 32, 32),
@@ -490,13 +491,15 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
             a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
             b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
             c = random_tensor(rng, (M, N), -1, 1)
-            gpu_wrapper.set_tuning(ks, 1)
-            for alpha, beta in [(1.0, 0.0), (-0.5, 1.0), (0.25, -2.0)]:
-                ref = oracle.dot(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
-                got = gpu_dot(gpu_wrapper, a, tA, b, tB, alpha, beta, c=c) if beta != 0 else \
-                    gpu_dot(gpu_wrapper, a, tA, b, tB, alpha, beta, c_shape=[M, N], prefill=float("nan"))
-                assert gpu_wrapper.last_tuning() == (ks, 1), (M, N, K)
-                assert np.max(np.abs(got - ref)) <= tol(K, a, b, alpha, beta, c), (M, N, K, alpha, beta)
+            for cfg in ks_all:
+                gpu_wrapper.set_tuning(cfg, 1)
+                for alpha, beta in [(1.0, 0.0), (-0.5, 1.0), (0.25, -2.0)]:
+                    ref = oracle.dot(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
+                    got = gpu_dot(gpu_wrapper, a, tA, b, tB, alpha, beta, c=c) if beta != 0 else \
+                        gpu_dot(gpu_wrapper, a, tA, b, tB, alpha, beta, c_shape=[M, N], prefill=float("nan"))
+                    assert gpu_wrapper.last_tuning() == (cfg, 1), (M, N, K)
+                    assert np.max(np.abs(got - ref)) <= tol(K, a, b, alpha, beta, c), (M, N, K, cfg, alpha, beta)
+        gpu_wrapper.set_tuning(ks, 1)
         # strided batch + bias through the row-major entry point
         batch, M, N, K = 3, 40, 52, 96
         a = random_tensor(rng, (batch, K, M) if tA else (batch, M, K), -1, 1)
@@ -508,12 +511,13 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
         assert gpu_wrapper.last_tuning() == (ks, 1)
         assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, tA, b, tB, 0.5))) <= tol(K, a, b, 0.5)
         gpu_wrapper.set_tuning(-1, 0)
-        # automatic choice: the Dense layer of benchmark configuration 1 and a square product of one tile per CU
-        for (M, N, K) in [(128, 256, 784), (512, 512, 512)]:
+        # automatic choice: the Dense layer of benchmark configuration 1, a square product of one 32 x 32 tile per
+        # CU, and a recurrent step (one 32 x 64 tile per CU)
+        for (M, N, K, want) in [(128, 256, 784, ks_all[0]), (512, 512, 512, ks_all[0]), (256, 2048, 512, ks_all[1])]:
             a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
             b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
             got = gpu_dot(gpu_wrapper, a, tA, b, tB, 1.0, 0.0, c_shape=[M, N], prefill=float("nan"))
-            assert gpu_wrapper.last_tuning() == (ks, 1)
+            assert gpu_wrapper.last_tuning() == (want, 1)
             assert np.max(np.abs(got - oracle.dot(a, tA, b, tB))) <= tol(K, a, b)
         # an operand view at an odd element offset cannot be read in 16-byte pieces: another kernel takes over
         big = GPUTensor([128 * 784 + 1], None, gpu_wrapper)
@@ -523,7 +527,7 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
         gw = GPUTensor(w_.shape, w_, gpu_wrapper)
         gy = GPUTensor([128, 256], None, gpu_wrapper)
         gy.Dot(view, False, gw, True, 1.0, 0.0)
-        assert gpu_wrapper.last_tuning()[0] != ks
+        assert gpu_wrapper.last_tuning()[0] not in ks_all
         assert np.all(gy.ToNumpy() == 0.0)
     finally:
         gpu_wrapper.set_tuning(-1, 0)
@@ -534,12 +538,13 @@ def test_k_split_kernel_padded_pitches_fuzz(oracle, gpu_wrapper):
     and ReLU, forced onto the K-split kernel; operands sit in NaN-filled buffers so that any read outside a matrix
     shows up in the result."""
     from sharpnet_amd import GPUTensor
-    ks = [c["id"] for c in gpu_wrapper.configs() if c["kind"] == "fp32-ksplit"][0]
+    ks_all = [c["id"] for c in gpu_wrapper.configs() if c["kind"] == "fp32-ksplit"]
     rng = np.random.default_rng(77)
     used = 0
     try:
-        gpu_wrapper.set_tuning(ks, 1)
         for it in range(60):
+            ks = ks_all[it % len(ks_all)]
+            gpu_wrapper.set_tuning(ks, 1)
             tA, tB = bool(rng.integers(2)), bool(rng.integers(2))
             M, N = int(rng.integers(1, 90)), int(rng.integers(1, 90))
             if tA:
