@@ -1,17 +1,21 @@
-// Element-wise halves of the recurrent cells; the matrix halves are the GEMM kernels.
+// Kernels of the recurrent layers' time steps.
 //
 // The reference gets its recurrent layers from cuDNN (cudnnRNNForward / cudnnRNNBackwardData_v8 /
-// cudnnRNNBackwardWeights_v8, Prod/Layers/RecurrentLayer.cs:353-374,456-503).  Here one time step of one
-// direction is a GEMM  gates[:, t] (+)= h[t-1] . R^T  followed by rnn_cell_fwd_kernel, and on the way back
-// rnn_cell_bwd_kernel followed by  dh = d(gates)[:, t] . R.  cuDNN's cell formulas:
+// cudnnRNNBackwardWeights_v8, Prod/Layers/RecurrentLayer.cs:353-374,456-503).  Here everything that spans all time
+// steps is a GEMM (rnn_layers.hpp); a time step itself is
+//   forward    gates[:, t] (+)= h[t-1] . R^T, then the cell          rnn_step_fused_kernel (one launch), or
+//                                                                    a GEMM + rnn_cell_fwd_kernel
+//   backward   dh = d(gates)[:, t+1] . R, then the cell gradient     rnn_step_bwd_fused_kernel (one launch), or
+//                                                                    rnn_cell_bwd_kernel + a GEMM
+// with cuDNN's cell formulas:
 //
 //   RELU / TANH   h' = act(W x + bW + R h + bR)
 //   LSTM          i, f, o = sigmoid(.), g = tanh(.) of W x + bW + R h + bR;   c' = f c + i g;   h' = o tanh(c')
 //   GRU           r, z = sigmoid(W x + bW + R h + bR);   n = tanh(Wn x + bWn + r (Rn h + bRn));   h' = (1 - z) n + z h
 //
-// Gate blocks follow each other along a row in the order i, f, g, o / r, z, n.  One thread owns one (sample,
-// hidden unit) pair: every access is coalesced along the hidden dimension, every buffer is read and written
-// once per step (HBM/L2-bound, a few hundred KB per step).  Must be included by exactly one translation unit.
+// Gate blocks follow each other along a row in the order i, f, g, o / r, z, n.  In the element-wise kernels one
+// thread owns one (sample, hidden unit) pair: every access is coalesced along the hidden dimension, every buffer is
+// read and written once per step.  Must be included by exactly one translation unit.
 #pragma once
 #include <hip/hip_runtime.h>
 

@@ -4,17 +4,18 @@
 //
 // Work of one layer and direction (n = batch * steps rows, G gates, H hidden units, I inputs):
 //   forward    gates (n x G*H) = X (n x I) . W^T + bW                                  one GEMM over all steps
-//              per step: gates[:, t] += h[t-1] . R^T (GRU: into a buffer of its own)   GEMM batch x G*H x H
-//                        cell kernel -> h[t] into y and into the slot the next step reads
-//   backward   per step, last to first: cell kernel -> d(gates)[:, t]; dh = d(gates)[:, t] . R   GEMM batch x H x G*H
+//              per step: gates[:, t] += h[t-1] . R^T (batch x G*H x H), cell -> h[t] into y and into the slot the
+//                        next step reads: one launch (rnn_step_fused_kernel) when H % 32 == 0, else GEMM + cell kernel
+//   backward   per step, last to first: dh = d(gates)[:, t+1] . R (batch x H x G*H), cell gradient -> d(gates)[:, t]:
+//                        one launch (rnn_step_bwd_fused_kernel) when H % 32 == 0, else cell kernel + GEMM
 //              dX (n x I) = d(gates) . W                                               one GEMM
 //   weights    dW += d(gates)^T . X, dR += d(gates_h)^T . Hprev, bias gradients = column sums     two GEMMs
 // Hprev (n x H) holds, for every (sample, step), the state that entered the step, so the recurrent weight gradient
 // is a single product over all steps.
-// Everything the library keeps between the calls is stored step-major ((steps, batch, width)): the rows of one
-// time step are contiguous, whereas in the caller's batch-major tensors they lie steps * width floats apart - a
-// power-of-two pitch of hundreds of KB that sends every row of a step to the same memory channel.  x is copied
-// into that order once per forward call; y, dy and dx are read and written in place through their row pitch.
+// Everything the library keeps between the calls is stored step-major ((steps, batch, width)): the rows one time
+// step works on are contiguous, whereas in the caller's batch-major tensors they lie steps * width floats apart.
+// x is copied into that order once per forward call; y, dy and dx are read and written in place through their
+// row pitch.
 #pragma once
 #include "rnn_cells.hpp"
 
