@@ -11,8 +11,8 @@
 // Operands: op(A) is M x K, op(B) is K x N, row-major storage with row pitch lda / ldb.  An operand whose storage
 // is contiguous along k (A not transposed, B transposed) is fetched 16 bytes per lane along k; one that is
 // contiguous along its rows (A transposed, B not transposed) is fetched 16 bytes per lane along the rows, kept in
-// that orientation in the patch and transposed by the reads.  Both need 16-byte aligned rows (the dispatcher checks pointers, pitches
-// and the contiguous extent); M, N are arbitrary, K is a multiple of 4.
+// that orientation in the patch and transposed by the reads.  Both need 16-byte aligned rows (the dispatcher
+// checks pointers, pitches and the contiguous extent); M, N are arbitrary, K is a multiple of 4.
 // Must be included by exactly one translation unit.
 #pragma once
 #include <hip/hip_runtime.h>

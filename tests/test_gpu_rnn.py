@@ -130,8 +130,8 @@ def test_cells_wider(gpu_wrapper, cell):
 @pytest.mark.parametrize("hidden,batch", [(32, 5), (64, 33), (96, 70), (160, 32)])
 def test_cells_one_launch_per_step(gpu_wrapper, cell, hidden, batch):
     """Hidden sizes that are multiples of 32 take the kernel that computes h . R^T and the cell in one launch
-    (K split over the wavefronts of a workgroup); checked against the oracle and against the GEMM + cell-kernel form selected through
-    snhip_rnn_set_step_mode (different summation orders: 2e-5)."""
+    (K split over the wavefronts of a workgroup); checked against the oracle and against the GEMM + cell-kernel form
+    selected through snhip_rnn_set_step_mode (different summation orders: 2e-5)."""
     rng = np.random.default_rng(hidden * 10 + batch + cell)
     desc = ro.RnnDesc(cell, input_size=20, hidden_size=hidden, num_layers=2, bidirectional=True, bias_mode=ro.DOUBLE_BIAS)
     Tn = 7
