@@ -444,31 +444,38 @@ def layer_timings(w, wl):
     B, Tn, I, H = 256, 128, 256, 512
     x, dyr = T((B, Tn, I)), T((B, Tn, H), -0.01, 0.01)
     yr, dxr = GPUTensor([B, Tn, H], None, w), GPUTensor([B, Tn, I], None, w)
-    for name, cell, bias in (("LSTM", recurrent.CUDNN_LSTM, recurrent.CUDNN_RNN_SINGLE_INP_BIAS),
-                             ("GRU", recurrent.CUDNN_GRU, recurrent.CUDNN_RNN_DOUBLE_BIAS)):
-        layer = recurrent.RecurrentLayer(w, I, H, cell, bias, True, False, 1)
+    for name, cell, bias, bidir in (("LSTM", recurrent.CUDNN_LSTM, recurrent.CUDNN_RNN_SINGLE_INP_BIAS, False),
+                                    ("GRU", recurrent.CUDNN_GRU, recurrent.CUDNN_RNN_DOUBLE_BIAS, False),
+                                    ("bidirectional LSTM", recurrent.CUDNN_LSTM, recurrent.CUDNN_RNN_SINGLE_INP_BIAS, True)):
+        K = 2 if bidir else 1
+        layer = recurrent.RecurrentLayer(w, I, H, cell, bias, True, bidir, 1)
         layer._weightsAndBiases.InitializeFromHostMemory(
             rng.uniform(-0.04, 0.04, layer._weightsAndBiases.Count).astype(np.float32))
+        yk = yr if not bidir else GPUTensor([B, Tn, K * H], None, w)
+        dyk = dyr if not bidir else T((B, Tn, K * H), -0.01, 0.01)
 
         def rnn_f():
-            layer.ForwardPropagation(x, yr, True)
+            layer.ForwardPropagation(x, yk, True)
             layer._reserveSpace.Dispose()
 
         def rnn_fb():
-            layer.ForwardPropagation(x, yr, True)
-            layer.BackwardPropagation(x, yr, dyr, dxr)
-        gates = 4 if name == "LSTM" else 3
-        flop = 2.0 * B * Tn * gates * H * (I + H)
+            layer.ForwardPropagation(x, yk, True)
+            layer.BackwardPropagation(x, yk, dyk, dxr)
+        gates = 3 if name == "GRU" else 4
+        flop = 2.0 * K * B * Tn * gates * H * (I + H)
         for form, mode in (("one launch per step (product with R + cell arithmetic)", 0),
                            ("GEMM + cell kernel per step (+ split-K reduction on the way back)", 1)):
             w.lib.snhip_rnn_set_step_mode(w.handle, mode)
             f = timed(rnn_f, 3, 1)
             fb = timed(rnn_fb, 3, 1)
             w.lib.snhip_rnn_set_step_mode(w.handle, 0)
-            res.append({"layer": "%s batch %d, %d steps, %d -> %d (forward %.1f GFLOP: %d sequential steps of %dx%dx%d)" %
-                                 (name, B, Tn, I, H, flop / 1e9, Tn, B, gates * H, H),
+            res.append({"layer": "%s batch %d, %d steps, %d -> %d (forward %.1f GFLOP: %d sequential steps of %dx%dx%d%s)" %
+                                 (name, B, Tn, I, H, flop / 1e9, Tn, B, gates * H, H, " per direction" if bidir else ""),
                         "form": form, "forward_ms": f, "backward_ms": round(fb - f, 4)})
         layer.Dispose()
+        if bidir:
+            yk.Dispose()
+            dyk.Dispose()
     for t in (x, dyr, yr, dxr):
         t.Dispose()
     w.use_memory_pool(False)

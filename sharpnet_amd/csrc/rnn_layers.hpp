@@ -31,7 +31,8 @@ struct RnnDims {
     long long out_off;                // start of the stacked layers' outputs, after all regions
     long long xt_off;                 // step-major copy of x
     long long total;                  // floats carried from forward to backward
-    long long rt_off;                 // inside the backward scratch: the transposed recurrent matrix of one direction
+    long long rt_off;                 // inside the backward scratch: the transposed recurrent matrix of direction 0
+    long long dir1_off;               // ... dh, dc and the transposed recurrent matrix of direction 1
     long long bwd_ws;                 // floats of scratch the backward calls need
 };
 
@@ -70,7 +71,8 @@ RnnDims rnn_dims(const snhip_rnn_desc* d, int batch, int steps) {
     r.total = r.xt_off + r.n * r.I;
     // dh, dc, one bias gradient, two buffers for the gradients that travel between stacked layers, and R^T
     r.rt_off = 2LL * batch * r.H + (long long)r.G * r.H + (r.L > 1 ? 2 * r.n * r.K * r.H : 0);
-    r.bwd_ws = r.rt_off + (long long)r.G * r.H * r.H;
+    r.dir1_off = r.rt_off + (long long)r.G * r.H * r.H;
+    r.bwd_ws = r.dir1_off + (r.K == 2 ? 2LL * batch * r.H + (long long)r.G * r.H * r.H : 0);
     return r;
 }
 
@@ -229,57 +231,69 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
         // rows of step t: the caller's y is batch-major, the stacked layers' outputs are step-major
         const long long out_step = top ? KH : (long long)B * KH, out_ld = top ? (long long)T * KH : KH;
         const long long I = rnn_layer_inputs(r, layer);
+        // per direction: where its buffers are, the input projections of every step at once, the initial state
+        struct Dir {
+            RnnWeights w;
+            float *gates, *hprev, *cells, *gh;
+            const float *hx, *cx;
+            int first, step;
+        } dirs[2];
+        bool fused = H % 32 == 0 && h->rnn_step_mode == 0;
         for (int d = 0; d < K; ++d) {
             const int p = layer * K + d;
-            const RnnWeights w = rnn_weights(r, const_cast<float*>(weights), p);
+            Dir& D = dirs[d];
+            D.w = rnn_weights(r, const_cast<float*>(weights), p);
             float* region = keep + (long long)p * r.per_p;
-            float* gates = region + r.gates_off;
-            float* hprev = region + r.hprev_off;
-            float* cells = region + r.cells_off;
-            float* gh = region + r.gh_off;
-            const float* hx_p = hx ? hx + (long long)p * B * H : nullptr;
-            const float* cx_p = cx ? cx + (long long)p * B * H : nullptr;
+            D.gates = region + r.gates_off, D.hprev = region + r.hprev_off;
+            D.cells = region + r.cells_off, D.gh = region + r.gh_off;
+            D.hx = hx ? hx + (long long)p * B * H : nullptr;
+            D.cx = cx ? cx + (long long)p * B * H : nullptr;
+            D.first = d == 0 ? 0 : T - 1, D.step = d == 0 ? 1 : -1;
 
-            GemmArgs g;  // input projections of every step at once
+            GemmArgs g;
             g.tB = true;
             g.M = (int)r.n, g.N = (int)GH, g.K = (int)I;
-            g.A = inp, g.lda = (int)I, g.B = w.W, g.ldb = (int)I, g.C = gates, g.ldc = (int)GH;
-            g.bias = w.bW;
+            g.A = inp, g.lda = (int)I, g.B = D.w.W, g.ldb = (int)I, g.C = D.gates, g.ldc = (int)GH;
+            g.bias = D.w.bW;
             st = gemm_core(h, g);
             if (st != SNHIP_STATUS_SUCCESS) return st;
-
-            const int first = d == 0 ? 0 : T - 1, dir = d == 0 ? 1 : -1;
-            st = rnn_set_rows(h, hprev + (long long)first * B * H, H, hx_p, H, B, H);
+            st = rnn_set_rows(h, D.hprev + (long long)D.first * B * H, H, D.hx, H, B, H);
             if (st != SNHIP_STATUS_SUCCESS) return st;
             // product and cell in one launch per step when the rows can be read in 16-byte pieces
-            const bool fused = H % 32 == 0 && (uintptr_t)hprev % 16 == 0 && (uintptr_t)w.R % 16 == 0 && h->rnn_step_mode == 0;
-            for (int k = 0; k < T; ++k) {
-                const int t = first + dir * k;
-                const bool last = k == T - 1;
-                const bool zero_state = k == 0 && hx_p == nullptr;
+            fused = fused && (uintptr_t)D.hprev % 16 == 0 && (uintptr_t)D.w.R % 16 == 0;
+        }
+        // the directions are independent and advance together (one launch per direction and step: a combined grid
+        // of both directions was measured and gains nothing, the second direction's workgroups queue behind the first's)
+        for (int k = 0; k < T; ++k) {
+            const bool last = k == T - 1;
+            for (int d = 0; d < K; ++d) {
+                const Dir& D = dirs[d];
+                const int p = layer * K + d;
+                const int t = D.first + D.step * k;
+                const bool zero_state = k == 0 && D.hx == nullptr;
                 if (!fused && (r.cell == RNN_GRU || !zero_state)) {
                     GemmArgs s;  // h[t-1] . R^T
                     s.tB = true;
                     s.M = B, s.N = (int)GH, s.K = H;
-                    s.A = hprev + (long long)t * B * H, s.lda = H;
-                    s.B = w.R, s.ldb = H;
+                    s.A = D.hprev + (long long)t * B * H, s.lda = H;
+                    s.B = D.w.R, s.ldb = H;
                     if (r.cell == RNN_GRU) {
-                        s.C = gh + (long long)t * B * 3 * H, s.ldc = 3 * H;
+                        s.C = D.gh + (long long)t * B * 3 * H, s.ldc = 3 * H;
                     } else {
-                        s.C = gates + (long long)t * B * GH, s.ldc = (int)GH, s.beta = 1.0f;
+                        s.C = D.gates + (long long)t * B * GH, s.ldc = (int)GH, s.beta = 1.0f;
                     }
                     st = gemm_core(h, s);
                     if (st != SNHIP_STATUS_SUCCESS) return st;
                 }
                 RnnStepFwd c;
-                c.gates = gates + (long long)t * B * GH, c.ld_gates = GH;
-                c.gh = gh + (long long)t * B * 3 * H, c.ld_gh = 3LL * H;
-                c.bias_r = w.bR;
-                c.h_prev = hprev + (long long)t * B * H, c.ld_hprev = H;
-                c.c_prev = k == 0 ? cx_p : cells + (long long)(t - dir) * B * H, c.ld_cprev = H;
-                c.c_out = cells + (long long)t * B * H, c.ld_c = H;
+                c.gates = D.gates + (long long)t * B * GH, c.ld_gates = GH;
+                c.gh = D.gh + (long long)t * B * 3 * H, c.ld_gh = 3LL * H;
+                c.bias_r = D.w.bR;
+                c.h_prev = D.hprev + (long long)t * B * H, c.ld_hprev = H;
+                c.c_prev = k == 0 ? D.cx : D.cells + (long long)(t - D.step) * B * H, c.ld_cprev = H;
+                c.c_out = D.cells + (long long)t * B * H, c.ld_c = H;
                 c.y = out + (long long)t * out_step + (long long)d * H, c.ld_y = out_ld;
-                c.h_next = last ? nullptr : hprev + (long long)(t + dir) * B * H, c.ld_hnext = H;
+                c.h_next = last ? nullptr : D.hprev + (long long)(t + D.step) * B * H, c.ld_hnext = H;
                 c.hy = (last && hy) ? hy + (long long)p * B * H : nullptr;
                 c.cy = (last && cy && r.cell == RNN_LSTM) ? cy + (long long)p * B * H : nullptr;
                 c.batch = B, c.hidden = H, c.cell = r.cell;
@@ -287,11 +301,11 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
                     const int U = G == 1 ? 32 : 16;
                     const dim3 grid((unsigned)((H + U - 1) / U), (unsigned)((B + 31) / 32));
                     if (G == 4)
-                        hipLaunchKernelGGL(rnn_step_fused_kernel<4>, grid, dim3(256), 0, h->stream, c, (const float*)w.R);
+                        hipLaunchKernelGGL(rnn_step_fused_kernel<4>, grid, dim3(256), 0, h->stream, c, (const float*)D.w.R);
                     else if (G == 3)
-                        hipLaunchKernelGGL(rnn_step_fused_kernel<3>, grid, dim3(256), 0, h->stream, c, (const float*)w.R);
+                        hipLaunchKernelGGL(rnn_step_fused_kernel<3>, grid, dim3(256), 0, h->stream, c, (const float*)D.w.R);
                     else
-                        hipLaunchKernelGGL(rnn_step_fused_kernel<1>, grid, dim3(256), 0, h->stream, c, (const float*)w.R);
+                        hipLaunchKernelGGL(rnn_step_fused_kernel<1>, grid, dim3(256), 0, h->stream, c, (const float*)D.w.R);
                 } else {
                     hipLaunchKernelGGL(rnn_cell_fwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
                                        h->stream, c);
@@ -321,8 +335,6 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
     if (ws == nullptr || workspace_bytes < (size_t)r.bwd_ws * sizeof(float)) return SNHIP_STATUS_INVALID_VALUE;
     const int B = batch, T = steps, H = r.H, G = r.G, K = r.K;
     const long long GH = (long long)G * H, KH = (long long)K * H;
-    float* dh = ws;
-    float* dc = ws + (long long)B * H;
     float* between[2] = {ws + 2LL * B * H + GH, ws + 2LL * B * H + GH + r.n * KH};
 
     for (int layer = r.L - 1; layer >= 0; --layer) {
@@ -332,85 +344,118 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
         const long long out_step = top ? KH : (long long)B * KH, out_ld = top ? (long long)T * KH : KH;
         float* dinp = layer == 0 ? dx : between[(layer - 1) & 1];
         const long long I = rnn_layer_inputs(r, layer);
+        struct Dir {
+            RnnWeights w;
+            float *gates, *hprev, *cells, *gh, *dh, *dc, *Rt;
+            const float* cx;
+            int first, step;
+        } dirs[2];
+        // every step but the first one processed runs as one launch (product with R, then the cell gradient) when
+        // rows can be read in 16-byte pieces; that kernel wants the rows of R^T
+        bool fused = H % 32 == 0 && T > 1 && h->rnn_step_mode == 0;
         for (int d = 0; d < K; ++d) {
             const int p = layer * K + d;
-            const RnnWeights w = rnn_weights(r, const_cast<float*>(weights), p);
+            Dir& D = dirs[d];
+            D.w = rnn_weights(r, const_cast<float*>(weights), p);
             float* region = keep + (long long)p * r.per_p;
-            float* gates = region + r.gates_off;
-            float* hprev = region + r.hprev_off;
-            float* cells = region + r.cells_off;
-            float* gh = region + r.gh_off;
-            const float* cx_p = cx ? cx + (long long)p * B * H : nullptr;
-            st = rnn_set_rows(h, dh, H, dhy ? dhy + (long long)p * B * H : nullptr, H, B, H);
+            D.gates = region + r.gates_off, D.hprev = region + r.hprev_off;
+            D.cells = region + r.cells_off, D.gh = region + r.gh_off;
+            D.dh = d == 0 ? ws : ws + r.dir1_off;
+            D.dc = D.dh + (long long)B * H;
+            D.Rt = d == 0 ? ws + r.rt_off : ws + r.dir1_off + 2LL * B * H;
+            D.cx = cx ? cx + (long long)p * B * H : nullptr;
+            D.first = d == 0 ? 0 : T - 1, D.step = d == 0 ? 1 : -1;
+            st = rnn_set_rows(h, D.dh, H, dhy ? dhy + (long long)p * B * H : nullptr, H, B, H);
             if (st != SNHIP_STATUS_SUCCESS) return st;
             if (r.cell == RNN_LSTM) {
-                st = rnn_set_rows(h, dc, H, dcy ? dcy + (long long)p * B * H : nullptr, H, B, H);
+                st = rnn_set_rows(h, D.dc, H, dcy ? dcy + (long long)p * B * H : nullptr, H, B, H);
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
-            const int first = d == 0 ? 0 : T - 1, dir = d == 0 ? 1 : -1;
-            // every step but the first one processed runs as one launch (product with R, then the cell gradient) when
-            // rows can be read in 16-byte pieces; that kernel wants the rows of R^T
-            float* Rt = ws + r.rt_off;
-            const bool fused = H % 32 == 0 && T > 1 && (uintptr_t)gates % 16 == 0 && (uintptr_t)Rt % 16 == 0 &&
-                               h->rnn_step_mode == 0;
-            if (fused) {
-                st = snhip_transpose_second_and_third_dimension(handle, w.R, Rt, 1, (int)GH, H, 1);
+            fused = fused && (uintptr_t)D.gates % 16 == 0 && (uintptr_t)D.Rt % 16 == 0;
+        }
+        if (fused)
+            for (int d = 0; d < K; ++d) {
+                st = snhip_transpose_second_and_third_dimension(handle, dirs[d].w.R, dirs[d].Rt, 1, (int)GH, H, 1);
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
-            for (int k = T - 1; k >= 0; --k) {
-                const int t = first + dir * k;
+        for (int k = T - 1; k >= 0; --k) {
+            const bool one_launch = fused && k < T - 1;
+            for (int d = 0; d < K; ++d) {
+                const Dir& D = dirs[d];
+                const int t = D.first + D.step * k;
                 RnnStepBwd c;
-                c.gates = gates + (long long)t * B * GH, c.ld_gates = GH;
-                c.gh = gh + (long long)t * B * 3 * H, c.ld_gh = 3LL * H;
-                c.h_prev = hprev + (long long)t * B * H, c.ld_hprev = H;
+                c.gates = D.gates + (long long)t * B * GH, c.ld_gates = GH;
+                c.gh = D.gh + (long long)t * B * 3 * H, c.ld_gh = 3LL * H;
+                c.h_prev = D.hprev + (long long)t * B * H, c.ld_hprev = H;
                 c.y = out + (long long)t * out_step + (long long)d * H, c.ld_y = out_ld;
-                c.c_prev = k == 0 ? cx_p : cells + (long long)(t - dir) * B * H, c.ld_cprev = H;
-                c.c = cells + (long long)t * B * H, c.ld_c = H;
+                c.c_prev = k == 0 ? D.cx : D.cells + (long long)(t - D.step) * B * H, c.ld_cprev = H;
+                c.c = D.cells + (long long)t * B * H, c.ld_c = H;
                 c.dy = dout + (long long)t * out_step + (long long)d * H, c.ld_dy = out_ld;
-                c.dh = dh, c.dc = dc;
+                c.dh = D.dh, c.dc = D.dc;
                 c.batch = B, c.hidden = H, c.cell = r.cell;
-                if (fused && k < T - 1) {
-                    const float* dg_next = ((r.cell == RNN_GRU) ? gh : gates) + (long long)(t + dir) * B * GH;
+                if (one_launch) {
+                    const float* dg_next = ((r.cell == RNN_GRU) ? D.gh : D.gates) + (long long)(t + D.step) * B * GH;
                     const dim3 grid((unsigned)((H + RnnBwdFusedCfg::U - 1) / RnnBwdFusedCfg::U), (unsigned)((B + 31) / 32));
                     if (G == 4)
                         hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<4>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
-                                           c, dg_next, GH, (const float*)Rt);
+                                           c, dg_next, GH, (const float*)D.Rt);
                     else if (G == 3)
                         hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<3>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
-                                           c, dg_next, GH, (const float*)Rt);
+                                           c, dg_next, GH, (const float*)D.Rt);
                     else
                         hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<1>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
-                                           c, dg_next, GH, (const float*)Rt);
-                } else {
-                    hipLaunchKernelGGL(rnn_cell_bwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
-                                       h->stream, c);
+                                           c, dg_next, GH, (const float*)D.Rt);
+                    st = hip_to_status(hipGetLastError());
+                    if (st != SNHIP_STATUS_SUCCESS) return st;
+                    continue;
                 }
+                hipLaunchKernelGGL(rnn_cell_bwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
+                                   h->stream, c);
                 st = hip_to_status(hipGetLastError());
                 if (st != SNHIP_STATUS_SUCCESS) return st;
-                if (k == 0 && dhx == nullptr) break;  // nobody asks for the gradient of the initial state
-                if (fused && k > 0) continue;         // the next launch multiplies by R itself
-                GemmArgs s;  // dh = d(R h)[:, t] . R  (GRU: added to dh * z)
+                // dh = d(R h)[:, t] . R for the step before (GRU: added to dh * z); with the one-launch steps only the
+                // gradient of the initial state is left to multiply, and only if somebody asks for it
+                if (fused ? (k > 0 || dhx == nullptr) : (k == 0 && dhx == nullptr)) continue;
+                GemmArgs s;
                 s.M = B, s.N = H, s.K = (int)GH;
-                s.A = (r.cell == RNN_GRU) ? gh + (long long)t * B * 3 * H : gates + (long long)t * B * GH;
+                s.A = (r.cell == RNN_GRU) ? D.gh + (long long)t * B * 3 * H : D.gates + (long long)t * B * GH;
                 s.lda = (int)GH;
-                s.B = w.R, s.ldb = H;
-                s.C = dh, s.ldc = H;
+                s.B = D.w.R, s.ldb = H;
+                s.C = D.dh, s.ldc = H;
                 s.beta = (r.cell == RNN_GRU) ? 1.0f : 0.0f;
                 st = gemm_core(h, s);
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
+            if (!one_launch) continue;
+            if (k == 0 && dhx != nullptr)
+                for (int d = 0; d < K; ++d) {  // the last launch left d(gates) of the first step: one more product for dhx
+                    const Dir& D = dirs[d];
+                    GemmArgs s;
+                    s.M = B, s.N = H, s.K = (int)GH;
+                    s.A = (r.cell == RNN_GRU) ? D.gh + (long long)D.first * B * 3 * H : D.gates + (long long)D.first * B * GH;
+                    s.lda = (int)GH;
+                    s.B = D.w.R, s.ldb = H;
+                    s.C = D.dh, s.ldc = H;
+                    s.beta = (r.cell == RNN_GRU) ? 1.0f : 0.0f;
+                    st = gemm_core(h, s);
+                    if (st != SNHIP_STATUS_SUCCESS) return st;
+                }
+        }
+        for (int d = 0; d < K; ++d) {
+            const Dir& D = dirs[d];
+            const int p = layer * K + d;
             if (dhx != nullptr) {
-                st = rnn_set_rows(h, dhx + (long long)p * B * H, H, dh, H, B, H);
+                st = rnn_set_rows(h, dhx + (long long)p * B * H, H, D.dh, H, B, H);
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
             if (dcx != nullptr && r.cell == RNN_LSTM) {
-                st = rnn_set_rows(h, dcx + (long long)p * B * H, H, dc, H, B, H);
+                st = rnn_set_rows(h, dcx + (long long)p * B * H, H, D.dc, H, B, H);
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
             if (dinp == nullptr) continue;
             GemmArgs g;  // gradient of the layer's input: both directions add up
             g.K = (int)GH, g.N = (int)I;
-            g.A = gates, g.lda = (int)GH, g.B = w.W, g.ldb = (int)I, g.C = dinp;
+            g.A = D.gates, g.lda = (int)GH, g.B = D.w.W, g.ldb = (int)I, g.C = dinp;
             g.beta = d == 0 ? 0.0f : 1.0f;
             if (layer == 0) {
                 // one product per step: step-major rows in, the caller's batch-major dx out
