@@ -265,3 +265,22 @@ def test_full_size_layer_properties(gpu_wrapper, cell):
     for key in ("dx", "dw", "dhx"):
         scale = max(1.0, float(np.max(np.abs(two[key]))))
         assert np.max(np.abs(one[key] - two[key])) <= 2e-4 * scale, key
+
+
+@pytest.mark.parametrize("cell", [ro.TANH, ro.LSTM, ro.GRU])
+@pytest.mark.parametrize("batch,steps,hidden", [(1, 1, 32), (3, 1, 5), (1, 4, 64), (2, 2, 32)])
+def test_degenerate_sequence_shapes(gpu_wrapper, cell, batch, steps, hidden):
+    """One sample, one step, two steps: the first / last step special cases of both step forms."""
+    rng = np.random.default_rng(batch * 100 + steps * 10 + hidden + cell)
+    desc = ro.RnnDesc(cell, input_size=8, hidden_size=hidden, num_layers=2, bidirectional=True, bias_mode=ro.DOUBLE_BIAS)
+    weights = rng.uniform(-0.3, 0.3, ro.weight_space_size(desc)).astype(np.float32)
+    x = rng.uniform(-1, 1, (batch, steps, 8)).astype(np.float32)
+    dy = rng.uniform(-1, 1, (batch, steps, 2 * hidden)).astype(np.float32)
+    st = lambda: rng.uniform(-1, 1, (desc.pseudo_layers, batch, hidden)).astype(np.float32)
+    hx, cx, dhy, dcy = st(), st(), st(), st()
+    if cell != ro.LSTM:
+        cx = dcy = None
+    got = run_gpu(gpu_wrapper, desc, x, weights, dy, hx, cx, dhy, dcy)
+    compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, 3e-5)
+    got = run_gpu(gpu_wrapper, desc, x, weights, dy)
+    compare(desc, got, x, weights, dy, None, None, None, None, 3e-5)
