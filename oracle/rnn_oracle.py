@@ -27,18 +27,25 @@ weight_space_size          RecurrentLayer.cs:170-184; the order    per-gate para
                            inside the weight space is this
                            build's own (the reference only ever
                            asks for addresses)
-rnn_forward                cudnnRNNForward, RecurrentLayer.cs:353  torch.nn.RNN / LSTM / GRU on the CPU (library
-                                                                   routine, same parameter convention), all cells,
-                                                                   both directions, 1-2 layers, every bias mode;
+rnn_forward                cudnnRNNForward, RecurrentLayer.cs:353  the reference's stored predictions of SimpleRNN /
+                                                                   LSTM / GRU networks after 10 epochs of training
+                                                                   (TestNetworkPropagation.cs:1193-1330, 13 cases:
+                                                                   sequences or last step, one or two directions);
                                                                    SimpleRNN loss before training
-                                                                   ParallelRunWithPyTorch.cs:949 (0.48370790481567383)
-rnn_backward               cudnnRNNBackwardData_v8 +               torch autograd through the same modules; SimpleRNN
-                           cudnnRNNBackwardWeights_v8, :456-503    loss after 10 epochs ParallelRunWithPyTorch.cs:951
-                                                                   (0.2722862660884857)
-layer_forward /            RecurrentLayer.ForwardPropagation /     the same stored losses (a 2-layer bidirectional
-layer_backward             BackwardPropagation :305-520            return-sequences layer feeding a last-step layer)
-                           (returnSequences == false: last step
-                           of the forward direction, first step
+                                                                   ParallelRunWithPyTorch.cs:949 (0.48370790481567383);
+                                                                   torch.nn.RNN / LSTM / GRU on the CPU (library
+                                                                   routine, same parameter convention): all cells,
+                                                                   both directions, 1-2 layers, every bias mode,
+                                                                   initial states, gate order with non-zero weights
+rnn_backward               cudnnRNNBackwardData_v8 +               the same 13 stored predictions (they are reached
+                           cudnnRNNBackwardWeights_v8, :456-503    through 10 gradient steps); SimpleRNN loss after
+                                                                   10 epochs ParallelRunWithPyTorch.cs:951
+                                                                   (0.2722862660884857); torch autograd through the
+                                                                   same modules
+layer_forward /            RecurrentLayer.ForwardPropagation /     the same stored predictions and losses (last-step
+layer_backward             BackwardPropagation :305-520            outputs of uni- and bidirectional layers; a 2-layer
+                           (returnSequences == false: last step    bidirectional sequence layer feeding a last-step
+                           of the forward direction, first step    layer)
                            of the reverse one)
 =========================  ======================================  ==================================================
 """

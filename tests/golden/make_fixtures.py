@@ -164,6 +164,33 @@ def main():
         "loss_before": losses[0], "loss_after": losses[1], "tolerance": 1e-6,
     }
 
+    # ---- Tests/NonReg/TestNetworkPropagation.cs:1193-1330  recurrent layers trained from zero weights ----
+    rnn_cases = []
+    for test, cell in (("Test_SimpleRNN", "tanh"), ("Test_LSTM", "lstm"), ("Test_GRU", "gru")):
+        i = tnp.index("public void %s(bool returnSequences" % test)
+        blk = tnp[tnp.rindex("\n\n", 0, i):i]
+        found = re.findall(r'\[TestCase\((true|false), (true|false), "([^"]*)", "([^"]*)", "([^"]*)"\)\]', blk)
+        assert len(found) == 4, (test, len(found))
+        for rs, bd, dense, before, after in found:
+            rnn_cases.append({"cell": cell, "return_sequences": rs == "true", "bidirectional": bd == "true", "hidden": 2,
+                              "dense_weight": json.loads(dense), "prediction_before": json.loads(before),
+                              "prediction_after": json.loads(after)})
+    blk = lines(tnp, 1198, 1226)
+    w = numpy_literals(blk)
+    assert len(w) == 3 and len(w[0]) == 3, w
+    rnn_cases.append({"cell": "tanh", "return_sequences": False, "bidirectional": False, "hidden": 3, "dense_weight": w[0],
+                      "prediction_before": w[1], "prediction_after": w[2]})
+    fx["ZeroWeightRecurrentLayers"] = {
+        "source": "Tests/NonReg/TestNetworkPropagation.cs:1193-1330 (Test_SimpleRNN_returnSequence_false, Test_SimpleRNN, "
+                  "Test_LSTM, Test_GRU): Input(2 steps, 1 feature) -> recurrent layer(hidden, returnSequences, bidirectional), all "
+                  "its weights zero -> Linear(1, bias, on the last dimension) with the given weights; Huber loss (delta 1, "
+                  "Prod/CPU/CpuTensor.cs:2420-2437), SGD(0.1, momentum 0.9) on the whole batch of 4 for 10 epochs, TensorFlow "
+                  "compatibility mode (SimpleRNN and LSTM: one bias vector on the input side, GRU: two, Prod/Networks/Network.cs:188-205)",
+        "x": const_literal(tnp, "X_RNN_4_2_1"), "y_sequences": const_literal(tnp, "Y_RNN_4_2_1"),
+        "y_last": const_literal(tnp, "Y_RNN_4_1_1"),
+        "lr": 0.1, "momentum": 0.9, "epochs": 10, "huber_delta": 1.0, "tolerance": 1e-4, "cases": rnn_cases,
+    }
+
     with open(OUT, "w") as f:
         json.dump(fx, f, indent=1)
     print("wrote", OUT, os.path.getsize(OUT), "bytes")

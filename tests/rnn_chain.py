@@ -44,3 +44,41 @@ def simple_rnn_chain(fx, forward=None, backward=None):
                 vel[k] = (np.float32(fx["momentum"]) * vel[k] - g * np.float32(fx["lr"] / bs)).astype(np.float32)
                 P[k] = (P[k] + vel[k]).astype(np.float32)
     return before, loss()
+
+
+CELLS = {"relu": ro.RELU, "tanh": ro.TANH, "lstm": ro.LSTM, "gru": ro.GRU}
+
+
+def zero_weight_chain(fx, case, forward=None, backward=None):
+    """The networks of Tests/NonReg/TestNetworkPropagation.cs:1193-1330: a recurrent layer whose weights start at zero
+    feeding Linear(1), Huber loss, SGD with momentum on the whole batch.  Returns (prediction before, after)."""
+    from oracle import dot_oracle as do
+    forward = forward or ro.layer_forward
+    backward = backward or ro.layer_backward
+    cell = CELLS[case["cell"]]
+    bias_mode = ro.DOUBLE_BIAS if cell == ro.GRU else ro.SINGLE_INP_BIAS          # Prod/Networks/Network.cs:188-205
+    desc = ro.RnnDesc(cell, 1, case["hidden"], 1, case["bidirectional"], bias_mode)
+    rs = case["return_sequences"]
+    X = np.array(fx["x"], np.float32)
+    Y = np.array(fx["y_sequences"] if rs else fx["y_last"], np.float32)
+    P = [np.zeros(ro.weight_space_size(desc), np.float32),
+         np.array(case["dense_weight"], np.float32).reshape(1, desc.dirs * case["hidden"]), np.zeros(1, np.float32)]
+    V = [np.zeros_like(p) for p in P]
+    batch = X.shape[0]
+
+    def predict():
+        y, cache = forward(desc, X, P[0], rs)
+        return do.dense_forward(y, P[1], P[2], flatten_last=True), (y, cache)
+
+    before = predict()[0]
+    for _ in range(fx["epochs"]):
+        out, (y, cache) = predict()
+        err = out.reshape(batch, -1) - Y.reshape(batch, -1)
+        # Huber gradient: the clipped error over the elements of a sample (Prod/CPU/CpuTensor.cs:2427-2437)
+        g = (np.clip(err, -fx["huber_delta"], fx["huber_delta"]) / err.shape[1]).reshape(out.shape).astype(np.float32)
+        dW, db, dy = do.dense_backward(y, g, P[1], flatten_last=True)
+        _, dw_rnn = backward(desc, dy.reshape(y.shape), cache)
+        for i, grad in enumerate((dw_rnn, dW, db)):          # CpuTensor.cs:470-489 with lr / batchSize (Optimizer.cs:26-29)
+            V[i] = (np.float32(fx["momentum"]) * V[i] - grad * np.float32(fx["lr"] / batch)).astype(np.float32)
+            P[i] = (P[i] + V[i]).astype(np.float32)
+    return before, predict()[0]

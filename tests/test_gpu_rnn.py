@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from oracle import rnn_oracle as ro
-from tests.rnn_chain import simple_rnn_chain
+from tests.rnn_chain import simple_rnn_chain, zero_weight_chain
 
 pytestmark = pytest.mark.gpu
 
@@ -216,6 +216,44 @@ def test_simple_rnn_training_losses_on_device(golden, gpu_wrapper):
     before, after = simple_rnn_chain(fx, forward, backward)
     assert abs(before - fx["loss_before"]) < 2e-6, (before, fx["loss_before"])
     assert abs(after - fx["loss_after"]) < 2e-6, (after, fx["loss_after"])
+
+
+def mirror_callbacks(gpu_wrapper):
+    """forward / backward in the oracle's signature, run by the RecurrentLayer mirror on the device."""
+    from sharpnet_amd import GPUTensor, recurrent
+    layers = {}
+
+    def forward(desc, x, weights, return_sequences):
+        key = (desc.cell, desc.input_size, desc.hidden_size, desc.num_layers, desc.bidirectional, return_sequences)
+        if key not in layers:
+            layers[key] = recurrent.RecurrentLayer(gpu_wrapper, desc.input_size, desc.hidden_size, desc.cell, desc.bias_mode,
+                                                   return_sequences, desc.bidirectional, desc.num_layers)
+        layer = layers[key]
+        layer._weightsAndBiases.InitializeFromHostMemory(weights)
+        gx = T(gpu_wrapper, x)
+        gy = GPUTensor(layer.OutputShape(x.shape[0], x.shape[1]), None, gpu_wrapper)
+        layer.ForwardPropagation(gx, gy, True)
+        return gy.ToNumpy(), (layer, gx, gy)
+
+    def backward(desc, dy, cache):
+        layer, gx, gy = cache
+        gdx = GPUTensor(gx.Shape, None, gpu_wrapper)
+        layer.BackwardPropagation(gx, gy, T(gpu_wrapper, dy), gdx)
+        return gdx.ToNumpy(), layer._weightsAndBiasesGradients.ToNumpy()
+
+    return forward, backward
+
+
+@pytest.mark.parametrize("index", range(13))
+def test_zero_weight_layers_reach_the_reference_predictions_on_device(golden, oracle, gpu_wrapper, index):
+    """Tests/NonReg/TestNetworkPropagation.cs:1193-1330 with the recurrent layer run by the mirror on the GPU: the
+    stored predictions after 10 epochs, within the reference's own tolerance (1e-4)."""
+    fx = golden["ZeroWeightRecurrentLayers"]
+    case = fx["cases"][index]
+    forward, backward = mirror_callbacks(gpu_wrapper)
+    before, after = zero_weight_chain(fx, case, forward, backward)
+    assert np.max(np.abs(before.reshape(-1) - np.array(case["prediction_before"], np.float32).reshape(-1))) <= fx["tolerance"]
+    assert np.max(np.abs(after.reshape(-1) - np.array(case["prediction_after"], np.float32).reshape(-1))) <= fx["tolerance"], case
 
 
 def test_rnn_argument_checks(gpu_wrapper):

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import rnn_oracle as ro
-from tests.rnn_chain import simple_rnn_chain
+from tests.rnn_chain import simple_rnn_chain, zero_weight_chain
 
 CELLS = {ro.RELU: ("RNN", "relu"), ro.TANH: ("RNN", "tanh"), ro.LSTM: ("LSTM", None), ro.GRU: ("GRU", None)}
 
@@ -125,3 +125,15 @@ def test_simple_rnn_chain_losses(golden):
     before, after = simple_rnn_chain(fx)
     assert abs(before - fx["loss_before"]) < fx["tolerance"], (before, fx["loss_before"])
     assert abs(after - fx["loss_after"]) < fx["tolerance"], (after, fx["loss_after"])
+
+
+@pytest.mark.parametrize("index", range(13))
+def test_zero_weight_layers_reach_the_reference_predictions(golden, oracle, index):
+    """SimpleRNN / LSTM / GRU, sequences or last step, one or two directions: the predictions the reference's tests
+    store after 10 epochs (tolerance 1e-4 there; reproduced to 1e-6).  Pins the LSTM and GRU cells, both
+    directions and the returnSequences handling with the reference's own numbers."""
+    fx = golden["ZeroWeightRecurrentLayers"]
+    case = fx["cases"][index]
+    before, after = zero_weight_chain(fx, case)
+    assert np.max(np.abs(before.reshape(-1) - np.array(case["prediction_before"], np.float32).reshape(-1))) <= 1e-6
+    assert np.max(np.abs(after.reshape(-1) - np.array(case["prediction_after"], np.float32).reshape(-1))) <= 2e-6, case
