@@ -281,9 +281,10 @@ int snhip_rnn_temp_space_sizes(const snhip_rnn_desc* desc, int training, int bat
 int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, int batch, int steps, const float* x,
                       float* y, const float* hx, float* hy, const float* cx, float* cy, const float* weights,
                       void* workspace, size_t workspace_bytes, void* reserve, size_t reserve_bytes);
-/* Tuning hook: 0 (default) runs a forward time step as one launch - the product with the recurrent matrix and the
- * cell arithmetic in one kernel - whenever hidden_size is a multiple of 32; 1 always issues the GEMM and the cell
- * kernel separately (what other hidden sizes get).  Same results within rounding (different summation order). */
+/* Tuning hook: 0 (default) runs a time step, forward or backward, as one launch - the product with the recurrent
+ * matrix and the cell arithmetic in one kernel - whenever hidden_size is a multiple of 4 and at least 32; 1 always
+ * issues the GEMM and the cell kernel separately (what other hidden sizes get).  Same results within rounding
+ * (different summation order). */
 int snhip_rnn_set_step_mode(void* handle, int mode);
 /* dx may be NULL (first layer of a network).  Leaves the gate gradients in reserve for snhip_rnn_backward_weights. */
 int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch, int steps, const float* y,

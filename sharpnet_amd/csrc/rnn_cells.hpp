@@ -84,9 +84,12 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd_kernel(const RnnStepFwd s) {
 // mbeg .. mend - 1.  Whole-line global loads, DEPTH groups in flight in registers; a group passes through the
 // wavefront's private LDS patches pa / pb (32 rows x PITCH floats each) to reach MFMA operand layout (row = l % 32,
 // sixteen consecutive k per half-wave).  No workgroup barrier inside.
-template <int D, int P>
+// TAIL: K is not a multiple of 32 (but of 4); a lane whose four k values of a group lie beyond K reads zeros instead.
+__device__ __attribute__((aligned(16))) const float rnn_zero_vector[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+
+template <int D, int P, bool TAIL>
 __device__ __forceinline__ void wave_product_32x32(const float* const (&ap)[4], const float* const (&bp)[4], int mbeg,
-                                                   int mend, float* pa, float* pb, int lane, f32x16 (&acc)[4]) {
+                                                   int mend, int K, float* pa, float* pb, int lane, f32x16 (&acc)[4]) {
     const int l32 = lane & 31, lhi = lane >> 5, lrow = lane >> 3, lcol = (lane & 7) * 4;
     f32x4 ra[D][4], rb[D][4];
 #pragma unroll
@@ -95,10 +98,11 @@ __device__ __forceinline__ void wave_product_32x32(const float* const (&ap)[4], 
         for (int r = 0; r < 16; ++r) acc[e][r] = 0.0f;
 
     auto load = [&](int slot, int m) {
+        const bool ok = !TAIL || 32 * m + lcol < K;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            ra[slot][i] = *reinterpret_cast<const f32x4*>(ap[i] + m * 32);
-            rb[slot][i] = *reinterpret_cast<const f32x4*>(bp[i] + m * 32);
+            ra[slot][i] = *reinterpret_cast<const f32x4*>(ok ? ap[i] + m * 32 : rnn_zero_vector);
+            rb[slot][i] = *reinterpret_cast<const f32x4*>(ok ? bp[i] + m * 32 : rnn_zero_vector);
         }
     };
     // stage(slot, f): a group goes from the registers it was loaded into, through the wavefront's LDS patch, into
@@ -181,7 +185,7 @@ __device__ __forceinline__ void wave_product_32x32(const float* const (&ap)[4], 
 // layout (row = lane % 32, sixteen consecutive k per half-wave), and multiplies - no workgroup barrier until the
 // partial tiles meet in LDS, where each thread picks up all gates of its (sample, unit) pairs, adds W x + bW from
 // the gates buffer and finishes the cell exactly as rnn_cell_fwd_kernel does.
-// Requires H % 32 == 0 and 16-byte aligned rows; the caller falls back to GEMM + cell kernel otherwise.
+// Requires H % 4 == 0, H >= 32 and 16-byte aligned rows; the caller falls back to GEMM + cell kernel otherwise.
 template <int G>
 struct RnnFusedCfg {
     static constexpr int U = (G == 1) ? 32 : 16;       // hidden units per workgroup
@@ -192,7 +196,7 @@ struct RnnFusedCfg {
     static constexpr int PITCH = 36;                   // floats per row of an LDS patch (32 + 4: conflict-free b128)
 };
 
-template <int G>
+template <int G, bool TAIL>
 __global__ void __launch_bounds__(256) rnn_step_fused_kernel(const RnnStepFwd s, const float* __restrict__ R) {
     using C = RnnFusedCfg<G>;
     constexpr int U = C::U, NT = C::NT, KS = C::KS, D = C::DEPTH, P = C::PITCH;
@@ -220,7 +224,7 @@ __global__ void __launch_bounds__(256) rnn_step_fused_kernel(const RnnStepFwd s,
     float* pa = &patch[wave][0][0];
     float* pb = &patch[wave][1][0];
 
-    const int groups = H / 32;                                   // groups of 32 k values
+    const int groups = (H + 31) / 32;                            // groups of 32 k values
     const int per = (groups + KS - 1) / KS;
     const int mbeg = kg * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
 
@@ -243,7 +247,7 @@ __global__ void __launch_bounds__(256) rnn_step_fused_kernel(const RnnStepFwd s,
     }
 
     f32x16 acc[4];
-    wave_product_32x32<D, P>(ap, bp, mbeg, mend, pa, pb, lane, acc);
+    wave_product_32x32<D, P, TAIL>(ap, bp, mbeg, mend, H, pa, pb, lane, acc);
     // accumulator register r holds row 8 (r / 4) + 4 lhi + r % 4, column l32 of the 32 x 32 tile
 #pragma unroll
     for (int r = 0; r < 16; ++r)
@@ -361,7 +365,7 @@ struct RnnBwdFusedCfg {
 
 typedef float f32x4_acc __attribute__((ext_vector_type(4)));
 
-template <int G>
+template <int G, bool TAIL>
 __global__ void __launch_bounds__(512) rnn_step_bwd_fused_kernel(const RnnStepBwd s, const float* __restrict__ dg_next,
                                                                  long long ld_dg, const float* __restrict__ Rt) {
     using C = RnnBwdFusedCfg;
@@ -388,7 +392,7 @@ __global__ void __launch_bounds__(512) rnn_step_bwd_fused_kernel(const RnnStepBw
         const int unit = (u0 + 8 * i + lrow < H) ? u0 + 8 * i + lrow : H - 1;
         bp[i] = Rt + (long long)unit * GH + lcol;
     }
-    const int groups = GH / 32;
+    const int groups = (GH + 31) / 32;
     const int per = (groups + KS - 1) / KS;
     const int mbeg = wave * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
 
@@ -429,10 +433,11 @@ __global__ void __launch_bounds__(512) rnn_step_bwd_fused_kernel(const RnnStepBw
 #pragma unroll
         for (int c = 0; c < 2; ++c) acc[hh][c] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
     auto load = [&](int slot, int m) {
+        const bool ok = !TAIL || 32 * m + lcol < GH;   // beyond K (not a multiple of 32): zeros
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ra[slot][i] = *reinterpret_cast<const f32x4*>(ap[i] + m * 32);
+        for (int i = 0; i < 4; ++i) ra[slot][i] = *reinterpret_cast<const f32x4*>(ok ? ap[i] + m * 32 : rnn_zero_vector);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) rb[slot][i] = *reinterpret_cast<const f32x4*>(bp[i] + m * 32);
+        for (int i = 0; i < 2; ++i) rb[slot][i] = *reinterpret_cast<const f32x4*>(ok ? bp[i] + m * 32 : rnn_zero_vector);
     };
     auto stage = [&](int slot, int f) {
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");

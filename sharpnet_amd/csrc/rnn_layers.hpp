@@ -5,9 +5,9 @@
 // Work of one layer and direction (n = batch * steps rows, G gates, H hidden units, I inputs):
 //   forward    gates (n x G*H) = X (n x I) . W^T + bW                                  one GEMM over all steps
 //              per step: gates[:, t] += h[t-1] . R^T (batch x G*H x H), cell -> h[t] into y and into the slot the
-//                        next step reads: one launch (rnn_step_fused_kernel) when H % 32 == 0, else GEMM + cell kernel
+//                        next step reads: one launch (rnn_step_fused_kernel) when H % 4 == 0, else GEMM + cell kernel
 //   backward   per step, last to first: dh = d(gates)[:, t+1] . R (batch x H x G*H), cell gradient -> d(gates)[:, t]:
-//                        one launch (rnn_step_bwd_fused_kernel) when H % 32 == 0, else cell kernel + GEMM
+//                        one launch (rnn_step_bwd_fused_kernel) when H % 4 == 0, else cell kernel + GEMM
 //              dX (n x I) = d(gates) . W                                               one GEMM
 //   weights    dW += d(gates)^T . X, dR += d(gates_h)^T . Hprev, bias gradients = column sums     two GEMMs
 // Hprev (n x H) holds, for every (sample, step), the state that entered the step, so the recurrent weight gradient
@@ -121,9 +121,12 @@ int rnn_set_rows(Handle* h, float* dst, long long ld_dst, const float* src, long
 
 // The backward step kernel stages more than the 64 KiB of LDS a kernel gets without asking.
 hipError_t rnn_prepare_kernels() {
-    const void* fns[3] = {reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<1>),
-                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<3>),
-                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<4>)};
+    const void* fns[6] = {reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<1, false>),
+                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<3, false>),
+                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<4, false>),
+                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<1, true>),
+                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<3, true>),
+                          reinterpret_cast<const void*>(rnn_step_bwd_fused_kernel<4, true>)};
     for (const void* f : fns) {
         const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, RnnBwdFusedCfg::LDS_BYTES);
         if (e != hipSuccess) return e;
@@ -238,7 +241,7 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
             const float *hx, *cx;
             int first, step;
         } dirs[2];
-        bool fused = H % 32 == 0 && h->rnn_step_mode == 0;
+        bool fused = H % 4 == 0 && H >= 32 && h->rnn_step_mode == 0;
         for (int d = 0; d < K; ++d) {
             const int p = layer * K + d;
             Dir& D = dirs[d];
@@ -300,12 +303,11 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
                 if (fused) {
                     const int U = G == 1 ? 32 : 16;
                     const dim3 grid((unsigned)((H + U - 1) / U), (unsigned)((B + 31) / 32));
-                    if (G == 4)
-                        hipLaunchKernelGGL(rnn_step_fused_kernel<4>, grid, dim3(256), 0, h->stream, c, (const float*)D.w.R);
-                    else if (G == 3)
-                        hipLaunchKernelGGL(rnn_step_fused_kernel<3>, grid, dim3(256), 0, h->stream, c, (const float*)D.w.R);
-                    else
-                        hipLaunchKernelGGL(rnn_step_fused_kernel<1>, grid, dim3(256), 0, h->stream, c, (const float*)D.w.R);
+                    const bool tail = H % 32 != 0;
+                    auto fn = G == 4   ? (tail ? rnn_step_fused_kernel<4, true> : rnn_step_fused_kernel<4, false>)
+                              : G == 3 ? (tail ? rnn_step_fused_kernel<3, true> : rnn_step_fused_kernel<3, false>)
+                                       : (tail ? rnn_step_fused_kernel<1, true> : rnn_step_fused_kernel<1, false>);
+                    hipLaunchKernelGGL(fn, grid, dim3(256), 0, h->stream, c, (const float*)D.w.R);
                 } else {
                     hipLaunchKernelGGL(rnn_cell_fwd_kernel, dim3((unsigned)(((long long)B * H + 255) / 256)), dim3(256), 0,
                                        h->stream, c);
@@ -352,7 +354,7 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
         } dirs[2];
         // every step but the first one processed runs as one launch (product with R, then the cell gradient) when
         // rows can be read in 16-byte pieces; that kernel wants the rows of R^T
-        bool fused = H % 32 == 0 && T > 1 && h->rnn_step_mode == 0;
+        bool fused = H % 4 == 0 && H >= 32 && T > 1 && h->rnn_step_mode == 0;
         for (int d = 0; d < K; ++d) {
             const int p = layer * K + d;
             Dir& D = dirs[d];
@@ -396,15 +398,12 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
                 if (one_launch) {
                     const float* dg_next = ((r.cell == RNN_GRU) ? D.gh : D.gates) + (long long)(t + D.step) * B * GH;
                     const dim3 grid((unsigned)((H + RnnBwdFusedCfg::U - 1) / RnnBwdFusedCfg::U), (unsigned)((B + 31) / 32));
-                    if (G == 4)
-                        hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<4>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
-                                           c, dg_next, GH, (const float*)D.Rt);
-                    else if (G == 3)
-                        hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<3>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
-                                           c, dg_next, GH, (const float*)D.Rt);
-                    else
-                        hipLaunchKernelGGL(rnn_step_bwd_fused_kernel<1>, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream,
-                                           c, dg_next, GH, (const float*)D.Rt);
+                    const bool tail = GH % 32 != 0;
+                    auto fn = G == 4   ? (tail ? rnn_step_bwd_fused_kernel<4, true> : rnn_step_bwd_fused_kernel<4, false>)
+                              : G == 3 ? (tail ? rnn_step_bwd_fused_kernel<3, true> : rnn_step_bwd_fused_kernel<3, false>)
+                                       : (tail ? rnn_step_bwd_fused_kernel<1, true> : rnn_step_bwd_fused_kernel<1, false>);
+                    hipLaunchKernelGGL(fn, grid, dim3(512), RnnBwdFusedCfg::LDS_BYTES, h->stream, c, dg_next, GH,
+                                       (const float*)D.Rt);
                     st = hip_to_status(hipGetLastError());
                     if (st != SNHIP_STATUS_SUCCESS) return st;
                     continue;

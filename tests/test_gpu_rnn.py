@@ -127,9 +127,9 @@ def test_cells_wider(gpu_wrapper, cell):
 
 
 @pytest.mark.parametrize("cell", [ro.RELU, ro.TANH, ro.LSTM, ro.GRU])
-@pytest.mark.parametrize("hidden,batch", [(32, 5), (64, 33), (96, 70), (160, 32)])
+@pytest.mark.parametrize("hidden,batch", [(32, 5), (64, 33), (96, 70), (160, 32), (36, 9), (100, 40), (44, 64)])
 def test_cells_one_launch_per_step(gpu_wrapper, cell, hidden, batch):
-    """Hidden sizes that are multiples of 32 take the kernel that computes h . R^T and the cell in one launch
+    """Hidden sizes that are multiples of 4 (from 32 up) take the kernel that computes h . R^T and the cell in one launch
     (K split over the wavefronts of a workgroup); checked against the oracle and against the GEMM + cell-kernel form
     selected through snhip_rnn_set_step_mode (different summation orders: 2e-5)."""
     rng = np.random.default_rng(hidden * 10 + batch + cell)
