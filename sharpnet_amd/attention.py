@@ -12,15 +12,19 @@ from . import hiplib
 from .gpu_tensor import GPUTensor
 from .hiplib import CublasStatus, check_status
 
-FUSED_ATTENTION_MAX_KEYS = 256      # limits of snhip_attention_forward
-FUSED_ATTENTION_MAX_HEAD_DIM = 64
+# limits of snhip_attention_forward: (keys, head dimension) pairs it has a kernel for
+FUSED_ATTENTION_LIMITS = ((256, 64), (128, 128))
+
+
+def fused_attention_supported(tkv, dk, dv):
+    return any(tkv <= keys and max(dk, dv) <= dim for keys, dim in FUSED_ATTENTION_LIMITS)
 
 
 def fused_attention_forward(Q, K, V, O, weights, *, batch, heads, tq, tkv, dk, dv, scale, is_causal, packed):
     """snhip_attention_forward.  packed=True: Q, K, V, O are (batch, steps, heads*dim) activations whose heads are
     addressed in place; False: contiguous (batch*heads, steps, dim) stacks.  Returns False (nothing launched) when
     the sizes are outside what the kernel handles."""
-    if tkv > FUSED_ATTENTION_MAX_KEYS or max(dk, dv) > FUSED_ATTENTION_MAX_HEAD_DIM:
+    if not fused_attention_supported(tkv, dk, dv):
         return False
 
     def strides(steps, dim):
@@ -64,8 +68,8 @@ def attention_backward(dQ, dK, dV, Q, K, V, dO, weights, scores_gradients, *, ba
 
 
 def ScaledDotProductAttentionForwardPropagation(Q, K, V, y, isTraining, use_scale, is_causal, fused=True):
-    """fused=True runs the whole chain as one launch when the sizes allow it (at most 256 keys, head dimension at
-    most 64); otherwise, or with fused=False, the reference's four calls."""
+    """fused=True runs the whole chain as one launch when the sizes allow it (at most 256 keys with a head dimension of at
+    most 64, or 128 keys with 128); otherwise, or with fused=False, the reference's four calls."""
     if V.Shape != K.Shape:
         raise ValueError("V.Shape and K.Shape must be equal, but are %s and %s" % (V.Shape, K.Shape))
     if V.Shape != y.Shape:

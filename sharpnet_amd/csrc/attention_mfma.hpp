@@ -38,7 +38,7 @@ constexpr int AT_BQ = 128;  // queries per workgroup
 
 template <int NT, int HD>
 struct AttnCfg {
-    static_assert(NT % 2 == 0 && NT <= 8 && (HD == 32 || HD == 64), "unsupported attention tile");
+    static_assert(NT % 2 == 0 && NT <= 8 && (HD == 32 || HD == 64 || HD == 128), "unsupported attention tile");
     static constexpr int KEYS = NT * 32;   // keys per (batch, head) at most
     static constexpr int KP = KEYS + 32;   // pitch of Ks[d][key]   (== 32 mod 64)
     static constexpr int VP = HD + 8;      // pitch of Vs[key][dv]  (4 * VP == 32 mod 64)

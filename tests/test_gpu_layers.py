@@ -361,6 +361,7 @@ def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrap
     (2, 3, 256, 256, 64, 64, True, True), (2, 3, 256, 256, 64, 64, False, False),   # the largest supported size
     (3, 2, 200, 130, 24, 40, False, True), (3, 2, 129, 65, 33, 7, True, False),     # Tq != Tk, dk != dv, odd sizes
     (1, 4, 1, 5, 3, 2, False, True),
+    (2, 2, 128, 128, 128, 128, True, True), (3, 1, 70, 100, 96, 128, False, False),  # head dimension up to 128: 128 keys
 ])
 def test_fused_attention_forward(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, causal, packed):
     """snhip_attention_forward (scores, mask, softmax and P.V in one launch) against the oracle's
@@ -399,17 +400,28 @@ def test_fused_attention_forward(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, caus
 
 
 def test_fused_attention_limits(gpu_wrapper):
-    """Beyond 256 keys or a head dimension of 64 nothing is launched and the caller is told so."""
+    """Beyond 256 keys (128 with a head dimension above 64) or a head dimension of 128 nothing is launched and the
+    caller is told so."""
     from sharpnet_amd import GPUTensor, attention
     w = gpu_wrapper
     big = GPUTensor([1, 300, 8], None, w)
     out = GPUTensor([1, 300, 8], None, w)
     assert attention.fused_attention_forward(big, big, big, out, None, batch=1, heads=1, tq=300, tkv=300, dk=8, dv=8,
                                              scale=1.0, is_causal=False, packed=False) is False
-    wide = GPUTensor([1, 16, 80], None, w)
-    outw = GPUTensor([1, 16, 80], None, w)
-    assert attention.fused_attention_forward(wide, wide, wide, outw, None, batch=1, heads=1, tq=16, tkv=16, dk=80, dv=80,
+    wide = GPUTensor([1, 16, 160], None, w)
+    outw = GPUTensor([1, 16, 160], None, w)
+    assert attention.fused_attention_forward(wide, wide, wide, outw, None, batch=1, heads=1, tq=16, tkv=16, dk=160, dv=160,
                                              scale=1.0, is_causal=False, packed=False) is False
+    long_wide = GPUTensor([1, 200, 80], None, w)
+    outl = GPUTensor([1, 200, 80], None, w)
+    assert attention.fused_attention_forward(long_wide, long_wide, long_wide, outl, None, batch=1, heads=1, tq=200, tkv=200,
+                                             dk=80, dv=80, scale=1.0, is_causal=False, packed=False) is False
+    # ... and the library says the same when asked directly
+    import ctypes
+    from sharpnet_amd import hiplib
+    d = hiplib.AttentionDesc(batch=1, Tq=200, Tk=200, dk=80, dv=80, Q=long_wide.Pointer, K=long_wide.Pointer,
+                             V=long_wide.Pointer, O=outl.Pointer, ldq=80, ldk=80, ldv=80, ldo=80)
+    assert w.lib.snhip_attention_forward(w.handle, ctypes.byref(d)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_SUPPORTED
     # the layer mirror falls back to the four-call sequence on its own
     y = GPUTensor([1, 300, 8], None, w)
     big.SetValue(0.5)
@@ -495,6 +507,8 @@ def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
     (5, 1, 37, 37, 16, 16, False), (2, 3, 256, 256, 64, 64, True), (2, 3, 256, 256, 64, 64, False),
     (3, 2, 200, 130, 24, 40, True), (3, 2, 129, 65, 33, 7, False), (1, 4, 1, 5, 3, 2, True),
     (1, 2, 40, 300, 8, 8, False),                                  # beyond 256 keys: the five-launch sequence
+    (2, 2, 128, 128, 128, 128, True), (3, 1, 70, 100, 96, 128, False),   # head dimension up to 128
+    (1, 2, 60, 200, 80, 80, False),                                # 200 keys x 80: the five-launch sequence
 ])
 def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, packed):
     """snhip_attention_backward (dV, score gradient through the softmax, dQ, dK; the middle two from one kernel when
