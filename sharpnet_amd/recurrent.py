@@ -4,7 +4,9 @@ The reference takes its SimpleRNN / LSTM / GRU layers from cuDNN; this class mak
 against libsharpnet_hip.so: weight space and per-gate views (RecurrentLayer.cs:138-190), forward with the reserve
 buffer kept for training (:305-408), backward data then backward weights into zeroed gradients (:410-520), with the
 reference's handling of ``returnSequences == false`` (last step of the forward direction, first step of the reverse
-one).  Encoder / decoder wiring (initial states taken from another layer) is available through ``hx`` / ``cx``.
+one) and of the encoder / decoder pair: an encoder's output is its final hidden states followed by its final cell
+states (two blocks of one buffer, RecurrentLayer.cs:526-533), a decoder takes that buffer as its initial states and
+returns their gradients in the same arrangement.
 """
 import ctypes
 
@@ -19,7 +21,10 @@ _GATES = {CUDNN_RNN_RELU: 1, CUDNN_RNN_TANH: 1, CUDNN_LSTM: 4, CUDNN_GRU: 3}
 
 class RecurrentLayer:
     def __init__(self, gpu_wrapper, inputSize, hiddenSize, cellMode, biasMode, returnSequences, isBidirectional,
-                 numLayers=1):
+                 numLayers=1, isEncoderThatWillBeFollowedByDecoder=False):
+        if isEncoderThatWillBeFollowedByDecoder and returnSequences:
+            raise ValueError("an Encoder can not return a sequence")            # RecurrentLayer.cs:128-131
+        self.IsEncoderThatWillBeFollowedByDecoder = isEncoderThatWillBeFollowedByDecoder
         self.Wrapper = gpu_wrapper
         self._lib = gpu_wrapper.lib
         self.desc = RnnDesc(cell_mode=cellMode, bias_mode=biasMode, bidirectional=bool(isBidirectional),
@@ -63,10 +68,18 @@ class RecurrentLayer:
                 t.Dispose()
 
     def OutputShape(self, batchSize, timeSteps):
-        # RNNDescriptor.Y_Shape (Prod/Layers/RNNDescriptor.cs:49-60), without the encoder variant
+        # RNNDescriptor.Y_Shape (Prod/Layers/RNNDescriptor.cs:49-60): an encoder returns hidden and cell states
+        K = self.K * (2 if self.IsEncoderThatWillBeFollowedByDecoder else 1)
         if self._returnSequences:
-            return [batchSize, timeSteps, self.K * self.hidden_size]
-        return [batchSize, self.K * self.hidden_size]
+            return [batchSize, timeSteps, K * self.hidden_size]
+        return [batchSize, K * self.hidden_size]
+
+    @staticmethod
+    def _ExtractEncoderContextVector(t):
+        """(hidden states, cell states): the two halves of an encoder's output buffer (RecurrentLayer.cs:526-533)."""
+        shape = list(t.Shape)
+        shape[-1] //= 2
+        return t.Slice(0, shape), t.Slice(t.Count // 2, shape)
 
     def _buffers(self, isTraining, batchSize, timeSteps):
         ws, rs = ctypes.c_size_t(), ctypes.c_size_t()
@@ -74,24 +87,28 @@ class RecurrentLayer:
                                                           ctypes.byref(ws), ctypes.byref(rs)), "snhip_rnn_temp_space_sizes")
         return ws.value, rs.value
 
-    def ForwardPropagation(self, x, y, isTraining, hx=None, cx=None, cy=None):
-        """x (batch, steps, input); y (batch, steps, K*hidden) or (batch, K*hidden) (RecurrentLayer.cs:305-408)."""
+    def ForwardPropagation(self, x, yFull, isTraining, encoderOutput=None):
+        """x (batch, steps, input); yFull (batch, steps, K*hidden) or (batch, K*hidden), twice as wide for an encoder;
+        encoderOutput: the output of the encoder this layer decodes (RecurrentLayer.cs:305-408)."""
         batchSize, timeSteps = x.Shape[0], x.Shape[1]
-        assert x.Shape[2] == self.input_size and y.Shape == self.OutputShape(batchSize, timeSteps)
+        assert x.Shape[2] == self.input_size and yFull.Shape == self.OutputShape(batchSize, timeSteps)
+        y, cy = self._ExtractEncoderContextVector(yFull) if self.IsEncoderThatWillBeFollowedByDecoder else (yFull, None)
+        hx, cx = self._ExtractEncoderContextVector(encoderOutput) if encoderOutput is not None else (None, None)
         ws_bytes, rs_bytes = self._buffers(isTraining, batchSize, timeSteps)
         workSpace = GPUTensor([ws_bytes // 4], None, self.Wrapper)
         self._reserveSpace = GPUTensor([rs_bytes // 4], None, self.Wrapper) if isTraining else None
         if self._returnSequences:
-            yFull, hy = y, None
+            ySeq, hy = y, None
         else:
-            yFull = GPUTensor([batchSize, timeSteps, self.K * self.hidden_size], None, self.Wrapper)
+            ySeq = GPUTensor([batchSize, timeSteps, self.K * self.hidden_size], None, self.Wrapper)
             # hy (K, batch, hidden) of the top layer; the lower layers' final states go to a scratch tensor
             hyAll = GPUTensor([self.K * self.num_layers, batchSize, self.hidden_size], None, self.Wrapper)
             hy = hyAll
+        cyAll = GPUTensor([self.K * self.num_layers, batchSize, self.hidden_size], None, self.Wrapper) if cy is not None else None
         check_status(self._lib.snhip_rnn_forward(
-            self.Wrapper.handle, ctypes.byref(self.desc), int(isTraining), batchSize, timeSteps, x.Pointer, yFull.Pointer,
+            self.Wrapper.handle, ctypes.byref(self.desc), int(isTraining), batchSize, timeSteps, x.Pointer, ySeq.Pointer,
             hx.Pointer if hx is not None else None, hy.Pointer if hy is not None else None,
-            cx.Pointer if cx is not None else None, cy.Pointer if cy is not None else None,
+            cx.Pointer if cx is not None else None, cyAll.Pointer if cyAll is not None else None,
             self._weightsAndBiases.Pointer, workSpace.Pointer, ws_bytes,
             self._reserveSpace.Pointer if isTraining else None, rs_bytes), "snhip_rnn_forward")
         if not self._returnSequences:
@@ -103,44 +120,62 @@ class RecurrentLayer:
                     y.Reshape(1, batchSize, self.K, self.hidden_size))
             else:
                 top.CopyTo(y)
+            if cyAll is not None:             # the top layer's cell states, (K, batch, hidden) as cuDNN leaves them
+                cyAll.Slice((self.num_layers - 1) * self.K * batchSize * self.hidden_size,
+                            [self.K, batchSize, self.hidden_size]).CopyTo(cy)
+                cyAll.Dispose()
             hyAll.Dispose()
             if isTraining:
-                self._yIfReturnSequences = yFull
+                self._yIfReturnSequences = ySeq
             else:
-                yFull.Dispose()
+                ySeq.Dispose()
         workSpace.Dispose()
 
-    def BackwardPropagation(self, x, y, dy, dx):
-        """RecurrentLayer.cs:410-520.  dx may be None (previous layer is the input)."""
+    def BackwardPropagation(self, x, yFull, dyFull, dx, encoderOutput=None, dEncoderOutput=None):
+        """RecurrentLayer.cs:410-520.  dx may be None (previous layer is the input).  A decoder also takes the encoder's
+        output again and writes the gradient with respect to it (hidden block, cell block) into dEncoderOutput."""
         assert self._reserveSpace is not None
         batchSize, timeSteps = x.Shape[0], x.Shape[1]
         H, K = self.hidden_size, self.K
+        y, _ = self._ExtractEncoderContextVector(yFull) if self.IsEncoderThatWillBeFollowedByDecoder else (yFull, None)
+        dy, dcy = self._ExtractEncoderContextVector(dyFull) if self.IsEncoderThatWillBeFollowedByDecoder else (dyFull, None)
+        hx, cx = self._ExtractEncoderContextVector(encoderOutput) if encoderOutput is not None else (None, None)
+        dhx, dcx = self._ExtractEncoderContextVector(dEncoderOutput) if dEncoderOutput is not None else (None, None)
         if self._returnSequences:
-            yFull, dyFull = y, dy
+            ySeq, dySeq = y, dy
         else:
-            yFull = self._yIfReturnSequences
-            dyFull = GPUTensor(yFull.Shape, None, self.Wrapper)
-            dyFull.ZeroMemory()
+            ySeq = self._yIfReturnSequences
+            dySeq = GPUTensor(ySeq.Shape, None, self.Wrapper)
+            dySeq.ZeroMemory()
             # last step takes the first half of dy, the first step (reverse direction) the second half (:437-454)
             for batchId in range(batchSize):
-                dy.Slice(batchId * K * H, [H]).CopyTo(dyFull.Slice((batchId * timeSteps + timeSteps - 1) * K * H, [H]))
+                dy.Slice(batchId * K * H, [H]).CopyTo(dySeq.Slice((batchId * timeSteps + timeSteps - 1) * K * H, [H]))
                 if K == 2:
-                    dy.Slice(batchId * K * H + H, [H]).CopyTo(dyFull.Slice(batchId * timeSteps * K * H + H, [H]))
+                    dy.Slice(batchId * K * H + H, [H]).CopyTo(dySeq.Slice(batchId * timeSteps * K * H + H, [H]))
         ws_bytes, rs_bytes = self._buffers(True, batchSize, timeSteps)
         workSpace = GPUTensor([ws_bytes // 4], None, self.Wrapper)
+        ptr = lambda t: t.Pointer if t is not None else None
+        # cell-state gradients travel as (K * layers, batch, hidden); with one layer that is the block itself
+        dcyAll = None
+        if dcy is not None:
+            dcyAll = GPUTensor([K * self.num_layers, batchSize, H], None, self.Wrapper)
+            dcyAll.ZeroMemory()
+            dcy.CopyTo(dcyAll.Slice((self.num_layers - 1) * K * batchSize * H, [K, batchSize, H]))
         check_status(self._lib.snhip_rnn_backward_data(
-            self.Wrapper.handle, ctypes.byref(self.desc), batchSize, timeSteps, yFull.Pointer, dyFull.Pointer,
-            dx.Pointer if dx is not None else None, None, None, None, None, None, None, self._weightsAndBiases.Pointer,
+            self.Wrapper.handle, ctypes.byref(self.desc), batchSize, timeSteps, ySeq.Pointer, dySeq.Pointer,
+            ptr(dx), ptr(hx), None, ptr(dhx), ptr(cx), ptr(dcyAll), ptr(dcx), self._weightsAndBiases.Pointer,
             workSpace.Pointer, ws_bytes, self._reserveSpace.Pointer, rs_bytes), "snhip_rnn_backward_data")
         self._weightsAndBiasesGradients.ZeroMemory()
         check_status(self._lib.snhip_rnn_backward_weights(
-            self.Wrapper.handle, ctypes.byref(self.desc), batchSize, timeSteps, x.Pointer, None, yFull.Pointer,
+            self.Wrapper.handle, ctypes.byref(self.desc), batchSize, timeSteps, x.Pointer, ptr(hx), ySeq.Pointer,
             self._weightsAndBiasesGradients.Pointer, workSpace.Pointer, ws_bytes, self._reserveSpace.Pointer, rs_bytes),
             "snhip_rnn_backward_weights")
         workSpace.Dispose()
+        if dcyAll is not None:
+            dcyAll.Dispose()
         self._reserveSpace.Dispose()
         self._reserveSpace = None
         if not self._returnSequences:
-            dyFull.Dispose()
+            dySeq.Dispose()
             self._yIfReturnSequences.Dispose()
             self._yIfReturnSequences = None

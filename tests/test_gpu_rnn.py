@@ -322,3 +322,52 @@ def test_degenerate_sequence_shapes(gpu_wrapper, cell, batch, steps, hidden):
     compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, 3e-5)
     got = run_gpu(gpu_wrapper, desc, x, weights, dy)
     compare(desc, got, x, weights, dy, None, None, None, None, 3e-5)
+
+
+@pytest.mark.parametrize("cell", [ro.LSTM, ro.GRU])
+def test_encoder_decoder_pair(gpu_wrapper, cell):
+    """An encoder (last step only, returns its final hidden and cell states as two blocks of one buffer) feeding a
+    decoder's initial states, forward and backward through the RecurrentLayer mirror, against the oracle run with
+    hx / cx / dhx / dcx passed by hand (RecurrentLayer.cs:318-319,421-423,526-533)."""
+    from sharpnet_amd import GPUTensor, recurrent
+    rng = np.random.default_rng(90 + cell)
+    B, T1, T2, I1, I2, H = 6, 5, 4, 7, 3, 32
+    de = ro.RnnDesc(cell, I1, H, 1, False, ro.DOUBLE_BIAS)
+    dd = ro.RnnDesc(cell, I2, H, 1, False, ro.DOUBLE_BIAS)
+    we = rng.uniform(-0.3, 0.3, ro.weight_space_size(de)).astype(np.float32)
+    wd = rng.uniform(-0.3, 0.3, ro.weight_space_size(dd)).astype(np.float32)
+    x1 = rng.uniform(-1, 1, (B, T1, I1)).astype(np.float32)
+    x2 = rng.uniform(-1, 1, (B, T2, I2)).astype(np.float32)
+    dy2 = rng.uniform(-1, 1, (B, T2, H)).astype(np.float32)
+    # oracle
+    _, hy1, cy1, c1 = ro.rnn_forward(de, x1, we)
+    y2, _, _, c2 = ro.rnn_forward(dd, x2, wd, hy1, cy1 if cell == ro.LSTM else None)
+    dx2, dw2, dhx2, dcx2 = ro.rnn_backward(dd, dy2, c2)
+    dseq = np.zeros((B, T1, H), np.float32)
+    dseq[:, -1, :] = dhx2[0]
+    dx1, dw1, _, _ = ro.rnn_backward(de, dseq, c1, None, dcx2 if cell == ro.LSTM else None)
+    # device
+    w = gpu_wrapper
+    enc = recurrent.RecurrentLayer(w, I1, H, cell, ro.DOUBLE_BIAS, False, False, 1, isEncoderThatWillBeFollowedByDecoder=True)
+    dec = recurrent.RecurrentLayer(w, I2, H, cell, ro.DOUBLE_BIAS, True, False, 1)
+    enc._weightsAndBiases.InitializeFromHostMemory(we)
+    dec._weightsAndBiases.InitializeFromHostMemory(wd)
+    gx1, gx2, gdy2 = T(w, x1), T(w, x2), T(w, dy2)
+    assert enc.OutputShape(B, T1) == [B, 2 * H]
+    enc_out, d_enc_out = GPUTensor([B, 2 * H], None, w), GPUTensor([B, 2 * H], None, w)
+    gy2, gdx2, gdx1 = GPUTensor([B, T2, H], None, w), GPUTensor([B, T2, I2], None, w), GPUTensor([B, T1, I1], None, w)
+    enc_out.ZeroMemory()
+    d_enc_out.ZeroMemory()
+    enc.ForwardPropagation(gx1, enc_out, True)
+    dec.ForwardPropagation(gx2, gy2, True, encoderOutput=enc_out)
+    dec.BackwardPropagation(gx2, gy2, gdy2, gdx2, encoderOutput=enc_out, dEncoderOutput=d_enc_out)
+    enc.BackwardPropagation(gx1, enc_out, d_enc_out, gdx1)
+    eo = enc_out.ToNumpy().reshape(-1)
+    assert np.max(np.abs(eo[:B * H].reshape(B, H) - hy1[0])) <= 2e-5
+    if cell == ro.LSTM:
+        assert np.max(np.abs(eo[B * H:].reshape(B, H) - cy1[0])) <= 2e-5
+    assert np.max(np.abs(gy2.ToNumpy() - y2)) <= 2e-5
+    assert np.max(np.abs(gdx2.ToNumpy() - dx2)) <= 5e-5 * max(1.0, float(np.max(np.abs(dx2))))
+    assert np.max(np.abs(dec._weightsAndBiasesGradients.ToNumpy() - dw2)) <= 5e-5 * max(1.0, float(np.max(np.abs(dw2))))
+    assert np.max(np.abs(gdx1.ToNumpy() - dx1)) <= 5e-5 * max(1.0, float(np.max(np.abs(dx1))))
+    assert np.max(np.abs(enc._weightsAndBiasesGradients.ToNumpy() - dw1)) <= 5e-5 * max(1.0, float(np.max(np.abs(dw1))))
