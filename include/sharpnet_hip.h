@@ -76,6 +76,23 @@ int snhip_sgemm_strided_batched(void* handle, int transa, int transb, int m, int
 int snhip_dot(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
               int transposeB, float* C, float alpha, float beta);
 
+/* snhip_dot for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same kernels, same choice
+ * of tile configuration and split-K factor, bit-identical results; the difference is where split-K partial sums
+ * go: into a fixed array of snhip_static_scratch_bytes() (32 MiB) that is part of the library's code object on
+ * every GPU, instead of the handle's lazily grown workspace.  The call never allocates, frees or synchronises.
+ * A product whose partial sums need more than the array holds is refused with status 15 (NOT_SUPPORTED) before
+ * anything is launched; snhip_get_last_error_message then says how many bytes were needed.  Products that run
+ * without split-K use no scratch and are never refused.  All handles of one GPU share that GPU's array: calls that
+ * overlap in time on one GPU (two handles on two streams) race on it. */
+int snhip_dot_noalloc(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
+                      int transposeB, float* C, float alpha, float beta);
+/* Size in bytes of the static scratch array (returns the size, not a status). */
+int snhip_static_scratch_bytes(void);
+/* Copies the text of the handle's last refusal that carries detail beyond its status code (empty if none) into
+ * buffer as a NUL-terminated string of at most capacity bytes. */
+int snhip_get_last_error_message(void* handle, char* buffer, int capacity);
+
 /* snhip_dot followed by C[m][n] += bias[n], in one kernel.  Replaces the pair
  * Dot + BroadcastAddVectorToOutput of Linear.DenseForwardPropagation
  * (Prod/Layers/Linear.cs:130-131; GPU bias add at GpuTensor.cs:633-644).

@@ -8,6 +8,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include <mutex>
 #include <new>
 
 #include "attention_mfma.hpp"
@@ -20,7 +21,33 @@ SNHIP_ALL_KERNEL_GROUPS(SNHIP_DECLARE_KERNELS)
 
 using namespace snhip;
 
+// Split-K partial sums of snhip_dot_noalloc: device memory that exists from the moment the code object is loaded,
+// so that entry point never has to allocate.  One copy per GPU, held until the process ends.  In host code this
+// name is only a handle for hipGetSymbolAddress; kernels and copies get the address that call returned.
+constexpr size_t kStaticScratchBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
+
+// Device address of `scratch` on each GPU, looked up once per device (with that device current) by snhip_create.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+hipError_t static_scratch_address(int dev, void** out) {
+    *out = nullptr;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (ptr == nullptr) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return hipSuccess;
+}
 
 constexpr int kVersion = 100;  // 0.1.0
 
@@ -39,6 +66,8 @@ struct Handle {
     int last_cfg = -1;
     int last_splitk = 0;
     int rnn_step_mode = 0;  // 0: recurrent forward steps as one launch when the shape allows, 1: always GEMM + cell kernel
+    float* static_scratch = nullptr;  // this device's copy of `scratch` (kStaticScratchBytes), never freed
+    char last_error[192] = {0};       // text of the last refusal that has more to say than its status code
 };
 
 // Upper bound for the split-K workspace; larger requests fall back to fewer splits.
@@ -358,6 +387,7 @@ struct GemmArgs {
     float act_param = 0.0f;
     float* colsum = nullptr;
     int math = -1;  // -1: the handle's math mode
+    bool no_alloc = false;  // split-K partial sums go to the static scratch array; nothing is allocated or freed
 };
 
 // Whether the product goes to sgemm_ksplit_kernel (32 x 32 tiles, K split inside the workgroup) instead of the
@@ -553,11 +583,22 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     bool fused_reduce = false;
     if (ch.splitk > 1) {
         const size_t need = (size_t)M * N * batch * ch.splitk * sizeof(float);
-        int st = ensure_workspace(h, need);
-        if (st != SNHIP_STATUS_SUCCESS) return st;
-        p.ws = h->ws;
+        int st = SNHIP_STATUS_SUCCESS;
+        if (g.no_alloc) {
+            if (need > kStaticScratchBytes || h->static_scratch == nullptr) {
+                snprintf(h->last_error, sizeof(h->last_error),
+                         "snhip_dot_noalloc: %d x %d x %d with split-K %d needs %zu bytes of partial sums, the static "
+                         "scratch holds %zu", M, N, K, ch.splitk, need, kStaticScratchBytes);
+                return SNHIP_STATUS_NOT_SUPPORTED;
+            }
+            p.ws = h->static_scratch;
+        } else {
+            st = ensure_workspace(h, need);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+            p.ws = h->ws;
+        }
         if (N % 4 == 0) p.flags |= GEMM_FLAG_WS_VEC;
-        fused_reduce = (h->splitk_mode == 2);
+        fused_reduce = (h->splitk_mode == 2) && !g.no_alloc;  // the arrival counters would have to be allocated
         if (fused_reduce) {
             st = ensure_counters(h, (size_t)(ntiles * batch));
             if (st != SNHIP_STATUS_SUCCESS) return st;
@@ -580,8 +621,8 @@ int gemm_core(Handle* h, const GemmArgs& g) {
         er.act = ep_kernel.act;
         const long long total = (long long)M * N * batch;
         const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, h->stream, h->ws, g.C, er, M, N, g.ldc, g.sC,
-                           g.sC2, inner, ch.splitk, batch, g.alpha, g.beta);
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, h->stream, (const float*)p.ws, g.C, er, M, N,
+                           g.ldc, g.sC, g.sC2, inner, ch.splitk, batch, g.alpha, g.beta);
         e = hipGetLastError();
         if (e != hipSuccess) return hip_to_status(e);
     }
@@ -654,8 +695,12 @@ int snhip_create(void** handle) {
     }
     e = rnn_prepare_kernels();
     if (e != hipSuccess) return hip_to_status(e);
+    void* scratch_ptr = nullptr;
+    e = static_scratch_address(dev, &scratch_ptr);
+    if (e != hipSuccess) return hip_to_status(e);
     Handle* h = new (std::nothrow) Handle();
     if (h == nullptr) return SNHIP_STATUS_ALLOC_FAILED;
+    h->static_scratch = static_cast<float*>(scratch_ptr);
     h->device = dev;
     h->num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     *handle = h;
@@ -945,6 +990,29 @@ int snhip_dot_bias(void* handle, const float* A, int aH, int aW, int transposeA,
 int snhip_dot(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
               int transposeB, float* C, float alpha, float beta) {
     return snhip_dot_bias(handle, A, aH, aW, transposeA, B, bH, bW, transposeB, C, alpha, beta, nullptr);
+}
+
+int snhip_dot_noalloc(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
+                      int transposeB, float* C, float alpha, float beta) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (aH < 0 || aW < 0 || bH < 0 || bW < 0) return SNHIP_STATUS_INVALID_VALUE;
+    GemmArgs g;  // BlasServices.DotMkl's derivation, as in snhip_dot
+    g.tA = transposeA != 0, g.tB = transposeB != 0;
+    g.M = transposeA ? aW : aH, g.N = transposeB ? bH : bW, g.K = transposeA ? aH : aW;
+    if (g.K != (transposeB ? bW : bH)) return SNHIP_STATUS_INVALID_VALUE;
+    g.alpha = alpha, g.beta = beta;
+    g.A = A, g.lda = aW, g.B = B, g.ldb = bW, g.C = C, g.ldc = g.N;
+    g.no_alloc = true;
+    return gemm_core(static_cast<Handle*>(handle), g);
+}
+
+int snhip_static_scratch_bytes(void) { return (int)kStaticScratchBytes; }
+
+int snhip_get_last_error_message(void* handle, char* buffer, int capacity) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (buffer == nullptr || capacity <= 0) return SNHIP_STATUS_INVALID_VALUE;
+    snprintf(buffer, (size_t)capacity, "%s", static_cast<Handle*>(handle)->last_error);
+    return SNHIP_STATUS_SUCCESS;
 }
 
 int snhip_bmm(void* handle, const float* A, int aH, int aW, int transposeA, long long strideA, const float* B, int bH,

@@ -161,6 +161,9 @@ SIGNATURES = {
     "snhip_sgemm_strided_batched": [_vp, _i, _i, _i, _i, _i, _c_float_p, _vp, _i, _ll, _vp, _i, _ll, _c_float_p, _vp,
                                     _i, _ll, _i],
     "snhip_dot": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f],
+    "snhip_dot_noalloc": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f],
+    "snhip_static_scratch_bytes": [],
+    "snhip_get_last_error_message": [_vp, ctypes.c_char_p, _i],
     "snhip_dot_bias": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f, _vp],
     "snhip_bmm": [_vp, _vp, _i, _i, _i, _ll, _vp, _i, _i, _i, _ll, _vp, _ll, _i, _f, _f],
     "snhip_gemm_rm": [_vp, _i, _i, _i, _i, _i, _f, _vp, _i, _ll, _vp, _i, _ll, _f, _vp, _i, _ll, _i, _vp],
