@@ -186,7 +186,8 @@ def main():
     from oracle import dot_oracle
     rng = np.random.default_rng(99)
     rows = np.sort(rng.choice(g.M, 16, replace=False))
-    got = gc.ToNumpy()[rows]
+    gpu_c = gc.ToNumpy()
+    got = gpu_c[rows]
     ref = dot_oracle.dot(np.ascontiguousarray(a[rows]), False, b, False)
     err = float(np.max(np.abs(got - ref)))
     bound = dot_oracle.tolerance(g.K, a, b)
@@ -195,11 +196,17 @@ def main():
         sys.exit("bench.py: timed result is outside the parity bound")
     gc.Dispose()
 
-    traffic = None
+    # HBM traffic per launch is a counter figure (two rocprofv3 --pmc runs); it cannot be collected from inside
+    # this process, so the line carries the stored figure together with where and when it was measured.
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "sgemm_8192_hbm_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+            tj = json.load(f)
+        traffic = tj.get("hbm_bytes_per_launch")
+        traffic_source = {"file": "profiles/sgemm_8192_hbm_traffic.json", "measured_in_this_run": False,
+                          "kernel": tj.get("workload"), "kernel_source_commit": tj.get("kernel_source_commit"),
+                          "summary": tj.get("source")}
 
     out = {
         "metric": "fp32 GEMM throughput, Tensor.Dot M=N=K=8192 (GEMM TFLOP/s + % of fp32 MFMA peak at 1 GPU)",
@@ -212,7 +219,7 @@ def main():
                    "device": {"cu": info["compute_units"], "clock_mhz": info["clock_khz"] / 1000.0}},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": wl.FP32_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / wl.FP32_MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
-                     "flops_per_launch": g.flops, "ms_per_launch_hip_events": round(ev_ms, 4)},
+                     "traffic_source": traffic_source, "flops_per_launch": g.flops, "ms_per_launch_hip_events": round(ev_ms, 4)},
         "parity": {"max_abs_err": err, "bound": bound, "rows_checked": 16},
     }
 
@@ -253,26 +260,80 @@ def main():
                       "median %.2f s per call; os.cpu_count()=%d" % (args.cpu_reps, route, cpu_s, os.cpu_count()),
         }
         log("[bench] cpu baseline:", out["cpu_baseline"])
+        # the whole timed GPU result against the whole MKL result of the same product
+        err_mkl = 0.0
+        for r0 in range(0, g.M, 1024):
+            err_mkl = max(err_mkl, float(np.max(np.abs(gpu_c[r0:r0 + 1024] - cpu_out[r0:r0 + 1024]))))
+        out["parity"]["max_abs_err_vs_mkl_full_result"] = err_mkl
+        log("[bench] timed GPU result against the MKL result, all %d x %d elements: max|d| = %.3e (bound %.3e)"
+            % (g.M, g.N, err_mkl, bound))
+        if not err_mkl <= bound:
+            sys.exit("bench.py: timed result differs from the MKL result by more than the parity bound")
         del cpu_out
-    del a, b
+    del a, b, gpu_c
 
-    # ------------------------------------------------------------------ the other configurations (GPU side)
+    # ------------------------------------------------------------------ the other configurations
+    # GPU figure and, beside it, the reference's CPU route for the same product on this box's host cores:
+    # cblas_sgemm RowMajor through MKL (BlasServices.cs:20), the bias pass of Linear.cs:131 where the layer has
+    # one, and the serial per-matrix loop of CpuTensor.cs:3018-3024 for the batched products.  The CPU side is a
+    # bounded sample (a few calls per product); its total is logged.
     if not args.no_extra:
         extra = {}
+        cpu_on = not args.no_cpu
+        cpu_cores = dot_oracle.mkl_threads() if cpu_on else 0
+        cpu_spent = [0.0]
 
-        def run(gm, seed, steps=10, warmup=3, bias=None):
+        def cpu_ms(gm, aa, bb, cc, reps, bias=None):
+            """Median ms of the product through MKL after one warm-up call."""
+            t_in = time.perf_counter()
+            out = np.array(cc, np.float32) if cc is not None else np.empty(gm.c_shape, np.float32)
+            ts = []
+            for rep in range(reps + 1):
+                t0 = time.perf_counter()
+                if gm.batch > 1:
+                    dot_oracle.mkl_bmm_serial(aa, gm.tA, bb, gm.tB, out, gm.alpha, gm.beta)
+                else:
+                    dot_oracle.mkl_dot(aa, gm.tA, bb, gm.tB, out, gm.alpha, gm.beta)
+                    if bias is not None:
+                        np.add(out, bias.reshape(1, -1), out=out)
+                if rep > 0:
+                    ts.append(time.perf_counter() - t0)
+            cpu_spent[0] += time.perf_counter() - t_in
+            return float(np.median(ts)) * 1e3
+
+        def run(gm, seed, steps=10, warmup=3, bias=None, cpu_reps=0):
             aa, bb, cc = wl.uniform_operands(gm, seed)
             _, ms, gcx = time_gemm(gm, aa, bb, cc, steps, warmup, bias=bias, min_warm_ms=40.0)
             gcx.Dispose()
             tf = gm.flops / (ms * 1e-3) / 1e12
-            return {"gemm": gm.label(), "ms": round(ms, 4), "tflops": round(tf, 2),
-                    "frac_of_roofline": round(gm.roofline_seconds() * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
-                    "splitk": w.last_tuning()[1]}
+            r = {"gemm": gm.label(), "ms": round(ms, 4), "tflops": round(tf, 2),
+                 "frac_of_roofline": round(gm.roofline_seconds() * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
+                 "splitk": w.last_tuning()[1]}
+            if cpu_on and cpu_reps > 0:
+                cms = cpu_ms(gm, aa, bb, cc, cpu_reps, bias=bias)
+                r["cpu_mkl_ms"] = round(cms, 4)
+                r["cpu_mkl_tflops"] = round(gm.flops / (cms * 1e-3) / 1e12, 4)
+            return r
 
-        extra["config1_dense_layer"] = [run(gm, 1, 50, 10, bias=np.zeros(gm.N, np.float32) if gm.bias else None)
-                                        for gm in wl.dense_layer_gemms()]
-        if not args.no_cpu:
-            # the same three products (and the bias add) on the host: the reference's CPU route through MKL
+        def cpu_summary(rows, gemms, sample):
+            """cpu_baseline object of one configuration from its per-product rows."""
+            timed = [(r, gm) for r, gm in zip(rows, gemms) if "cpu_mkl_ms" in r]
+            if not timed:
+                return None
+            total_ms = sum(r["cpu_mkl_ms"] for r, _ in timed)
+            flops = sum(gm.flops for _, gm in timed)
+            return {"value": round(flops / (total_ms * 1e-3) / 1e12, 4), "unit": "TFLOP/s", "cores": cpu_cores,
+                    "kind": "port", "ms": round(total_ms, 4),
+                    "gpu_ms_same_products": round(sum(r["ms"] for r, _ in timed), 4), "sample": sample}
+
+        dense = wl.dense_layer_gemms()
+        rows = [run(gm, 1, 50, 10, bias=np.zeros(gm.N, np.float32) if gm.bias else None, cpu_reps=200) for gm in dense]
+        extra["config1_dense_layer"] = {
+            "gemms": rows,
+            "cpu_baseline": cpu_summary(rows, dense, "forward (cblas_sgemm NT + bias pass), dW (TN), dx (NN) of the "
+                                        "128 x 784 -> 256 layer, each the median of 200 calls after a warm-up")}
+        if cpu_on:
+            # the same three products (and the bias add) back to back on the host, as a layer step runs them
             d = wl.dense_layer_inputs(seed=1)
             x, wt, dyv = d["x"], d["w_out_in"], d["dy"]
             y, dwv, dxv = (np.empty(sh, np.float32) for sh in ((x.shape[0], wt.shape[0]), wt.shape, x.shape))
@@ -288,40 +349,77 @@ def main():
             t0 = time.perf_counter()
             for _ in range(200):
                 cpu_layer()
-            cpu_ms = (time.perf_counter() - t0) * 1e3 / 200
-            gpu_ms = sum(r["ms"] for r in extra["config1_dense_layer"])
+            cpu_layer_ms = (time.perf_counter() - t0) * 1e3 / 200
+            cpu_spent[0] += time.perf_counter() - t0
+            gpu_ms = sum(r["ms"] for r in rows)
             extra["config1_dense_layer_fwd_bwd"] = {
-                "gpu_ms": round(gpu_ms, 4), "cpu_mkl_ms": round(cpu_ms, 4), "cpu_cores": dot_oracle.mkl_threads(),
+                "gpu_ms": round(gpu_ms, 4), "cpu_mkl_ms": round(cpu_layer_ms, 4), "cpu_cores": cpu_cores,
                 "note": "forward + dW + dx of the 128 x 784 -> 256 layer; GPU = sum of the three launches above, "
                         "CPU = cblas_sgemm x 3 + bias add, 200 repetitions"}
-        sweep = []
+        sweep, sweep_gemms = [], []
         for (M, N, K) in wl.SWEEP_SIZES:
-            for tA in (False, True):
-                for tB in (False, True):
-                    steps, warm = (5, 3) if M * N * K > 1e11 else (50, 20)
-                    sweep.append(run(wl.Gemm(M, N, K, tA, tB, 1.0, 0.0), 2, steps, warm))
-            sweep.append(run(wl.Gemm(M, N, K, False, False, 1.0, 1.0), 2, steps, warm))
-        extra["config2_sweep"] = sweep
-        mlp = [run(gm, 3, 20, 10, bias=np.zeros(gm.N, np.float32) if gm.bias else None) for gm in wl.mlp_gemms()]
+            steps, warm = (5, 3) if M * N * K > 1e11 else (50, 20)
+            for beta in (0.0, 1.0):
+                for tA in (False, True):
+                    for tB in (False, True):
+                        gm = wl.Gemm(M, N, K, tA, tB, 1.0, beta)
+                        # CPU side: one transpose form per size (NN, beta = 0); the 8192^3 one is the headline's
+                        cpu_reps = 2 if (not tA and not tB and beta == 0.0 and (M, N, K) != (8192, 8192, 8192)) else 0
+                        sweep.append(run(gm, 2, steps, warm, cpu_reps=cpu_reps))
+                        sweep_gemms.append(gm)
+        if cpu_on and "cpu_baseline" in out:
+            for r, gm in zip(sweep, sweep_gemms):
+                if (gm.M, gm.N, gm.K, gm.layout, gm.beta) == (8192, 8192, 8192, "NN", 0.0):
+                    r["cpu_mkl_tflops"] = out["cpu_baseline"]["value"]
+                    r["cpu_mkl_ms"] = round(gm.flops / (out["cpu_baseline"]["value"] * 1e12) * 1e3, 4)
+        extra["config2_sweep"] = {
+            "gemms": sweep,
+            "cpu_baseline": cpu_summary(sweep, sweep_gemms, "the NN beta=0 product of each of the seven sizes through "
+                                        "cblas_sgemm, median of 2 calls after a warm-up (8192^3: the headline's "
+                                        "cpu_baseline); per-size figures in the rows")}
+        mlp_g = wl.mlp_gemms()
+        mlp = [run(gm, 3, 20, 10, bias=np.zeros(gm.N, np.float32) if gm.bias else None, cpu_reps=1) for gm in mlp_g]
         extra["config3_mlp_step"] = {"gemms": mlp, "total_ms": round(sum(r["ms"] for r in mlp), 4),
-                                     "tflops": round(sum(gm.flops for gm in wl.mlp_gemms()) /
-                                                     (sum(r["ms"] for r in mlp) * 1e-3) / 1e12, 2)}
+                                     "tflops": round(sum(gm.flops for gm in mlp_g) /
+                                                     (sum(r["ms"] for r in mlp) * 1e-3) / 1e12, 2),
+                                     "cpu_baseline": cpu_summary(mlp, mlp_g, "all nine products of the step (forward ones "
+                                                                 "with the bias pass), one timed call each after a "
+                                                                 "warm-up")}
         proj, rec, seq = wl.lstm_gemms()
-        extra["config4_lstm"] = {"input_projection": run(proj, 4, 20, 10), "recurrent_step": run(rec, 4, seq, 20),
-                                 "recurrent_steps": seq}
-        extra["config5_attention_fp32"] = [run(gm, 5, 50, 10) for gm in wl.attention_gemms()]
+        lstm_rows = [run(proj, 4, 20, 10, cpu_reps=2), run(rec, 4, seq, 20, cpu_reps=16)]
+        cb = cpu_summary(lstm_rows, [proj, rec], "")
+        if cb is not None:
+            # the whole configuration: one projection + `seq` sequential recurrent products (beta = 1)
+            whole_ms = lstm_rows[0]["cpu_mkl_ms"] + seq * lstm_rows[1]["cpu_mkl_ms"]
+            cb.update({"value": round((proj.flops + seq * rec.flops) / (whole_ms * 1e-3) / 1e12, 4), "ms": round(whole_ms, 4),
+                       "gpu_ms_same_products": round(lstm_rows[0]["ms"] + seq * lstm_rows[1]["ms"], 4),
+                       "sample": "input projection: median of 2 calls; recurrent product (beta = 1): median of 16 of the "
+                                 "%d sequential calls, scaled to %d" % (seq, seq)})
+        extra["config4_lstm"] = {"gemms": lstm_rows, "input_projection": lstm_rows[0], "recurrent_step": lstm_rows[1],
+                                 "recurrent_steps": seq, "cpu_baseline": cb}
+        att_g = wl.attention_gemms()
+        att = [run(gm, 5, 50, 10, cpu_reps=3) for gm in att_g]
+        extra["config5_attention_fp32"] = {
+            "gemms": att,
+            "cpu_baseline": cpu_summary(att, att_g, "serial loop over the 512 matrices, one cblas_sgemm each "
+                                        "(CpuTensor.BatchMatrixMultiplication), median of 3 passes after a warm-up")}
         # bf16-input / fp32-accumulate variant (operands stay fp32 in HBM, rounded on the way into LDS)
         w.set_math_mode(w.MATH_BF16_INPUT)
         try:
-            bf = [run(gm, 5, 50, 10) for gm in wl.attention_gemms()]
-            for r, gm in zip(bf, wl.attention_gemms()):   # HBM-bound: roofline = bytes / 8 TB/s vs bf16 MFMA peak
+            bf = [run(gm, 5, 50, 10) for gm in att_g]
+            for r, gm in zip(bf, att_g):   # HBM-bound: roofline = bytes / 8 TB/s vs bf16 MFMA peak
                 r["frac_of_roofline"] = round(gm.roofline_seconds(wl.BF16_MFMA_PEAK_TFLOPS) * 1e3 / r["ms"], 4)
-            extra["config5_attention_bf16_input"] = bf
+            extra["config5_attention_bf16_input"] = {
+                "gemms": bf, "cpu_baseline": extra["config5_attention_fp32"]["cpu_baseline"],
+                "note": "the reference has no reduced-precision CPU route: the CPU figure is the fp32 one"}
             hb = run(wl.Gemm(8192, 8192, 8192, True, False, 1.0, 0.0), 2, 10, 5)
             hb["frac_of_roofline"] = round(hb["tflops"] / wl.BF16_MFMA_PEAK_TFLOPS, 4)
             extra["config2_8192_bf16_input_TN"] = hb
         finally:
             w.set_math_mode(w.MATH_FP32)
+        if cpu_on:
+            extra["cpu_leg_seconds"] = round(cpu_spent[0], 1)
+            log("[bench] CPU side of the other configurations took %.1f s" % cpu_spent[0])
         extra["layers_fused_vs_reference_sequence"] = layer_timings(w, wl)
         out["extra"] = extra
         for k, v in extra.items():
@@ -487,24 +585,29 @@ def write_table(path, out):
     rows = []
     layers = out["extra"].get("layers_fused_vs_reference_sequence", [])
     for name, v in out["extra"].items():
-        if name in ("layers_fused_vs_reference_sequence", "config1_dense_layer_fwd_bwd"):
+        if name in ("layers_fused_vs_reference_sequence", "config1_dense_layer_fwd_bwd") or not isinstance(v, (list, dict)):
             continue
-        items = v if isinstance(v, list) else v.get("gemms") or [x for x in v.values() if isinstance(x, dict)] or [v]
-        if isinstance(v, dict) and "gemm" in v:
-            items = [v]
+        items = v if isinstance(v, list) else v.get("gemms") or [v]
         for r in items:
-            rows.append("| %s | %s | %.4f | %.1f | %.3f | %d | %d |" % (name, r["gemm"], r["ms"], r["tflops"],
-                                                                       r["frac_of_roofline"], r["tile_config"], r["splitk"]))
+            rows.append("| %s | %s | %.4f | %.1f | %.3f | %d | %d | %s | %s |" % (
+                name, r["gemm"], r["ms"], r["tflops"], r["frac_of_roofline"], r["tile_config"], r["splitk"],
+                "%.4f" % r["cpu_mkl_ms"] if "cpu_mkl_ms" in r else "", "%.3f" % r["cpu_mkl_tflops"] if "cpu_mkl_ms" in r else ""))
         if isinstance(v, dict) and "total_ms" in v:
-            rows.append("| %s | all nine GEMMs | %.4f | %.1f | | | |" % (name, v["total_ms"], v["tflops"]))
+            rows.append("| %s | all nine GEMMs | %.4f | %.1f | | | | | |" % (name, v["total_ms"], v["tflops"]))
+        cb = v.get("cpu_baseline") if isinstance(v, dict) else None
+        if cb:
+            rows.append("| %s | CPU baseline of the configuration: %s | %.4f (GPU, same products) | | | | | %.4f | %.3f |" % (
+                name, cb["sample"], cb["gpu_ms_same_products"], cb["ms"], cb["value"]))
     cpu = out.get("cpu_baseline")
     with open(path, "w") as f:
         f.write("# Per-configuration GPU figures (MI355X, one GPU, fp32 unless noted)\n\n"
                 "Command: `python bench.py --table %s` (the table is the `extra` object of its JSON line). time = HIP events\n"
                 "around the timed launches; fraction = max(flops / 157.3 TFLOP/s, bytes / 8 TB/s) / time (bf16-input rows:\n"
                 "against the 2.5 PFLOP/s bf16 peak or 8 TB/s); tile config = index into `snhip_config_desc`.\n\n"
-                "| configuration | GEMM | ms | TFLOP/s | fraction of roofline | tile config | split-K |\n"
-                "|---|---|---|---|---|---|---|\n" % path)
+                "CPU columns: the same product through MKL cblas_sgemm on the box's host cores (%s threads), the reference's CPU route;\n"
+                "batched products as the reference's serial loop over the matrices.\n\n"
+                "| configuration | GEMM | ms | TFLOP/s | fraction of roofline | tile config | split-K | CPU (MKL) ms | CPU TFLOP/s |\n"
+                "|---|---|---|---|---|---|---|---|---|\n" % (path, cpu["cores"] if cpu else "no"))
         f.write("\n".join(rows) + "\n\n")
         fb = out["extra"].get("config1_dense_layer_fwd_bwd")
         if fb:

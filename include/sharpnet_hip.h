@@ -266,7 +266,7 @@ int snhip_sizeof_attention_bwd_desc(void);
  * gradients are (dirs * num_layers, batch, hidden_size), any of them may be NULL (zeros in, nothing out).
  * Each time step is one GEMM with the recurrent matrix plus one element-wise kernel; the input projections of all
  * steps, dx and both weight gradients are one GEMM each per layer and direction.  Dropout between stacked layers is
- * not implemented (the descriptor has no such field; the caller stacks single layers if it needs it). */
+ * not implemented: a descriptor that asks for it is refused in training (status 15), never silently ignored. */
 #define SNHIP_RNN_RELU 0 /* cudnnRNNMode_t, Prod/GPU/CudnnWrapper.cs:313-327 */
 #define SNHIP_RNN_TANH 1
 #define SNHIP_RNN_LSTM 2
@@ -281,6 +281,9 @@ typedef struct snhip_rnn_desc { /* the fields of Prod/Layers/RNNDescriptor.cs th
     int bidirectional;          /* 0 / 1 */
     int num_layers;
     int input_size, hidden_size;
+    float dropout;              /* RNNDescriptor.dropoutRate (Prod/Layers/RNNDescriptor.cs:21): applied by cuDNN between stacked
+                                   layers in training.  Not implemented: snhip_rnn_forward returns status 15 when it is
+                                   non-zero in training with num_layers > 1 (it has no effect otherwise, as in cuDNN). */
 } snhip_rnn_desc;
 int snhip_sizeof_rnn_desc(void);
 /* Bytes of the weight space.  Layout: all matrices (pseudo-layer by pseudo-layer = layer * dirs + direction: the
@@ -409,7 +412,9 @@ int snhip_set_splitk_mode(void* handle, int mode);
 int snhip_config_count(void);
 /* desc[0..5] = BM, BN, BK, threads, dynamic LDS bytes, kind (0 fp32 tiled kernel, 1 bf16-input kernel, 2 fp32 kernel
  * with 32 x 32 tiles and K split over the wavefronts of a workgroup: chosen by itself for products with few output
- * tiles, never part of a split-K launch, used only when the operands can be read in 16-byte pieces) */
+ * tiles, never part of a split-K launch, used only when the operands can be read in 16-byte pieces; 3 fp32 kernel
+ * with persistent workgroups and 32-wide k panels: chosen by itself for strided batches of small matrices with a
+ * short K, never part of a split-K launch) */
 int snhip_config_desc(int config, int desc[6]);
 
 #ifdef __cplusplus

@@ -460,6 +460,29 @@ def mkl_dot(a2, transposeA, b2, transposeB, out, alpha=1.0, beta=0.0):
     return "torch.mm (MKL build)"
 
 
+def mkl_bmm_serial(a3, transposeA, b3, transposeB, out3, alpha=1.0, beta=0.0):
+    """CpuTensor.BatchMatrixMultiplication as the reference runs it (CpuTensor.cs:3018-3024): a serial loop over the
+    matrices of the batch, one cblas_sgemm (BlasServices.cs:20) each.  a3, b3, out3: C-contiguous float32 3-D arrays."""
+    n = a3.shape[0]
+    assert b3.shape[0] == n and out3.shape[0] == n
+    lib = _find_mkl()
+    if lib is None:
+        for i in range(n):
+            mkl_dot(a3[i], transposeA, b3[i], transposeB, out3[i], alpha, beta)
+        return "torch.mm (MKL build), serial loop"
+    aH, aW = a3.shape[1:]
+    bH, bW = b3.shape[1:]
+    M, N, K, lda, ldb, ldc = dot_shapes(aH, aW, transposeA, bH, bW, transposeB)
+    ta, tb = (112 if transposeA else 111), (112 if transposeB else 111)
+    pa, pb, pc = a3.ctypes.data, b3.ctypes.data, out3.ctypes.data
+    sa, sb, sc = a3.strides[0], b3.strides[0], out3.strides[0]
+    fn, cast, al, be = lib.cblas_sgemm, ctypes.cast, float(alpha), float(beta)
+    for i in range(n):
+        fn(101, ta, tb, M, N, K, al, cast(pa + i * sa, _f32p), lda, cast(pb + i * sb, _f32p), ldb, be,
+           cast(pc + i * sc, _f32p), ldc)
+    return "libmkl_rt cblas_sgemm, serial loop"
+
+
 def mkl_threads():
     lib = _find_mkl()
     if lib is not None:

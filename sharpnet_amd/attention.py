@@ -172,6 +172,11 @@ def MultiheadAttentionForwardPropagation(Q, K, V, y, w_Q, w_K, w_V, out_proj_wei
         raise ValueError("V.Shape and y.Shape must be equal, but are %s and %s" % (V.Shape, y.Shape))
     if Q.Shape[2] != V.Shape[2]:
         raise ValueError("queries.Shape[2] and values.Shape[2] must be equal (same embedding dim)")
+    if Q.Shape[1] != V.Shape[1]:
+        # y has V's shape (checked above) but receives one row per query: with more queries than keys the products
+        # would write past y and the attention buffers (the reference fails its BatchMatrixMultiplication shape
+        # assertion at this point instead)
+        raise ValueError("queries.Shape[1] and values.Shape[1] must be equal, but are %d and %d" % (Q.Shape[1], V.Shape[1]))
     w = Q.Wrapper
     batch_size, tq, tkv = K.Shape[0], Q.Shape[1], V.Shape[1]
     H, dk, dv = num_heads, key_dim, value_dim

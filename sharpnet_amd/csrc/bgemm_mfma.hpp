@@ -184,11 +184,15 @@ __global__ void __launch_bounds__(CFG::NT) bgemm_mfma_kernel(const GemmParams p)
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, lhi = lane >> 5;
 
-    int tile_m, tile_n;
-    tile_coords(blockIdx.x, p.tiles_m * p.tiles_n, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
+    const WorkCoords wc = work_coords(blockIdx.x, p.tiles_m, p.tiles_n, p.nz, p.group_m);
+    const int tile_m = wc.tile_m, tile_n = wc.tile_n;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int zb = blockIdx.y;
-    const int batch = zb / p.splitk, split = zb - batch * p.splitk;
+    const int zb = wc.zb;
+    int batch = zb, split = 0;
+    if (p.splitk > 1) {
+        batch = zb / p.splitk;
+        split = zb - batch * p.splitk;
+    }
 
     const int kbeg = split * p.kchunk;
     const int kend = (kbeg + p.kchunk < p.K) ? (kbeg + p.kchunk) : p.K;
@@ -348,7 +352,8 @@ __global__ void __launch_bounds__(CFG::NT) bgemm_mfma_kernel(const GemmParams p)
         k_tile(P1{}, std::false_type{});
     }
 
-    store_accumulators_plain<TM, TN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch);
+    store_accumulators_plain<TM, TN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch,
+                                     tile_m * p.tiles_n + tile_n);
 }
 
 }  // namespace snhip

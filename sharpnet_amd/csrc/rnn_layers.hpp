@@ -44,7 +44,14 @@ int rnn_check_desc(const snhip_rnn_desc* d) {
     if (d->bias_mode < SNHIP_RNN_NO_BIAS || d->bias_mode > SNHIP_RNN_SINGLE_REC_BIAS) return SNHIP_STATUS_INVALID_VALUE;
     if (d->bidirectional != 0 && d->bidirectional != 1) return SNHIP_STATUS_INVALID_VALUE;
     if (d->num_layers < 1 || d->input_size < 1 || d->hidden_size < 1) return SNHIP_STATUS_INVALID_VALUE;
+    if (!(d->dropout >= 0.0f && d->dropout < 1.0f)) return SNHIP_STATUS_INVALID_VALUE;  // also refuses NaN
     return SNHIP_STATUS_SUCCESS;
+}
+
+// cuDNN drops units of the outputs that feed the next stacked layer, in training only; that is not implemented, so
+// the one combination in which the rate would change results is refused rather than computed without dropout.
+bool rnn_dropout_would_apply(const snhip_rnn_desc* d, int training) {
+    return training != 0 && d->dropout > 0.0f && d->num_layers > 1;
 }
 
 RnnDims rnn_dims(const snhip_rnn_desc* d, int batch, int steps) {
@@ -212,7 +219,10 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
                       float* y, const float* hx, float* hy, const float* cx, float* cy, const float* weights,
                       void* workspace, size_t workspace_bytes, void* reserve, size_t reserve_bytes) {
     Handle* h = static_cast<Handle*>(handle);
-    int st = rnn_common_checks(h, desc, batch, steps);
+    int st = rnn_check_desc(desc);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    if (rnn_dropout_would_apply(desc, training)) return SNHIP_STATUS_NOT_SUPPORTED;
+    st = rnn_common_checks(h, desc, batch, steps);
     if (st != SNHIP_STATUS_SUCCESS) return st;
     if (batch == 0 || steps == 0) return SNHIP_STATUS_SUCCESS;
     if (x == nullptr || y == nullptr || weights == nullptr) return SNHIP_STATUS_INVALID_VALUE;

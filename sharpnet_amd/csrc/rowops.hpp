@@ -183,14 +183,15 @@ __global__ void __launch_bounds__(256) transpose_2nd_3rd_kernel(const float* __r
 // Column-major C (m x n, ldc) = alpha * op(A) + beta * op(B): cublasSgeam, which the reference uses with
 // transa = T, beta = 0 as its matrix transpose (Prod/GPU/GpuTensor.cs:1256-1291).  A workgroup of 32 x 8 threads owns
 // a 32 x 32 tile of C; a transposed operand goes through a padded LDS tile so that both its reads and the writes
-// of C are contiguous.  B is not touched when beta == 0.
+// of C are contiguous.  An operand whose scalar is zero is never read (BLAS rule: 0 * NaN must not reach C).
 __global__ void __launch_bounds__(256) geam_kernel(int ta, int tb, int m, int n, float alpha, const float* __restrict__ A,
                                                    long long lda, float beta, const float* __restrict__ B, long long ldb,
                                                    float* C, long long ldc) {
     __shared__ float tA[32][33], tB[32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int i0 = blockIdx.x * 32, j0 = blockIdx.y * 32;
-    const bool use_b = (beta != 0.0f);
+    const bool use_a = (alpha != 0.0f), use_b = (beta != 0.0f);
+    ta = ta && use_a;
     if (ta || (tb && use_b)) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -207,7 +208,8 @@ __global__ void __launch_bounds__(256) geam_kernel(int ta, int tb, int m, int n,
         const int c = ty + 8 * k;  // index along j inside the tile; tx runs along i: contiguous in C
         const int i = i0 + tx, j = j0 + c;
         if (i < m && j < n) {
-            float v = alpha * (ta ? tA[tx][c] : A[(long long)j * lda + i]);
+            float v = 0.0f;
+            if (use_a) v = alpha * (ta ? tA[tx][c] : A[(long long)j * lda + i]);
             if (use_b) v += beta * (tb ? tB[tx][c] : B[(long long)j * ldb + i]);
             C[(long long)j * ldc + i] = v;
         }

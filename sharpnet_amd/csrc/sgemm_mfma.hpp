@@ -126,13 +126,18 @@ struct GemmParams {
     float alpha, beta;
     int flags;
     int group_m;  // tile rows per swizzle group
+    int nz;       // batch * splitk: the grid is one-dimensional, tiles_m * tiles_n * nz workgroups
 };
 
 // ---------------------------------------------------------------------------
 // Global -> register -> LDS staging of one operand tile of logical shape
 // [BK (k)] x [BMN (m or n)].  KCONTIG: global memory is contiguous along k.
 // ---------------------------------------------------------------------------
-template <int BMN, int BK, int NT, int PITCH, bool KCONTIG>
+// WAVE_SPLITS_K (k-contiguous operands with BK = 64 or 32): a wavefront covers 16 lines x 16 k (each lane one 16-byte
+// vector) instead of 4 lines x 64 k, and the wavefronts of the workgroup split k between them.  With BK = 64 the
+// plain assignment would put the four dword stores of a scattered vector on 16 banks (4-way conflicts; 2-way with
+// BK = 32); this one reaches 64 distinct banks again.
+template <int BMN, int BK, int NT, int PITCH, bool KCONTIG, bool WAVE_SPLITS_K = false>
 struct TileStage {
     static constexpr int NV = (BK * BMN) / (4 * NT);  // 16-byte vectors per thread
     static_assert((BK * BMN) % (4 * NT) == 0, "tile must split evenly over threads");
@@ -146,8 +151,15 @@ struct TileStage {
     long long ld;
 
     __device__ __forceinline__ void init(const float* base, long long ld_, int tile_mn, int kbeg, int tid) {
-        const int vec = tid % VEC_PER_LINE;
-        const int line = tid / VEC_PER_LINE;
+        int vec = tid % VEC_PER_LINE;
+        int line = tid / VEC_PER_LINE;
+        if constexpr (WAVE_SPLITS_K && KCONTIG) {
+            static_assert(!WAVE_SPLITS_K || ((BK == 64 || BK == 32) && NT == 256), "mapping written for 4 wavefronts");
+            constexpr int KW = BK / 16;  // wavefronts that split k between them; the others take further lines
+            const int wave = tid >> 6, lane = tid & 63;
+            vec = 4 * (wave % KW) + (lane >> 4);
+            line = (lane & 15) + 16 * (wave / KW);
+        }
         ld = ld_;
         if (KCONTIG) {
             k0 = vec * 4;
@@ -306,24 +318,39 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-// Workgroups are handed to the 8 XCDs round-robin by linear id.  Remap the id
-// so that each XCD (which has a private L2) works on a contiguous range of
-// tiles, then walk that range in groups of `group_m` tile rows so concurrently
-// resident tiles share A row panels and B column panels.
-__device__ __forceinline__ void tile_coords(int bid, int ntiles, int tiles_m, int tiles_n, int group_m, int& tm,
-                                            int& tn) {
-    constexpr int NXCD = 8;
-    const int q = ntiles / NXCD, r = ntiles % NXCD;
-    const int xcd = bid % NXCD, local = bid / NXCD;
+// Workgroups are handed to the 8 XCDs (each with a private L2) round-robin by linear workgroup id, so the grid is
+// one-dimensional and the id is remapped here: every XCD works on one contiguous range of the logical order
+// "matrix (batch entry x K split) by matrix, and inside a matrix tile after tile in groups of `group_m` tile
+// rows".  Tiles that are resident together then share A row panels and B column panels in their L2, and the tiles
+// of one matrix of a strided batch never spread over several XCDs unless a range boundary cuts through it.
+struct WorkCoords {
+    int zb;              // batch entry * splitk + split
+    int tile_m, tile_n;
+};
+__device__ __forceinline__ WorkCoords work_coords(unsigned lin, int tiles_m, int tiles_n, int nz, int group_m) {
+    constexpr unsigned NXCD = 8;
+    const unsigned ntiles = (unsigned)(tiles_m * tiles_n);
+    const unsigned total = ntiles * (unsigned)nz;  // the host keeps this below 2^31
+    const unsigned q = total / NXCD, r = total % NXCD;
+    const unsigned xcd = lin % NXCD, local = lin / NXCD;
+    const unsigned L = xcd * q + (xcd < r ? xcd : r) + local;
+    WorkCoords w;
+    unsigned t = L;
+    w.zb = 0;
+    if (nz > 1) {  // uniform; an unbatched product takes no division
+        w.zb = (int)(L / ntiles);
+        t = L - (unsigned)w.zb * ntiles;
+    }
     // reversed, so the ragged last tile row / column (slower, bounds-checked) is issued first
-    const int logical = ntiles - 1 - (xcd * q + (xcd < r ? xcd : r) + local);
+    const int logical = (int)(ntiles - 1 - t);
     const int per_group = group_m * tiles_n;
     const int g = logical / per_group;
     const int first_m = g * group_m;
     const int gsz = (tiles_m - first_m < group_m) ? (tiles_m - first_m) : group_m;
     const int in_g = logical - g * per_group;
-    tm = first_m + in_g % gsz;
-    tn = in_g / gsz;
+    w.tile_m = first_m + in_g % gsz;
+    w.tile_n = in_g / gsz;
+    return w;
 }
 
 // TN consecutive floats as one vector access (TN = 1, 2 or 4); the caller has checked alignment.
@@ -350,6 +377,66 @@ __device__ __forceinline__ void store_row_vec(float* p, const float (&v)[TN]) {
     }
 }
 
+// Write-out of a wavefront whose whole 32*TM x 32*TN patch lies inside the matrix and may be accessed in vectors
+// of TN floats:   C = act(alpha * acc + bias + beta * C + gamma * D).
+// There are no per-lane tests and no loads under conditions here, so the stores go out back to back.  (In the
+// general path every row is its own conditional block, and the compiler's wait-count bookkeeping, which merges the
+// paths through those blocks, makes each row wait until the previous row's store has been acknowledged.)
+// When old values are needed (beta != 0, or an addend D), rows go in chunks of four and the values of chunk k + 1
+// are requested before chunk k is stored, so a load never waits behind the stores issued just before it (the
+// compiler may not move loads across stores itself: for all it knows the rows alias).
+// c0 / d0 point at the lane's first row (row_base + 4 * TM * lhi) and first column; d0 == nullptr: no addend.
+template <int TM, int TN, bool EXT>
+__device__ __forceinline__ void store_patch_fast(const f32x16 (&acc)[TM][TN], float* c0, long long ldo, const float* d0,
+                                                 long long ldd, float alpha, float beta, float gamma,
+                                                 const float (&bv)[TN], int act, float act_param) {
+    auto row_off = [&](int k, int e) {  // chunk k = (tile row i, register group g), element e of the group
+        const int i = k / 4, r = 4 * (k % 4) + e;
+        return (long long)(TM * (8 * (r / 4) + (r % 4)) + i);
+    };
+    constexpr int CHUNKS = 4 * TM;
+    const bool use_c = (beta != 0.0f), use_d = EXT && (d0 != nullptr);
+    auto finish = [&](int k, int e, const float (&cv)[TN], const float (&dv)[TN]) {
+        const int i = k / 4, r = 4 * (k % 4) + e;
+        float v[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            v[j] = alpha * acc[i][j][r] + bv[j];
+            if (use_c) v[j] += beta * cv[j];
+            if constexpr (EXT) {
+                if (use_d) v[j] += gamma * dv[j];
+                if (act != ACT_NONE) v[j] = leaky_relu(v[j], act_param);
+            }
+        }
+        store_row_vec<TN>(c0 + row_off(k, e) * ldo, v);
+    };
+    if (!use_c && !use_d) {
+        const float zero[TN] = {};
+#pragma unroll
+        for (int k = 0; k < CHUNKS; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) finish(k, e, zero, zero);
+        return;
+    }
+    float cbuf[2][4][TN] = {}, dbuf[2][4][TN] = {};
+    auto request = [&](int k) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (use_c) load_row_vec<TN>(c0 + row_off(k, e) * ldo, cbuf[k & 1][e]);
+            if constexpr (EXT) {
+                if (use_d) load_row_vec<TN>(d0 + row_off(k, e) * ldd, dbuf[k & 1][e]);
+            }
+        }
+    };
+    request(0);
+#pragma unroll
+    for (int k = 0; k < CHUNKS; ++k) {
+        if (k + 1 < CHUNKS) request(k + 1);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) finish(k, e, cbuf[k & 1][e], dbuf[k & 1][e]);
+    }
+}
+
 // Epilogue shared by the fp32 and bf16-input kernels.  acc[i][j][r] holds
 // C[row][col] with  row = row_base + TM*(8*(r/4) + 4*lhi + r%4) + i  and
 // col = col0 + j  (row_base = first row of the wavefront, col0 = first of the
@@ -369,7 +456,7 @@ __device__ __forceinline__ void store_row_vec(float* p, const float (&v)[TN]) {
 // ---------------------------------------------------------------------------
 template <int TM, int TN>
 __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM][TN], const GemmParams& p, int row_base,
-                                                   int col0, int lhi, int zb, int batch) {
+                                                   int col0, int lhi, int zb, int batch, int tile_index) {
     const bool to_ws = (p.splitk > 1);
     float* out;
     long long ldo;
@@ -392,35 +479,52 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
         vec_ok = (p.flags & GEMM_FLAG_C_VEC) && (col0 + TN <= p.N);
     }
 
-    float bv[TN];
+    // a wavefront whose patch lies inside the matrix takes the branch-free write-out
+    const int row_w = __builtin_amdgcn_readfirstlane(row_base);
+    const int col_w = __builtin_amdgcn_readfirstlane(col0);  // lane 0 owns the wavefront's first column
+    const bool ws_or_c_vec = to_ws ? ((p.flags & GEMM_FLAG_WS_VEC) != 0) : ((p.flags & GEMM_FLAG_C_VEC) != 0);
+    if (ws_or_c_vec && row_w + 32 * TM <= p.M && col_w + 32 * TN <= p.N) {
+        float bv[TN];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) bv[j] = (bias != nullptr && col0 + j < p.N) ? bias[col0 + j] : 0.0f;
+        for (int j = 0; j < TN; ++j) bv[j] = 0.0f;
+        if (bias != nullptr) load_row_vec<TN>(bias + col0, bv);
+        store_patch_fast<TM, TN, false>(acc, out + (long long)(row_base + TM * 4 * lhi) * ldo + col0, ldo, nullptr, 0, alpha,
+                                        beta, 0.0f, bv, ACT_NONE, 0.0f);
+    } else {
+        float bv[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bv[j] = (bias != nullptr && col0 + j < p.N) ? bias[col0 + j] : 0.0f;
+        // the bias values are needed (and waited for) here, on every path: otherwise each row's block below
+        // would wait for "a load that may still be pending" and with it for the previous row's store
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bv[j]));
 
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
-            if (row >= p.M) continue;
-            float* crow = out + (long long)row * ldo + col0;
-            float v[TN];
+            for (int r = 0; r < 16; ++r) {
+                const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
+                if (row >= p.M) continue;
+                float* crow = out + (long long)row * ldo + col0;
+                float v[TN];
 #pragma unroll
-            for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r] + bv[j];
-            if (vec_ok) {
-                if (beta != 0.0f) {
-                    float c[TN];
-                    load_row_vec<TN>(crow, c);
+                for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r] + bv[j];
+                if (vec_ok) {
+                    if (beta != 0.0f) {
+                        float c[TN];
+                        load_row_vec<TN>(crow, c);
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) v[j] += beta * c[j];
-                }
-                store_row_vec<TN>(crow, v);
-            } else {
+                        for (int j = 0; j < TN; ++j) v[j] += beta * c[j];
+                    }
+                    store_row_vec<TN>(crow, v);
+                } else {
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    if (col0 + j < p.N) {
-                        float o = v[j];
-                        if (beta != 0.0f) o += beta * crow[j];
-                        crow[j] = o;
+                    for (int j = 0; j < TN; ++j) {
+                        if (col0 + j < p.N) {
+                            float o = v[j];
+                            if (beta != 0.0f) o += beta * crow[j];
+                            crow[j] = o;
+                        }
                     }
                 }
             }
@@ -434,7 +538,7 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
     __threadfence();  // release: this thread's partial sums are visible device-wide
     __syncthreads();
     if (threadIdx.x == 0) {
-        int* cnt = p.counters + (long long)batch * gridDim.x + blockIdx.x;
+        int* cnt = p.counters + (long long)batch * (p.tiles_m * p.tiles_n) + tile_index;
         const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         const int last = (old == p.splitk - 1);
         if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
@@ -547,7 +651,8 @@ __device__ __forceinline__ void finish_row(float (&v)[TN], float* crow, const fl
 
 template <int TM, int TN>
 __device__ __forceinline__ void store_accumulators_ext(const f32x16 (&acc)[TM][TN], const GemmParams& p, int row_base,
-                                                       int col0, int lhi, int zb, int batch, BatchIndex bi) {
+                                                       int col0, int lhi, int zb, int batch, BatchIndex bi,
+                                                       int tile_index) {
     const bool to_ws = (p.splitk > 1);
     float* const Cb = p.C + batch_offset(bi, p.strideC, p.strideC2);
     const float* const Db =
@@ -583,20 +688,33 @@ __device__ __forceinline__ void store_accumulators_ext(const f32x16 (&acc)[TM][T
 #pragma unroll
         for (int j = 0; j < TN; ++j) bv[j] = (p.ep.bias != nullptr && col0 + j < p.N) ? p.ep.bias[col0 + j] : 0.0f;
     }
+    // the bias values are needed (and waited for) here, on every path (see store_accumulators_plain)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bv[j]));
     const bool has_d = (dsrc != nullptr);
+    const int row_w = __builtin_amdgcn_readfirstlane(row_base);
+    const int col_w = __builtin_amdgcn_readfirstlane(col0);  // lane 0 owns the wavefront's first column
+    const bool ws_or_c_vec = to_ws ? ((p.flags & GEMM_FLAG_WS_VEC) != 0) : ((p.flags & GEMM_FLAG_C_VEC) != 0);
+    if (ws_or_c_vec && row_w + 32 * TM <= p.M && col_w + 32 * TN <= p.N) {
+        // the wavefront's patch lies inside the matrix: branch-free write-out
+        const long long first = (long long)(row_base + TM * 4 * lhi);
+        store_patch_fast<TM, TN, true>(acc, out + first * ldo + col0, ldo, has_d ? dsrc + first * ldd + col0 : nullptr, ldd,
+                                       alpha, beta, gamma, bv, act, p.ep.act_param);
+    } else {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
-            if (row >= p.M) continue;
-            float v[TN];
+            for (int r = 0; r < 16; ++r) {
+                const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
+                if (row >= p.M) continue;
+                float v[TN];
 #pragma unroll
-            for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r];
-            const float* drow = nullptr;
-            if (has_d) drow = dsrc + (long long)row * ldd + col0;
-            finish_row<TN>(v, out + (long long)row * ldo + col0, drow, has_d, bv, beta, gamma, act, p.ep.act_param,
-                           vec_ok, p.N - col0);
+                for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r];
+                const float* drow = nullptr;
+                if (has_d) drow = dsrc + (long long)row * ldd + col0;
+                finish_row<TN>(v, out + (long long)row * ldo + col0, drow, has_d, bv, beta, gamma, act, p.ep.act_param,
+                               vec_ok, p.N - col0);
+            }
         }
     }
 
@@ -608,7 +726,7 @@ __device__ __forceinline__ void store_accumulators_ext(const f32x16 (&acc)[TM][T
     __threadfence();  // release: this thread's partial sums are visible device-wide
     __syncthreads();
     if (threadIdx.x == 0) {
-        int* cnt = p.counters + (long long)batch * gridDim.x + blockIdx.x;
+        int* cnt = p.counters + (long long)batch * (p.tiles_m * p.tiles_n) + tile_index;
         const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         const int last = (old == p.splitk - 1);
         if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
@@ -657,11 +775,11 @@ __device__ __forceinline__ void store_accumulators_ext(const f32x16 (&acc)[TM][T
 
 template <int TM, int TN, bool EXT>
 __device__ __forceinline__ void store_accumulators(const f32x16 (&acc)[TM][TN], const GemmParams& p, int row_base,
-                                                   int col0, int lhi, int zb, int batch, BatchIndex bi) {
+                                                   int col0, int lhi, int zb, int batch, BatchIndex bi, int tile_index) {
     if constexpr (EXT)
-        store_accumulators_ext<TM, TN>(acc, p, row_base, col0, lhi, zb, batch, bi);
+        store_accumulators_ext<TM, TN>(acc, p, row_base, col0, lhi, zb, batch, bi, tile_index);
     else
-        store_accumulators_plain<TM, TN>(acc, p, row_base, col0, lhi, zb, batch);
+        store_accumulators_plain<TM, TN>(acc, p, row_base, col0, lhi, zb, batch, tile_index);
 }
 
 template <int TM_, int TN_, int WM_, int WN_, int BK_>
@@ -695,11 +813,15 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, lhi = lane >> 5;
 
-    int tile_m, tile_n;
-    tile_coords(blockIdx.x, p.tiles_m * p.tiles_n, p.tiles_m, p.tiles_n, p.group_m, tile_m, tile_n);
+    const WorkCoords wc = work_coords(blockIdx.x, p.tiles_m, p.tiles_n, p.nz, p.group_m);
+    const int tile_m = wc.tile_m, tile_n = wc.tile_n;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int zb = blockIdx.y;  // batch * splitk + split
-    const int batch = zb / p.splitk, split = zb - batch * p.splitk;
+    const int zb = wc.zb;  // batch * splitk + split
+    int batch = zb, split = 0;
+    if (p.splitk > 1) {
+        batch = zb / p.splitk;
+        split = zb - batch * p.splitk;
+    }
 
     const int kbeg = split * p.kchunk;
     const int kend = (kbeg + p.kchunk < p.K) ? (kbeg + p.kchunk) : p.K;
@@ -929,7 +1051,8 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         }
     }
 
-    store_accumulators<TM, TN, EXT>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch, bi);
+    store_accumulators<TM, TN, EXT>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch, bi,
+                                    tile_m * p.tiles_n + tile_n);
 }
 
 }  // namespace snhip

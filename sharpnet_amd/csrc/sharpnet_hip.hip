@@ -15,6 +15,7 @@
 #include "kernel_list.hpp"
 #include "rowops.hpp"
 #include "sgemm_ksplit.hpp"
+#include "sgemm_stream.hpp"
 
 // The GEMM kernels are compiled in gemm_kernels.hip; here they are only declared.
 SNHIP_ALL_KERNEL_GROUPS(SNHIP_DECLARE_KERNELS)
@@ -160,9 +161,24 @@ const ConfigEntry kConfigs[] = {
                 {{sgemm_ksplit_kernel<false, false, 2>, sgemm_ksplit_kernel<false, true, 2>},
                  {sgemm_ksplit_kernel<true, false, 2>, sgemm_ksplit_kernel<true, true, 2>}},
                 6, 0.5, 0.5, 1.0},  // 15: 32 x 64 (two column tiles), two K slices
+    // persistent streaming kernels for batches of small matrices with a short K (sgemm_stream.hpp): not part of
+    // the cost model's search either, see prefer_stream().  Panels of 32 k measured faster than panels of 64 on
+    // every attention-shaped product (49.0 against 52.6 us for 512 x (256 x 256 x 64)): a third (fourth) workgroup
+    // fits on a compute unit and the first MFMA starts after half the bytes.
+    ConfigEntry{128, 128, 32, 256, StreamCfg<4, 32>::LDS_BYTES, 4, 3,
+                {{sgemm_stream_kernel<4, false, false, 32>, sgemm_stream_kernel<4, false, true, 32>},
+                 {sgemm_stream_kernel<4, true, false, 32>, sgemm_stream_kernel<4, true, true, 32>}},
+                {{nullptr, nullptr}, {nullptr, nullptr}},
+                3, 0.8, 0.9, 1.1},  // 16: 128 x 128, k panels of 32, three workgroups per compute unit
+    ConfigEntry{128, 64, 32, 256, StreamCfg<2, 32>::LDS_BYTES, 2, 3,
+                {{sgemm_stream_kernel<2, false, false, 32>, sgemm_stream_kernel<2, false, true, 32>},
+                 {sgemm_stream_kernel<2, true, false, 32>, sgemm_stream_kernel<2, true, true, 32>}},
+                {{nullptr, nullptr}, {nullptr, nullptr}},
+                4, 0.7, 0.85, 1.1},  // 17: 128 x 64, k panels of 32, four workgroups per compute unit
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
-constexpr int kKsplitConfig = kNumConfigs - 2;   // and kKsplitConfig + 1
+constexpr int kKsplitConfig = 14;   // and kKsplitConfig + 1
+constexpr int kStreamConfig = 16;   // and kStreamConfig + 1
 
 // Fused attention forward kernels (attention_mfma.hpp)
 struct AttnEntry {
@@ -259,7 +275,7 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
 }
 
 Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
-    Choice best{kind == 0 ? 6 : kKsplitConfig - 1, 1};
+    Choice best{kind == 0 ? 6 : 13, 1};
     double best_cost = 1e300;
     const bool forced = h->force_cfg >= 0 && kConfigs[h->force_cfg].kind == kind;
     for (int c = 0; c < kNumConfigs; ++c) {
@@ -414,6 +430,24 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
     return -1;
 }
 
+// Whether the product goes to sgemm_stream_kernel (configuration 16 or 17) instead of what the cost model chose:
+// strided batches of small matrices whose K fits a few 64-wide panels, where the tiled kernels' pipeline never
+// fills and every workgroup is prologue and write-out.
+int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, bool wants_ext) {
+    if (math != SNHIP_MATH_FP32 || two_level || wants_ext) return -1;
+    const bool forced = h->force_cfg == kStreamConfig || h->force_cfg == kStreamConfig + 1;
+    if (h->force_cfg >= 0 && !forced) return -1;
+    if (h->force_splitk > 1) return -1;
+    if (forced) return h->force_cfg;
+    if (g.batch < 8 || g.K > 256 || g.M < 64) return -1;
+    const int cfg = g.N <= 64 ? kStreamConfig + 1 : kStreamConfig;
+    const long long tiles = (long long)ceil_div(g.M, 128) * ceil_div(g.N, kConfigs[cfg].BN) * g.batch;
+    if (tiles < 2LL * h->num_cu) return -1;
+    // mostly-empty tiles waste the streaming they are meant to save
+    if ((long long)ceil_div(g.M, 128) * 128 * ceil_div(g.N, kConfigs[cfg].BN) * kConfigs[cfg].BN > 2LL * g.M * g.N) return -1;
+    return cfg;
+}
+
 int gemm_core(Handle* h, const GemmArgs& g) {
     if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     const int math = (g.math < 0) ? h->math_mode : g.math;
@@ -508,6 +542,11 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     Choice ch = choose(h, M, N, K, batch, math);
     const int ks_cfg = prefer_ksplit(h, g, math, two_level);
     if (ks_cfg >= 0) ch = Choice{ks_cfg, 1};
+    {
+        const bool relu = (ep.act == ACT_RELU || ep.act == ACT_LEAKY_RELU);
+        const int st_cfg = prefer_stream(h, g, math, two_level, ep.addend != nullptr || relu || g.colsum != nullptr);
+        if (st_cfg >= 0 && ks_cfg < 0) ch = Choice{st_cfg, 1};
+    }
     const ConfigEntry& cfg = kConfigs[ch.cfg];
     if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
 
@@ -572,7 +611,8 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     p.flags = 0;
     p.counters = nullptr;
     const long long ntiles = (long long)p.tiles_m * p.tiles_n;
-    if (ntiles > 0x7fffffffLL) return SNHIP_STATUS_NOT_SUPPORTED;
+    if (ntiles * batch * ch.splitk > 0x7fffffffLL) return SNHIP_STATUS_NOT_SUPPORTED;  // one-dimensional grid
+    p.nz = batch * ch.splitk;
     const bool c_vec = ((uintptr_t)g.C % 16 == 0) && (g.ldc % 4 == 0) && (!multi || g.sC % 4 == 0) &&
                        (!two_level || g.sC2 % 4 == 0) && (g.bias == nullptr || (uintptr_t)g.bias % 16 == 0) &&
                        (ep_kernel.addend == nullptr ||
@@ -609,8 +649,16 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     h->last_splitk = ch.splitk;
 
     const KernelFn fn = use_ext ? fn_ext : cfg.fn[g.tA ? 1 : 0][g.tB ? 1 : 0];
-    hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)(batch * ch.splitk)), dim3(cfg.NT), cfg.lds_bytes,
-                       h->stream, p);
+    if (cfg.kind == 2) {  // the K-split kernel reads tile and matrix from a two-dimensional grid
+        hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)batch), dim3(cfg.NT), cfg.lds_bytes, h->stream, p);
+    } else if (cfg.kind == 3) {
+        // persistent workgroups: as many as fit on the chip at once, the same number on every XCD
+        long long wgs = (long long)cfg.occ * h->num_cu;
+        if (wgs > ntiles * p.nz) wgs = ntiles * p.nz;
+        if (wgs >= 8) wgs -= wgs % 8;
+        hipLaunchKernelGGL(fn, dim3((unsigned)wgs), dim3(cfg.NT), cfg.lds_bytes, h->stream, p);
+    } else
+        hipLaunchKernelGGL(fn, dim3((unsigned)(ntiles * p.nz)), dim3(cfg.NT), cfg.lds_bytes, h->stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return hip_to_status(e);
 
@@ -1123,14 +1171,11 @@ int snhip_sgeam(void* handle, int transa, int transb, int m, int n, const float*
     if (use_a && (A == nullptr || lda < (ta ? n : m))) return SNHIP_STATUS_INVALID_VALUE;
     if (use_b && (B == nullptr || ldb < (tb ? n : m))) return SNHIP_STATUS_INVALID_VALUE;
     if ((use_a && A == C && ta) || (use_b && B == C && tb)) return SNHIP_STATUS_NOT_SUPPORTED;  // in-place transpose
-    // alpha == 0 must not read A (it may be NULL): hand the kernel B's data under both names then
-    const float* a_eff = use_a ? A : (use_b ? B : C);
-    const int lda_eff = use_a ? lda : (use_b ? ldb : ldc);
-    const int ta_eff = use_a ? ta : (use_b ? tb : 0);
     if ((long long)ceil_div(n, 32) > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
+    // the kernel reads neither A when alpha == 0 nor B when beta == 0 (either may be NULL then)
     hipLaunchKernelGGL(geam_kernel, dim3((unsigned)ceil_div(m, 32), (unsigned)ceil_div(n, 32)), dim3(256), 0,
-                       static_cast<Handle*>(handle)->stream, (int)ta_eff, (int)tb, m, n, *alpha, a_eff, (long long)lda_eff,
-                       *beta, B, (long long)ldb, C, (long long)ldc);
+                       static_cast<Handle*>(handle)->stream, (int)ta, (int)tb, m, n, *alpha, A, (long long)lda, *beta, B,
+                       (long long)ldb, C, (long long)ldc);
     return hip_to_status(hipGetLastError());
 }
 

@@ -121,7 +121,7 @@ class AttentionBwdDesc(ctypes.Structure):
 class RnnDesc(ctypes.Structure):
     """snhip_rnn_desc of include/sharpnet_hip.h (field for field)."""
     _fields_ = [("struct_size", _i), ("cell_mode", _i), ("bias_mode", _i), ("bidirectional", _i), ("num_layers", _i),
-                ("input_size", _i), ("hidden_size", _i)]
+                ("input_size", _i), ("hidden_size", _i), ("dropout", _f)]
 
     def __init__(self, **kw):
         super().__init__()
@@ -130,7 +130,7 @@ class RnnDesc(ctypes.Structure):
         for k, v in kw.items():
             if k not in dict(self._fields_):
                 raise TypeError("snhip_rnn_desc has no field %r" % k)
-            setattr(self, k, int(v))
+            setattr(self, k, float(v) if k == "dropout" else int(v))
 
 
 # SNHIP_ACT_* and the reference's cudnnActivationMode_t names for them (Prod/GPU/CudnnWrapper.cs:267-281)

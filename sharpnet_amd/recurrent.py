@@ -21,14 +21,19 @@ _GATES = {CUDNN_RNN_RELU: 1, CUDNN_RNN_TANH: 1, CUDNN_LSTM: 4, CUDNN_GRU: 3}
 
 class RecurrentLayer:
     def __init__(self, gpu_wrapper, inputSize, hiddenSize, cellMode, biasMode, returnSequences, isBidirectional,
-                 numLayers=1, isEncoderThatWillBeFollowedByDecoder=False):
+                 numLayers=1, isEncoderThatWillBeFollowedByDecoder=False, dropoutRate=0.0):
         if isEncoderThatWillBeFollowedByDecoder and returnSequences:
             raise ValueError("an Encoder can not return a sequence")            # RecurrentLayer.cs:128-131
+        if isEncoderThatWillBeFollowedByDecoder and numLayers != 1:
+            # The context vector is two (batch, K*hidden) blocks, the library's states are (K*layers, batch, hidden):
+            # with more than one layer they do not have the same size and the state pointers would run past the buffer.
+            raise ValueError("an Encoder followed by a Decoder must have exactly one layer")
         self.IsEncoderThatWillBeFollowedByDecoder = isEncoderThatWillBeFollowedByDecoder
         self.Wrapper = gpu_wrapper
         self._lib = gpu_wrapper.lib
         self.desc = RnnDesc(cell_mode=cellMode, bias_mode=biasMode, bidirectional=bool(isBidirectional),
-                            num_layers=numLayers, input_size=inputSize, hidden_size=hiddenSize)
+                            num_layers=numLayers, input_size=inputSize, hidden_size=hiddenSize,
+                            dropout=dropoutRate)                                 # RecurrentLayer.cs:69,123
         self._returnSequences = returnSequences
         self.hidden_size, self.input_size, self.num_layers = hiddenSize, inputSize, numLayers
         self.K = 2 if isBidirectional else 1
@@ -81,6 +86,18 @@ class RecurrentLayer:
         shape[-1] //= 2
         return t.Slice(0, shape), t.Slice(t.Count // 2, shape)
 
+    def _CheckDecoderArguments(self, contextVector, batchSize):
+        """A context vector (an encoder's output or its gradient) holds K*batch*hidden floats per block, which is what
+        the library reads and writes as initial states only when this layer has one layer: refuse anything else
+        instead of letting the device run past the buffer."""
+        if contextVector is None:
+            return
+        if self.num_layers != 1:
+            raise ValueError("a Decoder that takes an encoder's output must have exactly one layer (has %d)" % self.num_layers)
+        if contextVector.Count != 2 * self.K * batchSize * self.hidden_size:
+            raise ValueError("encoder output has %d elements, expected 2 x %d x %d x %d"
+                             % (contextVector.Count, self.K, batchSize, self.hidden_size))
+
     def _buffers(self, isTraining, batchSize, timeSteps):
         ws, rs = ctypes.c_size_t(), ctypes.c_size_t()
         check_status(self._lib.snhip_rnn_temp_space_sizes(ctypes.byref(self.desc), int(isTraining), batchSize, timeSteps,
@@ -92,6 +109,7 @@ class RecurrentLayer:
         encoderOutput: the output of the encoder this layer decodes (RecurrentLayer.cs:305-408)."""
         batchSize, timeSteps = x.Shape[0], x.Shape[1]
         assert x.Shape[2] == self.input_size and yFull.Shape == self.OutputShape(batchSize, timeSteps)
+        self._CheckDecoderArguments(encoderOutput, batchSize)
         y, cy = self._ExtractEncoderContextVector(yFull) if self.IsEncoderThatWillBeFollowedByDecoder else (yFull, None)
         hx, cx = self._ExtractEncoderContextVector(encoderOutput) if encoderOutput is not None else (None, None)
         ws_bytes, rs_bytes = self._buffers(isTraining, batchSize, timeSteps)
@@ -137,6 +155,8 @@ class RecurrentLayer:
         assert self._reserveSpace is not None
         batchSize, timeSteps = x.Shape[0], x.Shape[1]
         H, K = self.hidden_size, self.K
+        self._CheckDecoderArguments(encoderOutput, batchSize)
+        self._CheckDecoderArguments(dEncoderOutput, batchSize)
         y, _ = self._ExtractEncoderContextVector(yFull) if self.IsEncoderThatWillBeFollowedByDecoder else (yFull, None)
         dy, dcy = self._ExtractEncoderContextVector(dyFull) if self.IsEncoderThatWillBeFollowedByDecoder else (dyFull, None)
         hx, cx = self._ExtractEncoderContextVector(encoderOutput) if encoderOutput is not None else (None, None)

@@ -99,6 +99,56 @@ def test_gemm_descriptor_layout_matches_the_library():
         hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
 
 
+def test_rnn_dropout_is_refused_not_ignored():
+    """RNNDescriptor.dropoutRate (Prod/Layers/RNNDescriptor.cs:21) travels in snhip_rnn_desc; the one combination in
+    which cuDNN would apply it (training, more than one layer) is refused, everything else is unaffected by it."""
+    import ctypes
+    from sharpnet_amd import hiplib
+    lib = hiplib.load_library()
+    S = hiplib.CublasStatus
+
+    def fwd(desc, training):
+        return lib.snhip_rnn_forward(None, ctypes.byref(desc), training, 1, 1, None, None, None, None, None, None, None,
+                                     None, 0, None, 0)
+    d = hiplib.RnnDesc(cell_mode=2, bias_mode=2, num_layers=2, input_size=3, hidden_size=5, dropout=0.25)
+    assert fwd(d, 1) == S.CUBLAS_STATUS_NOT_SUPPORTED
+    assert fwd(d, 0) == S.CUBLAS_STATUS_NOT_INITIALIZED          # inference: no dropout, goes on to the handle check
+    d1 = hiplib.RnnDesc(cell_mode=2, bias_mode=2, num_layers=1, input_size=3, hidden_size=5, dropout=0.25)
+    assert fwd(d1, 1) == S.CUBLAS_STATUS_NOT_INITIALIZED         # one layer: nothing to drop between layers
+    for bad in (-0.1, 1.0, float("nan")):
+        db = hiplib.RnnDesc(cell_mode=2, bias_mode=2, num_layers=2, input_size=3, hidden_size=5, dropout=bad)
+        assert fwd(db, 0) == S.CUBLAS_STATUS_INVALID_VALUE
+
+
+def test_host_mirrors_refuse_shapes_that_would_overrun_device_buffers():
+    """RecurrentLayer: an encoder / decoder pair exchanges (batch, K*hidden) blocks, which only match the library's
+    (K*layers, batch, hidden) states for one layer.  MultiheadAttention: y has the values' shape but one row per query."""
+    from sharpnet_amd import recurrent, attention
+
+    with pytest.raises(ValueError):
+        recurrent.RecurrentLayer(None, 4, 3, recurrent.CUDNN_LSTM, recurrent.CUDNN_RNN_DOUBLE_BIAS, False, False,
+                                 numLayers=2, isEncoderThatWillBeFollowedByDecoder=True)
+
+    class Stub:
+        def __init__(self, shape):
+            self.Shape = list(shape)
+            self.Count = 1
+            for s in shape:
+                self.Count *= s
+    layer = object.__new__(recurrent.RecurrentLayer)
+    layer.num_layers, layer.K, layer.hidden_size = 2, 1, 3
+    with pytest.raises(ValueError):
+        layer._CheckDecoderArguments(Stub((5, 6)), 5)
+    layer.num_layers = 1
+    layer._CheckDecoderArguments(Stub((5, 6)), 5)                  # 2 blocks of 5 x 3: accepted
+    layer._CheckDecoderArguments(None, 5)
+    with pytest.raises(ValueError):
+        layer._CheckDecoderArguments(Stub((5, 12)), 5)
+    q, kv = Stub((2, 9, 8)), Stub((2, 7, 8))
+    with pytest.raises(ValueError, match="queries.Shape\\[1\\]"):
+        attention.MultiheadAttentionForwardPropagation(q, kv, kv, kv, None, None, None, None, 2, 4, 4)
+
+
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     from sharpnet_amd import hiplib
     with pytest.raises(FileNotFoundError):

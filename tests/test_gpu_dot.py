@@ -458,6 +458,28 @@ def test_sgeam_transpose_and_sdgmm(oracle, gpu_wrapper):
     want = oracle.sgeam_colmajor(True, True, m, n, 0.5, A, n + 2, -2.0, B, n + 5, C0, m + 4)
     assert np.max(np.abs(gC.ToNumpy() - want)) <= 1e-6
     assert np.array_equal(gC.ToNumpy().reshape(n, m + 4)[:, m:], C0.reshape(n, m + 4)[:, m:])
+    # a zero scalar means "operand not referenced" (cuBLAS): NaN / Inf in that operand, or in the old C, never reach C
+    ld = max(m, n) + 1                     # fits either orientation of either operand
+    size = ld * max(m, n)
+    A2, B2 = random_tensor(rng, (size,), -1, 1), random_tensor(rng, (size,), -1, 1)
+    nanA, infB = np.full(size, np.nan, np.float32), np.full(size, np.inf, np.float32)
+    gA2, gB2, gNaN, gInf = (GPUTensor([size], x, w) for x in (A2, B2, nanA, infB))
+    for (alpha, beta, ta, tb, srcA, srcB, hostA, hostB) in (
+            (0.0, 0.0, 1, 0, gNaN, gInf, nanA, infB),          # C = 0 whatever A, B and the old C hold
+            (0.0, 1.5, 1, 1, gNaN, gB2, nanA, B2),             # C = 1.5 * B^T, A not read
+            (0.0, 1.5, 0, 0, None, gB2, nanA, B2),             # ... A may be NULL
+            (-0.75, 0.0, 1, 0, gA2, gInf, A2, infB),           # C = -0.75 * A^T, B not read
+            (-0.75, 0.0, 1, 0, gA2, None, A2, infB)):          # ... B may be NULL (the reference's Transpose call)
+        gC.SetValue(float("nan"))
+        al, be = ctypes.c_float(alpha), ctypes.c_float(beta)
+        st = w.lib.snhip_sgeam(w.handle, ta, tb, m, n, ctypes.byref(al), srcA.Pointer if srcA is not None else None, ld,
+                               ctypes.byref(be), srcB.Pointer if srcB is not None else None, ld, gC.Pointer, m + 4)
+        assert st == 0
+        want = oracle.sgeam_colmajor(bool(ta), bool(tb), m, n, alpha, hostA, ld, beta, hostB, ld,
+                                     np.full(C0.size, np.nan, np.float32), m + 4)
+        got = gC.ToNumpy().reshape(n, m + 4)[:, :m]
+        assert np.array_equal(got, want.reshape(n, m + 4)[:, :m]), (alpha, beta, ta, tb)
+        assert np.isfinite(got).all()
     # argument errors follow cuBLAS: bad op, short leading dimension, in-place transpose
     assert w.lib.snhip_sgeam(w.handle, 7, 0, m, n, ctypes.byref(al), gA.Pointer, n + 2, ctypes.byref(be), gB.Pointer, n + 5,
                              gC.Pointer, m + 4) == 7
@@ -531,6 +553,55 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
         assert np.all(gy.ToNumpy() == 0.0)
     finally:
         gpu_wrapper.set_tuning(-1, 0)
+
+
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_streaming_kernel_strided_batches(oracle, gpu_wrapper, tA, tB):
+    """The persistent kernel for batches of small matrices with a short K (k panels of 32, one LDS stage): more
+    tiles than workgroups so that every workgroup walks through several, ragged M / N, K below, at and above one
+    panel with tails, alpha / beta, a single matrix; forced through the tuning hook, and picked automatically for the
+    attention-shaped products."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    st_all = [c["id"] for c in w.configs() if c["kind"] == "fp32-stream"]
+    assert len(st_all) == 2
+    rng = np.random.default_rng(500 + 2 * tA + tB)
+    try:
+        for (batch, M, N, K) in [(700, 128, 128, 64), (40, 256, 256, 64), (40, 256, 64, 256), (9, 200, 100, 70),
+                                 (5, 130, 257, 130), (3, 64, 40, 7), (1, 300, 200, 129), (1100, 100, 60, 36)]:
+            a = random_tensor(rng, (batch, K, M) if tA else (batch, M, K), -1, 1)
+            b = random_tensor(rng, (batch, N, K) if tB else (batch, K, N), -1, 1)
+            c = random_tensor(rng, (batch, M, N), -1, 1)
+            ga, gb = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w)
+            for cfg in st_all:
+                w.set_tuning(cfg, 1)
+                for alpha, beta in [(0.125, 0.0), (-0.5, 1.0)]:
+                    gc = GPUTensor(c.shape, c, w)
+                    if beta == 0.0:
+                        gc.SetValue(float("nan"))
+                    gc.BatchMatrixMultiplication(ga, tA, gb, tB, alpha, beta)
+                    assert w.last_tuning() == (cfg, 1), (batch, M, N, K)
+                    got = gc.ToNumpy()
+                    gc.Dispose()
+                    ref = oracle.bmm(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
+                    assert np.all(np.isfinite(got)), (batch, M, N, K, cfg, alpha, beta)
+                    assert np.max(np.abs(got - ref)) <= tol(K, a, b, alpha, beta, c), (batch, M, N, K, cfg, alpha, beta)
+            ga.Dispose()
+            gb.Dispose()
+        w.set_tuning(-1, 0)
+        # automatic choice: the two attention products of benchmark configuration 5 (fewer matrices, same shape)
+        for (batch, M, N, K, want) in [(256, 256, 256, 64, st_all[0]), (256, 256, 64, 256, st_all[1])]:
+            a = random_tensor(rng, (batch, K, M) if tA else (batch, M, K), -1, 1)
+            b = random_tensor(rng, (batch, N, K) if tB else (batch, K, N), -1, 1)
+            ga, gb, gc = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w), GPUTensor([batch, M, N], None, w)
+            gc.SetValue(float("nan"))
+            gc.BatchMatrixMultiplication(ga, tA, gb, tB, 1.0, 0.0)
+            assert w.last_tuning() == (want, 1)
+            assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, tA, b, tB, 1.0))) <= tol(K, a, b)
+            for t in (ga, gb, gc):
+                t.Dispose()
+    finally:
+        w.set_tuning(-1, 0)
 
 
 def test_k_split_kernel_padded_pitches_fuzz(oracle, gpu_wrapper):

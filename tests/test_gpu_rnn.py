@@ -95,8 +95,6 @@ def compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, tol):
 @pytest.mark.parametrize("bidirectional,layers", [(False, 1), (True, 1), (False, 2), (True, 2)])
 @pytest.mark.parametrize("bias_mode", [ro.DOUBLE_BIAS, ro.SINGLE_INP_BIAS, ro.SINGLE_REC_BIAS, ro.NO_BIAS])
 def test_cells_small(gpu_wrapper, cell, bidirectional, layers, bias_mode):
-    if bias_mode != ro.DOUBLE_BIAS and (layers, bidirectional) != (2, True):
-        pytest.skip("bias modes are checked on the largest arrangement only")
     rng = np.random.default_rng(1000 + cell * 100 + layers * 10 + int(bidirectional) + bias_mode)
     desc = ro.RnnDesc(cell, input_size=5, hidden_size=3, num_layers=layers, bidirectional=bidirectional, bias_mode=bias_mode)
     B, Tn = 4, 6

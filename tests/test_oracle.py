@@ -260,6 +260,20 @@ def test_mkl_route_matches_closed_form(oracle):
         assert np.max(np.abs(out - ref)) <= oracle.tolerance(K, a, b)
 
 
+def test_mkl_serial_batch_loop_matches_the_batched_oracle(oracle):
+    """The batched baseline (one cblas_sgemm per matrix, in order: CpuTensor.cs:3018-3024) agrees with the oracle's bmm."""
+    rng = np.random.default_rng(23)
+    for tA, tB in itertools.product([False, True], repeat=2):
+        n, M, N, K = 5, 33, 18, 40
+        a = random_tensor(rng, (n, K, M) if tA else (n, M, K), -1, 1)
+        b = random_tensor(rng, (n, N, K) if tB else (n, K, N), -1, 1)
+        c = random_tensor(rng, (n, M, N), -1, 1)
+        out = c.copy()
+        oracle.mkl_bmm_serial(a, tA, b, tB, out, alpha=0.125, beta=1.0)
+        ref = oracle.bmm(a, tA, b, tB, 0.125, 1.0, c)
+        assert np.max(np.abs(out - ref)) <= oracle.tolerance(K, a, b)
+
+
 def test_round_to_bf16(oracle):
     """Ties go to the even 8-bit significand; agrees with torch's CPU bfloat16 cast on random data."""
     f = np.float32

@@ -76,8 +76,6 @@ def test_weight_space_is_a_partition():
 @pytest.mark.parametrize("bidirectional,layers", [(False, 1), (True, 1), (False, 2), (True, 2)])
 @pytest.mark.parametrize("bias_mode", [ro.DOUBLE_BIAS, ro.SINGLE_INP_BIAS, ro.SINGLE_REC_BIAS, ro.NO_BIAS])
 def test_against_torch_modules(cell, bidirectional, layers, bias_mode):
-    if bias_mode != ro.DOUBLE_BIAS and (layers, bidirectional) != (2, True):
-        pytest.skip("bias modes are checked on the largest arrangement only")
     rng = np.random.default_rng(cell * 100 + layers * 10 + int(bidirectional) + bias_mode)
     desc = ro.RnnDesc(cell, input_size=4, hidden_size=3, num_layers=layers, bidirectional=bidirectional, bias_mode=bias_mode)
     m = torch_module(desc)
