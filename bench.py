@@ -417,6 +417,57 @@ def main():
             extra["config2_8192_bf16_input_TN"] = hb
         finally:
             w.set_math_mode(w.MATH_FP32)
+
+        # The same arithmetic on operands STORED as bf16 (2 bytes per element in HBM; algorithmic bytes use s_in = 2).
+        # Operands are converted once by the library's own pass (timed separately: it is not part of the product).
+        def run_stored(gm, seed, steps, warmup):
+            from sharpnet_amd.hiplib import check_status
+            aa, bb, _ = wl.uniform_operands(gm, seed)
+            ga, gb = upload(aa), upload(bb)
+            gcs = GPUTensor(gm.c_shape, None, w)
+            pa, pb = w.allocate(2 * ga.Count), w.allocate(2 * gb.Count)
+
+            def convert():
+                check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, ga.Pointer, pa, ga.Count))
+                check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, gb.Pointer, pb, gb.Count))
+            aH, aW = aa.shape[-2:]
+            bH, bW = bb.shape[-2:]
+
+            def launch():
+                check_status(w.lib.snhip_bmm_bf16_stored(w.handle, pa, aH, aW, int(gm.tA), aH * aW, pb, bH, bW, int(gm.tB),
+                                                         bH * bW, gcs.Pointer, gm.M * gm.N, gm.batch, gm.alpha, gm.beta,
+                                                         None))
+
+            def timed(fn, n, nw):
+                for _ in range(nw):
+                    fn()
+                e0, e1 = w.new_event(), w.new_event()
+                w.synchronize()
+                w.record(e0)
+                for _ in range(n):
+                    fn()
+                w.record(e1)
+                ms = w.elapsed_ms(e0, e1) / n
+                w.destroy_event(e0)
+                w.destroy_event(e1)
+                return ms
+            conv_ms = timed(convert, 5, 2)
+            ms = timed(launch, steps, warmup)
+            by = gm.batch * (2.0 * (gm.M * gm.K + gm.K * gm.N) + 4.0 * gm.M * gm.N)
+            roof_s = max(gm.flops / (wl.BF16_MFMA_PEAK_TFLOPS * 1e12), by / (wl.HBM_PEAK_GBS * 1e9))
+            r = {"gemm": gm.label() + " (bf16 storage)", "ms": round(ms, 4), "tflops": round(gm.flops / (ms * 1e-3) / 1e12, 2),
+                 "frac_of_roofline": round(roof_s * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
+                 "splitk": w.last_tuning()[1], "algorithmic_bytes": by, "convert_both_operands_ms": round(conv_ms, 4)}
+            w.release(pa, 2 * ga.Count)
+            w.release(pb, 2 * gb.Count)
+            for t in (ga, gb, gcs):
+                t.Dispose()
+            return r
+        extra["config2_8192_bf16_stored"] = [run_stored(wl.Gemm(8192, 8192, 8192, tA, tB, 1.0, 0.0), 2, 10, 5)
+                                            for (tA, tB) in ((False, True), (False, False), (True, False))]
+        extra["config5_attention_bf16_stored"] = {"gemms": [run_stored(gm, 5, 50, 10) for gm in att_g],
+                                                  "cpu_baseline": extra["config5_attention_fp32"]["cpu_baseline"],
+                                                  "note": "CPU figure: the fp32 route (the reference has no other)"}
         if cpu_on:
             extra["cpu_leg_seconds"] = round(cpu_spent[0], 1)
             log("[bench] CPU side of the other configurations took %.1f s" % cpu_spent[0])

@@ -324,6 +324,7 @@ int snhip_rnn_backward_weights(void* handle, const snhip_rnn_desc* desc, int bat
  * <= 1e-2 * max|C|.  The reference has only the fp32 SGEMM (GpuTensor.cs:1218). */
 #define SNHIP_MATH_FP32 0
 #define SNHIP_MATH_BF16_INPUT 1
+#define SNHIP_MATH_BF16_STORED 2 /* per call only (snhip_gemm_desc.math, snhip_*_bf16_stored): A and B point at bf16 data */
 /* Selects the arithmetic used by every GEMM entry point of this handle
  * (the role cublasSetMathMode plays for cuBLAS handles). Default SNHIP_MATH_FP32. */
 int snhip_set_math_mode(void* handle, int mode);
@@ -333,6 +334,27 @@ int snhip_dot_bf16(void* handle, const float* A, int aH, int aW, int transposeA,
 int snhip_bmm_bf16(void* handle, const float* A, int aH, int aW, int transposeA, long long strideA, const float* B,
                    int bH, int bW, int transposeB, long long strideB, float* C, long long strideC, int batch,
                    float alpha, float beta);
+
+/* The same arithmetic on operands that are ALREADY bf16 in device memory (2 bytes per element: half the operand
+ * bytes from HBM and, what matters more for large products, half the bytes from L2 into LDS).  A and B point at
+ * bf16 data, aW / bW and the strides count bf16 elements, C and bias are fp32.  Results are bit-identical to
+ * snhip_dot_bf16 / snhip_bmm_bf16 on the fp32 operands these were converted from (same rounding, same products, same
+ * order of summation for a given tile configuration).  A, B must be 4-byte aligned and rows / matrices must start on
+ * even element offsets (aW, bW, strides even), else status 15.  snhip_gemm_ex takes the same operands with
+ * math = SNHIP_MATH_BF16_STORED (no column sum in that mode). */
+int snhip_dot_bf16_stored(void* handle, const void* A, int aH, int aW, int transposeA, const void* B, int bH, int bW,
+                          int transposeB, float* C, float alpha, float beta, const float* bias);
+int snhip_bmm_bf16_stored(void* handle, const void* A, int aH, int aW, int transposeA, long long strideA, const void* B,
+                          int bH, int bW, int transposeB, long long strideB, float* C, long long strideC, int batch,
+                          float alpha, float beta, const float* bias);
+/* dst[i] = bf16(src[i]) for count elements, round to nearest even: the one pass that produces such operands. */
+int snhip_convert_f32_to_bf16(void* handle, const float* src, void* dst, long long count);
+/* The same for a rows x cols matrix with row pitches (elements), optionally transposed on the way:
+ * dst[r][c] = bf16(src[r][c]) or, with transpose != 0, dst[c][r] = bf16(src[r][c]).  The bf16-stored products run
+ * fastest when both operands are contiguous along k (A not transposed, B transposed): an operand that is used many
+ * times (weights) can be brought into that form once. */
+int snhip_convert_f32_to_bf16_2d(void* handle, const float* src, int rows, int cols, long long ld_src, int transpose,
+                                 void* dst, long long ld_dst);
 
 /* ---- row / column helpers next to the GEMMs in Linear and attention ------- */
 /* bias_gradient[c] = sum_r dy[r][c].  Replaces Tensor.Compute_BiasGradient_from_dy

@@ -23,6 +23,12 @@
 // loaded as 4x4 blocks (4 k rows x 4 consecutive m/n, four 16-byte loads), which
 // are transposed in registers for free: each of the 4 rows gets 4 consecutive k
 // as one ds_write_b64.
+//
+// Operands stored as bf16 (TIN = __bf16).  The same kernel reads operands that are already bf16 in memory: a
+// 16-byte vector then carries 8 elements, a k-contiguous vector goes to LDS unchanged (one ds_write_b128) and an
+// m/n-contiguous operand is handled in units of 4 k rows x 8 columns, transposed in registers into eight
+// ds_write_b64.  Half the bytes per element on the way from L2 into LDS is what this variant is for: with fp32
+// storage a 256 x 256 tile needs the L2's whole bandwidth to feed the MFMAs at full rate.
 #pragma once
 #include "sgemm_mfma.hpp"
 
@@ -47,45 +53,52 @@ __device__ __forceinline__ constexpr int logical_row(int phys) {
 // T: MFMA tiles per wavefront along this dimension (row interleave factor).
 // A "piece" is the unit the pipeline stores to LDS and refills from global
 // memory in one go: one vector (KCONTIG) or one 4x4 block (otherwise).
-template <int BMN, int BK, int NT, int PITCH, int T, bool KCONTIG>
+template <int BMN, int BK, int NT, int PITCH, int T, bool KCONTIG, typename TIN = float>
 struct BStage {
-    static constexpr int NV = (BK * BMN) / (4 * NT);  // 16-byte vectors per thread
-    static_assert((BK * BMN) % (4 * NT) == 0, "tile must split evenly over threads");
+    static constexpr int EPV = 16 / (int)sizeof(TIN);   // elements per 16-byte vector: 4 (fp32 storage) or 8 (bf16)
+    static constexpr int NV = (BK * BMN) / (EPV * NT);  // 16-byte vectors per thread
+    static_assert((BK * BMN) % (EPV * NT) == 0, "tile must split evenly over threads");
     // KCONTIG: VPL vectors cover one row; thread = (vec, line); vector v -> physical row line + v*LINE_STEP
-    static constexpr int VPL = BK / 4;
+    static constexpr int VPL = BK / EPV;
     static constexpr int LINE_STEP = NT / VPL;
-    // !KCONTIG: UPL units cover one block of 4 k rows; thread = (g, kb); unit u -> k block kb + u*KB_STEP
-    static constexpr int UPL = BMN / 4;
+    // !KCONTIG: UPL units (4 k rows x EPV columns) cover one block of 4 k rows; thread = (g, kb);
+    // unit u -> k block kb + u*KB_STEP
+    static constexpr int UPL = BMN / EPV;
     static constexpr int KB_STEP = (NT >= UPL) ? NT / UPL : 1;
     static constexpr int NU = NV / 4;
     static constexpr int NPIECES = KCONTIG ? NV : NU;
     static constexpr int VEC_PER_PIECE = KCONTIG ? 1 : 4;
-    static_assert(!KCONTIG || (NT % VPL == 0 && LINE_STEP <= 32 && 32 % LINE_STEP == 0), "unsupported k-contiguous split");
+    // the logical row of vector v must separate into a per-thread part and a per-vector constant (see thread_row)
+    static_assert(!KCONTIG || (NT % VPL == 0 && ((LINE_STEP <= 32 && 32 % LINE_STEP == 0) ||
+                                                 (LINE_STEP % 32 == 0 && T % (LINE_STEP / 32) == 0))),
+                  "unsupported k-contiguous split");
     static_assert(KCONTIG || (NV % 4 == 0 && NT % UPL == 0), "unsupported m/n-contiguous split");
 
     int line, k0;       // KCONTIG: physical row of vector 0, k offset of this thread's vectors
-    int g, kb;          // !KCONTIG: group of 4 logical rows, k block of unit 0
-    const float* gptr;  // address of vector 0 for the current k tile
+    int g, kb;          // !KCONTIG: group of EPV logical rows, k block of unit 0
+    const TIN* gptr;    // address of vector 0 for the current k tile
     long long ld;
 
-    __device__ __forceinline__ void init(const float* base, long long ld_, int tile_mn, int kbeg, int tid) {
+    __device__ __forceinline__ void init(const TIN* base, long long ld_, int tile_mn, int kbeg, int tid) {
         ld = ld_;
         if (KCONTIG) {
-            k0 = (tid % VPL) * 4;
+            k0 = (tid % VPL) * EPV;
             line = tid / VPL;
-            gptr = base + (long long)(tile_mn + T * line) * ld + (kbeg + k0);
+            gptr = base + (long long)(tile_mn + thread_row()) * ld + (kbeg + k0);
         } else {
             g = tid % UPL;
             kb = tid / UPL;
-            gptr = base + (long long)(kbeg + 4 * kb) * ld + (tile_mn + 4 * g);
+            gptr = base + (long long)(kbeg + 4 * kb) * ld + (tile_mn + EPV * g);
         }
     }
     __device__ __forceinline__ void advance() { gptr += KCONTIG ? (long long)BK : (long long)BK * ld; }
 
-    // logical row of vector v is  row_const(v) + T*line  (line < LINE_STEP <= 32 never carries)
+    // logical row of vector v (physical row line + v * LINE_STEP) is  row_const(v) + thread_row(): with
+    // line = l + 32 * q the thread's part is T * l + q, and q + (tile index of v * LINE_STEP) never carries past T
     __device__ __forceinline__ static constexpr int row_const(int v) { return logical_row<T>(v * LINE_STEP); }
+    __device__ __forceinline__ int thread_row() const { return T * (line % 32) + line / 32; }
 
-    __device__ __forceinline__ const float* vec_ptr(int v) const {
+    __device__ __forceinline__ const TIN* vec_ptr(int v) const {
         if (KCONTIG) return gptr + (long long)row_const(v) * ld;
         return gptr + (long long)(4 * (v / 4) * KB_STEP + (v % 4)) * ld;
     }
@@ -94,25 +107,36 @@ struct BStage {
 
     // elements with m/n >= mn_rem or k >= k_rem (counted from the tile origin) read as zero, untouched in memory
     __device__ __forceinline__ void load_safe_vec(f32x4& r, int v, int mn_rem, int k_rem) const {
-        const float* p = vec_ptr(v);
+        const TIN* p = vec_ptr(v);
         int nval;
         if (KCONTIG) {
             // rows past the edge re-read the last valid row (their products are never stored)
-            const int mn = row_const(v) + T * line;
-            if (mn >= mn_rem) p = gptr + (long long)(mn_rem - 1 - T * line) * ld;
+            const int mn = row_const(v) + thread_row();
+            if (mn >= mn_rem) p = gptr + (long long)(mn_rem - 1 - thread_row()) * ld;
             nval = k_rem - k0;
         } else {
             const int k = 4 * (kb + (v / 4) * KB_STEP) + (v % 4);
-            nval = (k < k_rem) ? (mn_rem - 4 * g) : 0;
+            nval = (k < k_rem) ? (mn_rem - EPV * g) : 0;
         }
         f32x4 x;
-        if (nval >= 4) {
+        if (nval >= EPV) {
             __builtin_memcpy(&x, p, 16);
-        } else {
+        } else if constexpr (EPV == 4) {
             x.x = (nval > 0) ? p[0] : 0.0f;
             x.y = (nval > 1) ? p[1] : 0.0f;
             x.z = (nval > 2) ? p[2] : 0.0f;
             x.w = 0.0f;
+        } else {
+            // bf16 storage: the valid elements one by one as 16-bit words, the rest zero bits (= +0.0)
+            const unsigned short* ps = reinterpret_cast<const unsigned short*>(p);
+            unsigned int w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const unsigned int lo = (nval > 2 * e) ? ps[2 * e] : 0u;
+                const unsigned int hi = (nval > 2 * e + 1) ? ps[2 * e + 1] : 0u;
+                w[e] = lo | (hi << 16);
+            }
+            __builtin_memcpy(&x, w, 16);
         }
         r = x;
     }
@@ -129,7 +153,22 @@ struct BStage {
 
     // round to bf16 and write piece q to the LDS tile s[row][k]
     __device__ __forceinline__ void store_piece(__bf16* s, const f32x4 (&r)[NV], int q) const {
-        if (KCONTIG) {
+        if constexpr (EPV == 8) {
+            if (KCONTIG) {
+                *reinterpret_cast<f32x4*>(s + (line + q * LINE_STEP) * PITCH + k0) = r[q];  // 8 k, already bf16
+            } else {
+                // 4 k rows x 8 columns -> 8 rows of 4 k
+                const int kk = 4 * (kb + q * KB_STEP);
+                bf16x8 in[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) __builtin_memcpy(&in[i], &r[4 * q + i], 16);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const bf16x4 h = {in[0][e], in[1][e], in[2][e], in[3][e]};
+                    *reinterpret_cast<bf16x4*>(s + phys_row<T>(8 * g + e) * PITCH + kk) = h;
+                }
+            }
+        } else if (KCONTIG) {
             const bf16x4 h = __builtin_convertvector(r[q], bf16x4);
             *reinterpret_cast<bf16x4*>(s + (line + q * LINE_STEP) * PITCH + k0) = h;
         } else {
@@ -167,12 +206,14 @@ struct BTileCfg {
     static_assert(BK % 32 == 0, "BK must give an even number of 16-wide k steps");
 };
 
-template <class CFG, bool TA, bool TB>
+// TIN: how A and B are stored in memory (float, rounded to bf16 on the way into LDS, or __bf16); with __bf16 the
+// operand pointers of GemmParams point at bf16 data and leading dimensions / strides count bf16 elements.
+template <class CFG, bool TA, bool TB, typename TIN = float>
 __global__ void __launch_bounds__(CFG::NT) bgemm_mfma_kernel(const GemmParams p) {
     constexpr int TM = CFG::TM, TN = CFG::TN, WN = CFG::WN, BK = CFG::BK;
     constexpr int BM = CFG::BM, BN = CFG::BN, NT = CFG::NT, PITCH = CFG::PITCH;
-    using StageA = BStage<BM, BK, NT, PITCH, TM, !TA>;
-    using StageB = BStage<BN, BK, NT, PITCH, TN, TB>;
+    using StageA = BStage<BM, BK, NT, PITCH, TM, !TA, TIN>;
+    using StageB = BStage<BN, BK, NT, PITCH, TN, TB, TIN>;
 
     extern __shared__ __attribute__((aligned(16))) float smem_f[];
     __bf16* const smem = reinterpret_cast<__bf16*>(smem_f);
@@ -200,8 +241,8 @@ __global__ void __launch_bounds__(CFG::NT) bgemm_mfma_kernel(const GemmParams p)
     const int nk = (klen + BK - 1) / BK;
     const int nk_full = klen / BK;
 
-    const float* Ab = p.A + (long long)batch * p.strideA;
-    const float* Bb = p.B + (long long)batch * p.strideB;
+    const TIN* Ab = reinterpret_cast<const TIN*>(p.A) + (long long)batch * p.strideA;
+    const TIN* Bb = reinterpret_cast<const TIN*>(p.B) + (long long)batch * p.strideB;
     const int m_rem = p.M - m0, n_rem = p.N - n0;
     const bool full_mn = (m_rem >= BM) && (n_rem >= BN);
 

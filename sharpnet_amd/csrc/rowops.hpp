@@ -305,4 +305,55 @@ __global__ void __launch_bounds__(256) copy_f32_kernel(const float* __restrict__
     }
 }
 
+// dst[i] = bf16(src[i]), round to nearest even (the rounding the bf16-input GEMM applies on its way into LDS):
+// the one pass that turns an fp32 operand into the bf16 storage of the bf16-stored GEMM entry points.
+// Eight elements per thread and step (two 16-byte loads, one 16-byte store) when the pointers allow it.
+__global__ void __launch_bounds__(256) convert_f32_to_bf16_kernel(const float* __restrict__ src, __bf16* __restrict__ dst,
+                                                                  long long count, int vec) {
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    long long done = 0;
+    if (vec) {
+        const long long n8 = count / 8;
+        const f32x4* s4 = reinterpret_cast<const f32x4*>(src);
+        for (long long j = i; j < n8; j += stride) {
+            const f32x4 a = s4[2 * j], b = s4[2 * j + 1];
+            const bf16x4_t lo = __builtin_convertvector(a, bf16x4_t), hi = __builtin_convertvector(b, bf16x4_t);
+            bf16x4_t* d = reinterpret_cast<bf16x4_t*>(dst + 8 * j);
+            d[0] = lo;
+            d[1] = hi;
+        }
+        done = n8 * 8;
+    }
+    for (long long j = done + i; j < count; j += stride) dst[j] = (__bf16)src[j];
+}
+
+// dst (bf16) = src (fp32) or its transpose, both row-major with their own row pitch: brings an operand into bf16
+// storage with whichever dimension contiguous the caller wants (the bf16-stored GEMM is fastest when both operands
+// are contiguous along k).  32 x 32 tiles through LDS so that reads and writes are both along rows.
+__global__ void __launch_bounds__(256) convert_f32_to_bf16_2d_kernel(const float* __restrict__ src, long long ld_src,
+                                                                     int rows, int cols, int transpose,
+                                                                     __bf16* __restrict__ dst, long long ld_dst) {
+    __shared__ float t[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int r = r0 + ty + 8 * k, c = c0 + tx;
+        if (r < rows && c < cols) t[ty + 8 * k][tx] = src[(long long)r * ld_src + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        if (transpose) {
+            const int c = c0 + ty + 8 * k, r = r0 + tx;
+            if (r < rows && c < cols) dst[(long long)c * ld_dst + r] = (__bf16)t[tx][ty + 8 * k];
+        } else {
+            const int r = r0 + ty + 8 * k, c = c0 + tx;
+            if (r < rows && c < cols) dst[(long long)r * ld_dst + c] = (__bf16)t[ty + 8 * k][tx];
+        }
+    }
+}
+
 }  // namespace snhip

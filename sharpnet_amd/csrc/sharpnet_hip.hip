@@ -79,7 +79,8 @@ typedef void (*KernelFn)(const GemmParams);
 struct ConfigEntry {
     int BM, BN, BK, NT, lds_bytes;
     int mfma_per_k2;    // TM*TN: MFMA instructions one wavefront issues per MFMA k step
-    int kind;           // 0: fp32 kernel (k step 2, 64 cycles per MFMA), 1: bf16-input kernel (k step 16, 32 cycles)
+    int kind;           // 0: fp32 kernel (k step 2, 64 cycles per MFMA), 1: bf16-input kernel (k step 16, 32 cycles),
+                        // 2: K split inside the workgroup, 3: streaming kernel, 4: bf16-input kernel on bf16 storage
     KernelFn fn[2][2];  // [transposeA][transposeB]
     KernelFn fn_ext[2][2];  // the same with the extended write-out (addend, ReLU, two-level batch, column sum);
                             // nullptr if not built
@@ -120,6 +121,24 @@ constexpr ConfigEntry make_entry_bf16(int occ, double eff_alone, double eff_shar
                        1,
                        {{bgemm_mfma_kernel<CFG, false, false>, bgemm_mfma_kernel<CFG, false, true>},
                         {bgemm_mfma_kernel<CFG, true, false>, bgemm_mfma_kernel<CFG, true, true>}},
+                       {{nullptr, nullptr}, {nullptr, nullptr}},
+                       occ,
+                       eff_alone,
+                       eff_shared,
+                       edge_slow};
+}
+
+template <class CFG>
+constexpr ConfigEntry make_entry_bf16_stored(int occ, double eff_alone, double eff_shared, double edge_slow) {
+    return ConfigEntry{CFG::BM,
+                       CFG::BN,
+                       CFG::BK,
+                       CFG::NT,
+                       CFG::LDS_BYTES,
+                       CFG::TM * CFG::TN,
+                       4,
+                       {{bgemm_mfma_kernel<CFG, false, false, __bf16>, bgemm_mfma_kernel<CFG, false, true, __bf16>},
+                        {bgemm_mfma_kernel<CFG, true, false, __bf16>, bgemm_mfma_kernel<CFG, true, true, __bf16>}},
                        {{nullptr, nullptr}, {nullptr, nullptr}},
                        occ,
                        eff_alone,
@@ -175,6 +194,10 @@ const ConfigEntry kConfigs[] = {
                  {sgemm_stream_kernel<2, true, false, 32>, sgemm_stream_kernel<2, true, true, 32>}},
                 {{nullptr, nullptr}, {nullptr, nullptr}},
                 4, 0.7, 0.85, 1.1},  // 17: 128 x 64, k panels of 32, four workgroups per compute unit
+    // bf16-input kernels on operands stored as bf16 (SNHIP_MATH_BF16_STORED)
+    make_entry_bf16_stored<BTileCfg<4, 4, 2, 2, 64>>(1, 0.85, 0.85, 3.0),   // 18: 256 x 256, BK 64
+    make_entry_bf16_stored<BTileCfg<2, 2, 2, 2, 64>>(2, 0.65, 0.80, 1.3),   // 19: 128 x 128, BK 64
+    make_entry_bf16_stored<BTileCfg<1, 1, 2, 2, 128>>(2, 0.45, 0.60, 1.1),  // 20: 64 x 64, BK 128
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 constexpr int kKsplitConfig = 14;   // and kKsplitConfig + 1
@@ -248,6 +271,7 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
     const int kchunk = ceil_div(ceil_div(K, splitk), c.BK) * c.BK;
     const int nk = ((kchunk / c.BK + 1) / 2) * 2;  // the k loop runs pairs of tiles
     const double mfma_per_tile = c.kind == 0 ? (c.BK / 2) * 64.0 * c.mfma_per_k2 : (c.BK / 16) * 32.0 * c.mfma_per_k2;
+    const double elem = c.kind == 4 ? 2.0 : 4.0;  // bytes per operand element in memory
     const long long resident = per_cu < c.occ ? per_cu : c.occ;
     const double eff = resident >= 2 ? c.eff_shared : c.eff_alone;
     const bool has_edge = (M % c.BM != 0) || (N % c.BN != 0);
@@ -256,11 +280,11 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
     const double tile_alone = mfma_per_tile / c.eff_alone > kTileLatency ? mfma_per_tile / c.eff_alone : kTileLatency;
     const double t_lat = (double)((per_cu + c.occ - 1) / c.occ) *
                          (nk * tile_alone + kFixed + (double)c.BM * c.BN * 4.0 / kStoreBytesPerCycle);
-    const double bytes_hbm = (double)batch * (4.0 * ((double)M * K + (double)K * N) + 4.0 * M * N) +
+    const double bytes_hbm = (double)batch * (elem * ((double)M * K + (double)K * N) + 4.0 * M * N) +
                              (splitk > 1 ? (double)batch * M * N * 4.0 * splitk : 0.0);
     const double t_mem = bytes_hbm / kHbmBytesPerCycle;
-    const double t_l2 = (double)blocks * (c.BM + c.BN) * (double)kchunk * 4.0 / kL2BytesPerCycle;
-    const double t_cu = (double)per_cu * (c.BM + c.BN) * (double)kchunk * 4.0 / kCuBytesPerCycle + kFixed;
+    const double t_l2 = (double)blocks * (c.BM + c.BN) * (double)kchunk * elem / kL2BytesPerCycle;
+    const double t_cu = (double)per_cu * (c.BM + c.BN) * (double)kchunk * elem / kCuBytesPerCycle + kFixed;
     double t = t_mfma;
     if (t_cu > t) t = t_cu;
     if (t_lat > t) t = t_lat;
@@ -274,8 +298,11 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
     return t;
 }
 
+// kind of kernel that serves a math mode: 0 fp32, 1 bf16-input on fp32 storage, 4 bf16-input on bf16 storage
+inline int kind_of_math(int math) { return math == SNHIP_MATH_BF16_STORED ? 4 : math; }
+
 Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
-    Choice best{kind == 0 ? 6 : 13, 1};
+    Choice best{kind == 0 ? 6 : (kind == 1 ? 13 : 20), 1};
     double best_cost = 1e300;
     const bool forced = h->force_cfg >= 0 && kConfigs[h->force_cfg].kind == kind;
     for (int c = 0; c < kNumConfigs; ++c) {
@@ -460,9 +487,11 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     }
     const int M = g.M, N = g.N, K = g.K, batch = g.batch;
     if (M < 0 || N < 0 || K < 0 || batch < 0 || g.batch_inner < 0) return SNHIP_STATUS_INVALID_VALUE;
-    if (math != SNHIP_MATH_FP32 && math != SNHIP_MATH_BF16_INPUT) return SNHIP_STATUS_INVALID_VALUE;
+    if (math != SNHIP_MATH_FP32 && math != SNHIP_MATH_BF16_INPUT && math != SNHIP_MATH_BF16_STORED)
+        return SNHIP_STATUS_INVALID_VALUE;
     if (g.act < ACT_NONE || g.act > ACT_TANH) return SNHIP_STATUS_NOT_SUPPORTED;
     if (g.colsum != nullptr && !g.tA) return SNHIP_STATUS_NOT_SUPPORTED;  // only sums along the k of a transposed A
+    if (g.colsum != nullptr && math == SNHIP_MATH_BF16_STORED) return SNHIP_STATUS_NOT_SUPPORTED;  // sums read fp32
     if (M == 0 || N == 0 || batch == 0) return SNHIP_STATUS_SUCCESS;
     if (g.C == nullptr || g.ldc < N) return SNHIP_STATUS_INVALID_VALUE;
     if (g.D != nullptr && g.ldd < N) return SNHIP_STATUS_INVALID_VALUE;
@@ -539,7 +568,14 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     if (g.A == nullptr || g.B == nullptr) return SNHIP_STATUS_INVALID_VALUE;
     if (g.lda < (g.tA ? M : K) || g.ldb < (g.tB ? K : N)) return SNHIP_STATUS_INVALID_VALUE;
 
-    Choice ch = choose(h, M, N, K, batch, math);
+    if (math == SNHIP_MATH_BF16_STORED) {
+        // bf16 storage is read in 16-byte vectors of eight elements from 4-byte-aligned addresses: rows and
+        // matrices must start on even element offsets
+        if ((uintptr_t)g.A % 4 != 0 || (uintptr_t)g.B % 4 != 0 || g.lda % 2 != 0 || g.ldb % 2 != 0 ||
+            (multi && (g.sA % 2 != 0 || g.sB % 2 != 0)) || (two_level && (g.sA2 % 2 != 0 || g.sB2 % 2 != 0)))
+            return SNHIP_STATUS_NOT_SUPPORTED;
+    }
+    Choice ch = choose(h, M, N, K, batch, kind_of_math(math));
     const int ks_cfg = prefer_ksplit(h, g, math, two_level);
     if (ks_cfg >= 0) ch = Choice{ks_cfg, 1};
     {
@@ -1108,6 +1144,53 @@ int snhip_bmm_bf16(void* handle, const float* A, int aH, int aW, int transposeA,
                    bW, strideB, beta, C, N, strideC, batch, nullptr, SNHIP_MATH_BF16_INPUT);
 }
 
+int snhip_convert_f32_to_bf16(void* handle, const float* src, void* dst, long long count) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (count < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (count == 0) return SNHIP_STATUS_SUCCESS;
+    if (src == nullptr || dst == nullptr || (uintptr_t)dst % 2 != 0) return SNHIP_STATUS_INVALID_VALUE;
+    const int vec = ((uintptr_t)src % 16 == 0 && (uintptr_t)dst % 8 == 0) ? 1 : 0;
+    const long long work = vec ? (count + 7) / 8 : count;
+    const int blocks = (int)((work + 255) / 256 < 16384 ? (work + 255) / 256 : 16384);
+    hipLaunchKernelGGL(convert_f32_to_bf16_kernel, dim3(blocks), dim3(256), 0, static_cast<Handle*>(handle)->stream, src,
+                       static_cast<__bf16*>(dst), count, vec);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_convert_f32_to_bf16_2d(void* handle, const float* src, int rows, int cols, long long ld_src, int transpose,
+                                 void* dst, long long ld_dst) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (rows < 0 || cols < 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (rows == 0 || cols == 0) return SNHIP_STATUS_SUCCESS;
+    if (src == nullptr || dst == nullptr || (uintptr_t)dst % 2 != 0 || ld_src < cols || ld_dst < (transpose ? rows : cols))
+        return SNHIP_STATUS_INVALID_VALUE;
+    if (ceil_div(rows, 32) > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
+    hipLaunchKernelGGL(convert_f32_to_bf16_2d_kernel, dim3((unsigned)ceil_div(cols, 32), (unsigned)ceil_div(rows, 32)),
+                       dim3(256), 0, static_cast<Handle*>(handle)->stream, src, ld_src, rows, cols, transpose != 0,
+                       static_cast<__bf16*>(dst), ld_dst);
+    return hip_to_status(hipGetLastError());
+}
+
+int snhip_bmm_bf16_stored(void* handle, const void* A, int aH, int aW, int transposeA, long long strideA, const void* B,
+                          int bH, int bW, int transposeB, long long strideB, float* C, long long strideC, int batch,
+                          float alpha, float beta, const float* bias) {
+    if (aH < 0 || aW < 0 || bH < 0 || bW < 0) return SNHIP_STATUS_INVALID_VALUE;
+    const int M = transposeA ? aW : aH;
+    const int N = transposeB ? bH : bW;
+    const int K = transposeA ? aH : aW;
+    const int Kb = transposeB ? bW : bH;
+    if (K != Kb) return SNHIP_STATUS_INVALID_VALUE;
+    // the operand pointers travel as float* through the shared argument block; the bf16-stored kernels read them as bf16
+    return gemm_rm(static_cast<Handle*>(handle), transposeA != 0, transposeB != 0, M, N, K, alpha,
+                   static_cast<const float*>(A), aW, strideA, static_cast<const float*>(B), bW, strideB, beta, C, N,
+                   strideC, batch, bias, SNHIP_MATH_BF16_STORED);
+}
+
+int snhip_dot_bf16_stored(void* handle, const void* A, int aH, int aW, int transposeA, const void* B, int bH, int bW,
+                          int transposeB, float* C, float alpha, float beta, const float* bias) {
+    return snhip_bmm_bf16_stored(handle, A, aH, aW, transposeA, 0, B, bH, bW, transposeB, 0, C, 0, 1, alpha, beta, bias);
+}
+
 /* ---- row / column helpers of the Linear and attention layers ---- */
 
 static inline int grid_for(long long total) {
@@ -1384,10 +1467,11 @@ int snhip_set_tuning(void* handle, int config, int splitk) {
 
 int snhip_query_tuning(void* handle, int m, int n, int k, int batch, int math_mode, int* config, int* splitk) {
     if (m <= 0 || n <= 0 || k <= 0 || batch <= 0) return SNHIP_STATUS_INVALID_VALUE;
-    if (math_mode != SNHIP_MATH_FP32 && math_mode != SNHIP_MATH_BF16_INPUT) return SNHIP_STATUS_INVALID_VALUE;
+    if (math_mode != SNHIP_MATH_FP32 && math_mode != SNHIP_MATH_BF16_INPUT && math_mode != SNHIP_MATH_BF16_STORED)
+        return SNHIP_STATUS_INVALID_VALUE;
     Handle model;  // without a handle: an MI355X with 256 CUs, no overrides
     const Handle* h = handle != nullptr ? static_cast<const Handle*>(handle) : &model;
-    Choice ch = choose(h, m, n, k, batch, math_mode);
+    Choice ch = choose(h, m, n, k, batch, kind_of_math(math_mode));
     if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
     if (config != nullptr) *config = ch.cfg;
     if (splitk != nullptr) *splitk = ch.splitk;

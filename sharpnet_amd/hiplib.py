@@ -170,6 +170,10 @@ SIGNATURES = {
     "snhip_set_math_mode": [_vp, _i],
     "snhip_dot_bf16": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f, _vp],
     "snhip_bmm_bf16": [_vp, _vp, _i, _i, _i, _ll, _vp, _i, _i, _i, _ll, _vp, _ll, _i, _f, _f],
+    "snhip_dot_bf16_stored": [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _f, _f, _vp],
+    "snhip_bmm_bf16_stored": [_vp, _vp, _i, _i, _i, _ll, _vp, _i, _i, _i, _ll, _vp, _ll, _i, _f, _f, _vp],
+    "snhip_convert_f32_to_bf16": [_vp, _vp, _vp, _ll],
+    "snhip_convert_f32_to_bf16_2d": [_vp, _vp, _i, _i, _ll, _i, _vp, _ll],
     "snhip_gemm_ex": [_vp, ctypes.POINTER(GemmDesc)],
     "snhip_sizeof_gemm_desc": [],
     "snhip_attention_forward": [_vp, ctypes.POINTER(AttentionDesc)],

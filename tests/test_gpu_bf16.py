@@ -116,3 +116,157 @@ def test_bf16_bias_and_batched(oracle, gpu_wrapper):
                                     1.0, 0.0))
     ref = oracle.bmm(oracle.round_to_bf16(p_), False, oracle.round_to_bf16(v), False)
     assert np.max(np.abs(go.ToNumpy() - ref)) <= 1e-4 * np.sqrt(T) * np.max(np.abs(p_)) * np.max(np.abs(v))
+
+
+# ---------------------------------------------------------------------------
+# operands stored as bf16 in device memory
+# ---------------------------------------------------------------------------
+def to_bf16_on_device(w, t):
+    """Device buffer holding GPUTensor t converted to bf16 by the library's own pass; returns the raw pointer."""
+    from sharpnet_amd.hiplib import check_status
+    p = w.allocate(max(2 * t.Count, 8))
+    check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, t.Pointer, p, t.Count), "snhip_convert_f32_to_bf16")
+    return p
+
+
+def test_convert_f32_to_bf16_is_round_to_nearest_even(oracle, gpu_wrapper):
+    """Bit-exact against the oracle's rounding (itself pinned by hand-computed ties and torch's CPU cast): random
+    data, ties, infinities, zeros of both signs, the smallest normals; 16-byte-aligned and odd-offset views."""
+    import ctypes
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    rng = np.random.default_rng(41)
+    x = np.concatenate([
+        rng.normal(0, 1, 4099).astype(np.float32),
+        np.array([1.0, 1 + 2.0 ** -8, 1 + 2.0 ** -8 + 2.0 ** -20, 1 + 3 * 2.0 ** -8, -(1 + 2.0 ** -8), 0.0, -0.0,
+                  np.inf, -np.inf, 2.0 ** -126, 3.0e38, -3.0e38, 65504.0, 1e-30], np.float32)])
+    gx = GPUTensor([x.size], x, w)
+    for off in (0, 1, 3):                                   # element offsets of the source view
+        n = x.size - off
+        dst = w.allocate(2 * n + 8)
+        check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, gx.Pointer + 4 * off, dst, n))
+        host = np.empty(n, np.uint16)
+        check_status(w.lib.snhip_memcpy_dtoh(w.handle, host.ctypes.data, dst, 2 * n))
+        want = (oracle.round_to_bf16(x[off:]).view(np.uint32) >> 16).astype(np.uint16)
+        assert np.array_equal(host, want), off
+        w.release(dst, 2 * n + 8)
+
+
+def test_convert_2d_with_pitches_and_transpose(oracle, gpu_wrapper):
+    """Matrix form of the conversion: padded row pitches on both sides, with and without transposition, ragged sizes."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    rng = np.random.default_rng(44)
+    for rows, cols, pad_s, pad_d in [(1, 1, 0, 0), (33, 65, 3, 2), (100, 31, 0, 5), (256, 128, 4, 0)]:
+        src = random_tensor(rng, (rows, cols + pad_s), -2, 2)
+        gs = GPUTensor(src.shape, src, w)
+        for transpose in (0, 1):
+            dr, dc = (cols, rows) if transpose else (rows, cols)
+            ldd = dc + pad_d
+            nbytes = 2 * dr * ldd
+            dst = w.allocate(nbytes + 8)
+            check_status(w.lib.snhip_memset32(w.handle, dst, 0x7fc07fc0, (nbytes + 3) // 4))      # bf16 NaNs
+            check_status(w.lib.snhip_convert_f32_to_bf16_2d(w.handle, gs.Pointer, rows, cols, cols + pad_s, transpose, dst,
+                                                            ldd))
+            host = np.empty(dr * ldd, np.uint16)
+            check_status(w.lib.snhip_memcpy_dtoh(w.handle, host.ctypes.data, dst, nbytes))
+            host = host.reshape(dr, ldd)
+            m = src[:, :cols].T if transpose else src[:, :cols]
+            want = (oracle.round_to_bf16(np.ascontiguousarray(m)).view(np.uint32) >> 16).astype(np.uint16)
+            assert np.array_equal(host[:, :dc], want), (rows, cols, transpose)
+            assert np.all(host[:, dc:] == 0x7fc0)                  # padding untouched
+            w.release(dst, nbytes + 8)
+
+
+EVEN_SHAPES = [(36, 22, 124), (130, 258, 64), (256, 256, 64), (300, 130, 200), (64, 64, 16), (2, 2, 2), (258, 100, 34),
+               (6, 300, 1000), (512, 384, 512), (200, 520, 136)]
+
+
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_bf16_stored_all_configs_all_transposes(oracle, gpu_wrapper, tA, tB):
+    """bf16 storage: every tile configuration of that kind x transposes x split-K x alpha / beta on ragged shapes with
+    even row lengths, NaN-prefilled destinations, against the oracle on bf16-rounded inputs (tight fp32 bound) and the
+    fp32 oracle (1e-2); and bit-identical to the fp32-storage bf16-input kernel of the same tile shape is not asked
+    for (different k extent per stage), only the bound."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    lib, h = w.lib, w.handle
+    rng = np.random.default_rng(600 + 2 * tA + tB)
+    cfgs = [c["id"] for c in w.configs() if c["kind"] == "bf16-stored"]
+    assert len(cfgs) == 3
+    try:
+        for (M, N, K) in EVEN_SHAPES:
+            a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
+            b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
+            c = random_tensor(rng, (M, N), -1, 1)
+            ga, gb = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w)
+            pa, pb = to_bf16_on_device(w, ga), to_bf16_on_device(w, gb)
+            for cfg in cfgs:
+                for splitk in (1, 2):
+                    if splitk > 1 and K < 256:
+                        continue
+                    w.set_tuning(cfg, splitk)
+                    for alpha, beta in [(1.0, 0.0), (0.25, 0.0), (-1.0, 1.0)]:
+                        gc = GPUTensor([M, N], c if beta != 0 else None, w)
+                        if beta == 0:
+                            gc.SetValue(float("nan"))
+                        check_status(lib.snhip_dot_bf16_stored(h, pa, a.shape[0], a.shape[1], int(tA), pb, b.shape[0],
+                                                               b.shape[1], int(tB), gc.Pointer, alpha, beta, None))
+                        assert w.last_tuning() == (cfg, splitk), (M, N, K)
+                        check(oracle, gc.ToNumpy(), a, tA, b, tB, alpha, beta, c, K)
+                        gc.Dispose()
+            w.release(pa, max(2 * ga.Count, 8))
+            w.release(pb, max(2 * gb.Count, 8))
+            ga.Dispose()
+            gb.Dispose()
+    finally:
+        w.set_tuning(-1, 0)
+
+
+def test_bf16_stored_batched_bias_and_refusals(oracle, gpu_wrapper):
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status, CublasStatus
+    w = gpu_wrapper
+    lib, h = w.lib, w.handle
+    rng = np.random.default_rng(43)
+    # Linear forward with bias, automatic configuration
+    M, N, K = 128, 256, 784
+    x, wt, bias = rng.uniform(0, 1, (M, K)).astype(np.float32), random_tensor(rng, (N, K), -0.07, 0.07), \
+        random_tensor(rng, (N,), -1, 1)
+    gx, gw, gb, gy = (GPUTensor(t.shape, t, w) for t in (x, wt, bias, np.zeros((M, N), np.float32)))
+    px, pw = to_bf16_on_device(w, gx), to_bf16_on_device(w, gw)
+    check_status(lib.snhip_dot_bf16_stored(h, px, M, K, 0, pw, N, K, 1, gy.Pointer, 1.0, 0.0, gb.Pointer))
+    ref = oracle.dot(oracle.round_to_bf16(x), False, oracle.round_to_bf16(wt), True) + bias
+    assert np.max(np.abs(gy.ToNumpy() - ref)) <= 1e-4 * np.sqrt(K) * np.max(np.abs(x)) * np.max(np.abs(wt)) + 1e-6
+    # the same operands at fp32 storage through the bf16-input kernel: same rounding, so the two results agree to
+    # summation order
+    gy2 = GPUTensor([M, N], None, w)
+    check_status(lib.snhip_dot_bf16(h, gx.Pointer, M, K, 0, gw.Pointer, N, K, 1, gy2.Pointer, 1.0, 0.0, gb.Pointer))
+    assert np.max(np.abs(gy.ToNumpy() - gy2.ToNumpy())) <= 2e-4 * np.sqrt(K) * np.max(np.abs(x)) * np.max(np.abs(wt))
+    # strided batch: attention-shaped products, both orders
+    batch, T, d = 16, 256, 64
+    q, k = random_tensor(rng, (batch, T, d)), random_tensor(rng, (batch, T, d))
+    gq, gk, gs = GPUTensor(q.shape, q, w), GPUTensor(k.shape, k, w), GPUTensor([batch, T, T], None, w)
+    pq, pk = to_bf16_on_device(w, gq), to_bf16_on_device(w, gk)
+    gs.SetValue(float("nan"))
+    check_status(lib.snhip_bmm_bf16_stored(h, pq, T, d, 0, T * d, pk, T, d, 1, T * d, gs.Pointer, T * T, batch, 0.125, 0.0,
+                                           None))
+    ref = oracle.bmm(oracle.round_to_bf16(q), False, oracle.round_to_bf16(k), True, 0.125)
+    assert np.max(np.abs(gs.ToNumpy() - ref)) <= 1e-4 * np.sqrt(d) * np.max(np.abs(q)) * np.max(np.abs(k))
+    p_ = rng.uniform(0, 1, (batch, T, T)).astype(np.float32)
+    gp, go = GPUTensor(p_.shape, p_, w), GPUTensor([batch, T, d], None, w)
+    pp = to_bf16_on_device(w, gp)
+    check_status(lib.snhip_bmm_bf16_stored(h, pp, T, T, 0, T * T, pk, T, d, 0, T * d, go.Pointer, T * d, batch, 1.0, 0.0,
+                                           None))
+    ref = oracle.bmm(oracle.round_to_bf16(p_), False, oracle.round_to_bf16(k), False)
+    assert np.max(np.abs(go.ToNumpy() - ref)) <= 1e-4 * np.sqrt(T) * np.max(np.abs(p_)) * np.max(np.abs(k))
+    # rows that start on odd element offsets cannot be read in aligned pieces: refused, nothing written
+    go.SetValue(float("nan"))
+    assert lib.snhip_dot_bf16_stored(h, pp, 8, 7, 0, pk, 7, 8, 0, go.Pointer, 1.0, 0.0, None) == \
+        CublasStatus.CUBLAS_STATUS_NOT_SUPPORTED
+    assert lib.snhip_dot_bf16_stored(h, pp + 2, 8, 8, 0, pk, 8, 8, 0, go.Pointer, 1.0, 0.0, None) == \
+        CublasStatus.CUBLAS_STATUS_NOT_SUPPORTED
+    assert np.isnan(go.ToNumpy()).all()
