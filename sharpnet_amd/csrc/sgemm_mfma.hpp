@@ -223,43 +223,46 @@ struct TileStage {
 
     // Per-thread facts about a tile at the ragged edge of m/n, computed once per workgroup: they do not
     // change from k tile to k tile, so full-k tiles of an edge block can be loaded without re-deriving them.
+    //
+    // Nothing here zero-fills: a row (column) of op(A) (op(B)) past the edge only feeds rows (columns) of C that
+    // are never stored, so it may hold any value that can be read without leaving the matrix.  A k-contiguous
+    // operand re-reads its last valid row; an m/n-contiguous one reads its vector from a start clamped to
+    // `extent - 4` and rotates the elements that are inside the matrix back to their slots.  Both are plain
+    // 16-byte loads with no branch.  (Needs an extent of at least 4 along m/n; `usable` says so.)
     struct Edge {
-        long long off[KCONTIG ? NV : 1];  // KCONTIG: element offset of vector v from gptr, row clamped to the last valid one
-        int nv;                           // !KCONTIG: how many of this thread's 4 consecutive m/n are inside (<= 0: none)
+        long long off[KCONTIG ? NV : 1];  // KCONTIG: element offset of vector v from gptr (row clamped);
+                                          // otherwise off[0]: element offset of the clamped start from this thread's own
+        int shift;                        // !KCONTIG: how far the start was moved back (0..3 matter; more: nothing inside)
+        bool usable;
     };
-    __device__ __forceinline__ Edge edge_info(int mn_rem) const {
+    __device__ __forceinline__ Edge edge_info(int mn_rem, int tile_mn) const {
         Edge e;
+        e.shift = 0;
+        e.usable = true;
         if (KCONTIG) {
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
                 const int mn = mn0 + v * LINE_STEP;
                 e.off[v] = (long long)(((mn < mn_rem) ? mn : mn_rem - 1) - mn0) * ld;
             }
-            e.nv = 4;
         } else {
-            e.off[0] = 0;
-            e.nv = mn_rem - mn0;
+            // mn_rem counts from the tile origin; the matrix extent seen from this thread's vector is mn_rem - mn0
+            const int last_start = mn_rem - 4;  // latest start (relative to the tile origin) that stays inside
+            const int start = (mn0 <= last_start) ? mn0 : last_start;
+            e.shift = mn0 - start;
+            e.off[0] = (long long)(start - mn0);
+            e.usable = (mn_rem >= 4) || (tile_mn > 0);  // the clamped start may reach into the tile before this one
         }
         return e;
     }
-    // Load of a full-k tile of an edge block: plain vectors except for the (at most one per row) vector that
-    // straddles the edge of an m/n-contiguous operand; nothing past the matrix is touched.
+    // Load of a full-k tile of an edge block: a plain vector, nothing past the matrix is touched.  For an
+    // m/n-contiguous operand the elements arrive `shift` slots late; store_lds_vec_shifted puts them back (doing it
+    // here would make the load wait for its own data).
     __device__ __forceinline__ void load_edge_vec(f32x4& r, int v, const Edge& e) const {
-        if (KCONTIG) {
+        if (KCONTIG)
             __builtin_memcpy(&r, gptr + e.off[v], 16);
-        } else {
-            const float* p = gptr + (long long)(v * LINE_STEP) * ld;
-            if (e.nv >= 4) {
-                __builtin_memcpy(&r, p, 16);
-            } else {
-                f32x4 x;
-                x.x = (e.nv > 0) ? p[0] : 0.0f;
-                x.y = (e.nv > 1) ? p[1] : 0.0f;
-                x.z = (e.nv > 2) ? p[2] : 0.0f;
-                x.w = 0.0f;
-                r = x;
-            }
-        }
+        else
+            __builtin_memcpy(&r, gptr + (long long)(v * LINE_STEP) * ld + e.off[0], 16);
     }
 
     // vector v of this thread -> its place in the k-major LDS tile
@@ -274,6 +277,22 @@ struct TileStage {
             float* d = s + (k0 + v * LINE_STEP) * PITCH + mn0;
             *reinterpret_cast<f32x4*>(d) = r;
         }
+    }
+
+    // The same for a vector that was loaded from a start moved back by `sh` elements (load_edge_vec): element j of
+    // the wanted vector sits in slot j + sh; slots that would come from beyond slot 3 lie outside the matrix and
+    // may hold anything.  sh == 0: as loaded.
+    // `any_shift` is uniform over the workgroup (the extent along m/n is not a multiple of 4): without it the
+    // vector is stored as loaded and the selects cost nothing.  Returns what was stored.
+    __device__ __forceinline__ f32x4 store_lds_vec_shifted(float* s, const f32x4& r, int v, int sh, bool any_shift) const {
+        f32x4 y = r;
+        if (!KCONTIG && any_shift) {
+            y.x = sh == 0 ? r.x : (sh == 1 ? r.y : (sh == 2 ? r.z : r.w));
+            y.y = sh == 0 ? r.y : (sh == 1 ? r.z : r.w);
+            y.z = sh == 0 ? r.z : r.w;
+        }
+        store_lds_vec(s, y, v);
+        return y;
     }
 
     __device__ __forceinline__ void store_lds(float* s, const f32x4 (&r)[NV]) const {
@@ -883,15 +902,35 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     const float* const a_rd = As + lhi * PA + a_off;
     const float* const b_rd = Bs + lhi * PB + b_off;
 
+    // Edge blocks: per-thread facts for branch-free loads of full-k tiles (see TileStage::Edge).  rot_a / rot_b: how
+    // far this thread's vectors of an m/n-contiguous operand arrive shifted; zero when the extent is a multiple of 4
+    // (then a vector is either wholly inside or wholly outside, and what lies outside may hold anything).
+    // sh_a / sh_b [stage]: the shift of what the register stage currently holds (0: as loaded).
+    const typename StageA::Edge ea = sa.edge_info(m_rem, m0);
+    const typename StageB::Edge eb = sb.edge_info(n_rem, n0);
+    const bool edge_ok = ea.usable && eb.usable;  // uniform over the workgroup
+    const bool any_rot_a = (p.M % 4 != 0), any_rot_b = (p.N % 4 != 0);
+    const int rot_a = any_rot_a ? ea.shift : 0, rot_b = any_rot_b ? eb.shift : 0;
+    int sh_a[2] = {0, 0}, sh_b[2] = {0, 0};
+
     {
         // prologue: tile 0 -> LDS buffer 0, tile 1 -> stage 1, tile 2 -> stage 0
 #pragma unroll
         for (int t = 0; t < 3; ++t) {
             const int st = (t == 1) ? 1 : 0;
             const int k_rem = klen - fetch * BK;
+            sh_a[st] = 0;
+            sh_b[st] = 0;
             if (full_mn && fetch < nk_full) {
                 sa.load_fast(ra[st]);
                 sb.load_fast(rb[st]);
+            } else if (edge_ok && fetch < nk_full) {
+#pragma unroll
+                for (int v = 0; v < StageA::NV; ++v) sa.load_edge_vec(ra[st][v], v, ea);
+#pragma unroll
+                for (int v = 0; v < StageB::NV; ++v) sb.load_edge_vec(rb[st][v], v, eb);
+                sh_a[st] = rot_a;
+                sh_b[st] = rot_b;
             } else {
                 sa.load_safe(ra[st], m_rem, k_rem);
                 sb.load_safe(rb[st], n_rem, k_rem);
@@ -900,12 +939,13 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             sb.advance();
             ++fetch;
             if (t == 0) {
-                sa.store_lds(As, ra[0]);
-                sb.store_lds(Bs, rb[0]);
-                if constexpr (COLSUM) {
 #pragma unroll
-                    for (int v = 0; v < StageA::NV; ++v) cs += ra[0][v];
+                for (int v = 0; v < StageA::NV; ++v) {
+                    const f32x4 stored = sa.store_lds_vec_shifted(As, ra[0][v], v, sh_a[0], any_rot_a);
+                    if constexpr (COLSUM) cs += stored;
                 }
+#pragma unroll
+                for (int v = 0; v < StageB::NV; ++v) sb.store_lds_vec_shifted(Bs, rb[0][v], v, sh_b[0], any_rot_b);
             }
         }
         lds_barrier();
@@ -929,13 +969,17 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     // One k tile.  P selects the LDS buffer read; the register stage P^1 holds the
     // next tile and is refilled, piece by piece, with tile `fetch`.
     // MODE 0: tile `fetch` is a full tile of an interior block (unchecked loads);
-    // MODE 1: a full-k tile of an edge block (loads use the precomputed edge facts ea / eb);
-    // MODE 2: anything (each fetch decides between unchecked and fully checked loads).
+    // MODE 1: a full-k tile of an edge block (branch-free loads through the precomputed edge facts ea / eb);
+    // MODE 2: the last tiles of an interior block (each fetch decides between unchecked loads and, at or past the
+    //         end of K, checked ones);
+    // MODE 3: the last tiles of an edge block (edge loads for full-k tiles, fully checked loads otherwise).
     auto k_tile = [&](auto parity, auto mode, const typename StageA::Edge& ea, const typename StageB::Edge& eb) {
         constexpr int P = decltype(parity)::value;
         constexpr int Q = P ^ 1;
         constexpr int MODE = decltype(mode)::value;
-        const bool fast = (MODE == 0) || (MODE == 2 && full_mn && (fetch < nk_full));
+        const bool fast = (MODE == 0) || (MODE == 2 && (fetch < nk_full));
+        // the tail of an edge block: a full-k tile still takes the branch-free edge loads
+        const bool edge_fast = (MODE == 3) && edge_ok && (fetch < nk_full);
         const int k_rem = klen - fetch * BK;
         const float* as = a_rd + P * (BK * PA);
         const float* bs = b_rd + P * (BK * PB);
@@ -984,9 +1028,15 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                             if (q < StageA::NV) {
                                 const int v = q < StageA::NV ? q : 0;
                                 if (is_store) {
-                                    sa.store_lds_vec(as_next, ra[Q][v], v);
-                                    if constexpr (COLSUM) cs += ra[Q][v];
-                                } else if (MODE == 1)
+                                    if constexpr (MODE == 0 || MODE == 2) {
+                                        sa.store_lds_vec(as_next, ra[Q][v], v);
+                                        if constexpr (COLSUM) cs += ra[Q][v];
+                                    } else {
+                                        const f32x4 stored =
+                                            sa.store_lds_vec_shifted(as_next, ra[Q][v], v, sh_a[Q], any_rot_a);
+                                        if constexpr (COLSUM) cs += stored;
+                                    }
+                                } else if (MODE == 1 || edge_fast)
                                     sa.load_edge_vec(ra[Q][v], v, ea);
                                 else if (fast)
                                     sa.load_fast_vec(ra[Q][v], v);
@@ -994,9 +1044,13 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                                     sa.load_safe_vec(ra[Q][v], v, m_rem, k_rem);
                             } else {
                                 const int v = q >= StageA::NV ? q - StageA::NV : 0;
-                                if (is_store)
-                                    sb.store_lds_vec(bs_next, rb[Q][v], v);
-                                else if (MODE == 1)
+                                if (is_store) {
+                                    if constexpr (MODE == 0 || MODE == 2)
+                                        sb.store_lds_vec(bs_next, rb[Q][v], v);
+                                    else
+                                        sb.store_lds_vec_shifted(bs_next, rb[Q][v], v, sh_b[Q], any_rot_b);
+                                }
+                                else if (MODE == 1 || edge_fast)
                                     sb.load_edge_vec(rb[Q][v], v, eb);
                                 else if (fast)
                                     sb.load_fast_vec(rb[Q][v], v);
@@ -1009,12 +1063,16 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                 }
             }
         }
+        // what stage Q holds now was fetched in this tile: remember whether it arrived shifted
+        if constexpr (MODE == 1 || MODE == 3) {
+            const bool via_edge = (MODE == 1) || edge_fast;
+            sh_a[Q] = via_edge ? rot_a : 0;
+            sh_b[Q] = via_edge ? rot_b : 0;
+        }
     };
 
     using P0 = std::integral_constant<int, 0>;
     using P1 = std::integral_constant<int, 1>;
-    const typename StageA::Edge ea = sa.edge_info(m_rem);
-    const typename StageB::Edge eb = sb.edge_info(n_rem);
     int kt = 0;
     // branch-free pairs of tiles while both fetches (tiles kt+3, kt+4) are full k tiles
     if (full_mn) {
@@ -1022,16 +1080,23 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             k_tile(P0{}, std::integral_constant<int, 0>{}, ea, eb);
             k_tile(P1{}, std::integral_constant<int, 0>{}, ea, eb);
         }
-    } else {
+    } else if (edge_ok) {
         for (; kt + 4 < nk_full; kt += 2) {
             k_tile(P0{}, std::integral_constant<int, 1>{}, ea, eb);
             k_tile(P1{}, std::integral_constant<int, 1>{}, ea, eb);
         }
     }
     // the last few tiles (K tail included): same body, each fetch chooses checked or unchecked loads
-    for (; kt < nk; kt += 2) {
-        k_tile(P0{}, std::integral_constant<int, 2>{}, ea, eb);
-        k_tile(P1{}, std::integral_constant<int, 2>{}, ea, eb);
+    if (full_mn) {
+        for (; kt < nk; kt += 2) {
+            k_tile(P0{}, std::integral_constant<int, 2>{}, ea, eb);
+            k_tile(P1{}, std::integral_constant<int, 2>{}, ea, eb);
+        }
+    } else {
+        for (; kt < nk; kt += 2) {
+            k_tile(P0{}, std::integral_constant<int, 3>{}, ea, eb);
+            k_tile(P1{}, std::integral_constant<int, 3>{}, ea, eb);
+        }
     }
 
     if constexpr (COLSUM) {
