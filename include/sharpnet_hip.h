@@ -47,6 +47,15 @@ extern "C" {
 int snhip_create(void** handle);
 /* Replaces cublasDestroy_v2 (CublasWrapper.cs:225). Frees the split-K workspace. */
 int snhip_destroy(void* handle);
+/* The handle owns one scratch buffer: split-K partial sums and partial column sums.  It grows on demand, and growing
+ * means a stream synchronisation, hipFree and hipMalloc in the middle of a call - not allowed under HIP graph capture
+ * and unwelcome in a serving loop.  snhip_reserve_workspace sizes it ahead of time (it never shrinks): after it,
+ * no call whose need is at most `bytes` synchronises or allocates.  The largest need of any call is 1 GiB (the cap
+ * the split-K choice observes; larger values are refused with status 7); a product of M x N x batch floats split S
+ * ways needs 4 * M * N * batch * S bytes (S as reported by snhip_query_tuning).  No reference counterpart (cuBLAS
+ * manages its own workspace; cublasSetWorkspace is not bound by the reference). */
+int snhip_reserve_workspace(void* handle, size_t bytes);
+int snhip_get_workspace_size(void* handle, size_t* bytes);
 /* No counterpart is bound by the reference (it never calls cublasSetStream, so
  * GEMMs run on the legacy default stream); offered for callers with their own
  * hipStream_t.  stream == NULL selects the null stream again. */

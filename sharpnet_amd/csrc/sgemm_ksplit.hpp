@@ -25,13 +25,18 @@ namespace snhip {
 // column-tile index runs fastest in blockIdx.x
 constexpr int GEMM_FLAG_TILE_N_FASTEST = 4;
 
-// NT: 32-column tiles per workgroup (1 or 2); the four wavefronts are NT tiles x 4 / NT slices of K.
-template <int NT_>
+// NT: 32-column tiles per workgroup (1 or 2); the NW wavefronts (4, or 8 for products with so few tiles that even
+// four slices leave most of the chip idle) are NT tiles x NW / NT slices of K.
+template <int NT_, int NW_ = 4>
 struct KsplitCfg {
-    static constexpr int NT = NT_;
-    static constexpr int KS = 4 / NT_;  // K slices
+    static constexpr int NT = NT_, NW = NW_;
+    static constexpr int KS = NW_ / NT_;  // K slices
     static constexpr int DEPTH = 4;     // groups of 32 k values in flight per wavefront
     static constexpr int PITCH = 36;    // floats per patch row
+    // LDS (dynamic): a patch of 2 x 32 rows per wavefront during the k loop; afterwards the same memory holds the
+    // KS partial tiles
+    static constexpr int PATCH_FLOATS = NW_ * 2 * 32 * PITCH, PART_FLOATS = KS * NT_ * 32 * 33;
+    static constexpr int LDS_BYTES = 4 * (PATCH_FLOATS > PART_FLOATS ? PATCH_FLOATS : PART_FLOATS);
 };
 
 // One operand of one wavefront: 32 rows (m or n) x the k range.
@@ -93,12 +98,12 @@ struct KsplitOperand {
     }
 };
 
-template <bool TA, bool TB, int NT = 1>
-__global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
-    using C = KsplitCfg<NT>;
+template <bool TA, bool TB, int NT = 1, int NW = 4>
+__global__ void __launch_bounds__(64 * NW) sgemm_ksplit_kernel(const GemmParams p) {
+    using C = KsplitCfg<NT, NW>;
     constexpr int KS = C::KS, D = C::DEPTH, P = C::PITCH;
-    __shared__ float part[KS][NT][32][33];
-    __shared__ __attribute__((aligned(16))) float patch[4][2][32 * P];
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float(*const part)[NT][32][33] = reinterpret_cast<float(*)[NT][32][33]>(smem);  // [KS][NT][32][33], after the k loop
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
     const int nt = wave % NT, kg = wave / NT;
     // Workgroups go to the eight XCDs round-robin by their linear index.  The index that runs fastest spreads over
@@ -117,8 +122,8 @@ __global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
     KsplitOperand<!TB> ob;    // B not transposed: stored K x N, contiguous along n
     oa.init(Ab, p.lda, m0, p.M, lane);
     ob.init(Bb, p.ldb, n0, p.N, lane);
-    float* pa = &patch[wave][0][0];
-    float* pb = &patch[wave][1][0];
+    float* pa = smem + (wave * 2 + 0) * (32 * P);
+    float* pb = smem + (wave * 2 + 1) * (32 * P);
 
     const int K = p.K;
     const int groups = (K + 31) / 32;
@@ -199,6 +204,7 @@ __global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
             multiply(0);
         }
 
+    __syncthreads();  // every wavefront is done with its patch: the memory now takes the partial tiles
     // accumulator register r holds row 8 (r / 4) + 4 lhi + r % 4, column l32 of the tile
 #pragma unroll
     for (int r = 0; r < 16; ++r)
@@ -207,8 +213,8 @@ __global__ void __launch_bounds__(256) sgemm_ksplit_kernel(const GemmParams p) {
 
     const int nbase = tile_n * (32 * NT);
 #pragma unroll
-    for (int q = 0; q < 4 * NT; ++q) {
-        const int e = threadIdx.x + 256 * q;
+    for (int q = 0; q < (16 * NT) / NW; ++q) {
+        const int e = threadIdx.x + (64 * NW) * q;
         const int lr = e / (32 * NT), lc = e % (32 * NT);
         const int row = m0 + lr, col = nbase + lc;
         if (row >= p.M || col >= p.N) continue;

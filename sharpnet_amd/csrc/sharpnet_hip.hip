@@ -167,14 +167,14 @@ const ConfigEntry kConfigs[] = {
     make_entry_bf16<BTileCfg<1, 1, 2, 2, 64>>(3, 0.45, 0.60, 1.1),   // 13: 64 x 64, BK 64
     // K split over the wavefronts of a workgroup (sgemm_ksplit.hpp): not part of the cost model's search, see
     // prefer_ksplit()
-    ConfigEntry{32, 32, 32, 256, 0, 1, 2,
+    ConfigEntry{32, 32, 32, 256, KsplitCfg<1>::LDS_BYTES, 1, 2,
                 {{sgemm_ksplit_kernel<false, false>, sgemm_ksplit_kernel<false, true>},
                  {sgemm_ksplit_kernel<true, false>, sgemm_ksplit_kernel<true, true>}},
                 // the same kernels serve as the extended form: they always apply the addend and the (leaky) ReLU
                 {{sgemm_ksplit_kernel<false, false>, sgemm_ksplit_kernel<false, true>},
                  {sgemm_ksplit_kernel<true, false>, sgemm_ksplit_kernel<true, true>}},
                 6, 0.5, 0.5, 1.0},  // 14: 32 x 32, four K slices
-    ConfigEntry{32, 64, 32, 256, 0, 1, 2,
+    ConfigEntry{32, 64, 32, 256, KsplitCfg<2>::LDS_BYTES, 1, 2,
                 {{sgemm_ksplit_kernel<false, false, 2>, sgemm_ksplit_kernel<false, true, 2>},
                  {sgemm_ksplit_kernel<true, false, 2>, sgemm_ksplit_kernel<true, true, 2>}},
                 {{sgemm_ksplit_kernel<false, false, 2>, sgemm_ksplit_kernel<false, true, 2>},
@@ -198,10 +198,18 @@ const ConfigEntry kConfigs[] = {
     make_entry_bf16_stored<BTileCfg<4, 4, 2, 2, 64>>(1, 0.85, 0.85, 3.0),   // 18: 256 x 256, BK 64
     make_entry_bf16_stored<BTileCfg<2, 2, 2, 2, 64>>(2, 0.65, 0.80, 1.3),   // 19: 128 x 128, BK 64
     make_entry_bf16_stored<BTileCfg<1, 1, 2, 2, 128>>(2, 0.45, 0.60, 1.1),  // 20: 64 x 64, BK 128
+    // K split eight ways over a workgroup of eight wavefronts: see prefer_ksplit()
+    ConfigEntry{32, 32, 32, 512, KsplitCfg<1, 8>::LDS_BYTES, 1, 2,
+                {{sgemm_ksplit_kernel<false, false, 1, 8>, sgemm_ksplit_kernel<false, true, 1, 8>},
+                 {sgemm_ksplit_kernel<true, false, 1, 8>, sgemm_ksplit_kernel<true, true, 1, 8>}},
+                {{sgemm_ksplit_kernel<false, false, 1, 8>, sgemm_ksplit_kernel<false, true, 1, 8>},
+                 {sgemm_ksplit_kernel<true, false, 1, 8>, sgemm_ksplit_kernel<true, true, 1, 8>}},
+                1, 0.5, 0.5, 1.0},  // 21: 32 x 32, eight K slices
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 constexpr int kKsplitConfig = 14;   // and kKsplitConfig + 1
 constexpr int kStreamConfig = 16;   // and kStreamConfig + 1
+constexpr int kKsplit8Config = 21;
 
 // Fused attention forward kernels (attention_mfma.hpp)
 struct AttnEntry {
@@ -438,7 +446,7 @@ struct GemmArgs {
 // pays when the tiled kernels cannot fill the chip: few 32 x 32 tiles and a K of at least a few groups of 32.
 int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) {
     if (math != SNHIP_MATH_FP32 || two_level || g.K < 32 || g.K % 4 != 0) return -1;
-    const bool forced = h->force_cfg == kKsplitConfig || h->force_cfg == kKsplitConfig + 1;
+    const bool forced = h->force_cfg == kKsplitConfig || h->force_cfg == kKsplitConfig + 1 || h->force_cfg == kKsplit8Config;
     if (h->force_cfg >= 0 && !forced) return -1;
     const bool multi = g.batch > 1;
     auto aligned = [&](const float* ptr, int ld, long long stride, bool rows_contiguous, int rows) {
@@ -452,6 +460,8 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
     // 30.5 against 17.2 with split-K 16).  Up to one 32 x 32 tile per compute unit: four K slices; up to one
     // 32 x 64 tile per compute unit: two.
     const long long rows32 = (long long)ceil_div(g.M, 32) * g.batch;
+    // a quarter of the compute units or fewer, and a K that gives eight wavefronts a few groups of 32 each
+    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 4 && g.K >= 512) return kKsplit8Config;
     if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu) return kKsplitConfig;
     if (rows32 * ceil_div(g.N, 64) <= (long long)h->num_cu) return kKsplitConfig + 1;
     return -1;
@@ -735,6 +745,46 @@ inline bool op_is_trans(int op, bool* ok) {
     return op != SNHIP_OP_N;
 }
 
+// Kernels whose LDS stage exceeds the 64 KiB default need an explicit opt-in; it is a property of the function on a
+// device, so it is set once per device (every handle created later on that device finds it done).
+hipError_t prepare_kernels_once(int dev) {
+    static std::mutex mu;
+    static bool done[kMaxDevices] = {};
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (done[dev]) return hipSuccess;
+    hipError_t e = hipSuccess;
+    for (int c = 0; c < kNumConfigs; ++c) {
+        for (int ta = 0; ta < 2; ++ta)
+            for (int tb = 0; tb < 2; ++tb) {
+                e = hipFuncSetAttribute(reinterpret_cast<const void*>(kConfigs[c].fn[ta][tb]),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kConfigs[c].lds_bytes);
+                if (e != hipSuccess) return e;
+            }
+        for (int ta = 0; ta < 2; ++ta)
+            for (int tb = 0; tb < 2; ++tb) {
+                if (kConfigs[c].fn_ext[ta][tb] == nullptr) continue;
+                e = hipFuncSetAttribute(reinterpret_cast<const void*>(kConfigs[c].fn_ext[ta][tb]),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kConfigs[c].lds_bytes);
+                if (e != hipSuccess) return e;
+            }
+    }
+    for (const AttnEntry& c : kAttn) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                c.lds_bytes);
+        if (e != hipSuccess) return e;
+    }
+    for (const AttnEntry& c : kAttnBwd) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                c.lds_bytes);
+        if (e != hipSuccess) return e;
+    }
+    e = rnn_prepare_kernels();
+    if (e != hipSuccess) return e;
+    done[dev] = true;
+    return hipSuccess;
+}
+
 }  // namespace
 
 extern "C" {
@@ -751,33 +801,7 @@ int snhip_create(void** handle) {
     // The code objects in this library exist for gfx950 only.
     if (prop.gcnArchName[0] == '\0' || __builtin_strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return SNHIP_STATUS_ARCH_MISMATCH;
-    // Kernels whose LDS stage exceeds the 64 KiB default need an explicit opt-in.
-    for (int c = 0; c < kNumConfigs; ++c) {
-        for (int ta = 0; ta < 2; ++ta)
-            for (int tb = 0; tb < 2; ++tb) {
-                e = hipFuncSetAttribute(reinterpret_cast<const void*>(kConfigs[c].fn[ta][tb]),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kConfigs[c].lds_bytes);
-                if (e != hipSuccess) return hip_to_status(e);
-            }
-        for (int ta = 0; ta < 2; ++ta)
-            for (int tb = 0; tb < 2; ++tb) {
-                if (kConfigs[c].fn_ext[ta][tb] == nullptr) continue;
-                e = hipFuncSetAttribute(reinterpret_cast<const void*>(kConfigs[c].fn_ext[ta][tb]),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kConfigs[c].lds_bytes);
-                if (e != hipSuccess) return hip_to_status(e);
-            }
-    }
-    for (const AttnEntry& c : kAttn) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                c.lds_bytes);
-        if (e != hipSuccess) return hip_to_status(e);
-    }
-    for (const AttnEntry& c : kAttnBwd) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                c.lds_bytes);
-        if (e != hipSuccess) return hip_to_status(e);
-    }
-    e = rnn_prepare_kernels();
+    e = prepare_kernels_once(dev);
     if (e != hipSuccess) return hip_to_status(e);
     void* scratch_ptr = nullptr;
     e = static_scratch_address(dev, &scratch_ptr);
@@ -800,6 +824,23 @@ int snhip_destroy(void* handle) {
         if (h->counters != nullptr) (void)hipFree(h->counters);
     }
     delete h;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_reserve_workspace(void* handle, size_t bytes) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (bytes > kMaxWorkspaceBytes) return SNHIP_STATUS_INVALID_VALUE;
+    Handle* h = static_cast<Handle*>(handle);
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (cur != h->device && hipSetDevice(h->device) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    return ensure_workspace(h, bytes);
+}
+
+int snhip_get_workspace_size(void* handle, size_t* bytes) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (bytes == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    *bytes = static_cast<Handle*>(handle)->ws_bytes;
     return SNHIP_STATUS_SUCCESS;
 }
 

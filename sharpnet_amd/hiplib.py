@@ -156,6 +156,8 @@ SIGNATURES = {
     "snhip_create": [_vpp],
     "snhip_destroy": [_vp],
     "snhip_set_stream": [_vp, _vp],
+    "snhip_reserve_workspace": [_vp, _sz],
+    "snhip_get_workspace_size": [_vp, ctypes.POINTER(_sz)],
     "snhip_get_version": [_vp, _c_int_p],
     "snhip_sgemm": [_vp, _i, _i, _i, _i, _i, _c_float_p, _vp, _i, _vp, _i, _c_float_p, _vp, _i],
     "snhip_sgemm_strided_batched": [_vp, _i, _i, _i, _i, _i, _c_float_p, _vp, _i, _ll, _vp, _i, _ll, _c_float_p, _vp,

@@ -177,6 +177,39 @@ def test_aliased_operands_VanillaSgdOrtho_pattern(oracle, gpu_wrapper):
     assert np.max(np.abs(gX.ToNumpy() - ref2)) <= tol(m, ref, W, 0.5, 1.0, X) + 1e-5
 
 
+@pytest.mark.parametrize("m,n", [(37, 53), (64, 256), (130, 70)])
+def test_VanillaSgdOrtho_update_all_five_products(oracle, gpu_wrapper, m, n):
+    """The whole sequence of Prod/Optimizers/VanillaSgdOrtho.cs:82-88 on the device, buffer for buffer:
+    I - W.W^T (NT, alpha -1, beta 1, A == B), (..).dW (NN), W^T.dW (TN, beta 0), -= dW^T.W (TN, alpha -1, beta 1),
+    += 0.5 W.(..) (NN, alpha 0.5, beta 1); every intermediate against the oracle fed with the oracle's own chain."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    rng = np.random.default_rng(300 + m)
+    W, dW = random_tensor(rng, (m, n), -1, 1), random_tensor(rng, (m, n), -1, 1)
+    gW, gdW = GPUTensor(W.shape, W, w), GPUTensor(dW.shape, dW, w)
+    eye = np.eye(m, dtype=np.float32)
+    buffer_mm, buffer_mn, buffer_nn = GPUTensor([m, m], eye, w), GPUTensor([m, n], None, w), GPUTensor([n, n], None, w)
+    buffer_mn.SetValue(float("nan"))
+    buffer_nn.SetValue(float("nan"))
+    buffer_mm.Dot(gW, False, gW, True, -1.0, 1.0)
+    r_mm = oracle.dot(W, False, W, True, -1.0, 1.0, eye)
+    assert np.max(np.abs(buffer_mm.ToNumpy() - r_mm)) <= tol(n, W, W, 1.0, 1.0, eye)
+    buffer_mn.Dot(buffer_mm, gdW)                                     # two-argument form: (false, false, 1, 0)
+    r_mn = oracle.dot(r_mm, False, dW, False)
+    assert np.max(np.abs(buffer_mn.ToNumpy() - r_mn)) <= 2 * tol(m, r_mm, dW)
+    buffer_nn.Dot(gW, True, gdW, False, 1.0, 0.0)
+    r_nn = oracle.dot(W, True, dW, False, 1.0, 0.0)
+    assert np.max(np.abs(buffer_nn.ToNumpy() - r_nn)) <= tol(m, W, dW)
+    buffer_nn.Dot(gdW, True, gW, False, -1.0, 1.0)
+    r_nn2 = oracle.dot(dW, True, W, False, -1.0, 1.0, r_nn)
+    assert np.max(np.abs(buffer_nn.ToNumpy() - r_nn2)) <= 2 * tol(m, dW, W, 1.0, 1.0, r_nn)
+    # antisymmetric by construction: W^T dW - (W^T dW)^T
+    assert np.max(np.abs(buffer_nn.ToNumpy() + buffer_nn.ToNumpy().T)) <= 4 * tol(m, dW, W)
+    buffer_mn.Dot(gW, False, buffer_nn, False, 0.5, 1.0)
+    r_fin = oracle.dot(W, False, r_nn2, False, 0.5, 1.0, r_mn)
+    assert np.max(np.abs(buffer_mn.ToNumpy() - r_fin)) <= 4 * (tol(n, W, r_nn2, 0.5) + tol(m, r_mm, dW))
+
+
 def test_views_at_odd_element_offsets(oracle, gpu_wrapper):
     """Slices are views at Pointer + 4*startIndex (GpuTensor.cs:616): only 4-byte alignment may be assumed."""
     from sharpnet_amd import GPUTensor
@@ -533,9 +566,10 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
         assert gpu_wrapper.last_tuning() == (ks, 1)
         assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, tA, b, tB, 0.5))) <= tol(K, a, b, 0.5)
         gpu_wrapper.set_tuning(-1, 0)
-        # automatic choice: the Dense layer of benchmark configuration 1, a square product of one 32 x 32 tile per
-        # CU, and a recurrent step (one 32 x 64 tile per CU)
-        for (M, N, K, want) in [(128, 256, 784, ks_all[0]), (512, 512, 512, ks_all[0]), (256, 2048, 512, ks_all[1])]:
+        # automatic choice: the forward product of benchmark configuration 1's Dense layer (32 tiles: eight K slices),
+        # a square product of one 32 x 32 tile per CU, a recurrent step (one 32 x 64 tile per CU), the layer's dx
+        for (M, N, K, want) in [(128, 256, 784, ks_all[2]), (512, 512, 512, ks_all[0]), (256, 2048, 512, ks_all[1]),
+                                (128, 784, 256, ks_all[0])]:
             a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
             b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
             got = gpu_dot(gpu_wrapper, a, tA, b, tB, 1.0, 0.0, c_shape=[M, N], prefill=float("nan"))

@@ -56,6 +56,33 @@ def test_dense_layer_forward_backward_config1(oracle, gpu_wrapper):
         assert np.all(gdx.ToNumpy() == 7.0)                              # dx untouched when the previous layer is the input
 
 
+def test_dense_layer_config1_in_out_layout(oracle, gpu_wrapper):
+    """The same layer in the (in, out) weight layout of the benchmark's wording and of the TensorFlow-era vectors
+    (Tests/NonReg/TestNetworkPropagation.cs:80-105): Y = X.W + b (NN with the bias in the same launch),
+    dW = X^T.dY (TN: 784 x 256 x 128), dX = dY.W^T (NT), at the full shape, NaN-prefilled destinations."""
+    from sharpnet_amd import GPUTensor, workloads as wl
+    w = gpu_wrapper
+    d = wl.dense_layer_inputs(seed=1)
+    x, dy = d["x"], d["dy"]
+    W = np.ascontiguousarray(d["w_out_in"].T)                       # (784, 256)
+    bias = np.linspace(-0.5, 0.5, W.shape[1]).astype(np.float32)
+    gx, gW, gb, gdy = T(w, x), T(w, W), T(w, bias), T(w, dy)
+    gy, gdW, gdx = GPUTensor([128, 256], None, w), GPUTensor([784, 256], None, w), GPUTensor([128, 784], None, w)
+    for t in (gy, gdW, gdx):
+        t.SetValue(float("nan"))
+    gy.DotRowMajor(gx, False, gW, False, 1.0, 0.0, bias=gb)
+    assert np.max(np.abs(gy.ToNumpy() - (oracle.dot(x, False, W, False) + bias))) <= bound(784, x, W, 1e-6)
+    # the oracle's Linear forward on the (out, in) copy of the same weights is the same function
+    assert np.max(np.abs(gy.ToNumpy() - oracle.dense_forward(x, d["w_out_in"], bias))) <= bound(784, x, W, 1e-6)
+    gdW.Dot(gx, True, gdy, False, 1.0 / 128, 0.0)
+    assert np.max(np.abs(gdW.ToNumpy() - oracle.dot(x, True, dy, False, 1.0 / 128))) <= bound(128, x, dy) / 128 + 1e-9
+    gdx.Dot(gdy, False, gW, True, 1.0, 0.0)
+    assert np.max(np.abs(gdx.ToNumpy() - oracle.dot(dy, False, W, True))) <= bound(256, dy, W)
+    # consistent with the (out, in) layer: dW here is the transpose of dW there, dX is the same
+    _, _, rdx = oracle.dense_backward(x, dy, d["w_out_in"], multiplier=1.0 / 128)
+    assert np.max(np.abs(gdx.ToNumpy() - rdx)) <= bound(256, dy, W)
+
+
 ACTS = [("relu", "CUDNN_ACTIVATION_RELU", 0.0), ("leaky_relu", "CUDNN_ACTIVATION_LEAKY_RELU", 0.1),
         ("leaky_relu", "CUDNN_ACTIVATION_LEAKY_RELU", 0.3), ("sigmoid", "CUDNN_ACTIVATION_SIGMOID", 0.0),
         ("tanh", "CUDNN_ACTIVATION_TANH", 0.0)]

@@ -51,8 +51,7 @@ def test_config2_sweep_all_sizes_transposes_betas(oracle, gpu_wrapper):
                 a, b = bufs[sa], bufs[sb]
                 if a is b:                                     # square sizes: keep A and B distinct
                     b = bufs.setdefault((sb, "b"), rng.uniform(-1, 1, sb).astype(np.float32))
-                betas = (0.0, 1.0) if (M * N * K < 3e11 or (not tA and not tB)) else (0.0,)
-                for beta in betas:
+                for beta in (0.0, 1.0):
                     c = rng.uniform(-1, 1, (M, N)).astype(np.float32) if beta else None
                     sampled_rows_check(oracle, gpu_wrapper, wl.Gemm(M, N, K, tA, tB, 1.0, beta), a, b, c, nrows=6)
 
@@ -239,3 +238,32 @@ def test_calls_can_be_recorded_into_a_hip_graph_and_replayed(oracle, gpu_wrapper
         if graph:
             hip.hipGraphDestroy(graph)
         check_status(w.lib.snhip_stream_destroy(stream), "snhip_stream_destroy")
+
+
+def test_workspace_can_be_reserved_ahead_of_time(oracle, gpu_wrapper):
+    """snhip_reserve_workspace sizes the handle's scratch buffer so that later calls neither synchronise nor allocate:
+    a split-K product whose partial sums fit leaves the buffer as reserved, and gives the result it gives otherwise."""
+    import ctypes
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status, CublasStatus
+    from tests.helpers import random_tensor
+    w = gpu_wrapper
+    size = ctypes.c_size_t()
+    check_status(w.lib.snhip_get_workspace_size(w.handle, ctypes.byref(size)))
+    want = max(size.value, 48 << 20) + (1 << 20)
+    check_status(w.lib.snhip_reserve_workspace(w.handle, want))
+    check_status(w.lib.snhip_get_workspace_size(w.handle, ctypes.byref(size)))
+    assert size.value == want
+    check_status(w.lib.snhip_reserve_workspace(w.handle, 1024))                 # never shrinks
+    check_status(w.lib.snhip_get_workspace_size(w.handle, ctypes.byref(size)))
+    assert size.value == want
+    assert w.lib.snhip_reserve_workspace(w.handle, (1 << 30) + 1) == CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    rng = np.random.default_rng(5)
+    a, b = random_tensor(rng, (512, 8192), -1, 1), random_tensor(rng, (8192, 64), -1, 1)
+    ga, gb, gc = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w), GPUTensor([512, 64], None, w)
+    gc.SetValue(float("nan"))
+    gc.Dot(ga, False, gb, False, 1.0, 0.0)
+    assert w.last_tuning()[1] > 1                                             # split along K: the buffer is in use
+    assert np.max(np.abs(gc.ToNumpy() - oracle.dot(a, False, b, False))) <= 1e-4 * np.sqrt(8192)
+    check_status(w.lib.snhip_get_workspace_size(w.handle, ctypes.byref(size)))
+    assert size.value == want
