@@ -12,12 +12,16 @@ from . import hiplib
 from .gpu_tensor import GPUTensor
 from .hiplib import CublasStatus, check_status
 
-# limits of snhip_attention_forward: (keys, head dimension) pairs it has a kernel for
+# limits of snhip_attention_forward's single-block kernels: (keys, head dimension) pairs
 FUSED_ATTENTION_LIMITS = ((256, 64), (128, 128))
 
 
 def fused_attention_supported(tkv, dk, dv):
-    return any(tkv <= keys and max(dk, dv) <= dim for keys, dim in FUSED_ATTENTION_LIMITS)
+    """Whether snhip_attention_forward has a kernel for the sizes (it says the same with status 15): one key block, or
+    any number of keys with head dimensions that are multiples of 4 and at most 64."""
+    if any(tkv <= keys and max(dk, dv) <= dim for keys, dim in FUSED_ATTENTION_LIMITS):
+        return True
+    return max(dk, dv) <= 64 and dk % 4 == 0 and dv % 4 == 0
 
 
 def fused_attention_forward(Q, K, V, O, weights, *, batch, heads, tq, tkv, dk, dv, scale, is_causal, packed):
@@ -68,8 +72,9 @@ def attention_backward(dQ, dK, dV, Q, K, V, dO, weights, scores_gradients, *, ba
 
 
 def ScaledDotProductAttentionForwardPropagation(Q, K, V, y, isTraining, use_scale, is_causal, fused=True):
-    """fused=True runs the whole chain as one launch when the sizes allow it (at most 256 keys with a head dimension of at
-    most 64, or 128 keys with 128); otherwise, or with fused=False, the reference's four calls."""
+    """fused=True runs the whole chain as one launch when the sizes allow it (any number of keys with a head dimension
+    of at most 64 - beyond 256 keys a multiple of 4 -, or up to 128 keys with a head dimension of up to 128);
+    otherwise, or with fused=False, the reference's four calls."""
     if V.Shape != K.Shape:
         raise ValueError("V.Shape and K.Shape must be equal, but are %s and %s" % (V.Shape, K.Shape))
     if V.Shape != y.Shape:

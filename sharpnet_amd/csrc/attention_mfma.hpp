@@ -424,4 +424,274 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
     }  // query tiles
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same forward pass for any number of keys: the keys are walked in blocks of 256 in TWO passes.
+//   pass 1: scores of every block (K . Q^T as above), running row maximum and row sum of exponentials - nothing
+//           else is kept;
+//   pass 2: the scores again, now turned into the final probabilities p = exp(s - max) / sum at once (the softmax
+//           formula of the reference, Prod/CPU/CpuTensorActivationFunctions.cs:19-46, with its global maximum),
+//           written out if the caller keeps them, and multiplied into O += P_block . V_block.
+// Recomputing the scores costs half again the MFMA work of the single-block kernel, and buys exact, never rescaled
+// probabilities that are written exactly once - which is what a caller that keeps the (Tq, Tk) softmax output for
+// its backward pass needs.  With the causal mask, key blocks that lie wholly above the diagonal of a query tile are
+// not computed; their part of the stored probabilities is written as zeros.
+// A workgroup owns 128 queries (32 per wavefront) of one (batch, head) matrix; the K block (and in pass 2 the V
+// block) is staged in LDS exactly as in the kernel above.  Head dimensions: multiples of 4 up to HD.
+// ---------------------------------------------------------------------------------------------------------------
+template <int HD>
+__global__ void __launch_bounds__(256) attention_fwd_long_kernel(const AttnParams p) {
+    using CFG = AttnCfg<8, HD>;
+    constexpr int AT_TK = CFG::KEYS, AT_D = HD, AT_KP = CFG::KP, AT_VP = CFG::VP;
+    constexpr int NTILE = AT_TK / 32, MT = AT_D / 32;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float* const Ks = smem;                  // [AT_D][AT_KP]
+    float* const Vs = smem + AT_D * AT_KP;   // [AT_TK][AT_VP]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int z = blockIdx.y;
+    const BatchIndex bi = split_batch(z, p.batch_inner);
+    const float* Qz = p.Q + batch_offset(bi, p.sQ, p.sQ2);
+    const float* Kz = p.K + batch_offset(bi, p.sK, p.sK2);
+    const float* Vz = p.V + batch_offset(bi, p.sV, p.sV2);
+    float* Oz = p.O + batch_offset(bi, p.sO, p.sO2);
+
+    // last query tile first: with the causal mask the late tiles see the most key blocks, so they start first
+    const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * AT_BQ;
+    const int row = q0 + wave * 32 + l32;
+    const bool row_ok = row < p.Tq;
+
+    // this lane's query row as the B operand of the score product: qf[s] = Q[row][2 s + lane / 32]
+    float qf[AT_D / 2];
+    {
+        const float* qrow = Qz + (long long)(row_ok ? row : p.Tq - 1) * p.ldq;
+#pragma unroll
+        for (int j = 0; j < AT_D / 4; ++j) {
+            const f32x4 x = load4_select(qrow + (4 * j < p.dk ? 4 * j : 0), row_ok && 4 * j < p.dk);
+            qf[2 * j] = lhi ? x.y : x.x;
+            qf[2 * j + 1] = lhi ? x.w : x.z;
+        }
+    }
+
+    const int nblocks = (p.Tk + AT_TK - 1) / AT_TK;
+    // causal: the last query of the tile sees keys 0 .. q0 + 127
+    int nb_needed = nblocks;
+    if (p.causal) {
+        const int last_row = (q0 + AT_BQ - 1 < p.Tq - 1) ? q0 + AT_BQ - 1 : p.Tq - 1;
+        const int nb = last_row / AT_TK + 1;
+        nb_needed = nb < nblocks ? nb : nblocks;
+    }
+
+    constexpr int KIT = (AT_TK * AT_D / 4) / 256;
+    auto stage_k = [&](int kb) {
+        f32x4 kx[KIT];
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = kb * AT_TK + idx % AT_TK, v = idx / AT_TK;
+            const bool ok = key < p.Tk && 4 * v < p.dk;
+            kx[it] = load4_select(Kz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldk + (4 * v < p.dk ? 4 * v : 0), ok);
+        }
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = idx % AT_TK, v = idx / AT_TK;
+            Ks[(4 * v + 0) * AT_KP + key] = kx[it].x;
+            Ks[(4 * v + 1) * AT_KP + key] = kx[it].y;
+            Ks[(4 * v + 2) * AT_KP + key] = kx[it].z;
+            Ks[(4 * v + 3) * AT_KP + key] = kx[it].w;
+        }
+    };
+    auto stage_v = [&](int kb) {
+        f32x4 vx[KIT];
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = kb * AT_TK + idx / (AT_D / 4), v = idx % (AT_D / 4);
+            const bool ok = key < p.Tk && 4 * v < p.dv;
+            vx[it] = load4_select(Vz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldv + (4 * v < p.dv ? 4 * v : 0), ok);
+        }
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 256 + tid;
+            const int key = idx / (AT_D / 4), v = idx % (AT_D / 4);
+            *reinterpret_cast<f32x4*>(Vs + key * AT_VP + 4 * v) = vx[it];
+        }
+    };
+
+    constexpr float kLog2e = 1.44269504088896340736f;
+    constexpr float kMasked = -1e12f * kLog2e;
+    const float sl = p.scale * kLog2e;
+
+    // scores of key block kb in the log2 domain, masked: sacc[t][r] belongs to key kb*256 + t*32 + 8*(r/4) + r%4 + 4*lhi
+    f32x16 sacc[NTILE];
+    auto scores = [&](int kb) {
+#pragma unroll
+        for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[t][r] = 0.0f;
+        const float* kbase = Ks + lhi * AT_KP + l32;
+        float ka[2][NTILE];
+#pragma unroll
+        for (int t = 0; t < NTILE; ++t) ka[0][t] = kbase[t * 32];
+#pragma unroll
+        for (int s = 0; s < AT_D / 2; ++s) {
+            if (s + 1 < AT_D / 2) {
+#pragma unroll
+                for (int t = 0; t < NTILE; ++t) ka[(s + 1) & 1][t] = kbase[(2 * (s + 1)) * AT_KP + t * 32];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < NTILE; ++t)
+                sacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s & 1][t], qf[s], sacc[t], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // last key this lane's query may see, relative to the block and to the lane's own offset
+        int lim = p.Tk - 1;
+        if (p.causal && row < lim) lim = row;
+        lim -= kb * AT_TK + 4 * lhi;
+#pragma unroll
+        for (int t = 0; t < NTILE; ++t) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float v = sl * sacc[t][r];
+                sacc[t][r] = (t * 32 + 8 * (r / 4) + (r % 4) > lim) ? kMasked : v;
+            }
+        }
+    };
+
+    // ---- pass 1: row maximum and row sum over all needed blocks ----
+    float m = -3.402823466e+38f, l = 0.0f;
+    for (int kb = 0; kb < nb_needed; ++kb) {
+        stage_k(kb);
+        __syncthreads();
+        scores(kb);
+        float bm = -3.402823466e+38f;
+#pragma unroll
+        for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bm = fmaxf(bm, sacc[t][r]);
+        bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+        const float m_new = fmaxf(m, bm);
+        float bs = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bs += __builtin_amdgcn_exp2f(sacc[t][r] - m_new);
+        bs += __shfl_xor(bs, 32, 64);
+        l = l * __builtin_amdgcn_exp2f(m - m_new) + bs;
+        m = m_new;
+        __syncthreads();  // the block has been read by every wavefront: its LDS may be overwritten
+    }
+    const float inv = 1.0f / l;
+
+    // ---- pass 2: probabilities, P out, O += P . V ----
+    f32x16 oacc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[mt][r] = 0.0f;
+    float* const pbase = (p.P != nullptr) ? p.P + ((long long)z * p.Tq + (row_ok ? row : 0)) * p.Tk : nullptr;
+    for (int kb = 0; kb < nb_needed; ++kb) {
+        stage_k(kb);
+        stage_v(kb);
+        __syncthreads();
+        scores(kb);
+#pragma unroll
+        for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[t][r] = __builtin_amdgcn_exp2f(sacc[t][r] - m) * inv;
+
+        if (pbase != nullptr && row_ok) {
+            float* prow = pbase + kb * AT_TK;
+            const bool whole = (p.flags & 2) && (kb + 1) * AT_TK <= p.Tk;  // uniform
+#pragma unroll
+            for (int t = 0; t < NTILE; ++t) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int key0 = t * 32 + 8 * g + 4 * lhi;
+                    if (whole) {
+                        *reinterpret_cast<f32x4*>(prow + key0) =
+                            f32x4{sacc[t][4 * g], sacc[t][4 * g + 1], sacc[t][4 * g + 2], sacc[t][4 * g + 3]};
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (kb * AT_TK + key0 + j < p.Tk) prow[key0 + j] = sacc[t][4 * g + j];
+                    }
+                }
+            }
+        }
+
+        // O^T += V^T . P^T: even and odd k steps accumulate separately (no MFMA waits for its predecessor)
+        {
+            constexpr int NSTEP = NTILE * 16;
+            constexpr int LOOK = 2;
+            f32x16 part[2][MT];
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) part[h][mt][r] = 0.0f;
+            const float* vbase = Vs + (4 * lhi) * AT_VP + l32;
+            float va[4][MT];
+            auto v_off = [](int i) { return ((i / 16) * 32 + 8 * ((i % 16) / 4) + (i % 4)) * AT_VP; };
+#pragma unroll
+            for (int i = 0; i < LOOK; ++i)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) va[i][mt] = vbase[v_off(i) + mt * 32];
+#pragma unroll
+            for (int i = 0; i < NSTEP; ++i) {
+                if (i + LOOK < NSTEP) {
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) va[(i + LOOK) % 4][mt] = vbase[v_off(i + LOOK) + mt * 32];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    part[i & 1][mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[i % 4][mt], sacc[i / 16][i % 16],
+                                                                           part[i & 1][mt], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) oacc[mt] += part[0][mt] + part[1][mt];
+        }
+        __syncthreads();
+    }
+
+    // causal: the blocks that were skipped hold zeros in the stored probabilities
+    if (pbase != nullptr && row_ok) {
+        for (int kb = nb_needed; kb < nblocks; ++kb) {
+            float* prow = pbase + kb * AT_TK;
+            for (int c = 4 * lhi; c < AT_TK; c += 8) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (kb * AT_TK + c + j < p.Tk) prow[c + j] = 0.0f;
+            }
+        }
+    }
+
+    // oacc[mt][r] is O[row][mt*32 + 8*(r/4) + 4*lhi + r%4]
+    if (row_ok) {
+        float* orow = Oz + (long long)row * p.ldo;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int c0 = mt * 32 + 8 * g + 4 * lhi;
+                if (c0 >= p.dv) continue;
+                if ((p.flags & 1) && c0 + 4 <= p.dv) {
+                    *reinterpret_cast<f32x4*>(orow + c0) =
+                        f32x4{oacc[mt][4 * g], oacc[mt][4 * g + 1], oacc[mt][4 * g + 2], oacc[mt][4 * g + 3]};
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (c0 + j < p.dv) orow[c0 + j] = oacc[mt][4 * g + j];
+                }
+            }
+        }
+    }
+}
+
 }  // namespace snhip

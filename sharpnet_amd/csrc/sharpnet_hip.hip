@@ -779,6 +779,12 @@ hipError_t prepare_kernels_once(int dev) {
                                 c.lds_bytes);
         if (e != hipSuccess) return e;
     }
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd_long_kernel<32>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, AttnCfg<8, 32>::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd_long_kernel<64>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, AttnCfg<8, 64>::LDS_BYTES);
+    if (e != hipSuccess) return e;
     e = rnn_prepare_kernels();
     if (e != hipSuccess) return e;
     done[dev] = true;
@@ -918,7 +924,10 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
             e = &c;
             break;
         }
-    if (e == nullptr) return SNHIP_STATUS_NOT_SUPPORTED;
+    // more keys than one block holds: the two-pass kernel that walks the keys in blocks of 256 (head dimensions that
+    // are multiples of 4, up to 64)
+    const bool long_keys = (e == nullptr) && hd <= 64 && d->dk % 4 == 0 && d->dv % 4 == 0;
+    if (e == nullptr && !long_keys) return SNHIP_STATUS_NOT_SUPPORTED;
 
     AttnParams p;
     p.Q = d->Q, p.K = d->K, p.V = d->V, p.O = d->O, p.P = d->weights;
@@ -935,9 +944,20 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
         (!two_level || d->strideO_outer % 4 == 0))
         p.flags |= 1;
     if (d->weights != nullptr && (uintptr_t)d->weights % 16 == 0 && d->Tk % 4 == 0) p.flags |= 2;
+    const int tiles = ceil_div(d->Tq, AT_BQ);
+    if (long_keys) {
+        p.q_tiles = 1;
+        constexpr int lds32 = AttnCfg<8, 32>::LDS_BYTES, lds64 = AttnCfg<8, 64>::LDS_BYTES;
+        if (hd <= 32)
+            hipLaunchKernelGGL(attention_fwd_long_kernel<32>, dim3((unsigned)tiles, (unsigned)d->batch), dim3(256), lds32,
+                               h->stream, p);
+        else
+            hipLaunchKernelGGL(attention_fwd_long_kernel<64>, dim3((unsigned)tiles, (unsigned)d->batch), dim3(256), lds64,
+                               h->stream, p);
+        return hip_to_status(hipGetLastError());
+    }
     // K and V are staged once per workgroup: let one workgroup walk through all query tiles of its matrix unless
     // that would leave compute units without work
-    const int tiles = ceil_div(d->Tq, AT_BQ);
     int groups = 1;
     while (groups < tiles && (long long)d->batch * groups < 2LL * h->num_cu) ++groups;
     p.q_tiles = ceil_div(tiles, groups);

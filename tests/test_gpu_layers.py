@@ -389,6 +389,11 @@ def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrap
     (3, 2, 200, 130, 24, 40, False, True), (3, 2, 129, 65, 33, 7, True, False),     # Tq != Tk, dk != dv, odd sizes
     (1, 4, 1, 5, 3, 2, False, True),
     (2, 2, 128, 128, 128, 128, True, True), (3, 1, 70, 100, 96, 128, False, False),  # head dimension up to 128: 128 keys
+    # more than 256 keys: the two-pass kernel over key blocks (head dimensions that are multiples of 4, up to 64)
+    (2, 2, 512, 512, 64, 64, False, True), (2, 2, 512, 512, 64, 64, True, False),
+    (1, 2, 1024, 1024, 32, 32, True, True), (1, 1, 1024, 1024, 64, 64, False, False),
+    (1, 3, 300, 700, 24, 40, False, False), (1, 2, 700, 300, 64, 16, True, True), (1, 1, 2048, 2048, 64, 64, True, False),
+    (2, 1, 257, 257, 8, 4, True, False),
 ])
 def test_fused_attention_forward(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, causal, packed):
     """snhip_attention_forward (scores, mask, softmax and P.V in one launch) against the oracle's
@@ -427,13 +432,13 @@ def test_fused_attention_forward(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, caus
 
 
 def test_fused_attention_limits(gpu_wrapper):
-    """Beyond 256 keys (128 with a head dimension above 64) or a head dimension of 128 nothing is launched and the
-    caller is told so."""
+    """Beyond 256 keys with a head dimension that is not a multiple of 4 or above 64, beyond 128 keys with a head
+    dimension above 64, or with a head dimension above 128, nothing is launched and the caller is told so."""
     from sharpnet_amd import GPUTensor, attention
     w = gpu_wrapper
-    big = GPUTensor([1, 300, 8], None, w)
-    out = GPUTensor([1, 300, 8], None, w)
-    assert attention.fused_attention_forward(big, big, big, out, None, batch=1, heads=1, tq=300, tkv=300, dk=8, dv=8,
+    big = GPUTensor([1, 300, 6], None, w)
+    out = GPUTensor([1, 300, 6], None, w)
+    assert attention.fused_attention_forward(big, big, big, out, None, batch=1, heads=1, tq=300, tkv=300, dk=6, dv=6,
                                              scale=1.0, is_causal=False, packed=False) is False
     wide = GPUTensor([1, 16, 160], None, w)
     outw = GPUTensor([1, 16, 160], None, w)
@@ -450,7 +455,7 @@ def test_fused_attention_limits(gpu_wrapper):
                              V=long_wide.Pointer, O=outl.Pointer, ldq=80, ldk=80, ldv=80, ldo=80)
     assert w.lib.snhip_attention_forward(w.handle, ctypes.byref(d)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_SUPPORTED
     # the layer mirror falls back to the four-call sequence on its own
-    y = GPUTensor([1, 300, 8], None, w)
+    y = GPUTensor([1, 300, 6], None, w)
     big.SetValue(0.5)
     wts = attention.ScaledDotProductAttentionForwardPropagation(big, big, big, y, True, True, False)
     assert abs(float(wts.ToNumpy()[0, 0, 0]) - 1.0 / 300) < 1e-6 and abs(float(y.ToNumpy()[0, 7, 3]) - 0.5) < 1e-6
