@@ -19,6 +19,7 @@
 // Work items are assigned so that each XCD gets one contiguous range of the (matrix, tile) order: the tiles of a
 // matrix share its operand panels in one L2.
 #pragma once
+#include "bgemm_mfma.hpp"
 #include "sgemm_mfma.hpp"
 
 namespace snhip {
@@ -137,6 +138,139 @@ __global__ void __launch_bounds__(256, stream_occupancy(TN, BK_)) sgemm_stream_k
 
         // The next panel goes into LDS before this tile's results go out: the stores of the write-out are then in
         // flight during the next panel's MFMAs, and nothing waits for them until the panel after that is staged.
+        lds_barrier();  // every wavefront has finished reading the current panel
+        if (has_next) {
+            sa.store_lds(As, ra);
+            sb.store_lds(Bs, rb);
+        }
+        if (last_panel) {
+            store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[0][j][e] = 0.0f;
+        }
+        if (!has_next) break;
+        lds_barrier();
+        cur = nxt;
+        idx = idx_next;
+        kp = kp_next;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same persistent streaming scheme with bf16-input / fp32-accumulate arithmetic (v_mfma_f32_32x32x16_bf16,
+// staging and LDS layout of bgemm_mfma.hpp: tiles kept [row][k] in bf16, rows of the TN column tiles stored
+// tile-major).  TIN = float: operands are fp32 in memory and rounded on their way into LDS; TIN = __bf16: they are
+// stored as bf16.  With eight times the MFMA rate of the fp32 kernel these products are plain streaming: the k
+// panel is 64 wide (one panel for an attention head of 64; 128 for the 64-column tile), one LDS stage, the next work
+// item's loads in flight during the MFMAs and the write-out of the current one.
+// ---------------------------------------------------------------------------------------------------------------
+template <int TN_>
+struct BStreamCfg {
+    static constexpr int TN = TN_;
+    // the 64-column tile takes k panels of 128 (its operands then split evenly over the threads in every layout)
+    static constexpr int BM = 128, BN = 32 * TN, BK = (TN_ == 2) ? 128 : 64, NT = 256;
+    static constexpr int PITCH = BK + 8;  // bf16 elements
+    static constexpr int LDS_BYTES = (BM + BN) * PITCH * 2;
+};
+
+// workgroups per compute unit the register budget is set for: fp32 storage keeps twice the bytes in flight
+constexpr int bstream_occupancy(int bytes_per_element) { return bytes_per_element == 4 ? 2 : 3; }
+
+template <int TN, bool TA, bool TB, typename TIN>
+__global__ void __launch_bounds__(256, bstream_occupancy(sizeof(TIN))) bgemm_stream_kernel(const GemmParams p) {
+    using CFG = BStreamCfg<TN>;
+    constexpr int BM = CFG::BM, BN = CFG::BN, BK = CFG::BK, NT = CFG::NT, PITCH = CFG::PITCH;
+    using StageA = BStage<BM, BK, NT, PITCH, 1, !TA, TIN>;
+    using StageB = BStage<BN, BK, NT, PITCH, TN, TB, TIN>;
+
+    extern __shared__ __attribute__((aligned(16))) float smem_f[];
+    __bf16* const As = reinterpret_cast<__bf16*>(smem_f);  // [BM][PITCH]
+    __bf16* const Bs = As + BM * PITCH;                    // [BN][PITCH]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    constexpr unsigned NXCD = 8;
+    const unsigned ntiles = (unsigned)(p.tiles_m * p.tiles_n);
+    const unsigned total = ntiles * (unsigned)p.nz;
+    const unsigned xcd = blockIdx.x % NXCD, slot = blockIdx.x / NXCD;
+    const unsigned nwg = (gridDim.x - xcd + NXCD - 1) / NXCD;
+    const unsigned q = total / NXCD, r = total % NXCD;
+    const unsigned start = xcd * q + (xcd < r ? xcd : r), cnt = q + (xcd < r ? 1u : 0u);
+    if (slot >= cnt) return;  // uniform over the workgroup
+    const int nkp = (p.K + BK - 1) / BK;
+
+    struct Tile {
+        int z, m0, n0;
+    };
+    auto tile_at = [&](unsigned idx) {
+        const unsigned L = start + idx;
+        Tile t;
+        t.z = (int)(L / ntiles);
+        const int logical = (int)(L - (unsigned)t.z * ntiles);
+        t.m0 = (logical % p.tiles_m) * BM;
+        t.n0 = (logical / p.tiles_m) * BN;
+        return t;
+    };
+
+    StageA sa;
+    StageB sb;
+    f32x4 ra[StageA::NV], rb[StageB::NV];
+    auto fetch = [&](const Tile& t, int kp) {
+        sa.init(reinterpret_cast<const TIN*>(p.A) + (long long)t.z * p.strideA, p.lda, t.m0, kp * BK, tid);
+        sb.init(reinterpret_cast<const TIN*>(p.B) + (long long)t.z * p.strideB, p.ldb, t.n0, kp * BK, tid);
+        const int m_rem = p.M - t.m0, n_rem = p.N - t.n0, k_rem = p.K - kp * BK;
+        if (m_rem >= BM && n_rem >= BN && k_rem >= BK) {
+            sa.load_fast(ra);
+            sb.load_fast(rb);
+        } else {
+            sa.load_safe(ra, m_rem, k_rem);
+            sb.load_safe(rb, n_rem, k_rem);
+        }
+    };
+
+    f32x16 acc[1][TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[0][j][e] = 0.0f;
+
+    // physical row of this lane: the wavefront's 32 rows of A; in tile j of B row 32 j + l32
+    const __bf16* const a_rd = As + (wave * 32 + l32) * PITCH + 8 * lhi;
+    const __bf16* const b_rd = Bs + l32 * PITCH + 8 * lhi;
+
+    unsigned idx = slot;
+    int kp = 0;
+    Tile cur = tile_at(idx);
+    fetch(cur, kp);
+    sa.store_lds(As, ra);
+    sb.store_lds(Bs, rb);
+    lds_barrier();
+    for (;;) {
+        const bool last_panel = (kp + 1 == nkp);
+        const unsigned idx_next = last_panel ? idx + nwg : idx;
+        const int kp_next = last_panel ? 0 : kp + 1;
+        const bool has_next = idx_next < cnt;
+        Tile nxt = cur;
+        if (has_next) {
+            if (last_panel) nxt = tile_at(idx_next);
+            fetch(nxt, kp_next);
+        }
+
+#pragma unroll
+        for (int s = 0; s < BK / 16; ++s) {
+            const bf16x8 fa = *reinterpret_cast<const bf16x8*>(a_rd + 16 * s);
+            bf16x8 fb[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const bf16x8*>(b_rd + (32 * j) * PITCH + 16 * s);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb[j], acc[0][j], 0, 0, 0);
+        }
+
         lds_barrier();  // every wavefront has finished reading the current panel
         if (has_next) {
             sa.store_lds(As, ra);

@@ -80,7 +80,8 @@ struct ConfigEntry {
     int BM, BN, BK, NT, lds_bytes;
     int mfma_per_k2;    // TM*TN: MFMA instructions one wavefront issues per MFMA k step
     int kind;           // 0: fp32 kernel (k step 2, 64 cycles per MFMA), 1: bf16-input kernel (k step 16, 32 cycles),
-                        // 2: K split inside the workgroup, 3: streaming kernel, 4: bf16-input kernel on bf16 storage
+                        // 2: K split inside the workgroup, 3: streaming kernel, 4: bf16-input kernel on bf16 storage,
+                        // 5 / 6: bf16-input streaming kernel on fp32 / bf16 storage
     KernelFn fn[2][2];  // [transposeA][transposeB]
     KernelFn fn_ext[2][2];  // the same with the extended write-out (addend, ReLU, two-level batch, column sum);
                             // nullptr if not built
@@ -205,11 +206,35 @@ const ConfigEntry kConfigs[] = {
                 {{sgemm_ksplit_kernel<false, false, 1, 8>, sgemm_ksplit_kernel<false, true, 1, 8>},
                  {sgemm_ksplit_kernel<true, false, 1, 8>, sgemm_ksplit_kernel<true, true, 1, 8>}},
                 1, 0.5, 0.5, 1.0},  // 21: 32 x 32, eight K slices
+    // persistent streaming kernels in bf16-input arithmetic (sgemm_stream.hpp), fp32 storage (kind 5) ...
+    ConfigEntry{128, 128, 64, 256, BStreamCfg<4>::LDS_BYTES, 4, 5,
+                {{bgemm_stream_kernel<4, false, false, float>, bgemm_stream_kernel<4, false, true, float>},
+                 {bgemm_stream_kernel<4, true, false, float>, bgemm_stream_kernel<4, true, true, float>}},
+                {{nullptr, nullptr}, {nullptr, nullptr}},
+                2, 0.8, 0.9, 1.1},  // 22: 128 x 128, k panels of 64
+    ConfigEntry{128, 64, 128, 256, BStreamCfg<2>::LDS_BYTES, 2, 5,
+                {{bgemm_stream_kernel<2, false, false, float>, bgemm_stream_kernel<2, false, true, float>},
+                 {bgemm_stream_kernel<2, true, false, float>, bgemm_stream_kernel<2, true, true, float>}},
+                {{nullptr, nullptr}, {nullptr, nullptr}},
+                2, 0.7, 0.85, 1.1},  // 23: 128 x 64, k panels of 128
+    // ... and bf16 storage (kind 6)
+    ConfigEntry{128, 128, 64, 256, BStreamCfg<4>::LDS_BYTES, 4, 6,
+                {{bgemm_stream_kernel<4, false, false, __bf16>, bgemm_stream_kernel<4, false, true, __bf16>},
+                 {bgemm_stream_kernel<4, true, false, __bf16>, bgemm_stream_kernel<4, true, true, __bf16>}},
+                {{nullptr, nullptr}, {nullptr, nullptr}},
+                3, 0.8, 0.9, 1.1},  // 24: 128 x 128, k panels of 64
+    ConfigEntry{128, 64, 128, 256, BStreamCfg<2>::LDS_BYTES, 2, 6,
+                {{bgemm_stream_kernel<2, false, false, __bf16>, bgemm_stream_kernel<2, false, true, __bf16>},
+                 {bgemm_stream_kernel<2, true, false, __bf16>, bgemm_stream_kernel<2, true, true, __bf16>}},
+                {{nullptr, nullptr}, {nullptr, nullptr}},
+                3, 0.7, 0.85, 1.1},  // 25: 128 x 64, k panels of 128
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 constexpr int kKsplitConfig = 14;   // and kKsplitConfig + 1
 constexpr int kStreamConfig = 16;   // and kStreamConfig + 1
 constexpr int kKsplit8Config = 21;
+constexpr int kBStreamConfig = 22;        // bf16-input streaming, fp32 storage: 22, 23
+constexpr int kBStreamStoredConfig = 24;  // ... bf16 storage: 24, 25
 
 // Fused attention forward kernels (attention_mfma.hpp)
 struct AttnEntry {
@@ -471,13 +496,15 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
 // strided batches of small matrices whose K fits a few 64-wide panels, where the tiled kernels' pipeline never
 // fills and every workgroup is prologue and write-out.
 int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, bool wants_ext) {
-    if (math != SNHIP_MATH_FP32 || two_level || wants_ext) return -1;
-    const bool forced = h->force_cfg == kStreamConfig || h->force_cfg == kStreamConfig + 1;
+    if (two_level || wants_ext) return -1;
+    const int first = math == SNHIP_MATH_FP32 ? kStreamConfig
+                                              : (math == SNHIP_MATH_BF16_INPUT ? kBStreamConfig : kBStreamStoredConfig);
+    const bool forced = h->force_cfg == first || h->force_cfg == first + 1;
     if (h->force_cfg >= 0 && !forced) return -1;
     if (h->force_splitk > 1) return -1;
     if (forced) return h->force_cfg;
     if (g.batch < 8 || g.K > 256 || g.M < 64) return -1;
-    const int cfg = g.N <= 64 ? kStreamConfig + 1 : kStreamConfig;
+    const int cfg = g.N <= 64 ? first + 1 : first;
     const long long tiles = (long long)ceil_div(g.M, 128) * ceil_div(g.N, kConfigs[cfg].BN) * g.batch;
     if (tiles < 2LL * h->num_cu) return -1;
     // mostly-empty tiles waste the streaming they are meant to save
@@ -697,7 +724,7 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     const KernelFn fn = use_ext ? fn_ext : cfg.fn[g.tA ? 1 : 0][g.tB ? 1 : 0];
     if (cfg.kind == 2) {  // the K-split kernel reads tile and matrix from a two-dimensional grid
         hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)batch), dim3(cfg.NT), cfg.lds_bytes, h->stream, p);
-    } else if (cfg.kind == 3) {
+    } else if (cfg.kind == 3 || cfg.kind == 5 || cfg.kind == 6) {
         // persistent workgroups: as many as fit on the chip at once, the same number on every XCD
         long long wgs = (long long)cfg.occ * h->num_cu;
         if (wgs > ntiles * p.nz) wgs = ntiles * p.nz;

@@ -270,3 +270,77 @@ def test_bf16_stored_batched_bias_and_refusals(oracle, gpu_wrapper):
     assert lib.snhip_dot_bf16_stored(h, pp + 2, 8, 8, 0, pk, 8, 8, 0, go.Pointer, 1.0, 0.0, None) == \
         CublasStatus.CUBLAS_STATUS_NOT_SUPPORTED
     assert np.isnan(go.ToNumpy()).all()
+
+
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_bf16_streaming_kernels_strided_batches(oracle, gpu_wrapper, tA, tB):
+    """The persistent streaming kernels in bf16-input arithmetic, fp32 storage and bf16 storage: more tiles than
+    workgroups, ragged M / N, K below, at and above one panel, alpha / beta; forced through the tuning hook, and picked
+    automatically for the attention-shaped products.  Bar: the fp32 bound against the oracle on bf16-rounded inputs."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    lib, h = w.lib, w.handle
+    kinds = {c["kind"]: [] for c in w.configs()}
+    for c in w.configs():
+        kinds[c["kind"]].append(c["id"])
+    assert len(kinds["bf16-stream"]) == 2 and len(kinds["bf16-stored-stream"]) == 2
+    rng = np.random.default_rng(700 + 2 * tA + tB)
+
+    def run(stored, pa, pb, a, b, gc, alpha, beta):
+        batch = a.shape[0]
+        aH, aW, bH, bW = a.shape[1], a.shape[2], b.shape[1], b.shape[2]
+        M, N = gc.Shape[1], gc.Shape[2]
+        if stored:
+            check_status(lib.snhip_bmm_bf16_stored(h, pa, aH, aW, int(tA), aH * aW, pb, bH, bW, int(tB), bH * bW, gc.Pointer,
+                                                   M * N, batch, alpha, beta, None))
+        else:
+            check_status(lib.snhip_bmm_bf16(h, pa, aH, aW, int(tA), aH * aW, pb, bH, bW, int(tB), bH * bW, gc.Pointer, M * N,
+                                            batch, alpha, beta))
+    try:
+        for (batch, M, N, K) in [(600, 128, 128, 64), (40, 256, 256, 64), (40, 256, 64, 256), (9, 200, 100, 72),
+                                 (5, 130, 258, 130), (3, 64, 40, 8), (1, 300, 200, 136), (1100, 100, 60, 36)]:
+            a = random_tensor(rng, (batch, K, M) if tA else (batch, M, K), -1, 1)
+            b = random_tensor(rng, (batch, N, K) if tB else (batch, K, N), -1, 1)
+            c = random_tensor(rng, (batch, M, N), -1, 1)
+            ar, br = oracle.round_to_bf16(a), oracle.round_to_bf16(b)
+            ga, gb = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w)
+            pa, pb = to_bf16_on_device(w, ga), to_bf16_on_device(w, gb)
+            for stored, kind in ((False, "bf16-stream"), (True, "bf16-stored-stream")):
+                for cfg in kinds[kind]:
+                    w.set_tuning(cfg, 1)
+                    for alpha, beta in [(0.125, 0.0), (-0.5, 1.0)]:
+                        gc = GPUTensor(c.shape, c, w)
+                        if beta == 0.0:
+                            gc.SetValue(float("nan"))
+                        run(stored, pa if stored else ga.Pointer, pb if stored else gb.Pointer, a, b, gc, alpha, beta)
+                        assert w.last_tuning() == (cfg, 1), (batch, M, N, K, kind)
+                        got = gc.ToNumpy()
+                        gc.Dispose()
+                        ref = oracle.bmm(ar, tA, br, tB, alpha, beta, c if beta != 0 else None)
+                        bound = 1e-4 * np.sqrt(K) * abs(alpha) + (1e-6 * abs(beta) if beta else 0.0)
+                        assert np.all(np.isfinite(got)), (batch, M, N, K, cfg, alpha, beta)
+                        assert np.max(np.abs(got - ref)) <= bound, (batch, M, N, K, cfg, alpha, beta)
+            w.release(pa, max(2 * ga.Count, 8))
+            w.release(pb, max(2 * gb.Count, 8))
+            ga.Dispose()
+            gb.Dispose()
+        w.set_tuning(-1, 0)
+        # automatic choice for the two attention products of benchmark configuration 5 (fewer matrices, same shape)
+        for (batch, M, N, K, which) in [(256, 256, 256, 64, 0), (256, 256, 64, 256, 1)]:
+            a = random_tensor(rng, (batch, K, M) if tA else (batch, M, K), -1, 1)
+            b = random_tensor(rng, (batch, N, K) if tB else (batch, K, N), -1, 1)
+            ga, gb, gc = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w), GPUTensor([batch, M, N], None, w)
+            pa, pb = to_bf16_on_device(w, ga), to_bf16_on_device(w, gb)
+            ref = oracle.bmm(oracle.round_to_bf16(a), tA, oracle.round_to_bf16(b), tB, 1.0)
+            for stored, kind in ((False, "bf16-stream"), (True, "bf16-stored-stream")):
+                gc.SetValue(float("nan"))
+                run(stored, pa if stored else ga.Pointer, pb if stored else gb.Pointer, a, b, gc, 1.0, 0.0)
+                assert w.last_tuning() == (kinds[kind][which], 1)
+                assert np.max(np.abs(gc.ToNumpy() - ref)) <= 1e-4 * np.sqrt(K)
+            w.release(pa, max(2 * ga.Count, 8))
+            w.release(pb, max(2 * gb.Count, 8))
+            for t in (ga, gb, gc):
+                t.Dispose()
+    finally:
+        w.set_tuning(-1, 0)
