@@ -107,6 +107,50 @@ def main():
             gbias.Dispose()
         return wall_ms, ev_ms, gc
 
+    def run_stored(gm, seed, steps, warmup):
+        from sharpnet_amd.hiplib import check_status
+        aa, bb, _ = wl.uniform_operands(gm, seed)
+        ga, gb = upload(aa), upload(bb)
+        gcs = GPUTensor(gm.c_shape, None, w)
+        pa, pb = w.allocate(2 * ga.Count), w.allocate(2 * gb.Count)
+
+        def convert():
+            check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, ga.Pointer, pa, ga.Count))
+            check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, gb.Pointer, pb, gb.Count))
+        aH, aW = aa.shape[-2:]
+        bH, bW = bb.shape[-2:]
+
+        def launch():
+            check_status(w.lib.snhip_bmm_bf16_stored(w.handle, pa, aH, aW, int(gm.tA), aH * aW, pb, bH, bW, int(gm.tB),
+                                                     bH * bW, gcs.Pointer, gm.M * gm.N, gm.batch, gm.alpha, gm.beta,
+                                                     None))
+
+        def timed(fn, n, nw):
+            for _ in range(nw):
+                fn()
+            e0, e1 = w.new_event(), w.new_event()
+            w.synchronize()
+            w.record(e0)
+            for _ in range(n):
+                fn()
+            w.record(e1)
+            ms = w.elapsed_ms(e0, e1) / n
+            w.destroy_event(e0)
+            w.destroy_event(e1)
+            return ms
+        conv_ms = timed(convert, 5, 2)
+        ms = timed(launch, steps, warmup)
+        by = gm.batch * (2.0 * (gm.M * gm.K + gm.K * gm.N) + 4.0 * gm.M * gm.N)
+        roof_s = max(gm.flops / (wl.BF16_MFMA_PEAK_TFLOPS * 1e12), by / (wl.HBM_PEAK_GBS * 1e9))
+        r = {"gemm": gm.label() + " (bf16 storage)", "ms": round(ms, 4), "tflops": round(gm.flops / (ms * 1e-3) / 1e12, 2),
+             "frac_of_roofline": round(roof_s * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
+             "splitk": w.last_tuning()[1], "algorithmic_bytes": by, "convert_both_operands_ms": round(conv_ms, 4)}
+        w.release(pa, 2 * ga.Count)
+        w.release(pb, 2 * gb.Count)
+        for t in (ga, gb, gcs):
+            t.Dispose()
+        return r
+
     if args.attention_probe:
         from sharpnet_amd import attention
         rng = np.random.default_rng(5)
@@ -117,6 +161,17 @@ def main():
             for _ in range(20):
                 attention.fused_attention_forward(q, k, v, o, keep, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
                                                   scale=0.125, is_causal=False, packed=False)
+            w.synchronize()
+        for t in (q, k, v, o, wts):
+            t.Dispose()
+        # more than 256 keys: the two-pass kernel over key blocks (64 sequences of 1024 positions, weights kept, then causal)
+        Z, Tn = 64, 1024
+        q, k, v = (GPUTensor([Z, Tn, d], rng.uniform(-1, 1, (Z, Tn, d)).astype(np.float32), w) for _ in range(3))
+        o, wts = GPUTensor([Z, Tn, d], None, w), GPUTensor([Z, Tn, Tn], None, w)
+        for causal in (False, True):
+            for _ in range(20):
+                attention.fused_attention_forward(q, k, v, o, wts, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
+                                                  scale=0.125, is_causal=causal, packed=False)
             w.synchronize()
         return
     if args.rnn_probe:
@@ -145,6 +200,10 @@ def main():
         shapes += [("attention " + gm.name, gm, 0) for gm in wl.attention_gemms()]
         shapes += [("bf16-input 8192^3 TN", wl.Gemm(8192, 8192, 8192, True, False), 1),
                    ("bf16-input 4096^3 NN", wl.Gemm(4096, 4096, 4096), 1)]
+        shapes += [("bf16-input attention " + gm.name, gm, 1) for gm in wl.attention_gemms()]
+        shapes += [("square %d^3 NN" % n, wl.Gemm(n, n, n), 0) for n in (1024, 2048, 4096)]
+        shapes += [("ragged 1000^3 NN", wl.Gemm(1000, 1000, 1000), 0),
+                   ("ragged 4097x3001x2049 NN", wl.Gemm(4097, 3001, 2049), 0)]
         for name, gm, math_mode in shapes:
             w.set_math_mode(math_mode)
             aa, bb, cc = wl.uniform_operands(gm, 2)
@@ -154,6 +213,13 @@ def main():
                               "flops": gm.flops, "bytes": gm.bytes, "event_ms": round(ms, 5),
                               "tile_config": w.last_tuning()[0], "splitk": w.last_tuning()[1]}), flush=True)
         w.set_math_mode(0)
+        # operands stored as bf16 (converted once, outside the 30 launches of each product)
+        stored = [wl.Gemm(8192, 8192, 8192, tA, tB, 1.0, 0.0) for (tA, tB) in ((False, True), (False, False), (True, False))]
+        for gm in stored + list(wl.attention_gemms()):
+            r = run_stored(gm, 2, 20, 10)
+            print(json.dumps({"shape": "bf16-stored " + gm.label(), "M": gm.M, "N": gm.N, "K": gm.K, "batch": gm.batch,
+                              "launches": 30, "flops": gm.flops, "bytes": r["algorithmic_bytes"], "event_ms": r["ms"],
+                              "tile_config": r["tile_config"], "splitk": r["splitk"]}), flush=True)
         return
     if args.probe:
         # known-size launch: copy_f32_kernel reads 2**30 bytes and writes 2**30 bytes
@@ -420,49 +486,6 @@ def main():
 
         # The same arithmetic on operands STORED as bf16 (2 bytes per element in HBM; algorithmic bytes use s_in = 2).
         # Operands are converted once by the library's own pass (timed separately: it is not part of the product).
-        def run_stored(gm, seed, steps, warmup):
-            from sharpnet_amd.hiplib import check_status
-            aa, bb, _ = wl.uniform_operands(gm, seed)
-            ga, gb = upload(aa), upload(bb)
-            gcs = GPUTensor(gm.c_shape, None, w)
-            pa, pb = w.allocate(2 * ga.Count), w.allocate(2 * gb.Count)
-
-            def convert():
-                check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, ga.Pointer, pa, ga.Count))
-                check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, gb.Pointer, pb, gb.Count))
-            aH, aW = aa.shape[-2:]
-            bH, bW = bb.shape[-2:]
-
-            def launch():
-                check_status(w.lib.snhip_bmm_bf16_stored(w.handle, pa, aH, aW, int(gm.tA), aH * aW, pb, bH, bW, int(gm.tB),
-                                                         bH * bW, gcs.Pointer, gm.M * gm.N, gm.batch, gm.alpha, gm.beta,
-                                                         None))
-
-            def timed(fn, n, nw):
-                for _ in range(nw):
-                    fn()
-                e0, e1 = w.new_event(), w.new_event()
-                w.synchronize()
-                w.record(e0)
-                for _ in range(n):
-                    fn()
-                w.record(e1)
-                ms = w.elapsed_ms(e0, e1) / n
-                w.destroy_event(e0)
-                w.destroy_event(e1)
-                return ms
-            conv_ms = timed(convert, 5, 2)
-            ms = timed(launch, steps, warmup)
-            by = gm.batch * (2.0 * (gm.M * gm.K + gm.K * gm.N) + 4.0 * gm.M * gm.N)
-            roof_s = max(gm.flops / (wl.BF16_MFMA_PEAK_TFLOPS * 1e12), by / (wl.HBM_PEAK_GBS * 1e9))
-            r = {"gemm": gm.label() + " (bf16 storage)", "ms": round(ms, 4), "tflops": round(gm.flops / (ms * 1e-3) / 1e12, 2),
-                 "frac_of_roofline": round(roof_s * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
-                 "splitk": w.last_tuning()[1], "algorithmic_bytes": by, "convert_both_operands_ms": round(conv_ms, 4)}
-            w.release(pa, 2 * ga.Count)
-            w.release(pb, 2 * gb.Count)
-            for t in (ga, gb, gcs):
-                t.Dispose()
-            return r
         extra["config2_8192_bf16_stored"] = [run_stored(wl.Gemm(8192, 8192, 8192, tA, tB, 1.0, 0.0), 2, 10, 5)
                                             for (tA, tB) in ((False, True), (False, False), (True, False))]
         extra["config5_attention_bf16_stored"] = {"gemms": [run_stored(gm, 5, 50, 10) for gm in att_g],

@@ -447,7 +447,8 @@ int snhip_config_count(void);
  * with 32 x 32 tiles and K split over the wavefronts of a workgroup: chosen by itself for products with few output
  * tiles, never part of a split-K launch, used only when the operands can be read in 16-byte pieces; 3 fp32 kernel
  * with persistent workgroups and 32-wide k panels: chosen by itself for strided batches of small matrices with a
- * short K, never part of a split-K launch) */
+ * short K, never part of a split-K launch; 4 tiled kernel for operands stored as bf16 (SNHIP_MATH_BF16_STORED);
+ * 5 / 6 the persistent kernel of kind 3 with bf16 arithmetic on fp32-stored / bf16-stored operands) */
 int snhip_config_desc(int config, int desc[6]);
 
 #ifdef __cplusplus

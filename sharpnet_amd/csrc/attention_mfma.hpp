@@ -450,15 +450,16 @@ __global__ void __launch_bounds__(256) attention_fwd_long_kernel(const AttnParam
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
-    const int z = blockIdx.y;
+    const int z = blockIdx.x;  // matrices run fastest in the grid, query tiles slowest (see q0)
     const BatchIndex bi = split_batch(z, p.batch_inner);
     const float* Qz = p.Q + batch_offset(bi, p.sQ, p.sQ2);
     const float* Kz = p.K + batch_offset(bi, p.sK, p.sK2);
     const float* Vz = p.V + batch_offset(bi, p.sV, p.sV2);
     float* Oz = p.O + batch_offset(bi, p.sO, p.sO2);
 
-    // last query tile first: with the causal mask the late tiles see the most key blocks, so they start first
-    const int q0 = (int)(gridDim.x - 1 - blockIdx.x) * AT_BQ;
+    // last query tile first, for all matrices, then the tile before it, ...: with the causal mask the late tiles see
+    // the most key blocks, and started first they leave the short ones to fill the end of the launch
+    const int q0 = (int)(gridDim.y - 1 - blockIdx.y) * AT_BQ;
     const int row = q0 + wave * 32 + l32;
     const bool row_ok = row < p.Tq;
 
@@ -661,13 +662,15 @@ __global__ void __launch_bounds__(256) attention_fwd_long_kernel(const AttnParam
     }
 
     // causal: the blocks that were skipped hold zeros in the stored probabilities
-    if (pbase != nullptr && row_ok) {
-        for (int kb = nb_needed; kb < nblocks; ++kb) {
-            float* prow = pbase + kb * AT_TK;
-            for (int c = 4 * lhi; c < AT_TK; c += 8) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (kb * AT_TK + c + j < p.Tk) prow[c + j] = 0.0f;
+    // (a wavefront clears whole rows, lanes along the keys: consecutive 16-byte stores, full lines)
+    if (p.P != nullptr && nb_needed < nblocks) {  // uniform
+        const int first = nb_needed * AT_TK, ncol = p.Tk - first;
+        for (int r = wave; r < AT_BQ && q0 + r < p.Tq; r += 4) {
+            float* prow = p.P + ((long long)z * p.Tq + q0 + r) * p.Tk + first;
+            if (p.flags & 2) {  // rows are 16-byte aligned and Tk is a multiple of 4
+                for (int c = 4 * lane; c < ncol; c += 256) *reinterpret_cast<f32x4*>(prow + c) = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            } else {
+                for (int c = lane; c < ncol; c += 64) prow[c] = 0.0f;
             }
         }
     }

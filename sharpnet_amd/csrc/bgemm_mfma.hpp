@@ -393,8 +393,12 @@ __global__ void __launch_bounds__(CFG::NT) bgemm_mfma_kernel(const GemmParams p)
         k_tile(P1{}, std::false_type{});
     }
 
-    store_accumulators_plain<TM, TN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch,
-                                     tile_m * p.tiles_n + tile_n);
+    // Reading the full-size accumulator set through pinned accumulation registers (see acc_value) pays with
+    // bf16 storage only: with fp32 storage the k loop needs every ordinary register, and the allocation the
+    // pinned write-out leads to puts spill reloads inside that loop (8192^3: 725 against 924 TFLOP/s).
+    constexpr bool PIN = (TM * TN >= 16) && (sizeof(TIN) == 2);
+    store_accumulators_plain<TM, TN, PIN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, zb, batch,
+                                          tile_m * p.tiles_n + tile_n);
 }
 
 }  // namespace snhip

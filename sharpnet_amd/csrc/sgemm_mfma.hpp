@@ -396,6 +396,22 @@ __device__ __forceinline__ void store_row_vec(float* p, const float (&v)[TN]) {
     }
 }
 
+// One accumulator element, read where it is used.  The operand constraint keeps the element in an accumulation
+// register up to this point.  Without it the register allocator, which may hold these values in either half of the
+// register file, moves most of a full-size accumulator set (256 values) into ordinary registers right behind the
+// k loop and then spills to memory in the write-out.
+// Only for the full-size set (PIN): smaller ones live wherever the allocator likes and need no help.
+template <bool PIN>
+__device__ __forceinline__ float acc_value(float x) {
+    if constexpr (PIN) {
+        float y;
+        asm("v_accvgpr_read_b32 %0, %1" : "=v"(y) : "a"(x));
+        return y;
+    } else {
+        return x;
+    }
+}
+
 // Write-out of a wavefront whose whole 32*TM x 32*TN patch lies inside the matrix and may be accessed in vectors
 // of TN floats:   C = act(alpha * acc + bias + beta * C + gamma * D).
 // There are no per-lane tests and no loads under conditions here, so the stores go out back to back.  (In the
@@ -405,7 +421,7 @@ __device__ __forceinline__ void store_row_vec(float* p, const float (&v)[TN]) {
 // are requested before chunk k is stored, so a load never waits behind the stores issued just before it (the
 // compiler may not move loads across stores itself: for all it knows the rows alias).
 // c0 / d0 point at the lane's first row (row_base + 4 * TM * lhi) and first column; d0 == nullptr: no addend.
-template <int TM, int TN, bool EXT>
+template <int TM, int TN, bool EXT, bool PIN = (TM * TN >= 16)>
 __device__ __forceinline__ void store_patch_fast(const f32x16 (&acc)[TM][TN], float* c0, long long ldo, const float* d0,
                                                  long long ldd, float alpha, float beta, float gamma,
                                                  const float (&bv)[TN], int act, float act_param) {
@@ -420,7 +436,7 @@ __device__ __forceinline__ void store_patch_fast(const f32x16 (&acc)[TM][TN], fl
         float v[TN];
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            v[j] = alpha * acc[i][j][r] + bv[j];
+            v[j] = alpha * acc_value<PIN>(acc[i][j][r]) + bv[j];
             if (use_c) v[j] += beta * cv[j];
             if constexpr (EXT) {
                 if (use_d) v[j] += gamma * dv[j];
@@ -432,9 +448,13 @@ __device__ __forceinline__ void store_patch_fast(const f32x16 (&acc)[TM][TN], fl
     if (!use_c && !use_d) {
         const float zero[TN] = {};
 #pragma unroll
-        for (int k = 0; k < CHUNKS; ++k)
+        for (int k = 0; k < CHUNKS; ++k) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) finish(k, e, zero, zero);
+            // keep the arithmetic of one chunk next to its stores: left alone, the scheduler computes all
+            // 16 * TM * TN results first, which needs more registers than there are
+            __builtin_amdgcn_sched_barrier(0);
+        }
         return;
     }
     float cbuf[2][4][TN] = {}, dbuf[2][4][TN] = {};
@@ -453,6 +473,7 @@ __device__ __forceinline__ void store_patch_fast(const f32x16 (&acc)[TM][TN], fl
         if (k + 1 < CHUNKS) request(k + 1);
 #pragma unroll
         for (int e = 0; e < 4; ++e) finish(k, e, cbuf[k & 1][e], dbuf[k & 1][e]);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -473,7 +494,7 @@ __device__ __forceinline__ void store_patch_fast(const f32x16 (&acc)[TM][TN], fl
 // uses, and the extended one (also gamma * D, (leaky) ReLU, two-level batch) compiled only into the kernels
 // instantiated with EXT, so that the extra tests and registers cost the plain product nothing.
 // ---------------------------------------------------------------------------
-template <int TM, int TN>
+template <int TM, int TN, bool PIN = (TM * TN >= 16)>
 __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM][TN], const GemmParams& p, int row_base,
                                                    int col0, int lhi, int zb, int batch, int tile_index) {
     const bool to_ws = (p.splitk > 1);
@@ -507,7 +528,7 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
 #pragma unroll
         for (int j = 0; j < TN; ++j) bv[j] = 0.0f;
         if (bias != nullptr) load_row_vec<TN>(bias + col0, bv);
-        store_patch_fast<TM, TN, false>(acc, out + (long long)(row_base + TM * 4 * lhi) * ldo + col0, ldo, nullptr, 0, alpha,
+        store_patch_fast<TM, TN, false, PIN>(acc, out + (long long)(row_base + TM * 4 * lhi) * ldo + col0, ldo, nullptr, 0, alpha,
                                         beta, 0.0f, bv, ACT_NONE, 0.0f);
     } else {
         float bv[TN];
@@ -527,7 +548,7 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
                 float* crow = out + (long long)row * ldo + col0;
                 float v[TN];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r] + bv[j];
+                for (int j = 0; j < TN; ++j) v[j] = alpha * acc_value<PIN>(acc[i][j][r]) + bv[j];
                 if (vec_ok) {
                     if (beta != 0.0f) {
                         float c[TN];
@@ -728,7 +749,7 @@ __device__ __forceinline__ void store_accumulators_ext(const f32x16 (&acc)[TM][T
                 if (row >= p.M) continue;
                 float v[TN];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) v[j] = alpha * acc[i][j][r];
+                for (int j = 0; j < TN; ++j) v[j] = alpha * acc_value<(TM * TN >= 16)>(acc[i][j][r]);
                 const float* drow = nullptr;
                 if (has_d) drow = dsrc + (long long)row * ldd + col0;
                 finish_row<TN>(v, out + (long long)row * ldo + col0, drow, has_d, bv, beta, gamma, act, p.ep.act_param,
@@ -906,10 +927,21 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     // far this thread's vectors of an m/n-contiguous operand arrive shifted; zero when the extent is a multiple of 4
     // (then a vector is either wholly inside or wholly outside, and what lies outside may hold anything).
     // sh_a / sh_b [stage]: the shift of what the register stage currently holds (0: as loaded).
-    const typename StageA::Edge ea = sa.edge_info(m_rem, m0);
-    const typename StageB::Edge eb = sb.edge_info(n_rem, n0);
-    const bool edge_ok = ea.usable && eb.usable;  // uniform over the workgroup
-    const bool any_rot_a = (p.M % 4 != 0), any_rot_b = (p.N % 4 != 0);
+    //
+    // Interior blocks and edge blocks run two disjoint copies of everything from here to the end of the k loop
+    // (run<true> / run<false>): the edge facts then do not exist on the interior path at all.  With one copy they were
+    // live across the interior loop (the edge loops are reachable from it as far as the compiler can tell), and in the
+    // configurations that use all 512 registers they were spilled around it, in every block.
+    auto run = [&](auto interior_tag) {
+    constexpr bool INTERIOR = decltype(interior_tag)::value;
+    typename StageA::Edge ea = {};
+    typename StageB::Edge eb = {};
+    if constexpr (!INTERIOR) {
+        ea = sa.edge_info(m_rem, m0);
+        eb = sb.edge_info(n_rem, n0);
+    }
+    const bool edge_ok = !INTERIOR && ea.usable && eb.usable;  // uniform over the workgroup
+    const bool any_rot_a = !INTERIOR && (p.M % 4 != 0), any_rot_b = !INTERIOR && (p.N % 4 != 0);
     const int rot_a = any_rot_a ? ea.shift : 0, rot_b = any_rot_b ? eb.shift : 0;
     int sh_a[2] = {0, 0}, sh_b[2] = {0, 0};
 
@@ -921,7 +953,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             const int k_rem = klen - fetch * BK;
             sh_a[st] = 0;
             sh_b[st] = 0;
-            if (full_mn && fetch < nk_full) {
+            if (INTERIOR && fetch < nk_full) {
                 sa.load_fast(ra[st]);
                 sb.load_fast(rb[st]);
             } else if (edge_ok && fetch < nk_full) {
@@ -941,11 +973,21 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             if (t == 0) {
 #pragma unroll
                 for (int v = 0; v < StageA::NV; ++v) {
-                    const f32x4 stored = sa.store_lds_vec_shifted(As, ra[0][v], v, sh_a[0], any_rot_a);
-                    if constexpr (COLSUM) cs += stored;
+                    if constexpr (INTERIOR) {
+                        sa.store_lds_vec(As, ra[0][v], v);
+                        if constexpr (COLSUM) cs += ra[0][v];
+                    } else {
+                        const f32x4 stored = sa.store_lds_vec_shifted(As, ra[0][v], v, sh_a[0], any_rot_a);
+                        if constexpr (COLSUM) cs += stored;
+                    }
                 }
 #pragma unroll
-                for (int v = 0; v < StageB::NV; ++v) sb.store_lds_vec_shifted(Bs, rb[0][v], v, sh_b[0], any_rot_b);
+                for (int v = 0; v < StageB::NV; ++v) {
+                    if constexpr (INTERIOR)
+                        sb.store_lds_vec(Bs, rb[0][v], v);
+                    else
+                        sb.store_lds_vec_shifted(Bs, rb[0][v], v, sh_b[0], any_rot_b);
+                }
             }
         }
         lds_barrier();
@@ -1075,29 +1117,33 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     using P1 = std::integral_constant<int, 1>;
     int kt = 0;
     // branch-free pairs of tiles while both fetches (tiles kt+3, kt+4) are full k tiles
-    if (full_mn) {
+    // then the last few tiles (K tail included): same body, each fetch chooses checked or unchecked loads
+    if constexpr (INTERIOR) {
         for (; kt + 4 < nk_full; kt += 2) {
             k_tile(P0{}, std::integral_constant<int, 0>{}, ea, eb);
             k_tile(P1{}, std::integral_constant<int, 0>{}, ea, eb);
         }
-    } else if (edge_ok) {
-        for (; kt + 4 < nk_full; kt += 2) {
-            k_tile(P0{}, std::integral_constant<int, 1>{}, ea, eb);
-            k_tile(P1{}, std::integral_constant<int, 1>{}, ea, eb);
-        }
-    }
-    // the last few tiles (K tail included): same body, each fetch chooses checked or unchecked loads
-    if (full_mn) {
         for (; kt < nk; kt += 2) {
             k_tile(P0{}, std::integral_constant<int, 2>{}, ea, eb);
             k_tile(P1{}, std::integral_constant<int, 2>{}, ea, eb);
         }
     } else {
+        if (edge_ok) {
+            for (; kt + 4 < nk_full; kt += 2) {
+                k_tile(P0{}, std::integral_constant<int, 1>{}, ea, eb);
+                k_tile(P1{}, std::integral_constant<int, 1>{}, ea, eb);
+            }
+        }
         for (; kt < nk; kt += 2) {
             k_tile(P0{}, std::integral_constant<int, 3>{}, ea, eb);
             k_tile(P1{}, std::integral_constant<int, 3>{}, ea, eb);
         }
     }
+    };  // run
+    if (full_mn)
+        run(std::true_type{});
+    else
+        run(std::false_type{});
 
     if constexpr (COLSUM) {
         if (p.colsum != nullptr && tile_n == 0) {  // uniform over the workgroup

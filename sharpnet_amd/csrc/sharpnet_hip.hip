@@ -338,6 +338,19 @@ Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
     Choice best{kind == 0 ? 6 : (kind == 1 ? 13 : 20), 1};
     double best_cost = 1e300;
     const bool forced = h->force_cfg >= 0 && kConfigs[h->force_cfg].kind == kind;
+    // A tall operand against a narrow one (N <= 64) with a long K streams op(A) from memory once: measured on
+    // 8192 x 64 x 8192, all transposes, 128 x 64 tiles with 32-wide k panels (whole 128-byte lines of a k-contiguous
+    // operand per row and tile) and one workgroup per compute unit (split 4) take 78-85 us, against 84-92 us for what the
+    // cost model picks (16-wide panels, split 8).
+    if (kind == 0 && !forced && h->force_splitk <= 0 && batch == 1 && N <= 64 && K >= 2048 &&
+        (long long)M * K >= (1LL << 24)) {
+        const ConfigEntry& e = kConfigs[8];
+        const long long tiles = (long long)ceil_div(M, e.BM) * ceil_div(N, e.BN);
+        int s = 1;
+        while (tiles * s < h->num_cu && s < 32 && K / (2 * s) >= 8 * e.BK) s *= 2;
+        const int kchunk = ceil_div(ceil_div(K, s), e.BK) * e.BK;
+        if ((long long)kchunk * (s - 1) < K && (size_t)M * N * s * sizeof(float) <= kMaxWorkspaceBytes) return Choice{8, s};
+    }
     for (int c = 0; c < kNumConfigs; ++c) {
         const ConfigEntry& e = kConfigs[c];
         if (e.kind != kind) continue;
@@ -973,13 +986,14 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
     if (d->weights != nullptr && (uintptr_t)d->weights % 16 == 0 && d->Tk % 4 == 0) p.flags |= 2;
     const int tiles = ceil_div(d->Tq, AT_BQ);
     if (long_keys) {
+        if (tiles > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
         p.q_tiles = 1;
         constexpr int lds32 = AttnCfg<8, 32>::LDS_BYTES, lds64 = AttnCfg<8, 64>::LDS_BYTES;
         if (hd <= 32)
-            hipLaunchKernelGGL(attention_fwd_long_kernel<32>, dim3((unsigned)tiles, (unsigned)d->batch), dim3(256), lds32,
+            hipLaunchKernelGGL(attention_fwd_long_kernel<32>, dim3((unsigned)d->batch, (unsigned)tiles), dim3(256), lds32,
                                h->stream, p);
         else
-            hipLaunchKernelGGL(attention_fwd_long_kernel<64>, dim3((unsigned)tiles, (unsigned)d->batch), dim3(256), lds64,
+            hipLaunchKernelGGL(attention_fwd_long_kernel<64>, dim3((unsigned)d->batch, (unsigned)tiles), dim3(256), lds64,
                                h->stream, p);
         return hip_to_status(hipGetLastError());
     }
