@@ -383,6 +383,7 @@ __global__ void __launch_bounds__(CFG::NT) bgemm_mfma_kernel(const GemmParams p)
     using P1 = std::integral_constant<int, 1>;
     int kt = 0;
     if (full_mn) {
+        wait_for_all_loads();  // makes the wait counts inside the loop exact (see the fp32 kernel)
         for (; kt + 4 < nk_full; kt += 2) {
             k_tile(P0{}, std::true_type{});
             k_tile(P1{}, std::true_type{});

@@ -396,6 +396,10 @@ __device__ __forceinline__ void store_row_vec(float* p, const float (&v)[TN]) {
     }
 }
 
+// s_waitcnt vmcnt(0) as an instruction the compiler's own wait-count bookkeeping sees (expcnt and lgkmcnt fields at
+// their maxima: not waited for).
+__device__ __forceinline__ void wait_for_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // One accumulator element, read where it is used.  The operand constraint keeps the element in an accumulation
 // register up to this point.  Without it the register allocator, which may hold these values in either half of the
 // register file, moves most of a full-size accumulator set (256 values) into ordinary registers right behind the
@@ -941,7 +945,8 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         eb = sb.edge_info(n_rem, n0);
     }
     const bool edge_ok = !INTERIOR && ea.usable && eb.usable;  // uniform over the workgroup
-    const bool any_rot_a = !INTERIOR && (p.M % 4 != 0), any_rot_b = !INTERIOR && (p.N % 4 != 0);
+    // (StageA is k-contiguous when A is not transposed, StageB when B is: their vectors never arrive shifted)
+    const bool any_rot_a = !INTERIOR && TA && (p.M % 4 != 0), any_rot_b = !INTERIOR && !TB && (p.N % 4 != 0);
     const int rot_a = any_rot_a ? ea.shift : 0, rot_b = any_rot_b ? eb.shift : 0;
     int sh_a[2] = {0, 0}, sh_b[2] = {0, 0};
 
@@ -1014,7 +1019,10 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     // MODE 1: a full-k tile of an edge block (branch-free loads through the precomputed edge facts ea / eb);
     // MODE 2: the last tiles of an interior block (each fetch decides between unchecked loads and, at or past the
     //         end of K, checked ones);
-    // MODE 3: the last tiles of an edge block (edge loads for full-k tiles, fully checked loads otherwise).
+    // MODE 3: the last tiles of an edge block (edge loads for full-k tiles, fully checked loads otherwise);
+    // MODE 4: MODE 1 for a block none of whose vectors arrives shifted (M and N multiples of 4, or the operand is
+    //         k-contiguous): plain LDS stores.  The element selects of the shifted store, executed for nothing, made
+    //         the 64-wide-tile kernels VALU-bound in edge blocks (12 instructions per MFMA).
     auto k_tile = [&](auto parity, auto mode, const typename StageA::Edge& ea, const typename StageB::Edge& eb) {
         constexpr int P = decltype(parity)::value;
         constexpr int Q = P ^ 1;
@@ -1070,7 +1078,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                             if (q < StageA::NV) {
                                 const int v = q < StageA::NV ? q : 0;
                                 if (is_store) {
-                                    if constexpr (MODE == 0 || MODE == 2) {
+                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4) {
                                         sa.store_lds_vec(as_next, ra[Q][v], v);
                                         if constexpr (COLSUM) cs += ra[Q][v];
                                     } else {
@@ -1078,7 +1086,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                                             sa.store_lds_vec_shifted(as_next, ra[Q][v], v, sh_a[Q], any_rot_a);
                                         if constexpr (COLSUM) cs += stored;
                                     }
-                                } else if (MODE == 1 || edge_fast)
+                                } else if (MODE == 1 || MODE == 4 || edge_fast)
                                     sa.load_edge_vec(ra[Q][v], v, ea);
                                 else if (fast)
                                     sa.load_fast_vec(ra[Q][v], v);
@@ -1087,12 +1095,12 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                             } else {
                                 const int v = q >= StageA::NV ? q - StageA::NV : 0;
                                 if (is_store) {
-                                    if constexpr (MODE == 0 || MODE == 2)
+                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4)
                                         sb.store_lds_vec(bs_next, rb[Q][v], v);
                                     else
                                         sb.store_lds_vec_shifted(bs_next, rb[Q][v], v, sh_b[Q], any_rot_b);
                                 }
-                                else if (MODE == 1 || edge_fast)
+                                else if (MODE == 1 || MODE == 4 || edge_fast)
                                     sb.load_edge_vec(rb[Q][v], v, eb);
                                 else if (fast)
                                     sb.load_fast_vec(rb[Q][v], v);
@@ -1119,6 +1127,13 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     // branch-free pairs of tiles while both fetches (tiles kt+3, kt+4) are full k tiles
     // then the last few tiles (K tail included): same body, each fetch chooses checked or unchecked loads
     if constexpr (INTERIOR) {
+        // All loads of the prologue are waited for here, once per block.  The compiler derives the wait counts in
+        // front of the loop's LDS stores from the loads that may be in flight on any path into the loop; with the
+        // prologue's loads among them (issued in an order of its own choosing, some under conditions) it made the
+        // first store of every pass wait for ALL loads, including the ones issued a few MFMAs earlier, and the loop
+        // ran at one memory latency per pair of tiles (64 x 64 tiles: 885 cycles per tile for 512 cycles of MFMAs).
+        // With nothing in flight at the entry the counts are exact (all but the newest 2 * NP - 1 loads).
+        wait_for_all_loads();
         for (; kt + 4 < nk_full; kt += 2) {
             k_tile(P0{}, std::integral_constant<int, 0>{}, ea, eb);
             k_tile(P1{}, std::integral_constant<int, 0>{}, ea, eb);
@@ -1128,10 +1143,16 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             k_tile(P1{}, std::integral_constant<int, 2>{}, ea, eb);
         }
     } else {
-        if (edge_ok) {
+        if (edge_ok && (any_rot_a || any_rot_b)) {  // uniform
             for (; kt + 4 < nk_full; kt += 2) {
                 k_tile(P0{}, std::integral_constant<int, 1>{}, ea, eb);
                 k_tile(P1{}, std::integral_constant<int, 1>{}, ea, eb);
+            }
+        } else if (edge_ok) {
+            wait_for_all_loads();  // exact wait counts inside the loop, as for interior blocks
+            for (; kt + 4 < nk_full; kt += 2) {
+                k_tile(P0{}, std::integral_constant<int, 4>{}, ea, eb);
+                k_tile(P1{}, std::integral_constant<int, 4>{}, ea, eb);
             }
         }
         for (; kt < nk; kt += 2) {
