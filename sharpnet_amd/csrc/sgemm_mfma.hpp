@@ -903,16 +903,18 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     constexpr int KS = BK / 2;                   // MFMA k steps per tile
     constexpr int NP = StageA::NV + StageB::NV;  // LDS store pieces per tile
 
-    // Two register stages per operand: while tile kt is multiplied out of LDS,
-    // tile kt+1 sits in registers and is written to the other LDS buffer in small
-    // pieces between MFMAs, and tile kt+2 is in flight from global memory.  Each
-    // piece's registers are refilled with tile kt+3 right after they have been
-    // stored, so a global load has two full tiles of MFMA work to land.
+    // NS register stages per operand (tile t lives in stage t % NS): while tile kt is multiplied out of LDS,
+    // tile kt+1 sits in registers and is written to the other LDS buffer in small pieces between MFMAs, and
+    // tiles kt+2 .. kt+NS are in flight from global memory.  Each piece's registers are refilled with tile
+    // kt+1+NS right after they have been stored, so a global load has NS full tiles of MFMA work to land.
+    // Two stages everywhere.  Four were measured for the 64-wide tiles (a tile lasts 512-1024 cycles there, less
+    // than a memory latency): 1024 x 1024 x 2048 38.9 -> 37.0 us, but 1024^3 and 1000^3 unchanged or slower (five
+    // tiles of prologue loads) and twice the registers (137 against 68: fewer co-resident workgroups).
     //
-    // The k loop is one straight-line body of two tiles with no special cases:
-    // tiles at or beyond the end of K are fetched as zeros (no memory access), so
-    // an odd tile count simply multiplies one tile of zeros.
-    f32x4 ra[2][StageA::NV], rb[2][StageB::NV];
+    // The k loop is one straight-line body of NS tiles with no special cases: tiles at or beyond the end of K are
+    // fetched as zeros (no memory access), so a tile count that is not a multiple of two multiplies one tile of zeros.
+    constexpr int NS = 2;
+    f32x4 ra[NS][StageA::NV], rb[NS][StageB::NV];
     int fetch = 0;  // index of the k tile the stage pointers address; tiles are fetched in order
 
     // MFMA operand fragments: a ring of NB buffers over k steps, read D = NB-1 steps ahead of their use.
@@ -948,13 +950,13 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     // (StageA is k-contiguous when A is not transposed, StageB when B is: their vectors never arrive shifted)
     const bool any_rot_a = !INTERIOR && TA && (p.M % 4 != 0), any_rot_b = !INTERIOR && !TB && (p.N % 4 != 0);
     const int rot_a = any_rot_a ? ea.shift : 0, rot_b = any_rot_b ? eb.shift : 0;
-    int sh_a[2] = {0, 0}, sh_b[2] = {0, 0};
+    int sh_a[NS] = {}, sh_b[NS] = {};
 
     {
-        // prologue: tile 0 -> LDS buffer 0, tile 1 -> stage 1, tile 2 -> stage 0
+        // prologue: tile 0 -> stage 0 -> LDS buffer 0, tiles 1 .. NS-1 -> their stages, tile NS -> stage 0
 #pragma unroll
-        for (int t = 0; t < 3; ++t) {
-            const int st = (t == 1) ? 1 : 0;
+        for (int t = 0; t <= NS; ++t) {
+            const int st = t % NS;
             const int k_rem = klen - fetch * BK;
             sh_a[st] = 0;
             sh_b[st] = 0;
@@ -1023,9 +1025,12 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     // MODE 4: MODE 1 for a block none of whose vectors arrives shifted (M and N multiples of 4, or the operand is
     //         k-contiguous): plain LDS stores.  The element selects of the shifted store, executed for nothing, made
     //         the 64-wide-tile kernels VALU-bound in edge blocks (12 instructions per MFMA).
-    auto k_tile = [&](auto parity, auto mode, const typename StageA::Edge& ea, const typename StageB::Edge& eb) {
+    // R: the register stage that holds the next tile (it is stored to LDS buffer P ^ 1 and refilled).
+    auto k_tile = [&](auto parity, auto stage, auto mode, const typename StageA::Edge& ea,
+                      const typename StageB::Edge& eb) {
         constexpr int P = decltype(parity)::value;
         constexpr int Q = P ^ 1;
+        constexpr int R = decltype(stage)::value;
         constexpr int MODE = decltype(mode)::value;
         const bool fast = (MODE == 0) || (MODE == 2 && (fetch < nk_full));
         // the tail of an edge block: a full-k tile still takes the branch-free edge loads
@@ -1079,33 +1084,33 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                                 const int v = q < StageA::NV ? q : 0;
                                 if (is_store) {
                                     if constexpr (MODE == 0 || MODE == 2 || MODE == 4) {
-                                        sa.store_lds_vec(as_next, ra[Q][v], v);
-                                        if constexpr (COLSUM) cs += ra[Q][v];
+                                        sa.store_lds_vec(as_next, ra[R][v], v);
+                                        if constexpr (COLSUM) cs += ra[R][v];
                                     } else {
                                         const f32x4 stored =
-                                            sa.store_lds_vec_shifted(as_next, ra[Q][v], v, sh_a[Q], any_rot_a);
+                                            sa.store_lds_vec_shifted(as_next, ra[R][v], v, sh_a[R], any_rot_a);
                                         if constexpr (COLSUM) cs += stored;
                                     }
                                 } else if (MODE == 1 || MODE == 4 || edge_fast)
-                                    sa.load_edge_vec(ra[Q][v], v, ea);
+                                    sa.load_edge_vec(ra[R][v], v, ea);
                                 else if (fast)
-                                    sa.load_fast_vec(ra[Q][v], v);
+                                    sa.load_fast_vec(ra[R][v], v);
                                 else
-                                    sa.load_safe_vec(ra[Q][v], v, m_rem, k_rem);
+                                    sa.load_safe_vec(ra[R][v], v, m_rem, k_rem);
                             } else {
                                 const int v = q >= StageA::NV ? q - StageA::NV : 0;
                                 if (is_store) {
                                     if constexpr (MODE == 0 || MODE == 2 || MODE == 4)
-                                        sb.store_lds_vec(bs_next, rb[Q][v], v);
+                                        sb.store_lds_vec(bs_next, rb[R][v], v);
                                     else
-                                        sb.store_lds_vec_shifted(bs_next, rb[Q][v], v, sh_b[Q], any_rot_b);
+                                        sb.store_lds_vec_shifted(bs_next, rb[R][v], v, sh_b[R], any_rot_b);
                                 }
                                 else if (MODE == 1 || MODE == 4 || edge_fast)
-                                    sb.load_edge_vec(rb[Q][v], v, eb);
+                                    sb.load_edge_vec(rb[R][v], v, eb);
                                 else if (fast)
-                                    sb.load_fast_vec(rb[Q][v], v);
+                                    sb.load_fast_vec(rb[R][v], v);
                                 else
-                                    sb.load_safe_vec(rb[Q][v], v, n_rem, k_rem);
+                                    sb.load_safe_vec(rb[R][v], v, n_rem, k_rem);
                             }
                         }
                     }
@@ -1113,18 +1118,31 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                 }
             }
         }
-        // what stage Q holds now was fetched in this tile: remember whether it arrived shifted
+        // what stage R holds now was fetched in this tile: remember whether it arrived shifted
         if constexpr (MODE == 1 || MODE == 3) {
             const bool via_edge = (MODE == 1) || edge_fast;
-            sh_a[Q] = via_edge ? rot_a : 0;
-            sh_b[Q] = via_edge ? rot_b : 0;
+            sh_a[R] = via_edge ? rot_a : 0;
+            sh_b[R] = via_edge ? rot_b : 0;
         }
     };
 
-    using P0 = std::integral_constant<int, 0>;
-    using P1 = std::integral_constant<int, 1>;
+    // NS tiles in a row, starting at a tile index that is a multiple of NS (tile kt reads LDS buffer kt & 1, the
+    // next tile sits in stage (kt + 1) % NS).  `limit`: tiles at or past it are skipped, in pairs (NS = 4 only).
+    auto tiles = [&](auto mode, int first, int limit) {
+        using M = decltype(mode);
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        k_tile(I0{}, std::integral_constant<int, 1 % NS>{}, M{}, ea, eb);
+        k_tile(I1{}, std::integral_constant<int, 2 % NS>{}, M{}, ea, eb);
+        if constexpr (NS == 4) {
+            if (first + 2 >= limit) return;  // uniform
+            k_tile(I0{}, std::integral_constant<int, 3>{}, M{}, ea, eb);
+            k_tile(I1{}, std::integral_constant<int, 0>{}, M{}, ea, eb);
+        }
+    };
+    constexpr int kNoLimit = 0x7fffffff;
     int kt = 0;
-    // branch-free pairs of tiles while both fetches (tiles kt+3, kt+4) are full k tiles
+    // branch-free groups of NS tiles while all their fetches (tiles kt+NS+1 .. kt+2*NS) are full k tiles,
     // then the last few tiles (K tail included): same body, each fetch chooses checked or unchecked loads
     if constexpr (INTERIOR) {
         // All loads of the prologue are waited for here, once per block.  The compiler derives the wait counts in
@@ -1132,33 +1150,18 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         // prologue's loads among them (issued in an order of its own choosing, some under conditions) it made the
         // first store of every pass wait for ALL loads, including the ones issued a few MFMAs earlier, and the loop
         // ran at one memory latency per pair of tiles (64 x 64 tiles: 885 cycles per tile for 512 cycles of MFMAs).
-        // With nothing in flight at the entry the counts are exact (all but the newest 2 * NP - 1 loads).
+        // With nothing in flight at the entry the counts are exact (all but the newest NS * NP - 1 loads).
         wait_for_all_loads();
-        for (; kt + 4 < nk_full; kt += 2) {
-            k_tile(P0{}, std::integral_constant<int, 0>{}, ea, eb);
-            k_tile(P1{}, std::integral_constant<int, 0>{}, ea, eb);
-        }
-        for (; kt < nk; kt += 2) {
-            k_tile(P0{}, std::integral_constant<int, 2>{}, ea, eb);
-            k_tile(P1{}, std::integral_constant<int, 2>{}, ea, eb);
-        }
+        for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 0>{}, kt, kNoLimit);
+        for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 2>{}, kt, nk);
     } else {
         if (edge_ok && (any_rot_a || any_rot_b)) {  // uniform
-            for (; kt + 4 < nk_full; kt += 2) {
-                k_tile(P0{}, std::integral_constant<int, 1>{}, ea, eb);
-                k_tile(P1{}, std::integral_constant<int, 1>{}, ea, eb);
-            }
+            for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 1>{}, kt, kNoLimit);
         } else if (edge_ok) {
             wait_for_all_loads();  // exact wait counts inside the loop, as for interior blocks
-            for (; kt + 4 < nk_full; kt += 2) {
-                k_tile(P0{}, std::integral_constant<int, 4>{}, ea, eb);
-                k_tile(P1{}, std::integral_constant<int, 4>{}, ea, eb);
-            }
+            for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 4>{}, kt, kNoLimit);
         }
-        for (; kt < nk; kt += 2) {
-            k_tile(P0{}, std::integral_constant<int, 3>{}, ea, eb);
-            k_tile(P1{}, std::integral_constant<int, 3>{}, ea, eb);
-        }
+        for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 3>{}, kt, nk);
     }
     };  // run
     if (full_mn)
