@@ -463,6 +463,54 @@ def test_random_shapes_offsets_and_pitches(oracle, gpu_wrapper):
             t.Dispose()
 
 
+def test_random_aligned_shapes_every_tiled_configuration(oracle, gpu_wrapper):
+    """160 seeded cases on whole, tightly packed tensors (16-byte-aligned rows whenever the extents allow: the
+    vector write-out, the branch-free edge loads with and without shifted vectors), sizes up to 1100 with a bias
+    towards multiples of 4 and of the tile sizes plus or minus a little, every fp32 tiled configuration in turn with
+    split-K 1 or 2, beta 0 / 1 / -0.5.  Reference: the oracle's float64 closed form."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    tiled = [i for i, c in enumerate(w.configs()) if c["kind"] == "fp32"]
+    assert len(tiled) == 10
+    rng = np.random.default_rng(77)
+
+    def extent():
+        base = int(rng.choice([64, 128, 256, 512, 1024]))
+        kind = int(rng.integers(4))
+        if kind == 0:
+            return base
+        if kind == 1:
+            return base + int(rng.choice([-8, -4, 4, 8, 12, 40]))      # ragged, multiple of 4
+        if kind == 2:
+            return base + int(rng.choice([-3, -1, 1, 2, 3, 5]))        # ragged, odd
+        return int(rng.integers(1, 1100))
+    try:
+        for case in range(160):
+            M, N, K = extent(), extent(), extent()
+            if M * N * K > 6e8:
+                K = max(16, K // 4)
+            tA, tB = bool(rng.integers(2)), bool(rng.integers(2))
+            alpha = float(rng.choice([1.0, -0.5, 2.0]))
+            beta = float(rng.choice([0.0, 0.0, 1.0, -0.5]))
+            a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
+            b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
+            c = random_tensor(rng, (M, N), -1, 1)
+            cfg = tiled[case % len(tiled)]
+            sk = 2 if (case // len(tiled)) % 3 == 2 and K >= 256 else 1
+            w.set_tuning(cfg, sk)
+            ga, gb, gc = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w), GPUTensor(c.shape, c, w)
+            gc.Dot(ga, tA, gb, tB, alpha, beta)
+            assert w.last_tuning() == (cfg, sk), (case, w.last_tuning())
+            got = gc.ToNumpy()
+            ref = oracle.dot_f64(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
+            err = float(np.max(np.abs(got - ref)))
+            assert err <= tol(K, a, b, alpha, beta, c) + 1e-6, (case, cfg, sk, M, N, K, tA, tB, alpha, beta, err)
+            for t in (ga, gb, gc):
+                t.Dispose()
+    finally:
+        w.set_tuning(-1, 0)
+
+
 def test_sgeam_transpose_and_sdgmm(oracle, gpu_wrapper):
     """Tensor.Transpose (cublasSgeam with the reference's arguments, Tests/TestParallelRunCpuVersusGpu.cs:522-533 sizes and
     larger ones that span several tiles), the general Sgeam form, and Tensor.MultiplyTensor (cublasSdgmm, same file
