@@ -231,4 +231,173 @@ __global__ void __launch_bounds__(64 * NW) sgemm_ksplit_kernel(const GemmParams 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same scheme on 16 x 16 tiles (v_mfma_f32_16x16x4_f32) with K split over the eight wavefronts of a workgroup,
+// for products with so few 32 x 32 tiles that most compute units would get none (the forward product of a Dense
+// layer on a small batch, 128 x 256 x 784: 32 tiles of 32 x 32, 128 of 16 x 16).
+// ---------------------------------------------------------------------------------------------------------------
+typedef float f32x4_acc16 __attribute__((ext_vector_type(4)));
+
+struct Ksplit16Cfg {
+    static constexpr int NW = 8;        // wavefronts = K slices
+    static constexpr int DEPTH = 4;     // groups of 32 k values in flight per wavefront
+    static constexpr int PITCH = 36;    // floats per row of a patch[16 rows][32 k]
+    static constexpr int PITCH_K = 20;  // floats per row of a patch[32 k][16 rows]
+    static constexpr int PATCH_FLOATS = NW * 2 * 32 * PITCH_K;  // >= NW * 2 * 16 * PITCH
+    static constexpr int PART_FLOATS = NW * 16 * 17;
+    static constexpr int LDS_BYTES = 4 * (PATCH_FLOATS > PART_FLOATS ? PATCH_FLOATS : PART_FLOATS);
+};
+
+// One operand of one wavefront: 16 rows (m or n) x the k range, two 16-byte loads per lane and group of 32 k.
+//   KMAJOR = false: storage [row][k]; instruction i reads row 8 i + lane / 8, k 4 (lane % 8) .. + 3.
+//   KMAJOR = true:  storage [k][row]; instruction i reads k 16 i + lane / 4, rows 4 (lane % 4) .. + 3.
+template <bool KMAJOR>
+struct KsplitOperand16 {
+    const float* ptr[2];
+    long long step;
+    bool row_ok[2];
+    int k_first[2];
+
+    __device__ __forceinline__ void init(const float* base, long long ld, int row0, int rows, int lane) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            if constexpr (KMAJOR) {
+                const int lcol = (lane & 3) * 4;
+                row_ok[i] = row0 + lcol < rows;  // rows % 4 == 0: all four or none
+                k_first[i] = 16 * i + (lane >> 2);
+                ptr[i] = base + (long long)k_first[i] * ld + (row_ok[i] ? row0 + lcol : 0);
+            } else {
+                const int lrow = lane >> 3, lcol = (lane & 7) * 4;
+                const int r = (row0 + 8 * i + lrow < rows) ? row0 + 8 * i + lrow : rows - 1;
+                row_ok[i] = true;
+                k_first[i] = lcol;
+                ptr[i] = base + (long long)r * ld + lcol;
+            }
+        }
+        step = KMAJOR ? 32 * ld : 32;
+    }
+    __device__ __forceinline__ f32x4 load(int i, int m, int K) const {
+        const bool ok = 32 * m + k_first[i] < K;
+        return *reinterpret_cast<const f32x4*>(ptr[i] + (ok ? (long long)m * step : 0));
+    }
+    __device__ __forceinline__ f32x4 keep(f32x4 v, int i, int m, int K) const {
+        const bool ok = (32 * m + k_first[i] < K) && row_ok[i];
+        f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
+        return ok ? v : z;
+    }
+    __device__ __forceinline__ void to_patch(float* patch, int i, int lane, f32x4 v) const {
+        if constexpr (KMAJOR)
+            *reinterpret_cast<f32x4*>(patch + (16 * i + (lane >> 2)) * Ksplit16Cfg::PITCH_K + (lane & 3) * 4) = v;
+        else
+            *reinterpret_cast<f32x4*>(patch + (8 * i + (lane >> 3)) * Ksplit16Cfg::PITCH + (lane & 7) * 4) = v;
+    }
+    // The eight MFMAs of a group: MFMA j takes k = 8 q + j from lane group q = lane / 16 (any assignment of the 32 k
+    // values to (j, q) will do as long as both operands use the same one).  f[j] = operand[row lane % 16][8 q + j].
+    __device__ __forceinline__ void fragment(const float* patch, int lane, float (&f)[8]) const {
+        const int r = lane & 15, q = lane >> 4;
+        if constexpr (KMAJOR) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) f[j] = patch[(8 * q + j) * Ksplit16Cfg::PITCH_K + r];
+        } else {
+            const f32x4 lo = *reinterpret_cast<const f32x4*>(patch + r * Ksplit16Cfg::PITCH + 8 * q);
+            const f32x4 hi = *reinterpret_cast<const f32x4*>(patch + r * Ksplit16Cfg::PITCH + 8 * q + 4);
+            f[0] = lo.x, f[1] = lo.y, f[2] = lo.z, f[3] = lo.w, f[4] = hi.x, f[5] = hi.y, f[6] = hi.z, f[7] = hi.w;
+        }
+    }
+};
+
+template <bool TA, bool TB>
+__global__ void __launch_bounds__(512) sgemm_ksplit16_kernel(const GemmParams p) {
+    using C = Ksplit16Cfg;
+    constexpr int NW = C::NW, D = C::DEPTH;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float(*const part)[16][17] = reinterpret_cast<float(*)[16][17]>(smem);  // [NW][16][17], after the k loop
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const bool n_fastest = (p.flags & GEMM_FLAG_TILE_N_FASTEST) != 0;
+    const int tile_m = n_fastest ? blockIdx.x / p.tiles_n : blockIdx.x % p.tiles_m;
+    const int tile_n = n_fastest ? blockIdx.x % p.tiles_n : blockIdx.x / p.tiles_m;
+    const int m0 = tile_m * 16, n0 = tile_n * 16;
+    const int z = blockIdx.y;
+    const float* Ab = p.A + (long long)z * p.strideA;
+    const float* Bb = p.B + (long long)z * p.strideB;
+    float* Cb = p.C + (long long)z * p.strideC;
+
+    KsplitOperand16<TA> oa;
+    KsplitOperand16<!TB> ob;
+    oa.init(Ab, p.lda, m0, p.M, lane);
+    ob.init(Bb, p.ldb, n0, p.N, lane);
+    float* pa = smem + (wave * 2 + 0) * (32 * C::PITCH_K);
+    float* pb = smem + (wave * 2 + 1) * (32 * C::PITCH_K);
+
+    const int K = p.K;
+    const int groups = (K + 31) / 32;
+    const int per = (groups + NW - 1) / NW;
+    const int mbeg = wave * per, mend = (mbeg + per < groups) ? mbeg + per : groups;
+
+    f32x4 ra[D][2], rb[D][2];
+    float fa[8], fb[8];
+    f32x4_acc16 acc[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[e][r] = 0.0f;
+
+    // all of a wavefront's groups are requested before the first one is used (up to D at a time)
+    for (int m = mbeg; m < mend; m += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if (m + d < mend) {  // uniform
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    ra[d][i] = oa.load(i, m + d, K);
+                    rb[d][i] = ob.load(i, m + d, K);
+                }
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if (m + d < mend) {
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    oa.to_patch(pa, i, lane, oa.keep(ra[d][i], i, m + d, K));
+                    ob.to_patch(pb, i, lane, ob.keep(rb[d][i], i, m + d, K));
+                }
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                oa.fragment(pa, lane, fa);
+                ob.fragment(pb, lane, fb);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    acc[j & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[j], fb[j], acc[j & 1], 0, 0, 0);
+            }
+        }
+    }
+
+    __syncthreads();  // every wavefront is done with its patch: the memory now takes the partial tiles
+    // accumulator register e holds row 4 (lane / 16) + e, column lane % 16 of the tile
+#pragma unroll
+    for (int e = 0; e < 4; ++e) part[wave][4 * (lane >> 4) + e][lane & 15] = acc[0][e] + acc[1][e];
+    __syncthreads();
+
+    if (threadIdx.x < 256) {
+        const int lr = threadIdx.x / 16, lc = threadIdx.x % 16;
+        const int row = m0 + lr, col = n0 + lc;
+        if (row < p.M && col < p.N) {
+            float v = 0.0f;
+#pragma unroll
+            for (int k = 0; k < NW; ++k) v += part[k][lr][lc];
+            v *= p.alpha;
+            if (p.ep.bias != nullptr) v += p.ep.bias[col];
+            float* c = Cb + (long long)row * p.ldc + col;
+            if (p.beta != 0.0f) v += p.beta * *c;
+            if (p.ep.addend != nullptr)
+                v += p.ep.gamma * p.ep.addend[(long long)z * p.ep.strideD + (long long)row * p.ep.ldd + col];
+            if (p.ep.act == ACT_RELU || p.ep.act == ACT_LEAKY_RELU) v = leaky_relu(v, p.ep.act_param);
+            *c = v;
+        }
+    }
+}
+
 }  // namespace snhip

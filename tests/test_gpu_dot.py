@@ -614,9 +614,11 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
         assert gpu_wrapper.last_tuning() == (ks, 1)
         assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, tA, b, tB, 0.5))) <= tol(K, a, b, 0.5)
         gpu_wrapper.set_tuning(-1, 0)
-        # automatic choice: the forward product of benchmark configuration 1's Dense layer (32 tiles: eight K slices),
-        # a square product of one 32 x 32 tile per CU, a recurrent step (one 32 x 64 tile per CU), the layer's dx
-        for (M, N, K, want) in [(128, 256, 784, ks_all[2]), (512, 512, 512, ks_all[0]), (256, 2048, 512, ks_all[1]),
+        # automatic choice: the forward product of benchmark configuration 1's Dense layer (32 tiles of 32 x 32: the
+        # 16 x 16-tile kernel), a square product of one 32 x 32 tile per CU, a recurrent step (one 32 x 64 tile per
+        # CU), the layer's dx
+        assert len(ks_all) == 4
+        for (M, N, K, want) in [(128, 256, 784, ks_all[3]), (512, 512, 512, ks_all[0]), (256, 2048, 512, ks_all[1]),
                                 (128, 784, 256, ks_all[0])]:
             a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
             b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
