@@ -107,21 +107,36 @@ def main():
             gbias.Dispose()
         return wall_ms, ev_ms, gc
 
-    def run_stored(gm, seed, steps, warmup):
+    def run_stored(gm, seed, steps, warmup, to_nt=False):
+        """One product with operands stored as bf16.  to_nt (single matrices only): a transposed A / a plain B is
+        transposed by the conversion pass, so that the product itself runs in the NT form."""
         from sharpnet_amd.hiplib import check_status
         aa, bb, _ = wl.uniform_operands(gm, seed)
         ga, gb = upload(aa), upload(bb)
         gcs = GPUTensor(gm.c_shape, None, w)
         pa, pb = w.allocate(2 * ga.Count), w.allocate(2 * gb.Count)
-
-        def convert():
-            check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, ga.Pointer, pa, ga.Count))
-            check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, gb.Pointer, pb, gb.Count))
         aH, aW = aa.shape[-2:]
         bH, bW = bb.shape[-2:]
+        flip_a, flip_b = to_nt and gm.tA, to_nt and not gm.tB
+        assert not to_nt or gm.batch == 1
+
+        def convert():
+            if flip_a:
+                check_status(w.lib.snhip_convert_f32_to_bf16_2d(w.handle, ga.Pointer, aH, aW, aW, 1, pa, aH))
+            else:
+                check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, ga.Pointer, pa, ga.Count))
+            if flip_b:
+                check_status(w.lib.snhip_convert_f32_to_bf16_2d(w.handle, gb.Pointer, bH, bW, bW, 1, pb, bH))
+            else:
+                check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, gb.Pointer, pb, gb.Count))
+        if flip_a:
+            aH, aW = aW, aH
+        if flip_b:
+            bH, bW = bW, bH
+        tA, tB = (False if flip_a else gm.tA), (True if flip_b else gm.tB)
 
         def launch():
-            check_status(w.lib.snhip_bmm_bf16_stored(w.handle, pa, aH, aW, int(gm.tA), aH * aW, pb, bH, bW, int(gm.tB),
+            check_status(w.lib.snhip_bmm_bf16_stored(w.handle, pa, aH, aW, int(tA), aH * aW, pb, bH, bW, int(tB),
                                                      bH * bW, gcs.Pointer, gm.M * gm.N, gm.batch, gm.alpha, gm.beta,
                                                      None))
 
@@ -142,7 +157,8 @@ def main():
         ms = timed(launch, steps, warmup)
         by = gm.batch * (2.0 * (gm.M * gm.K + gm.K * gm.N) + 4.0 * gm.M * gm.N)
         roof_s = max(gm.flops / (wl.BF16_MFMA_PEAK_TFLOPS * 1e12), by / (wl.HBM_PEAK_GBS * 1e9))
-        r = {"gemm": gm.label() + " (bf16 storage)", "ms": round(ms, 4), "tflops": round(gm.flops / (ms * 1e-3) / 1e12, 2),
+        r = {"gemm": gm.label() + (" (bf16 storage, operands transposed to the NT form by the conversion)" if to_nt
+                                 else " (bf16 storage)"), "ms": round(ms, 4), "tflops": round(gm.flops / (ms * 1e-3) / 1e12, 2),
              "frac_of_roofline": round(roof_s * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
              "splitk": w.last_tuning()[1], "algorithmic_bytes": by, "convert_both_operands_ms": round(conv_ms, 4)}
         w.release(pa, 2 * ga.Count)
@@ -488,6 +504,10 @@ def main():
         # Operands are converted once by the library's own pass (timed separately: it is not part of the product).
         extra["config2_8192_bf16_stored"] = [run_stored(wl.Gemm(8192, 8192, 8192, tA, tB, 1.0, 0.0), 2, 10, 5)
                                             for (tA, tB) in ((False, True), (False, False), (True, False))]
+        # the NN and TN products again with their operands brought into the k-contiguous (NT) form by the transposing
+        # conversion: what a caller that converts an operand once and multiplies it many times would do
+        extra["config2_8192_bf16_stored"] += [run_stored(wl.Gemm(8192, 8192, 8192, tA, tB, 1.0, 0.0), 2, 10, 5, to_nt=True)
+                                             for (tA, tB) in ((False, False), (True, False))]
         extra["config5_attention_bf16_stored"] = {"gemms": [run_stored(gm, 5, 50, 10) for gm in att_g],
                                                   "cpu_baseline": extra["config5_attention_fp32"]["cpu_baseline"],
                                                   "note": "CPU figure: the fp32 route (the reference has no other)"}

@@ -180,6 +180,45 @@ def test_convert_2d_with_pitches_and_transpose(oracle, gpu_wrapper):
             w.release(dst, nbytes + 8)
 
 
+def test_transposing_conversion_brings_a_product_into_the_nt_form(oracle, gpu_wrapper):
+    """A plain B (K x N) converted with transpose = 1 becomes an (N x K) operand for transposeB = 1, a transposed A
+    (K x M) likewise an (M x K) one: the product in the NT form equals the product on the operands as they were, bit
+    for bit (same tile configuration, same summation order), ragged even sizes included."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    L, h = w.lib, w.handle
+    rng = np.random.default_rng(45)
+    for (M, N, K) in [(512, 384, 640), (130, 258, 72), (36, 22, 124)]:
+        at = random_tensor(rng, (K, M), -1, 1)     # A stored transposed
+        b = random_tensor(rng, (K, N), -1, 1)      # B stored plain
+        gat, gb = GPUTensor(at.shape, at, w), GPUTensor(b.shape, b, w)
+        pat, pb = w.allocate(2 * K * M), w.allocate(2 * K * N)
+        pa_nt, pb_nt = w.allocate(2 * K * M), w.allocate(2 * K * N)
+        check_status(L.snhip_convert_f32_to_bf16(h, gat.Pointer, pat, K * M))
+        check_status(L.snhip_convert_f32_to_bf16(h, gb.Pointer, pb, K * N))
+        check_status(L.snhip_convert_f32_to_bf16_2d(h, gat.Pointer, K, M, M, 1, pa_nt, K))
+        check_status(L.snhip_convert_f32_to_bf16_2d(h, gb.Pointer, K, N, N, 1, pb_nt, K))
+        c_tn, c_nt = GPUTensor([M, N], None, w), GPUTensor([M, N], None, w)
+        for t in (c_tn, c_nt):
+            t.SetValue(float("nan"))
+        check_status(L.snhip_dot_bf16_stored(h, pat, K, M, 1, pb, K, N, 0, c_tn.Pointer, 1.0, 0.0, None))
+        cfg = w.last_tuning()
+        w.set_tuning(*cfg)
+        try:
+            check_status(L.snhip_dot_bf16_stored(h, pa_nt, M, K, 0, pb_nt, N, K, 1, c_nt.Pointer, 1.0, 0.0, None))
+        finally:
+            w.set_tuning(-1, 0)
+        got_tn, got_nt = c_tn.ToNumpy(), c_nt.ToNumpy()
+        assert np.array_equal(got_tn, got_nt), (M, N, K)
+        ref = oracle.dot(oracle.round_to_bf16(at), True, oracle.round_to_bf16(b), False)
+        assert np.max(np.abs(got_nt - ref)) <= 1e-4 * np.sqrt(K), (M, N, K)
+        for ptr, n in ((pat, 2 * K * M), (pb, 2 * K * N), (pa_nt, 2 * K * M), (pb_nt, 2 * K * N)):
+            w.release(ptr, n)
+        for t in (gat, gb, c_tn, c_nt):
+            t.Dispose()
+
+
 EVEN_SHAPES = [(36, 22, 124), (130, 258, 64), (256, 256, 64), (300, 130, 200), (64, 64, 16), (2, 2, 2), (258, 100, 34),
                (6, 300, 1000), (512, 384, 512), (200, 520, 136)]
 
