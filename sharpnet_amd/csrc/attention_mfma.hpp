@@ -105,22 +105,42 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 
     const bool vec4 = (p.dk % 4 == 0) && (p.dv % 4 == 0);  // uniform: whole 16-byte vectors are inside or outside
 
-    // this lane's query row as the B operand of the score product: qf[s] = Q[row][2 s + lane / 32]
+    // This lane's query row as the B operand of the score product.  The product sums over d in any order as long as
+    // both operands agree on it: k step s of lane half h (= lane / 32) stands for d = h * D/2 + s, so a lane reads
+    // D/2 consecutive floats of its row - whole 16-byte loads that land in their registers with nothing to select.
+    // qf[s] = Q[row][(lane / 32) * D/2 + s].  Rows past Tq read the last row instead: a query is one column of both
+    // products, so what such a lane computes never meets another row and is never stored.
     auto load_q = [&](float (&dst)[AT_D / 2], int qrow_index) {
         const bool ok = qrow_index < p.Tq;
-        const float* qrow = Qz + (long long)(ok ? qrow_index : p.Tq - 1) * p.ldq;
-        if (vec4) {
+        const int d0 = lhi * (AT_D / 2);
+        const float* qrow = Qz + (long long)(ok ? qrow_index : p.Tq - 1) * p.ldq + d0;
+        if (vec4 && p.dk == AT_D) {
 #pragma unroll
-            for (int j = 0; j < AT_D / 4; ++j) {
-                const f32x4 x = load4_select(qrow + (4 * j < p.dk ? 4 * j : 0), ok && 4 * j < p.dk);
-                dst[2 * j] = lhi ? x.y : x.x;
-                dst[2 * j + 1] = lhi ? x.w : x.z;
+            for (int j = 0; j < AT_D / 8; ++j) {
+                f32x4 x;
+                __builtin_memcpy(&x, qrow + 4 * j, 16);
+                dst[4 * j] = x.x;
+                dst[4 * j + 1] = x.y;
+                dst[4 * j + 2] = x.z;
+                dst[4 * j + 3] = x.w;
+            }
+        } else if (vec4) {
+#pragma unroll
+            for (int j = 0; j < AT_D / 8; ++j) {
+                const bool in = d0 + 4 * j < p.dk;
+                const f32x4 x = load4_select(in ? qrow + 4 * j : Qz, ok && in);
+                dst[4 * j] = x.x;
+                dst[4 * j + 1] = x.y;
+                dst[4 * j + 2] = x.z;
+                dst[4 * j + 3] = x.w;
             }
         } else {
-            for (int j = 0; j < AT_D / 4; ++j) {
-                const f32x4 x = load4_guarded(qrow + 4 * j, ok ? (p.dk - 4 * j) : 0);
-                dst[2 * j] = lhi ? x.y : x.x;
-                dst[2 * j + 1] = lhi ? x.w : x.z;
+            for (int j = 0; j < AT_D / 8; ++j) {
+                const f32x4 x = load4_guarded(qrow + 4 * j, ok ? (p.dk - d0 - 4 * j) : 0);
+                dst[4 * j] = x.x;
+                dst[4 * j + 1] = x.y;
+                dst[4 * j + 2] = x.z;
+                dst[4 * j + 3] = x.w;
             }
         }
     };
@@ -203,7 +223,7 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
     // from sinking the reads back next to their use).
     {
         constexpr int NTILE = AT_TK / 32;
-        const float* kbase = Ks + lhi * AT_KP + l32;
+        const float* kbase = Ks + (lhi * (AT_D / 2)) * AT_KP + l32;  // row d = lhi * D/2 + s in step s, as in load_q
         float ka[2][NTILE];
 #pragma unroll
         for (int t = 0; t < NTILE; ++t) ka[0][t] = kbase[t * 32];
@@ -211,7 +231,7 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
         for (int s = 0; s < AT_D / 2; ++s) {
             if (s + 1 < AT_D / 2) {
 #pragma unroll
-                for (int t = 0; t < NTILE; ++t) ka[(s + 1) & 1][t] = kbase[(2 * (s + 1)) * AT_KP + t * 32];
+                for (int t = 0; t < NTILE; ++t) ka[(s + 1) & 1][t] = kbase[(s + 1) * AT_KP + t * 32];
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -324,7 +344,9 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 
     // ---- P out (four consecutive keys per register group).  With all keys present and aligned rows the stores
     //      are spread over the second product's MFMAs instead (below); this is the general form. ----
-    const bool p_inline = p.P != nullptr && (p.flags & 2) && p.Tk == AT_TK;  // uniform
+    // (uniform; a tile with query rows past Tq takes the general form, so that the spread stores need no predicate
+    // and the second product stays one straight run of instructions)
+    const bool p_inline = p.P != nullptr && (p.flags & 2) && p.Tk == AT_TK && q0 + AT_BQ <= p.Tq;
     if (p.P != nullptr && !p_inline && row_ok) {
         float* prow = p.P + ((long long)z * p.Tq + row) * p.Tk;
 #pragma unroll
@@ -365,7 +387,7 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 #pragma unroll
                 for (int r = 0; r < 16; ++r) part[h][mt][r] = 0.0f;
         const float* vbase = Vs + (4 * lhi) * AT_VP + l32;
-        float* const prow = STORE_P ? p.P + ((long long)z * p.Tq + (row_ok ? row : 0)) * p.Tk + 4 * lhi : nullptr;
+        float* const prow = STORE_P ? p.P + ((long long)z * p.Tq + row) * p.Tk + 4 * lhi : nullptr;
         float va[4][MT];
         auto v_off = [](int i) { return ((i / 16) * 32 + 8 * ((i % 16) / 4) + (i % 4)) * AT_VP; };
 #pragma unroll
@@ -381,9 +403,8 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
             if (STORE_P && i % 4 == 0) {
                 // one 16-byte store of P every four k steps: the write-out rides in the MFMAs' shadow
                 const int t = i / 16, g = (i % 16) / 4;
-                if (row_ok)
-                    *reinterpret_cast<f32x4*>(prow + t * 32 + 8 * g) =
-                        f32x4{sacc[t][4 * g], sacc[t][4 * g + 1], sacc[t][4 * g + 2], sacc[t][4 * g + 3]};
+                *reinterpret_cast<f32x4*>(prow + t * 32 + 8 * g) =
+                    f32x4{sacc[t][4 * g], sacc[t][4 * g + 1], sacc[t][4 * g + 2], sacc[t][4 * g + 3]};
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
