@@ -58,6 +58,7 @@ struct AttnParams {
     long long sQ2, sK2, sV2, sO2;  // ... of the outer level
     int batch_inner;
     int q_tiles;  // 128-query tiles one workgroup walks through (K and V stay in LDS across them)
+    int batch;    // number of (batch, head) matrices
     float scale;
     int causal;
     int flags;  // bit 0: O rows may be written as aligned 16-byte vectors, bit 1: P rows likewise
@@ -443,6 +444,281 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 #pragma unroll
     for (int j = 0; j < AT_D / 2; ++j) qf[j] = qf_next[j];
     }  // query tiles
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The forward pass once more for the common full-size case (head dimension exactly 64 on both sides, up to KEYS
+// keys, aligned outputs), laid out so that TWO wavefronts share each SIMD: eight wavefronts per workgroup, each owning
+// 16 queries of the 128-query tile and working in 16x16x4 MFMAs.  A wavefront then holds KEYS/4 score registers
+// instead of KEYS/2 (64 for 256 keys), everything fits in half the register file, and while one wavefront of a SIMD is
+// in its softmax (VALU only) the other keeps the matrix pipe busy.  A workgroup takes several matrices in turn and
+// has the next one's K and V in flight while it finishes the current one.
+// Both MFMA shapes deliver the same flops per cycle; the 16x16 one reads twice the LDS bytes per flop (32 of the
+// 128 bytes per clock a compute unit has).
+//   S^T = K . Q^T      A[i = key][k] from Ks[d][key], B[k][j = query] from registers.  k step s of lane group
+//                      g = lane / 16 stands for d = 16 g + s, so a lane holds 16 consecutive floats of its query row.
+//                      sacc[t][r] = S[query lane % 16][key 16 t + 4 g + r]: four consecutive keys per register group.
+//   O^T = V^T . P^T    step (t, r): B = sacc[t][r] as it lies, A[i = dv][k = g] = Vs[16 t + 4 g + r][16 mt + lane % 16].
+//                      oacc[mt][r] = O[query][16 mt + 4 g + r].
+// Pitches: 16 KP == 16 and 4 VP == 16 (mod 64), so the four lane groups of an operand read hit four different
+// sixteen-bank groups.
+// ---------------------------------------------------------------------------------------------------------------
+template <int KEYS>
+struct Attn16Cfg {
+    static_assert(KEYS % 32 == 0 && KEYS <= 256, "unsupported key count");
+    static constexpr int D = 64;
+    static constexpr int KP = KEYS + 1;  // pitch of Ks[d][key]
+    static constexpr int VP = D + 4;     // pitch of Vs[key][dv]
+    static constexpr int LDS_BYTES = (D * KP + KEYS * VP) * 4;
+};
+
+template <int KEYS>
+__global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p) {
+    using CFG = Attn16Cfg<KEYS>;
+    constexpr int D = CFG::D, KP = CFG::KP, VP = CFG::VP;
+    constexpr int NKT = KEYS / 16;  // key tiles of 16
+    constexpr int NDT = D / 16;     // output column tiles of 16
+    constexpr int NQ = D / 4;       // k steps of the score product = query floats per lane
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float* const Ks = smem;            // [D][KP]
+    float* const Vs = smem + D * KP;   // [KEYS][VP]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int qt0 = blockIdx.x * p.q_tiles;
+    const int qt_end = min(qt0 + p.q_tiles, (p.Tq + AT_BQ - 1) / AT_BQ);
+
+    // Rows past Tq read the last row instead: a query is one column of both products, so what such a lane computes
+    // never meets another row and is never stored.
+    auto load_q = [&](float (&dst)[NQ], int zz, int qrow_index) {
+        const float* qrow = p.Q + batch_offset(split_batch(zz, p.batch_inner), p.sQ, p.sQ2) +
+                            (long long)(qrow_index < p.Tq ? qrow_index : p.Tq - 1) * p.ldq + NQ * g;
+#pragma unroll
+        for (int j = 0; j < NQ / 4; ++j) {
+            f32x4 x;
+            __builtin_memcpy(&x, qrow + 4 * j, 16);
+            dst[4 * j] = x.x, dst[4 * j + 1] = x.y, dst[4 * j + 2] = x.z, dst[4 * j + 3] = x.w;
+        }
+    };
+    // K and V of one matrix on their way to LDS: 16 consecutive threads read one 256-byte row.  The transposing
+    // stores into Ks[d][key] are conflict-free because KP == 1 (mod 64): the 16 x 4 (vector, key) pairs of a
+    // wavefront land in banks 4 v + c + key.  Addresses are clamped and rows past Tk are zeroed only when they are
+    // stored, so nothing waits for these loads before then.
+    constexpr int KIT = (KEYS * (D / 4)) / 512;
+    f32x4 kx[KIT], vx[KIT];
+    // (the thread index goes through an empty asm in both helpers: their address arithmetic is then redone at each
+    // call instead of being carried in registers across the products, where every register counts)
+    auto load_kv = [&](int zz) {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const BatchIndex bz = split_batch(zz, p.batch_inner);
+        const float* Kz = p.K + batch_offset(bz, p.sK, p.sK2);
+        const float* Vz = p.V + batch_offset(bz, p.sV, p.sV2);
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = idx / (D / 4), v = idx % (D / 4);
+            __builtin_memcpy(&kx[it], Kz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldk + 4 * v, 16);
+        }
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = idx / (D / 4), v = idx % (D / 4);
+            __builtin_memcpy(&vx[it], Vz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldv + 4 * v, 16);
+        }
+    };
+    auto store_kv = [&]() {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = idx / (D / 4), v = idx % (D / 4);
+            const f32x4 x = key < p.Tk ? kx[it] : zero;
+            Ks[(4 * v + 0) * KP + key] = x.x;
+            Ks[(4 * v + 1) * KP + key] = x.y;
+            Ks[(4 * v + 2) * KP + key] = x.z;
+            Ks[(4 * v + 3) * KP + key] = x.w;
+        }
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = idx / (D / 4), v = idx % (D / 4);
+            *reinterpret_cast<f32x4*>(Vs + key * VP + 4 * v) = key < p.Tk ? vx[it] : zero;
+        }
+    };
+
+    // A workgroup walks through the matrices z, z + gridDim.y, ...: while it works on the last query tile of one, K
+    // and V of the next are already travelling into registers, so only the first matrix pays for the round trip.
+    // The two wavefronts of a SIMD (w and w + 4: wavefronts are dealt to the four SIMDs in turn) share its matrix
+    // pipe.  Left alone the older one wins most issue slots and finishes a matrix well ahead of the other; a small
+    // standing priority for the younger one evens that out (measured: the pair stays half a product apart, which is
+    // what lets one's softmax run under the other's MFMAs; pacing the two into lockstep is slower).
+    const int mfma_prio = wave >= 4 ? 1 : 0;
+    if (mfma_prio) __builtin_amdgcn_s_setprio(1);
+    int z = blockIdx.y;
+    if (z >= p.batch || qt0 >= qt_end) return;  // uniform
+    float qf[NQ];
+    load_q(qf, z, qt0 * AT_BQ + wave * 16 + l16);
+    load_kv(z);
+
+    for (; z < p.batch; z += gridDim.y) {
+    const int z_next = z + (int)gridDim.y;
+    const bool has_next = z_next < p.batch;  // uniform
+    float* Oz = p.O + batch_offset(split_batch(z, p.batch_inner), p.sO, p.sO2);
+    __syncthreads();  // every wavefront is done with the previous matrix in LDS
+    store_kv();
+    __syncthreads();
+
+    for (int qt = qt0; qt < qt_end; ++qt) {
+        const int q0 = qt * AT_BQ;
+        const int row = q0 + wave * 16 + l16;
+        const bool row_ok = row < p.Tq;
+        const bool last_tile = qt + 1 == qt_end;  // uniform
+
+        // ---- S^T = K . Q^T ----
+        f32x4 sacc[NKT];
+#pragma unroll
+        for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        {
+            const float* kbase = Ks + (NQ * g) * KP + l16;
+            float ka[2][NKT];
+#pragma unroll
+            for (int t = 0; t < NKT; ++t) ka[0][t] = kbase[t * 16];
+#pragma unroll
+            for (int s = 0; s < NQ; ++s) {
+                if (s + 1 < NQ) {
+#pragma unroll
+                    for (int t = 0; t < NKT; ++t) ka[(s + 1) & 1][t] = kbase[(s + 1) * KP + t * 16];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < NKT; ++t)
+                    sacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s & 1][t], qf[s], sacc[t], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // The next matrix is asked for here, behind the score product: the wait the compiler puts in front of that
+        // product's first MFMA (for the queries) covers every load in flight, and these should not be among them.
+        if (last_tile && has_next) load_kv(z_next);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- softmax over the keys of this lane's query (log2 domain: exp(s - max) is one v_exp_f32; a masked score
+        //      - above the diagonal, the reference's -1e12, ScaledDotProductAttentionLayer.cs:73-76, or a key past
+        //      Tk - becomes so negative that its exponential is exactly zero).  Key of register (t, r): 16 t + 4 g + r.
+        //      The VALU stretch runs at raised priority: the SIMD's other wavefront is then usually inside a product,
+        //      always has an MFMA ready, and would otherwise keep winning the issue slot for a pipe that is still busy.
+        __builtin_amdgcn_s_setprio(3);
+        constexpr float kLog2e = 1.44269504088896340736f;
+        constexpr float kMasked = -1e12f * kLog2e;
+        const float sl = p.scale * kLog2e;
+        float m = -3.402823466e+38f;
+        if (p.causal || p.Tk < KEYS) {  // uniform
+            int lim = p.Tk - 1;
+            if (p.causal && row < lim) lim = row;
+            lim -= 4 * g;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float v = sl * sacc[t][r];
+                    v = (t * 16 + r > lim) ? kMasked : v;
+                    sacc[t][r] = v;
+                    m = fmaxf(m, v);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float v = sl * sacc[t][r];
+                    sacc[t][r] = v;
+                    m = fmaxf(m, v);
+                }
+        }
+        m = fmaxf(m, __shfl_xor(m, 16, 64));
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float e = __builtin_amdgcn_exp2f(sacc[t][r] - m);
+                sacc[t][r] = e;
+                sum += e;
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sacc[t][r] *= inv;
+        if (mfma_prio) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
+
+        // ---- P out: 16 bytes (four consecutive keys) per register group.  In a full tile with all keys present the
+        //      stores are spread over the second product instead (uniform choice). ----
+        const bool p_inline = p.P != nullptr && p.Tk == KEYS && q0 + AT_BQ <= p.Tq;
+        if (p.P != nullptr && !p_inline && row_ok) {
+            float* prow = p.P + ((long long)z * p.Tq + row) * p.Tk + 4 * g;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+                if (t * 16 + 4 * g < p.Tk) *reinterpret_cast<f32x4*>(prow + t * 16) = sacc[t];
+        }
+
+        // the next tile's queries (the next matrix's first tile after the last one) travel while this tile's second
+        // product runs
+        float qf_next[NQ];
+        if (!last_tile)
+            load_q(qf_next, z, q0 + AT_BQ + wave * 16 + l16);
+        else
+            load_q(qf_next, has_next ? z_next : z, qt0 * AT_BQ + wave * 16 + l16);
+
+        // ---- O^T = V^T . P^T ----
+        f32x4 oacc[NDT];
+#pragma unroll
+        for (int mt = 0; mt < NDT; ++mt) oacc[mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        auto second_product = [&](auto store_tag) {
+            constexpr bool STORE_P = decltype(store_tag)::value;
+            constexpr int NSTEP = NKT * 4;
+            constexpr int LOOK = 3;  // k steps of look-ahead for the LDS reads of V
+            const float* vbase = Vs + (4 * g) * VP + l16;
+            float* const prow = STORE_P ? p.P + ((long long)z * p.Tq + row) * p.Tk + 4 * g : nullptr;
+            float va[4][NDT];
+            auto v_off = [](int i) { return ((i / 4) * 16 + (i % 4)) * VP; };
+#pragma unroll
+            for (int i = 0; i < LOOK; ++i)
+#pragma unroll
+                for (int mt = 0; mt < NDT; ++mt) va[i][mt] = vbase[v_off(i) + mt * 16];
+#pragma unroll
+            for (int i = 0; i < NSTEP; ++i) {
+                if (i + LOOK < NSTEP) {
+#pragma unroll
+                    for (int mt = 0; mt < NDT; ++mt) va[(i + LOOK) % 4][mt] = vbase[v_off(i + LOOK) + mt * 16];
+                }
+                if (STORE_P && i % 4 == 0) *reinterpret_cast<f32x4*>(prow + (i / 4) * 16) = sacc[i / 4];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int mt = 0; mt < NDT; ++mt)
+                    oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(va[i % 4][mt], sacc[i / 4][i % 4], oacc[mt], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        if (p_inline)
+            second_product(std::true_type{});
+        else
+            second_product(std::false_type{});
+        if (row_ok) {
+            float* orow = Oz + (long long)row * p.ldo + 4 * g;
+#pragma unroll
+            for (int mt = 0; mt < NDT; ++mt) *reinterpret_cast<f32x4*>(orow + mt * 16) = oacc[mt];
+        }
+#pragma unroll
+        for (int j = 0; j < NQ; ++j) qf[j] = qf_next[j];
+    }  // query tiles
+    }  // matrices
 }
 
 // ---------------------------------------------------------------------------------------------------------------

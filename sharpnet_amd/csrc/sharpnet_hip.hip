@@ -830,6 +830,9 @@ hipError_t prepare_kernels_once(int dev) {
                                 c.lds_bytes);
         if (e != hipSuccess) return e;
     }
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_kernel<256>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
+    if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd_long_kernel<32>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, AttnCfg<8, 32>::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -987,6 +990,7 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
     p.sQ = d->strideQ, p.sK = d->strideK, p.sV = d->strideV, p.sO = d->strideO;
     p.sQ2 = d->strideQ_outer, p.sK2 = d->strideK_outer, p.sV2 = d->strideV_outer, p.sO2 = d->strideO_outer;
     p.batch_inner = inner;
+    p.batch = d->batch;
     p.scale = d->scale;
     p.causal = d->causal != 0;
     p.flags = 0;
@@ -1013,8 +1017,19 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
     int groups = 1;
     while (groups < tiles && (long long)d->batch * groups < 2LL * h->num_cu) ++groups;
     p.q_tiles = ceil_div(tiles, groups);
-    hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256), e->lds_bytes,
-                       h->stream, p);
+    // the full-size case (head dimension exactly 64 on both sides, 129 to 256 keys, outputs that take 16-byte
+    // stores) has a form of its own with two wavefronts per SIMD
+    if (e->keys == 256 && e->hd == 64 && d->dk == 64 && d->dv == 64 && d->Tk % 4 == 0 && (p.flags & 1) &&
+        (d->weights == nullptr || (p.flags & 2))) {
+        // one workgroup per compute unit (136 KB of LDS), each walking through its share of the matrices
+        const int gx = ceil_div(tiles, p.q_tiles);
+        int gy = h->num_cu / gx;
+        gy = gy < 1 ? 1 : (gy > d->batch ? d->batch : gy);
+        hipLaunchKernelGGL(attention_fwd16_kernel<256>, dim3((unsigned)gx, (unsigned)gy), dim3(512),
+                           Attn16Cfg<256>::LDS_BYTES, h->stream, p);
+    } else
+        hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256),
+                           e->lds_bytes, h->stream, p);
     return hip_to_status(hipGetLastError());
 }
 
@@ -1063,6 +1078,7 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
         p.sQ = d->strideO, p.sK = d->strideV, p.sV = d->strideK, p.sO = d->strideQ;
         p.sQ2 = d->strideO_outer, p.sK2 = d->strideV_outer, p.sV2 = d->strideK_outer, p.sO2 = d->strideQ_outer;
         p.batch_inner = inner;
+        p.batch = d->batch;
         p.scale = d->scale;
         p.causal = 0;
         p.flags = 0;

@@ -387,6 +387,10 @@ def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrap
     (5, 1, 37, 37, 16, 16, False, False), (5, 1, 37, 37, 16, 16, True, False),      # ragged, small tiles
     (2, 3, 256, 256, 64, 64, True, True), (2, 3, 256, 256, 64, 64, False, False),   # the largest supported size
     (3, 2, 200, 130, 24, 40, False, True), (3, 2, 129, 65, 33, 7, True, False),     # Tq != Tk, dk != dv, odd sizes
+    # head dimension exactly 64 and 129 to 256 keys (the form with two wavefronts per SIMD): ragged last query tile,
+    # keys short of 256, three tiles per matrix; 255 keys (not a multiple of 4) stay on the general kernel
+    (3, 2, 200, 132, 64, 64, True, False), (2, 2, 300, 256, 64, 64, False, True), (1, 3, 77, 252, 64, 64, False, False),
+    (2, 1, 384, 200, 64, 64, True, True), (1, 3, 77, 255, 64, 64, True, True),
     (1, 4, 1, 5, 3, 2, False, True),
     (2, 2, 128, 128, 128, 128, True, True), (3, 1, 70, 100, 96, 128, False, False),  # head dimension up to 128: 128 keys
     # more than 256 keys: the two-pass kernel over key blocks (head dimensions that are multiples of 4, up to 64)
