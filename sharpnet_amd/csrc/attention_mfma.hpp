@@ -472,7 +472,12 @@ struct Attn16Cfg {
     static constexpr int LDS_BYTES = (D * KP + KEYS * VP) * 4;
 };
 
-template <int KEYS>
+//
+// BWD: the first half of the backward pass, as in attention_fwd_kernel (Q <- dO, K <- V, V <- K, O <- dQ, P <- dS out,
+// Pin <- the stored softmax output): the first product leaves dP^T in the accumulators, the softmax stretch becomes
+// dS = scale * P * (dP - sum_keys dP * P), the second product is dQ = dS . K.  A lane's 64 values of P are asked for
+// before the first product and wait in registers, so P is read once and its latency is hidden.
+template <int KEYS, bool BWD = false>
 __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p) {
     using CFG = Attn16Cfg<KEYS>;
     constexpr int D = CFG::D, KP = CFG::KP, VP = CFG::VP;
@@ -602,7 +607,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p
         }
         // The next matrix is asked for here, behind the score product: the wait the compiler puts in front of that
         // product's first MFMA (for the queries) covers every load in flight, and these should not be among them.
-        if (last_tile && has_next) load_kv(z_next);
+        if (!BWD && last_tile && has_next) load_kv(z_next);
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- softmax over the keys of this lane's query (log2 domain: exp(s - max) is one v_exp_f32; a masked score
@@ -611,6 +616,28 @@ __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p
         //      The VALU stretch runs at raised priority: the SIMD's other wavefront is then usually inside a product,
         //      always has an MFMA ready, and would otherwise keep winning the issue slot for a pipe that is still busy.
         __builtin_amdgcn_s_setprio(3);
+        if constexpr (BWD) {
+            // keys past Tk: dP is zero there (zero rows of the staged operand) and so is what is taken for P
+            f32x4 pin[NKT];
+            {
+                const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + 4 * g;
+#pragma unroll
+                for (int t = 0; t < NKT; ++t)
+                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : 0), 16);  // past Tk: any valid address
+            }
+            float rs = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t) {
+                if (p.Tk < KEYS && t * 16 + 4 * g >= p.Tk) pin[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                rs += sacc[t].x * pin[t].x + sacc[t].y * pin[t].y + sacc[t].z * pin[t].z + sacc[t].w * pin[t].w;
+            }
+            rs += __shfl_xor(rs, 16, 64);
+            rs += __shfl_xor(rs, 32, 64);
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sacc[t][r] = p.scale * pin[t][r] * (sacc[t][r] - rs);
+        } else {
         constexpr float kLog2e = 1.44269504088896340736f;
         constexpr float kMasked = -1e12f * kLog2e;
         const float sl = p.scale * kLog2e;
@@ -656,7 +683,10 @@ __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p
         for (int t = 0; t < NKT; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) sacc[t][r] *= inv;
+        }
         if (mfma_prio) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
+        if (BWD && last_tile && has_next) load_kv(z_next);  // (behind the stretch that still holds P in registers)
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- P out: 16 bytes (four consecutive keys) per register group.  In a full tile with all keys present the
         //      stores are spread over the second product instead (uniform choice). ----

@@ -833,6 +833,9 @@ hipError_t prepare_kernels_once(int dev) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_kernel<256>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_kernel<256, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
+    if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd_long_kernel<32>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, AttnCfg<8, 32>::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -1092,8 +1095,17 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
         int groups = 1;
         while (groups < tiles && (long long)d->batch * groups < 2LL * h->num_cu) ++groups;
         p.q_tiles = ceil_div(tiles, groups);
-        hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256), e->lds_bytes,
-                           h->stream, p);
+        if (e->keys == 256 && e->hd == 64 && d->dk == 64 && d->dv == 64 && (p.flags & 7) == 7) {
+            // the full-size case, as in the forward call: two wavefronts per SIMD, one workgroup per compute unit
+            const int gx = ceil_div(tiles, p.q_tiles);
+            int gy = h->num_cu / gx;
+            gy = gy < 1 ? 1 : (gy > d->batch ? d->batch : gy);
+            hipLaunchKernelGGL((attention_fwd16_kernel<256, true>), dim3((unsigned)gx, (unsigned)gy), dim3(512),
+                               Attn16Cfg<256>::LDS_BYTES, h->stream, p);
+        } else {
+            hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256),
+                               e->lds_bytes, h->stream, p);
+        }
         st = hip_to_status(hipGetLastError());
         if (st != SNHIP_STATUS_SUCCESS) return st;
     } else {

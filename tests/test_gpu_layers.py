@@ -545,6 +545,9 @@ def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
     (1, 2, 40, 300, 8, 8, False),                                  # beyond 256 keys: the five-launch sequence
     (2, 2, 128, 128, 128, 128, True), (3, 1, 70, 100, 96, 128, False),   # head dimension up to 128
     (1, 2, 60, 200, 80, 80, False),                                # 200 keys x 80: the five-launch sequence
+    # head dimension exactly 64, 129 to 256 keys (two wavefronts per SIMD): ragged query tiles, keys short of 256
+    (3, 2, 200, 132, 64, 64, False), (2, 2, 300, 256, 64, 64, True), (1, 3, 77, 252, 64, 64, False),
+    (2, 1, 384, 200, 64, 64, True),
 ])
 def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, packed):
     """snhip_attention_backward (dV, score gradient through the softmax, dQ, dK; the middle two from one kernel when
