@@ -1024,4 +1024,263 @@ __global__ void __launch_bounds__(256) attention_fwd_long_kernel(const AttnParam
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The two-pass kernel for any number of keys in the layout of attention_fwd16_kernel (head dimension exactly 64 on
+// both sides, a multiple of 4 keys, aligned outputs): eight wavefronts of 16 queries, 16x16x4 MFMAs, two wavefronts per
+// SIMD, and the next key block's K (pass 1) or K and V (pass 2) travelling in registers while the current block is
+// worked on, so that a block change costs the two barriers and the LDS stores but not the round trip to memory.
+// Same passes, same skipping of causal blocks and the same zero-fill of the skipped weights as
+// attention_fwd_long_kernel.
+// ---------------------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnParams p) {
+    constexpr int KEYS = 256;
+    using CFG = Attn16Cfg<KEYS>;
+    constexpr int D = CFG::D, KP = CFG::KP, VP = CFG::VP;
+    constexpr int NKT = KEYS / 16, NDT = D / 16, NQ = D / 4;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float* const Ks = smem;            // [D][KP]
+    float* const Vs = smem + D * KP;   // [KEYS][VP]
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int z = blockIdx.x;  // matrices run fastest in the grid, query tiles slowest, last tile first
+    const BatchIndex bi = split_batch(z, p.batch_inner);
+    const float* Kz = p.K + batch_offset(bi, p.sK, p.sK2);
+    const float* Vz = p.V + batch_offset(bi, p.sV, p.sV2);
+    const int q0 = (int)(gridDim.y - 1 - blockIdx.y) * AT_BQ;
+    const int row = q0 + wave * 16 + l16;
+    const bool row_ok = row < p.Tq;
+
+    // qf[s] = Q[row][16 (lane / 16) + s]; rows past Tq read the last row (never stored)
+    float qf[NQ];
+    {
+        const float* qrow = p.Q + batch_offset(bi, p.sQ, p.sQ2) + (long long)(row_ok ? row : p.Tq - 1) * p.ldq + NQ * g;
+#pragma unroll
+        for (int j = 0; j < NQ / 4; ++j) {
+            f32x4 x;
+            __builtin_memcpy(&x, qrow + 4 * j, 16);
+            qf[4 * j] = x.x, qf[4 * j + 1] = x.y, qf[4 * j + 2] = x.z, qf[4 * j + 3] = x.w;
+        }
+    }
+
+    const int nblocks = (p.Tk + KEYS - 1) / KEYS;
+    int nb_needed = nblocks;  // causal: the last query of the tile sees keys 0 .. q0 + 127
+    if (p.causal) {
+        const int last_row = (q0 + AT_BQ - 1 < p.Tq - 1) ? q0 + AT_BQ - 1 : p.Tq - 1;
+        const int nb = last_row / KEYS + 1;
+        nb_needed = nb < nblocks ? nb : nblocks;
+    }
+
+    // one key block on its way to LDS (16 lanes to a 256-byte row; clamped addresses, rows past Tk zeroed when stored;
+    // the thread index goes through an empty asm so that the address arithmetic is redone at each call instead of
+    // being carried in registers across the products)
+    constexpr int KIT = (KEYS * (D / 4)) / 512;
+    f32x4 kx[KIT], vx[KIT];
+    auto load_block = [&](const float* base, int ld, int kb, f32x4 (&dst)[KIT]) {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = kb * KEYS + idx / (D / 4), v = idx % (D / 4);
+            __builtin_memcpy(&dst[it], base + (long long)(key < p.Tk ? key : p.Tk - 1) * ld + 4 * v, 16);
+        }
+    };
+    auto store_k = [&](int kb) {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = idx / (D / 4), v = idx % (D / 4);
+            const f32x4 x = kb * KEYS + key < p.Tk ? kx[it] : zero;
+            Ks[(4 * v + 0) * KP + key] = x.x;
+            Ks[(4 * v + 1) * KP + key] = x.y;
+            Ks[(4 * v + 2) * KP + key] = x.z;
+            Ks[(4 * v + 3) * KP + key] = x.w;
+        }
+    };
+    auto store_v = [&](int kb) {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = idx / (D / 4), v = idx % (D / 4);
+            *reinterpret_cast<f32x4*>(Vs + key * VP + 4 * v) = kb * KEYS + key < p.Tk ? vx[it] : zero;
+        }
+    };
+
+    constexpr float kLog2e = 1.44269504088896340736f;
+    constexpr float kMasked = -1e12f * kLog2e;
+    const float sl = p.scale * kLog2e;
+    const int mfma_prio = wave >= 4 ? 1 : 0;  // see attention_fwd16_kernel
+    auto product_priority = [&]() {
+        if (mfma_prio)
+            __builtin_amdgcn_s_setprio(1);
+        else
+            __builtin_amdgcn_s_setprio(0);
+    };
+
+    // raw scores of the block in LDS: sacc[t][r] belongs to key kb * 256 + 16 t + 4 g + r
+    f32x4 sacc[NKT];
+    auto score_product = [&]() {
+#pragma unroll
+        for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        const float* kbase = Ks + (NQ * g) * KP + l16;
+        float ka[2][NKT];
+#pragma unroll
+        for (int t = 0; t < NKT; ++t) ka[0][t] = kbase[t * 16];
+#pragma unroll
+        for (int s = 0; s < NQ; ++s) {
+            if (s + 1 < NQ) {
+#pragma unroll
+                for (int t = 0; t < NKT; ++t) ka[(s + 1) & 1][t] = kbase[(s + 1) * KP + t * 16];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+                sacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s & 1][t], qf[s], sacc[t], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // log2-domain scores with the mask (a key past Tk or above the diagonal becomes kMasked: its exponential is 0)
+    auto scale_and_mask = [&](int kb) {
+        int lim = p.Tk - 1;
+        if (p.causal && row < lim) lim = row;
+        lim -= kb * KEYS + 4 * g;
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float v = sl * sacc[t][r];
+                sacc[t][r] = (t * 16 + r > lim) ? kMasked : v;
+            }
+    };
+
+    // ---- pass 1: row maximum and row sum over all needed blocks ----
+    float m = -3.402823466e+38f, l = 0.0f;
+    load_block(Kz, p.ldk, 0, kx);
+    product_priority();
+    for (int kb = 0; kb < nb_needed; ++kb) {
+        __syncthreads();  // every wavefront is done with the previous block
+        store_k(kb);
+        __syncthreads();
+        score_product();
+        // the next block is asked for behind the product (the wait in front of a loop body's first MFMA covers every
+        // load in flight); after the last block of this pass that is the first block of the next one
+        if (kb + 1 < nb_needed) {
+            load_block(Kz, p.ldk, kb + 1, kx);
+        } else {
+            load_block(Kz, p.ldk, 0, kx);
+            load_block(Vz, p.ldv, 0, vx);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(3);
+        scale_and_mask(kb);
+        float bm = -3.402823466e+38f;
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) bm = fmaxf(bm, sacc[t][r]);
+        bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+        bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+        const float m_new = fmaxf(m, bm);
+        float bs = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) bs += __builtin_amdgcn_exp2f(sacc[t][r] - m_new);
+        bs += __shfl_xor(bs, 16, 64);
+        bs += __shfl_xor(bs, 32, 64);
+        l = l * __builtin_amdgcn_exp2f(m - m_new) + bs;
+        m = m_new;
+        product_priority();
+    }
+    const float inv = 1.0f / l;
+
+    // ---- pass 2: probabilities, P out, O += P . V ----
+    f32x4 oacc[NDT];
+#pragma unroll
+    for (int mt = 0; mt < NDT; ++mt) oacc[mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    float* const pbase = (p.P != nullptr) ? p.P + ((long long)z * p.Tq + (row_ok ? row : 0)) * p.Tk + 4 * g : nullptr;
+    for (int kb = 0; kb < nb_needed; ++kb) {
+        __syncthreads();
+        store_k(kb);
+        store_v(kb);
+        __syncthreads();
+        score_product();
+        if (kb + 1 < nb_needed) {
+            load_block(Kz, p.ldk, kb + 1, kx);
+            load_block(Vz, p.ldv, kb + 1, vx);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(3);
+        scale_and_mask(kb);
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sacc[t][r] = __builtin_amdgcn_exp2f(sacc[t][r] - m) * inv;
+        product_priority();
+
+        // P out: inside the second product when the whole block and the whole tile exist (uniform), else here
+        const bool p_inline = pbase != nullptr && (kb + 1) * KEYS <= p.Tk && q0 + AT_BQ <= p.Tq;
+        if (pbase != nullptr && !p_inline && row_ok) {
+            float* prow = pbase + kb * KEYS;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+                if (kb * KEYS + t * 16 + 4 * g < p.Tk) *reinterpret_cast<f32x4*>(prow + t * 16) = sacc[t];
+        }
+        auto second_product = [&](auto store_tag) {
+            constexpr bool STORE_P = decltype(store_tag)::value;
+            constexpr int NSTEP = NKT * 4;
+            constexpr int LOOK = 3;  // k steps of look-ahead for the LDS reads of V
+            const float* vbase = Vs + (4 * g) * VP + l16;
+            float* const prow = STORE_P ? pbase + kb * KEYS : nullptr;
+            float va[4][NDT];
+            auto v_off = [](int i) { return ((i / 4) * 16 + (i % 4)) * VP; };
+#pragma unroll
+            for (int i = 0; i < LOOK; ++i)
+#pragma unroll
+                for (int mt = 0; mt < NDT; ++mt) va[i][mt] = vbase[v_off(i) + mt * 16];
+#pragma unroll
+            for (int i = 0; i < NSTEP; ++i) {
+                if (i + LOOK < NSTEP) {
+#pragma unroll
+                    for (int mt = 0; mt < NDT; ++mt) va[(i + LOOK) % 4][mt] = vbase[v_off(i + LOOK) + mt * 16];
+                }
+                if (STORE_P && i % 4 == 0) *reinterpret_cast<f32x4*>(prow + (i / 4) * 16) = sacc[i / 4];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int mt = 0; mt < NDT; ++mt)
+                    oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(va[i % 4][mt], sacc[i / 4][i % 4], oacc[mt], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        if (p_inline)
+            second_product(std::true_type{});
+        else
+            second_product(std::false_type{});
+    }
+    __builtin_amdgcn_s_setprio(0);
+
+    // causal: the blocks that were skipped hold zeros in the stored probabilities (a wavefront clears whole rows, lanes
+    // along the keys: consecutive 16-byte stores, full lines)
+    if (p.P != nullptr && nb_needed < nblocks) {  // uniform
+        const int first = nb_needed * KEYS, ncol = p.Tk - first;
+        for (int r = wave; r < AT_BQ && q0 + r < p.Tq; r += 8) {
+            float* prow = p.P + ((long long)z * p.Tq + q0 + r) * p.Tk + first;
+            for (int c = 4 * lane; c < ncol; c += 256) *reinterpret_cast<f32x4*>(prow + c) = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+
+    if (row_ok) {
+        float* orow = p.O + batch_offset(bi, p.sO, p.sO2) + (long long)row * p.ldo + 4 * g;
+#pragma unroll
+        for (int mt = 0; mt < NDT; ++mt) *reinterpret_cast<f32x4*>(orow + mt * 16) = oacc[mt];
+    }
+}
+
 }  // namespace snhip

@@ -836,6 +836,9 @@ hipError_t prepare_kernels_once(int dev) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_kernel<256, true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
+    if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd_long_kernel<32>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, AttnCfg<8, 32>::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -1007,7 +1010,11 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
         if (tiles > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
         p.q_tiles = 1;
         constexpr int lds32 = AttnCfg<8, 32>::LDS_BYTES, lds64 = AttnCfg<8, 64>::LDS_BYTES;
-        if (hd <= 32)
+        // head dimension exactly 64 and outputs that take 16-byte stores: the form with two wavefronts per SIMD
+        if (d->dk == 64 && d->dv == 64 && d->Tk % 4 == 0 && (p.flags & 1) && (d->weights == nullptr || (p.flags & 2)))
+            hipLaunchKernelGGL(attention_fwd16_long_kernel, dim3((unsigned)d->batch, (unsigned)tiles), dim3(512),
+                               Attn16Cfg<256>::LDS_BYTES, h->stream, p);
+        else if (hd <= 32)
             hipLaunchKernelGGL(attention_fwd_long_kernel<32>, dim3((unsigned)d->batch, (unsigned)tiles), dim3(256), lds32,
                                h->stream, p);
         else

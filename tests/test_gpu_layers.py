@@ -398,6 +398,9 @@ def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrap
     (1, 2, 1024, 1024, 32, 32, True, True), (1, 1, 1024, 1024, 64, 64, False, False),
     (1, 3, 300, 700, 24, 40, False, False), (1, 2, 700, 300, 64, 16, True, True), (1, 1, 2048, 2048, 64, 64, True, False),
     (2, 1, 257, 257, 8, 4, True, False),
+    # ... head dimension exactly 64 (two wavefronts per SIMD): ragged query tiles and a last key block short of 256,
+    # with and without the mask; 770 keys (not a multiple of 4) stay on the general two-pass kernel
+    (2, 2, 300, 700, 64, 64, True, False), (1, 3, 650, 516, 64, 64, False, True), (1, 1, 130, 770, 64, 64, True, True),
 ])
 def test_fused_attention_forward(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, causal, packed):
     """snhip_attention_forward (scores, mask, softmax and P.V in one launch) against the oracle's
