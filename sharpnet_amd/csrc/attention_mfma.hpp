@@ -1030,8 +1030,10 @@ __global__ void __launch_bounds__(256) attention_fwd_long_kernel(const AttnParam
 // SIMD, and the next key block's K (pass 1) or K and V (pass 2) travelling in registers while the current block is
 // worked on, so that a block change costs the two barriers and the LDS stores but not the round trip to memory.
 // Same passes, same skipping of causal blocks and the same zero-fill of the skipped weights as
-// attention_fwd_long_kernel.
+// attention_fwd_long_kernel.  ONE_PASS is for callers that do not keep the weights (P == nullptr, inference): a single
+// walk over the key blocks with a running maximum and sum (two thirds of the MFMA work).
 // ---------------------------------------------------------------------------------------------------------------
+template <bool ONE_PASS>
 __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnParams p) {
     constexpr int KEYS = 256;
     using CFG = Attn16Cfg<KEYS>;
@@ -1163,8 +1165,9 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
     // ---- pass 1: row maximum and row sum over all needed blocks ----
     float m = -3.402823466e+38f, l = 0.0f;
     load_block(Kz, p.ldk, 0, kx);
+    if constexpr (ONE_PASS) load_block(Vz, p.ldv, 0, vx);
     product_priority();
-    for (int kb = 0; kb < nb_needed; ++kb) {
+    for (int kb = 0; !ONE_PASS && kb < nb_needed; ++kb) {
         __syncthreads();  // every wavefront is done with the previous block
         store_k(kb);
         __syncthreads();
@@ -1199,9 +1202,11 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         m = m_new;
         product_priority();
     }
-    const float inv = 1.0f / l;
+    const float inv = ONE_PASS ? 1.0f : 1.0f / l;
 
-    // ---- pass 2: probabilities, P out, O += P . V ----
+    // ---- pass 2: probabilities, P out, O += P . V.  ONE_PASS (no weights kept): this is the only pass; maximum and
+    //      sum run along with the blocks, the output is rescaled whenever the maximum moves (a multiplication by
+    //      exp2(0) = 1 otherwise) and divided by the sum at the end. ----
     f32x4 oacc[NDT];
 #pragma unroll
     for (int mt = 0; mt < NDT; ++mt) oacc[mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -1219,10 +1224,38 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(3);
         scale_and_mask(kb);
+        if constexpr (ONE_PASS) {
+            float bm = -3.402823466e+38f;
 #pragma unroll
-        for (int t = 0; t < NKT; ++t)
+            for (int t = 0; t < NKT; ++t)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sacc[t][r] = __builtin_amdgcn_exp2f(sacc[t][r] - m) * inv;
+                for (int r = 0; r < 4; ++r) bm = fmaxf(bm, sacc[t][r]);
+            bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+            bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+            const float m_new = fmaxf(m, bm);
+            const float shrink = __builtin_amdgcn_exp2f(m - m_new);
+            float bs = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float e = __builtin_amdgcn_exp2f(sacc[t][r] - m_new);
+                    sacc[t][r] = e;
+                    bs += e;
+                }
+            bs += __shfl_xor(bs, 16, 64);
+            bs += __shfl_xor(bs, 32, 64);
+            l = l * shrink + bs;
+            m = m_new;
+            // oacc[mt][r] belongs to query lane % 16 as well (O^T: the query is the column), so the lane's own factor applies
+#pragma unroll
+            for (int mt = 0; mt < NDT; ++mt) oacc[mt] *= shrink;
+        } else {
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sacc[t][r] = __builtin_amdgcn_exp2f(sacc[t][r] - m) * inv;
+        }
         product_priority();
 
         // P out: inside the second product when the whole block and the whole tile exist (uniform), else here
@@ -1278,8 +1311,9 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
 
     if (row_ok) {
         float* orow = p.O + batch_offset(bi, p.sO, p.sO2) + (long long)row * p.ldo + 4 * g;
+        const float norm = ONE_PASS ? 1.0f / l : 1.0f;
 #pragma unroll
-        for (int mt = 0; mt < NDT; ++mt) *reinterpret_cast<f32x4*>(orow + mt * 16) = oacc[mt];
+        for (int mt = 0; mt < NDT; ++mt) *reinterpret_cast<f32x4*>(orow + mt * 16) = oacc[mt] * norm;
     }
 }
 

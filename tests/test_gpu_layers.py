@@ -431,11 +431,16 @@ def test_fused_attention_forward(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, caus
                                              scale=scale, is_causal=causal, packed=packed)
     assert np.max(np.abs(gw.ToNumpy() - wref)) <= 2e-6 + 1e-5 * float(np.max(wref))
     assert np.max(np.abs(go.ToNumpy() - lay(oref, Tq, dv))) <= 1e-5 * max(1.0, float(np.max(np.abs(v))))
-    # inference form: no weights requested, same output
+    # inference form: no weights requested, same output - bit for bit where the same kernel runs without its stores;
+    # beyond 256 keys a call without weights may take a single pass with a running maximum instead (other rounding)
     go2 = GPUTensor(go.Shape, None, gpu_wrapper)
+    go2.SetValue(float("nan"))
     assert attention.fused_attention_forward(gq, gk, gv, go2, None, batch=B, heads=H, tq=Tq, tkv=Tk, dk=dk, dv=dv,
                                              scale=scale, is_causal=causal, packed=packed)
-    assert np.array_equal(go2.ToNumpy(), go.ToNumpy())
+    if Tk <= 256:
+        assert np.array_equal(go2.ToNumpy(), go.ToNumpy())
+    else:
+        assert np.max(np.abs(go2.ToNumpy() - lay(oref, Tq, dv))) <= 1e-5 * max(1.0, float(np.max(np.abs(v))))
 
 
 def test_fused_attention_limits(gpu_wrapper):
