@@ -217,7 +217,8 @@ int snhip_activation_backward(void* handle, int activation, float activation_par
  * Q is Tq x dk, K is Tk x dk, V is Tk x dv, O is Tq x dv, each with its own row pitch and two-level batch strides as in
  * snhip_gemm_desc, so heads can be read from and written to a (batch, steps, heads * dim) activation in place.
  * Supported: any Tk with dk, dv <= 64 (beyond 256 keys: dk and dv multiples of 4; the keys are then walked in blocks
- * of 256 in two passes, row maximum and sum first, so the stored weights are final when they are written), or
+ * of 256 in two passes, row maximum and sum first, so the stored weights are final when they are written; without
+ * `weights` the output may come from a single pass with a running maximum, which rounds differently), or
  * Tk <= 128 with dk, dv <= 128; anything else returns status 15 (NOT_SUPPORTED) and the caller issues the reference's
  * sequence of calls instead. */
 typedef struct snhip_attention_desc {
