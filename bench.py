@@ -597,6 +597,25 @@ def layer_timings(w, wl):
                     "forward_ms": f, "backward_ms": round(fb - f, 4)})
     for t in (q, k, v, o, dq, dk_, dv_, do):
         t.Dispose()
+    # more than 256 keys: 64 matrices of 1024 x 1024, head dimension 64 (key blocks of 256; two passes when the weights
+    # are kept, one with a running maximum when they are not)
+    Z, Tn, d = 64, 1024, 64
+    q, k, v = T((Z, Tn, d)), T((Z, Tn, d)), T((Z, Tn, d))
+    o = GPUTensor([Z, Tn, d], None, w)
+    for training in (True, False):
+        for fused in (True, False):
+            for causal in (False, True):
+                def sdpa_long():
+                    wts = attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, training, True, causal, fused=fused)
+                    if wts is not None:
+                        wts.Dispose()
+                ms = timed(sdpa_long, 10, 5)
+                res.append({"layer": "ScaledDotProductAttention forward 64 x (1024 x 64)%s, weights %s" %
+                                     (", causal" if causal else "", "kept" if training else "not kept"),
+                            "form": "one launch" if fused else "reference sequence (4 calls)", "forward_ms": ms,
+                            "backward_ms": float("nan")})
+    for t in (q, k, v, o):
+        t.Dispose()
     B, Tn, H, d = 64, 256, 8, 64
     E = H * d
     Q, K, V, dy = T((B, Tn, E)), T((B, Tn, E)), T((B, Tn, E)), T((B, Tn, E))
