@@ -447,7 +447,7 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// The forward pass once more for the common full-size case (head dimension exactly 64 on both sides, up to KEYS
+// The forward pass once more for the common sizes (head dimension exactly HD = 32 or 64 on both sides, up to KEYS
 // keys, aligned outputs), laid out so that TWO wavefronts share each SIMD: eight wavefronts per workgroup, each owning
 // 16 queries of the 128-query tile and working in 16x16x4 MFMAs.  A wavefront then holds KEYS/4 score registers
 // instead of KEYS/2 (64 for 256 keys), everything fits in half the register file, and while one wavefront of a SIMD is
@@ -456,18 +456,21 @@ __global__ void __launch_bounds__(256) attention_fwd_kernel(const AttnParams p) 
 // Both MFMA shapes deliver the same flops per cycle; the 16x16 one reads twice the LDS bytes per flop (32 of the
 // 128 bytes per clock a compute unit has).
 //   S^T = K . Q^T      A[i = key][k] from Ks[d][key], B[k][j = query] from registers.  k step s of lane group
-//                      g = lane / 16 stands for d = 16 g + s, so a lane holds 16 consecutive floats of its query row.
+//                      g = lane / 16 stands for d = (HD / 4) g + s, so a lane holds HD / 4 consecutive floats of its
+//                      query row.
 //                      sacc[t][r] = S[query lane % 16][key 16 t + 4 g + r]: four consecutive keys per register group.
 //   O^T = V^T . P^T    step (t, r): B = sacc[t][r] as it lies, A[i = dv][k = g] = Vs[16 t + 4 g + r][16 mt + lane % 16].
 //                      oacc[mt][r] = O[query][16 mt + 4 g + r].
-// Pitches: 16 KP == 16 and 4 VP == 16 (mod 64), so the four lane groups of an operand read hit four different
+// Pitches: (HD / 4) KP == 16 and 4 VP == 16 (mod 64), so the four lane groups of an operand read hit four different
 // sixteen-bank groups.
 // ---------------------------------------------------------------------------------------------------------------
-template <int KEYS>
+template <int KEYS, int HD = 64>
 struct Attn16Cfg {
-    static_assert(KEYS % 32 == 0 && KEYS <= 256, "unsupported key count");
-    static constexpr int D = 64;
-    static constexpr int KP = KEYS + 1;  // pitch of Ks[d][key]
+    static_assert(KEYS % 32 == 0 && KEYS <= 256 && (HD == 32 || HD == 64), "unsupported attention tile");
+    static constexpr int D = HD;
+    // pitch of Ks[d][key]: (D / 4) * KP == 16 (mod 64) spreads the four lane groups of an operand read, and the
+    // transposing stores of a wavefront (D / 4 vectors of 64 / (D / 4) keys) land in 64 different banks
+    static constexpr int KP = KEYS + (HD == 64 ? 1 : 2);
     static constexpr int VP = D + 4;     // pitch of Vs[key][dv]
     static constexpr int LDS_BYTES = (D * KP + KEYS * VP) * 4;
 };
@@ -477,9 +480,9 @@ struct Attn16Cfg {
 // Pin <- the stored softmax output): the first product leaves dP^T in the accumulators, the softmax stretch becomes
 // dS = scale * P * (dP - sum_keys dP * P), the second product is dQ = dS . K.  A lane's 64 values of P are asked for
 // before the first product and wait in registers, so P is read once and its latency is hidden.
-template <int KEYS, bool BWD = false>
+template <int KEYS, bool BWD = false, int HD = 64>
 __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p) {
-    using CFG = Attn16Cfg<KEYS>;
+    using CFG = Attn16Cfg<KEYS, HD>;
     constexpr int D = CFG::D, KP = CFG::KP, VP = CFG::VP;
     constexpr int NKT = KEYS / 16;  // key tiles of 16
     constexpr int NDT = D / 16;     // output column tiles of 16

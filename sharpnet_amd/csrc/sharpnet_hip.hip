@@ -265,6 +265,26 @@ constexpr AttnEntry attn_bwd_entry() {
 const AttnEntry kAttnBwd[] = {attn_bwd_entry<2, 32>(), attn_bwd_entry<4, 32>(), attn_bwd_entry<8, 32>(),
                               attn_bwd_entry<2, 64>(), attn_bwd_entry<4, 64>(), attn_bwd_entry<8, 64>()};
 
+// The same for head dimension exactly 32 or 64 and 65 to 256 keys: attention_fwd16_kernel (two wavefronts per SIMD)
+struct Attn16Entry {
+    int keys, hd, lds_bytes;
+    void (*fn)(const AttnParams);
+};
+template <int KEYS, int HD, bool BWD>
+constexpr Attn16Entry attn16_entry() {
+    return Attn16Entry{KEYS, HD, Attn16Cfg<KEYS, HD>::LDS_BYTES, attention_fwd16_kernel<KEYS, BWD, HD>};
+}
+const Attn16Entry kAttn16[] = {attn16_entry<128, 32, false>(), attn16_entry<256, 32, false>(),
+                               attn16_entry<128, 64, false>(), attn16_entry<256, 64, false>()};
+const Attn16Entry kAttn16Bwd[] = {attn16_entry<128, 32, true>(), attn16_entry<256, 32, true>(),
+                                  attn16_entry<128, 64, true>(), attn16_entry<256, 64, true>()};
+template <int N>
+const Attn16Entry* find_attn16(const Attn16Entry (&table)[N], int keys, int hd) {
+    for (const Attn16Entry& c : table)
+        if (c.keys == keys && c.hd == hd) return &c;
+    return nullptr;
+}
+
 int hip_to_status(hipError_t e) {
     switch (e) {
         case hipSuccess:
@@ -830,12 +850,16 @@ hipError_t prepare_kernels_once(int dev) {
                                 c.lds_bytes);
         if (e != hipSuccess) return e;
     }
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_kernel<256>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_kernel<256, true>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
-    if (e != hipSuccess) return e;
+    for (const Attn16Entry& c : kAttn16) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                c.lds_bytes);
+        if (e != hipSuccess) return e;
+    }
+    for (const Attn16Entry& c : kAttn16Bwd) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(c.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                c.lds_bytes);
+        if (e != hipSuccess) return e;
+    }
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -1032,14 +1056,14 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
     p.q_tiles = ceil_div(tiles, groups);
     // the full-size case (head dimension exactly 64 on both sides, 129 to 256 keys, outputs that take 16-byte
     // stores) has a form of its own with two wavefronts per SIMD
-    if (e->keys == 256 && e->hd == 64 && d->dk == 64 && d->dv == 64 && d->Tk % 4 == 0 && (p.flags & 1) &&
+    const Attn16Entry* e16 = find_attn16(kAttn16, e->keys, e->hd);
+    if (e16 != nullptr && d->dk == e->hd && d->dv == e->hd && d->Tk % 4 == 0 && (p.flags & 1) &&
         (d->weights == nullptr || (p.flags & 2))) {
-        // one workgroup per compute unit (136 KB of LDS), each walking through its share of the matrices
+        // one workgroup per compute unit, each walking through its share of the matrices
         const int gx = ceil_div(tiles, p.q_tiles);
         int gy = h->num_cu / gx;
         gy = gy < 1 ? 1 : (gy > d->batch ? d->batch : gy);
-        hipLaunchKernelGGL(attention_fwd16_kernel<256>, dim3((unsigned)gx, (unsigned)gy), dim3(512),
-                           Attn16Cfg<256>::LDS_BYTES, h->stream, p);
+        hipLaunchKernelGGL(e16->fn, dim3((unsigned)gx, (unsigned)gy), dim3(512), e16->lds_bytes, h->stream, p);
     } else
         hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256),
                            e->lds_bytes, h->stream, p);
@@ -1105,13 +1129,14 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
         int groups = 1;
         while (groups < tiles && (long long)d->batch * groups < 2LL * h->num_cu) ++groups;
         p.q_tiles = ceil_div(tiles, groups);
-        if (e->keys == 256 && e->hd == 64 && d->dk == 64 && d->dv == 64 && (p.flags & 7) == 7) {
-            // the full-size case, as in the forward call: two wavefronts per SIMD, one workgroup per compute unit
+        const Attn16Entry* e16 = find_attn16(kAttn16Bwd, e->keys, e->hd);
+        if (e16 != nullptr && d->dk == e->hd && d->dv == e->hd && (p.flags & 7) == 7) {
+            // head dimension exactly 32 or 64, as in the forward call: two wavefronts per SIMD, one workgroup per
+            // compute unit
             const int gx = ceil_div(tiles, p.q_tiles);
             int gy = h->num_cu / gx;
             gy = gy < 1 ? 1 : (gy > d->batch ? d->batch : gy);
-            hipLaunchKernelGGL((attention_fwd16_kernel<256, true>), dim3((unsigned)gx, (unsigned)gy), dim3(512),
-                               Attn16Cfg<256>::LDS_BYTES, h->stream, p);
+            hipLaunchKernelGGL(e16->fn, dim3((unsigned)gx, (unsigned)gy), dim3(512), e16->lds_bytes, h->stream, p);
         } else {
             hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256),
                                e->lds_bytes, h->stream, p);

@@ -391,6 +391,10 @@ def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrap
     # keys short of 256, three tiles per matrix; 255 keys (not a multiple of 4) stay on the general kernel
     (3, 2, 200, 132, 64, 64, True, False), (2, 2, 300, 256, 64, 64, False, True), (1, 3, 77, 252, 64, 64, False, False),
     (2, 1, 384, 200, 64, 64, True, True), (1, 3, 77, 255, 64, 64, True, True),
+    # ... and 65 to 128 keys
+    (4, 2, 128, 128, 64, 64, True, True), (3, 2, 100, 68, 64, 64, False, False), (2, 1, 300, 100, 64, 64, True, False),
+    # ... and head dimension exactly 32
+    (2, 2, 256, 256, 32, 32, True, True), (3, 1, 200, 132, 32, 32, False, False), (2, 2, 130, 100, 32, 32, True, False),
     (1, 4, 1, 5, 3, 2, False, True),
     (2, 2, 128, 128, 128, 128, True, True), (3, 1, 70, 100, 96, 128, False, False),  # head dimension up to 128: 128 keys
     # more than 256 keys: the two-pass kernel over key blocks (head dimensions that are multiples of 4, up to 64)
@@ -555,7 +559,8 @@ def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
     (1, 2, 60, 200, 80, 80, False),                                # 200 keys x 80: the five-launch sequence
     # head dimension exactly 64, 129 to 256 keys (two wavefronts per SIMD): ragged query tiles, keys short of 256
     (3, 2, 200, 132, 64, 64, False), (2, 2, 300, 256, 64, 64, True), (1, 3, 77, 252, 64, 64, False),
-    (2, 1, 384, 200, 64, 64, True),
+    (2, 1, 384, 200, 64, 64, True), (2, 3, 128, 128, 64, 64, True), (3, 2, 100, 68, 64, 64, False),
+    (2, 2, 256, 256, 32, 32, True), (3, 1, 200, 132, 32, 32, False), (2, 2, 130, 100, 32, 32, False),
 ])
 def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, packed):
     """snhip_attention_backward (dV, score gradient through the softmax, dQ, dK; the middle two from one kernel when
