@@ -503,6 +503,42 @@ def test_fused_attention_on_views_at_odd_element_offsets(oracle, gpu_wrapper):
     assert o[0] == -3.0 and np.all(o[1 + Z * Tn * d:] == -3.0) and wt[0] == -3.0 and wt[-1] == -3.0
 
 
+@pytest.mark.parametrize("Tq,Tk,d", [(150, 200, 64), (150, 100, 32), (140, 520, 64)])
+def test_fused_attention_inputs_at_odd_element_offsets_outputs_aligned(oracle, gpu_wrapper, Tq, Tk, d):
+    """The kernels with two wavefronts per SIMD ask for 16-byte-aligned outputs but read Q, K and V wherever they lie:
+    inputs that start 1, 2 and 3 floats into their buffers, outputs at the start of theirs; nothing outside the
+    outputs is written."""
+    from sharpnet_amd import GPUTensor, attention
+    rng = np.random.default_rng(43)
+    Z = 3
+    q, k, v = random_tensor(rng, (Z, Tq, d), -1, 1), random_tensor(rng, (Z, Tk, d), -1, 1), random_tensor(rng, (Z, Tk, d), -1, 1)
+    ref, wref = oracle.sdpa_forward(q, k, v, use_scale=True, is_causal=False)
+    views = []
+    for off, x in zip((1, 2, 3), (q, k, v)):
+        flat = np.concatenate([np.full(off, 7.0, np.float32), x.reshape(-1)])
+        g = GPUTensor([flat.size], flat, gpu_wrapper)
+        views.append((g, g.Slice(off, list(x.shape))))
+    obuf = GPUTensor([Z * Tq * d + 8], None, gpu_wrapper)
+    obuf.SetValue(-3.0)
+    wbuf = GPUTensor([Z * Tq * Tk + 8], None, gpu_wrapper)
+    wbuf.SetValue(-3.0)
+    assert attention.fused_attention_forward(views[0][1], views[1][1], views[2][1], obuf.Slice(0, [Z, Tq, d]),
+                                             wbuf.Slice(0, [Z, Tq, Tk]), batch=Z, heads=1, tq=Tq, tkv=Tk, dk=d, dv=d,
+                                             scale=1.0 / np.sqrt(d), is_causal=False, packed=False)
+    o, wt = obuf.ToNumpy(), wbuf.ToNumpy()
+    assert np.max(np.abs(o[:Z * Tq * d].reshape(Z, Tq, d) - ref)) <= 1e-5
+    assert np.max(np.abs(wt[:Z * Tq * Tk].reshape(Z, Tq, Tk) - wref)) <= 1e-5
+    assert np.all(o[Z * Tq * d:] == -3.0) and np.all(wt[Z * Tq * Tk:] == -3.0)
+    # without weights (beyond 256 keys: the single-pass form)
+    obuf.SetValue(-3.0)
+    assert attention.fused_attention_forward(views[0][1], views[1][1], views[2][1], obuf.Slice(0, [Z, Tq, d]), None,
+                                             batch=Z, heads=1, tq=Tq, tkv=Tk, dk=d, dv=d, scale=1.0 / np.sqrt(d),
+                                             is_causal=False, packed=False)
+    o = obuf.ToNumpy()
+    assert np.max(np.abs(o[:Z * Tq * d].reshape(Z, Tq, d) - ref)) <= 1e-5
+    assert np.all(o[Z * Tq * d:] == -3.0)
+
+
 def test_gemm_ex_degenerate_products_keep_the_rest_of_the_epilogue(oracle, gpu_wrapper):
     """alpha == 0 or K == 0: A and B are not read (BLAS rule) but bias, beta * C, gamma * D and the activation still apply,
     and a requested column sum is still produced (zeros for K == 0)."""
