@@ -543,31 +543,44 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
 #pragma unroll
         for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bv[j]));
 
+        // Old values (beta != 0) are asked for four rows at a time, from addresses clamped into the matrix and outside
+        // the per-row conditions, before any of the four rows is stored: one wait per four rows instead of a
+        // load - wait - store round trip per row (the compiler may not move a load across the store of the row
+        // before it: for all it knows they alias).
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
-                if (row >= p.M) continue;
-                float* crow = out + (long long)row * ldo + col0;
-                float v[TN];
+            for (int rc = 0; rc < 4; ++rc) {
+                float cold[4][TN];
+                if (vec_ok && beta != 0.0f) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j) v[j] = alpha * acc_value<PIN>(acc[i][j][r]) + bv[j];
-                if (vec_ok) {
-                    if (beta != 0.0f) {
-                        float c[TN];
-                        load_row_vec<TN>(crow, c);
-#pragma unroll
-                        for (int j = 0; j < TN; ++j) v[j] += beta * c[j];
+                    for (int q = 0; q < 4; ++q) {
+                        const int rq = row_base + TM * (8 * rc + 4 * lhi + q) + i;
+                        load_row_vec<TN>(out + (long long)(rq < p.M ? rq : p.M - 1) * ldo + col0, cold[q]);
                     }
-                    store_row_vec<TN>(crow, v);
-                } else {
+                }
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) {
-                        if (col0 + j < p.N) {
-                            float o = v[j];
-                            if (beta != 0.0f) o += beta * crow[j];
-                            crow[j] = o;
+                for (int r = 4 * rc; r < 4 * rc + 4; ++r) {
+                    const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
+                    if (row >= p.M) continue;
+                    float* crow = out + (long long)row * ldo + col0;
+                    float v[TN];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) v[j] = alpha * acc_value<PIN>(acc[i][j][r]) + bv[j];
+                    if (vec_ok) {
+                        if (beta != 0.0f) {
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) v[j] += beta * cold[r % 4][j];
+                        }
+                        store_row_vec<TN>(crow, v);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) {
+                            if (col0 + j < p.N) {
+                                float o = v[j];
+                                if (beta != 0.0f) o += beta * crow[j];
+                                crow[j] = o;
+                            }
                         }
                     }
                 }
