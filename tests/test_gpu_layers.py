@@ -395,6 +395,8 @@ def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrap
     (4, 2, 128, 128, 64, 64, True, True), (3, 2, 100, 68, 64, 64, False, False), (2, 1, 300, 100, 64, 64, True, False),
     # ... and head dimension exactly 32
     (2, 2, 256, 256, 32, 32, True, True), (3, 1, 200, 132, 32, 32, False, False), (2, 2, 130, 100, 32, 32, True, False),
+    # ... more matrices than compute units: a workgroup walks through several, the next one's K and V prefetched
+    (75, 8, 130, 132, 64, 64, True, True), (700, 1, 100, 100, 64, 64, False, False), (90, 7, 140, 136, 32, 32, True, False),
     (1, 4, 1, 5, 3, 2, False, True),
     (2, 2, 128, 128, 128, 128, True, True), (3, 1, 70, 100, 96, 128, False, False),  # head dimension up to 128: 128 keys
     # more than 256 keys: the two-pass kernel over key blocks (head dimensions that are multiples of 4, up to 64)
@@ -597,6 +599,7 @@ def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
     (3, 2, 200, 132, 64, 64, False), (2, 2, 300, 256, 64, 64, True), (1, 3, 77, 252, 64, 64, False),
     (2, 1, 384, 200, 64, 64, True), (2, 3, 128, 128, 64, 64, True), (3, 2, 100, 68, 64, 64, False),
     (2, 2, 256, 256, 32, 32, True), (3, 1, 200, 132, 32, 32, False), (2, 2, 130, 100, 32, 32, False),
+    (75, 8, 130, 132, 64, 64, True), (700, 1, 100, 100, 64, 64, False), (90, 7, 140, 136, 32, 32, False),
 ])
 def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, packed):
     """snhip_attention_backward (dV, score gradient through the softmax, dQ, dK; the middle two from one kernel when
