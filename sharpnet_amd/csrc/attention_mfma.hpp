@@ -475,6 +475,63 @@ struct Attn16Cfg {
     static constexpr int LDS_BYTES = (D * KP + KEYS * VP) * 4;
 };
 
+// The two products of the 16-query layout, shared by attention_fwd16_kernel and attention_fwd16_long_kernel.
+// S^T = K . Q^T for one wavefront: NKT tiles of 16 keys x 16 queries, K from Ks[d][key] (pitch KP), the lane's NQ query
+// floats as the B operand; the A operands are read from LDS one k step ahead of the MFMAs that use them (the fences
+// keep the scheduler from sinking the reads back next to their use).
+template <int NKT, int NQ, int KP>
+__device__ __forceinline__ void attn16_score_product(const float* Ks, int g, int l16, const float (&qf)[NQ],
+                                                     f32x4 (&sacc)[NKT]) {
+#pragma unroll
+    for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const float* kbase = Ks + (NQ * g) * KP + l16;
+    float ka[2][NKT];
+#pragma unroll
+    for (int t = 0; t < NKT; ++t) ka[0][t] = kbase[t * 16];
+#pragma unroll
+    for (int s = 0; s < NQ; ++s) {
+        if (s + 1 < NQ) {
+#pragma unroll
+            for (int t = 0; t < NKT; ++t) ka[(s + 1) & 1][t] = kbase[(s + 1) * KP + t * 16];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+            sacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s & 1][t], qf[s], sacc[t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// O^T += V^T . P^T for one wavefront: k step (t, r) takes the score register sacc[t][r] as the B operand as it lies and
+// A[i = dv][k = g] = Vs[16 t + 4 g + r][16 mt + lane % 16] (pitch VP), read LOOK steps ahead.  STORE_P: the lane's
+// probabilities go out on the way, one 16-byte store (four consecutive keys, at prow + 16 t) every four k steps.
+template <int NKT, int NDT, int VP, bool STORE_P>
+__device__ __forceinline__ void attn16_second_product(const float* Vs, int g, int l16, const f32x4 (&sacc)[NKT],
+                                                      f32x4 (&oacc)[NDT], float* prow) {
+    constexpr int NSTEP = NKT * 4;
+    constexpr int LOOK = 3;
+    const float* vbase = Vs + (4 * g) * VP + l16;
+    float va[4][NDT];
+    auto v_off = [](int i) { return ((i / 4) * 16 + (i % 4)) * VP; };
+#pragma unroll
+    for (int i = 0; i < LOOK; ++i)
+#pragma unroll
+        for (int mt = 0; mt < NDT; ++mt) va[i][mt] = vbase[v_off(i) + mt * 16];
+#pragma unroll
+    for (int i = 0; i < NSTEP; ++i) {
+        if (i + LOOK < NSTEP) {
+#pragma unroll
+            for (int mt = 0; mt < NDT; ++mt) va[(i + LOOK) % 4][mt] = vbase[v_off(i + LOOK) + mt * 16];
+        }
+        if (STORE_P && i % 4 == 0) *reinterpret_cast<f32x4*>(prow + (i / 4) * 16) = sacc[i / 4];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mt = 0; mt < NDT; ++mt)
+            oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(va[i % 4][mt], sacc[i / 4][i % 4], oacc[mt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 //
 // BWD: the first half of the backward pass, as in attention_fwd_kernel (Q <- dO, K <- V, V <- K, O <- dQ, P <- dS out,
 // Pin <- the stored softmax output): the first product leaves dP^T in the accumulators, the softmax stretch becomes
@@ -588,26 +645,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p
 
         // ---- S^T = K . Q^T ----
         f32x4 sacc[NKT];
-#pragma unroll
-        for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        {
-            const float* kbase = Ks + (NQ * g) * KP + l16;
-            float ka[2][NKT];
-#pragma unroll
-            for (int t = 0; t < NKT; ++t) ka[0][t] = kbase[t * 16];
-#pragma unroll
-            for (int s = 0; s < NQ; ++s) {
-                if (s + 1 < NQ) {
-#pragma unroll
-                    for (int t = 0; t < NKT; ++t) ka[(s + 1) & 1][t] = kbase[(s + 1) * KP + t * 16];
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int t = 0; t < NKT; ++t)
-                    sacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s & 1][t], qf[s], sacc[t], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
+        attn16_score_product<NKT, NQ, KP>(Ks, g, l16, qf, sacc);
         // The next matrix is asked for here, behind the score product: the wait the compiler puts in front of that
         // product's first MFMA (for the queries) covers every load in flight, and these should not be among them.
         if (!BWD && last_tile && has_next) load_kv(z_next);
@@ -713,36 +751,11 @@ __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p
         f32x4 oacc[NDT];
 #pragma unroll
         for (int mt = 0; mt < NDT; ++mt) oacc[mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        auto second_product = [&](auto store_tag) {
-            constexpr bool STORE_P = decltype(store_tag)::value;
-            constexpr int NSTEP = NKT * 4;
-            constexpr int LOOK = 3;  // k steps of look-ahead for the LDS reads of V
-            const float* vbase = Vs + (4 * g) * VP + l16;
-            float* const prow = STORE_P ? p.P + ((long long)z * p.Tq + row) * p.Tk + 4 * g : nullptr;
-            float va[4][NDT];
-            auto v_off = [](int i) { return ((i / 4) * 16 + (i % 4)) * VP; };
-#pragma unroll
-            for (int i = 0; i < LOOK; ++i)
-#pragma unroll
-                for (int mt = 0; mt < NDT; ++mt) va[i][mt] = vbase[v_off(i) + mt * 16];
-#pragma unroll
-            for (int i = 0; i < NSTEP; ++i) {
-                if (i + LOOK < NSTEP) {
-#pragma unroll
-                    for (int mt = 0; mt < NDT; ++mt) va[(i + LOOK) % 4][mt] = vbase[v_off(i + LOOK) + mt * 16];
-                }
-                if (STORE_P && i % 4 == 0) *reinterpret_cast<f32x4*>(prow + (i / 4) * 16) = sacc[i / 4];
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int mt = 0; mt < NDT; ++mt)
-                    oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(va[i % 4][mt], sacc[i / 4][i % 4], oacc[mt], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        };
         if (p_inline)
-            second_product(std::true_type{});
+            attn16_second_product<NKT, NDT, VP, true>(Vs, g, l16, sacc, oacc,
+                                                      p.P + ((long long)z * p.Tq + row) * p.Tk + 4 * g);
         else
-            second_product(std::false_type{});
+            attn16_second_product<NKT, NDT, VP, false>(Vs, g, l16, sacc, oacc, nullptr);
         if (row_ok) {
             float* orow = Oz + (long long)row * p.ldo + 4 * g;
 #pragma unroll
@@ -1131,26 +1144,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
 
     // raw scores of the block in LDS: sacc[t][r] belongs to key kb * 256 + 16 t + 4 g + r
     f32x4 sacc[NKT];
-    auto score_product = [&]() {
-#pragma unroll
-        for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        const float* kbase = Ks + (NQ * g) * KP + l16;
-        float ka[2][NKT];
-#pragma unroll
-        for (int t = 0; t < NKT; ++t) ka[0][t] = kbase[t * 16];
-#pragma unroll
-        for (int s = 0; s < NQ; ++s) {
-            if (s + 1 < NQ) {
-#pragma unroll
-                for (int t = 0; t < NKT; ++t) ka[(s + 1) & 1][t] = kbase[(s + 1) * KP + t * 16];
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int t = 0; t < NKT; ++t)
-                sacc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s & 1][t], qf[s], sacc[t], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
+    auto score_product = [&]() { attn16_score_product<NKT, NQ, KP>(Ks, g, l16, qf, sacc); };
     // log2-domain scores with the mask (a key past Tk or above the diagonal becomes kMasked: its exponential is 0)
     auto scale_and_mask = [&](int kb) {
         int lim = p.Tk - 1;
@@ -1269,36 +1263,10 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
             for (int t = 0; t < NKT; ++t)
                 if (kb * KEYS + t * 16 + 4 * g < p.Tk) *reinterpret_cast<f32x4*>(prow + t * 16) = sacc[t];
         }
-        auto second_product = [&](auto store_tag) {
-            constexpr bool STORE_P = decltype(store_tag)::value;
-            constexpr int NSTEP = NKT * 4;
-            constexpr int LOOK = 3;  // k steps of look-ahead for the LDS reads of V
-            const float* vbase = Vs + (4 * g) * VP + l16;
-            float* const prow = STORE_P ? pbase + kb * KEYS : nullptr;
-            float va[4][NDT];
-            auto v_off = [](int i) { return ((i / 4) * 16 + (i % 4)) * VP; };
-#pragma unroll
-            for (int i = 0; i < LOOK; ++i)
-#pragma unroll
-                for (int mt = 0; mt < NDT; ++mt) va[i][mt] = vbase[v_off(i) + mt * 16];
-#pragma unroll
-            for (int i = 0; i < NSTEP; ++i) {
-                if (i + LOOK < NSTEP) {
-#pragma unroll
-                    for (int mt = 0; mt < NDT; ++mt) va[(i + LOOK) % 4][mt] = vbase[v_off(i + LOOK) + mt * 16];
-                }
-                if (STORE_P && i % 4 == 0) *reinterpret_cast<f32x4*>(prow + (i / 4) * 16) = sacc[i / 4];
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int mt = 0; mt < NDT; ++mt)
-                    oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(va[i % 4][mt], sacc[i / 4][i % 4], oacc[mt], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        };
         if (p_inline)
-            second_product(std::true_type{});
+            attn16_second_product<NKT, NDT, VP, true>(Vs, g, l16, sacc, oacc, pbase + kb * KEYS);
         else
-            second_product(std::false_type{});
+            attn16_second_product<NKT, NDT, VP, false>(Vs, g, l16, sacc, oacc, nullptr);
     }
     __builtin_amdgcn_s_setprio(0);
 
