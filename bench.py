@@ -581,6 +581,20 @@ def layer_timings(w, wl):
                                  (", causal" if causal else ""),
                         "form": "one launch" if fused else "reference sequence (4 calls)", "forward_ms": ms,
                         "backward_ms": float("nan")})
+    # the same launch on a handle in the bf16-input math mode (Q, K, V and the probabilities rounded to bf16 for the MFMAs)
+    w.set_math_mode(1)
+    try:
+        for training in (True, False):
+            def sdpa_bf16():
+                wts = attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, training, True, False, fused=True)
+                if wts is not None:
+                    wts.Dispose()
+            ms = timed(sdpa_bf16, 20, 10)
+            res.append({"layer": "ScaledDotProductAttention forward 512 x (256 x 64), bf16-input math, weights %s" %
+                                 ("kept" if training else "not kept"),
+                        "form": "one launch", "forward_ms": ms, "backward_ms": float("nan")})
+    finally:
+        w.set_math_mode(0)
     dq, dk_, dv_, do = (GPUTensor([Z, Tn, d], None, w) for _ in range(4))
     do.SetValue(0.01)
     for fused in (True, False):

@@ -1041,6 +1041,240 @@ __global__ void __launch_bounds__(256) attention_fwd_long_kernel(const AttnParam
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// attention_fwd16_kernel with bf16-input MFMAs, for handles in the bf16-input math mode (forward, head dimension
+// exactly 64): Q, K and V are rounded to bf16 (nearest even) on their way in, the probabilities on their way into the
+// second product; sums, the softmax and the stored weights stay fp32.  v_mfma_f32_16x16x16_bf16 takes four consecutive
+// k per lane, and its accumulator layout is that of the fp32 16x16x4 shape, so one score register group
+// sacc[t] (keys 16 t + 4 g .. + 3 of query lane % 16), rounded, IS the B operand of a k = 16 step of the second product.
+//   S^T = K . Q^T      A[i = key][k = 4 g ..] = Kb[key][16 s + 4 g ..] (K row-major in LDS, 8-byte reads),
+//                      B = the lane's query floats 16 s + 4 g .. + 3.
+//   O^T = V^T . P^T    A[i = dv][k = 4 g ..] = Vt[dv][16 t + 4 g ..] (V transposed in LDS: keys contiguous).
+// Pitches (in 4-byte words) are 4 (mod 64): the 16 rows x 4 lane groups of an operand read hit 64 different banks.
+// The matrix work shrinks to a sixteenth; what is left is the softmax and the traffic to memory.
+// ---------------------------------------------------------------------------------------------------------------
+typedef short bf16x4_bits __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x4_bits round_to_bf16x4(f32x4 x) {
+    const bf16x4_t h = __builtin_convertvector(x, bf16x4_t);
+    bf16x4_bits b;
+    __builtin_memcpy(&b, &h, 8);
+    return b;
+}
+
+template <int KEYS>
+struct Attn16BCfg {
+    static_assert(KEYS % 32 == 0 && KEYS <= 256, "unsupported key count");
+    static constexpr int D = 64;
+    static constexpr int KP = D + 8;      // pitch of Kb[key][d], bf16 elements (36 words)
+    static constexpr int VP = KEYS + 8;   // pitch of Vt[dv][key], bf16 elements
+    static constexpr int LDS_BYTES = (KEYS * KP + D * VP) * 2;
+};
+
+template <int KEYS>
+__global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnParams p) {
+    using CFG = Attn16BCfg<KEYS>;
+    constexpr int D = CFG::D, KP = CFG::KP, VP = CFG::VP;
+    constexpr int NKT = KEYS / 16, NDT = D / 16, NS = D / 16;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    __bf16* const Kb = reinterpret_cast<__bf16*>(smem);  // [KEYS][KP]
+    __bf16* const Vt = Kb + KEYS * KP;                    // [D][VP]
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int qt0 = blockIdx.x * p.q_tiles;
+    const int qt_end = min(qt0 + p.q_tiles, (p.Tq + AT_BQ - 1) / AT_BQ);
+
+    // the lane's share of its query row, rounded: qb[s] = Q[row][16 s + 4 g .. + 3] (rows past Tq read the last row)
+    auto load_q = [&](f32x4 (&dst)[NS], int zz, int qrow_index) {
+        const float* qrow = p.Q + batch_offset(split_batch(zz, p.batch_inner), p.sQ, p.sQ2) +
+                            (long long)(qrow_index < p.Tq ? qrow_index : p.Tq - 1) * p.ldq + 4 * g;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) __builtin_memcpy(&dst[s], qrow + 16 * s, 16);
+    };
+    // K: 16 lanes to a 256-byte row.  V: a thread takes the same four columns of two adjacent keys, so that it can
+    // write pairs of keys as whole words into the transposed tile.
+    constexpr int KIT = (KEYS * (D / 4)) / 512;
+    f32x4 kx[KIT], vx[KIT];
+    auto load_kv = [&](int zz) {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const BatchIndex bz = split_batch(zz, p.batch_inner);
+        const float* Kz = p.K + batch_offset(bz, p.sK, p.sK2);
+        const float* Vz = p.V + batch_offset(bz, p.sV, p.sV2);
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = idx / (D / 4), v = idx % (D / 4);
+            __builtin_memcpy(&kx[it], Kz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldk + 4 * v, 16);
+        }
+#pragma unroll
+        for (int it = 0; it < KIT / 2; ++it) {
+            const int idx = it * 512 + tid;
+            const int kp = idx % (KEYS / 2), v = idx / (KEYS / 2);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int key = 2 * kp + h;
+                __builtin_memcpy(&vx[2 * it + h], Vz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldv + 4 * v, 16);
+            }
+        }
+    };
+    auto store_kv = [&]() {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int it = 0; it < KIT; ++it) {
+            const int idx = it * 512 + tid;
+            const int key = idx / (D / 4), v = idx % (D / 4);
+            const bf16x4_bits h = round_to_bf16x4(key < p.Tk ? kx[it] : zero);
+            *reinterpret_cast<bf16x4_bits*>(Kb + key * KP + 4 * v) = h;
+        }
+#pragma unroll
+        for (int it = 0; it < KIT / 2; ++it) {
+            const int idx = it * 512 + tid;
+            const int kp = idx % (KEYS / 2), v = idx / (KEYS / 2);
+            const bf16x4_bits lo = round_to_bf16x4(2 * kp < p.Tk ? vx[2 * it] : zero);
+            const bf16x4_bits hi = round_to_bf16x4(2 * kp + 1 < p.Tk ? vx[2 * it + 1] : zero);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const unsigned int w = (unsigned int)(unsigned short)lo[c] | ((unsigned int)(unsigned short)hi[c] << 16);
+                *reinterpret_cast<unsigned int*>(Vt + (4 * v + c) * VP + 2 * kp) = w;
+            }
+        }
+    };
+
+    int z = blockIdx.y;
+    if (z >= p.batch || qt0 >= qt_end) return;  // uniform
+    f32x4 qf[NS];
+    load_q(qf, z, qt0 * AT_BQ + wave * 16 + l16);
+    load_kv(z);
+
+    for (; z < p.batch; z += gridDim.y) {
+    const int z_next = z + (int)gridDim.y;
+    const bool has_next = z_next < p.batch;  // uniform
+    float* Oz = p.O + batch_offset(split_batch(z, p.batch_inner), p.sO, p.sO2);
+    __syncthreads();  // every wavefront is done with the previous matrix in LDS
+    store_kv();
+    __syncthreads();
+
+    for (int qt = qt0; qt < qt_end; ++qt) {
+        const int q0 = qt * AT_BQ;
+        const int row = q0 + wave * 16 + l16;
+        const bool row_ok = row < p.Tq;
+        const bool last_tile = qt + 1 == qt_end;  // uniform
+
+        // ---- S^T = K . Q^T ----
+        f32x4 sacc[NKT];
+#pragma unroll
+        for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        {
+            const __bf16* kbase = Kb + l16 * KP + 4 * g;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const bf16x4_bits qb = round_to_bf16x4(qf[s]);
+                bf16x4_bits ka[NKT];
+#pragma unroll
+                for (int t = 0; t < NKT; ++t) ka[t] = *reinterpret_cast<const bf16x4_bits*>(kbase + t * 16 * KP + 16 * s);
+#pragma unroll
+                for (int t = 0; t < NKT; ++t)
+                    sacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[t], qb, sacc[t], 0, 0, 0);
+            }
+        }
+        // (behind the product: the wait in front of it covers every load in flight, see attention_fwd16_kernel)
+        if (last_tile && has_next) load_kv(z_next);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- softmax over the keys, as in attention_fwd16_kernel ----
+        constexpr float kLog2e = 1.44269504088896340736f;
+        constexpr float kMasked = -1e12f * kLog2e;
+        const float sl = p.scale * kLog2e;
+        float m = -3.402823466e+38f;
+        if (p.causal || p.Tk < KEYS) {  // uniform
+            int lim = p.Tk - 1;
+            if (p.causal && row < lim) lim = row;
+            lim -= 4 * g;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float v = sl * sacc[t][r];
+                    v = (t * 16 + r > lim) ? kMasked : v;
+                    sacc[t][r] = v;
+                    m = fmaxf(m, v);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float v = sl * sacc[t][r];
+                    sacc[t][r] = v;
+                    m = fmaxf(m, v);
+                }
+        }
+        m = fmaxf(m, __shfl_xor(m, 16, 64));
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float e = __builtin_amdgcn_exp2f(sacc[t][r] - m);
+                sacc[t][r] = e;
+                sum += e;
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int t = 0; t < NKT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sacc[t][r] *= inv;
+
+        // ---- P out (fp32, as computed) ----
+        if (p.P != nullptr && row_ok) {
+            float* prow = p.P + ((long long)z * p.Tq + row) * p.Tk + 4 * g;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+                if (p.Tk == KEYS || t * 16 + 4 * g < p.Tk) *reinterpret_cast<f32x4*>(prow + t * 16) = sacc[t];
+        }
+
+        // the next tile's queries (the next matrix's first tile after the last one) travel during the second product
+        f32x4 qf_next[NS];
+        if (!last_tile)
+            load_q(qf_next, z, q0 + AT_BQ + wave * 16 + l16);
+        else
+            load_q(qf_next, has_next ? z_next : z, qt0 * AT_BQ + wave * 16 + l16);
+
+        // ---- O^T = V^T . P^T ----
+        f32x4 oacc[NDT];
+#pragma unroll
+        for (int mt = 0; mt < NDT; ++mt) oacc[mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        {
+            const __bf16* vbase = Vt + l16 * VP + 4 * g;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t) {
+                const bf16x4_bits pb = round_to_bf16x4(sacc[t]);
+#pragma unroll
+                for (int mt = 0; mt < NDT; ++mt) {
+                    const bf16x4_bits va = *reinterpret_cast<const bf16x4_bits*>(vbase + mt * 16 * VP + 16 * t);
+                    oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb, oacc[mt], 0, 0, 0);
+                }
+            }
+        }
+        if (row_ok) {
+            float* orow = Oz + (long long)row * p.ldo + 4 * g;
+#pragma unroll
+            for (int mt = 0; mt < NDT; ++mt) *reinterpret_cast<f32x4*>(orow + mt * 16) = oacc[mt];
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s) qf[s] = qf_next[s];
+    }  // query tiles
+    }  // matrices
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // The two-pass kernel for any number of keys in the layout of attention_fwd16_kernel (head dimension exactly 64 on
 // both sides, a multiple of 4 keys, aligned outputs): eight wavefronts of 16 queries, 16x16x4 MFMAs, two wavefronts per
 // SIMD, and the next key block's K (pass 1) or K and V (pass 2) travelling in registers while the current block is

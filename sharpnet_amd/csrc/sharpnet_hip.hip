@@ -860,6 +860,12 @@ hipError_t prepare_kernels_once(int dev) {
                                 c.lds_bytes);
         if (e != hipSuccess) return e;
     }
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_bf16_kernel<256>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<256>::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_bf16_kernel<128>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<128>::LDS_BYTES);
+    if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -1063,7 +1069,15 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
         const int gx = ceil_div(tiles, p.q_tiles);
         int gy = h->num_cu / gx;
         gy = gy < 1 ? 1 : (gy > d->batch ? d->batch : gy);
-        hipLaunchKernelGGL(e16->fn, dim3((unsigned)gx, (unsigned)gy), dim3(512), e16->lds_bytes, h->stream, p);
+        // a handle in the bf16-input math mode multiplies in bf16 here as it does in its GEMMs (head dimension 64)
+        if (h->math_mode == SNHIP_MATH_BF16_INPUT && e->hd == 64 && e->keys == 256)
+            hipLaunchKernelGGL(attention_fwd16_bf16_kernel<256>, dim3((unsigned)gx, (unsigned)gy), dim3(512),
+                               Attn16BCfg<256>::LDS_BYTES, h->stream, p);
+        else if (h->math_mode == SNHIP_MATH_BF16_INPUT && e->hd == 64 && e->keys == 128)
+            hipLaunchKernelGGL(attention_fwd16_bf16_kernel<128>, dim3((unsigned)gx, (unsigned)gy), dim3(512),
+                               Attn16BCfg<128>::LDS_BYTES, h->stream, p);
+        else
+            hipLaunchKernelGGL(e16->fn, dim3((unsigned)gx, (unsigned)gy), dim3(512), e16->lds_bytes, h->stream, p);
     } else
         hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256),
                            e->lds_bytes, h->stream, p);

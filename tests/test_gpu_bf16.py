@@ -383,3 +383,58 @@ def test_bf16_streaming_kernels_strided_batches(oracle, gpu_wrapper, tA, tB):
                 t.Dispose()
     finally:
         w.set_tuning(-1, 0)
+
+
+@pytest.mark.parametrize("B,H,Tq,Tk,causal,packed", [(2, 3, 256, 256, True, True), (3, 2, 200, 132, False, False),
+                                                       (2, 2, 130, 100, True, False), (70, 8, 130, 136, False, True)])
+def test_attention_forward_in_bf16_input_mode(oracle, gpu_wrapper, B, H, Tq, Tk, causal, packed):
+    """snhip_attention_forward on a handle in the bf16-input math mode (head dimension 64, up to 256 keys): Q, K, V and
+    the probabilities entering the second product are rounded to bf16, sums and softmax stay fp32.
+    Two bars: against the fp32 oracle, 1e-2 of max|V| for the output and 1e-2 of the row maximum ... of the weights
+    (the scores of |q|,|k| <= 1 at scale 1/8 move by at most 64 * 2 * 2^-9 / 8 = 0.03, their exponentials by 3 %);
+    against the same chain on rounded operands: the weights against softmax(scale * Qb . Kb^T) as the fp32 kernels
+    are, and the output against round(weights the kernel wrote) . Vb at 2e-5 (the kernel's own weights, because a
+    weight that lies next to a bf16 rounding boundary may round either way after a last-bit difference in the
+    softmax, and one such flip moves the output by 2^-9 of that weight)."""
+    from sharpnet_amd import GPUTensor, attention
+    rng = np.random.default_rng(71)
+    Z, d = B * H, 64
+    q, k, v = random_tensor(rng, (Z, Tq, d), -1, 1), random_tensor(rng, (Z, Tk, d), -1, 1), random_tensor(rng, (Z, Tk, d), -1, 1)
+    scale = 1.0 / np.sqrt(d)
+
+    def chain(q_, k_, v_, round_p):
+        s = np.stack([oracle.dot(q_[z], False, k_[z], True, scale) for z in range(Z)])
+        if causal:
+            s[:, np.triu_indices(Tq, 1, Tk)[0], np.triu_indices(Tq, 1, Tk)[1]] = -1e12
+        wts = oracle.softmax_last_dim(s)
+        return oracle.bmm(oracle.round_to_bf16(wts) if round_p else wts, False, v_, False), wts
+    o32, w32 = chain(q, k, v, False)
+    obf, wbf = chain(oracle.round_to_bf16(q), oracle.round_to_bf16(k), oracle.round_to_bf16(v), True)
+
+    def lay(x, steps):
+        if not packed:
+            return x
+        return np.ascontiguousarray(x.reshape(B, H, steps, d).transpose(0, 2, 1, 3)).reshape(B, steps, H * d)
+    w = gpu_wrapper
+    gq, gk, gv = (GPUTensor(list(lay(x, t).shape), lay(x, t), w) for x, t in ((q, Tq), (k, Tk), (v, Tk)))
+    go = GPUTensor(list(lay(o32, Tq).shape), None, w)
+    gw = GPUTensor([Z, Tq, Tk], None, w)
+    go.SetValue(float("nan"))
+    gw.SetValue(float("nan"))
+    w.set_math_mode(1)
+    try:
+        assert attention.fused_attention_forward(gq, gk, gv, go, gw, batch=B, heads=H, tq=Tq, tkv=Tk, dk=d, dv=d,
+                                                 scale=scale, is_causal=causal, packed=packed)
+        got_o, got_w = go.ToNumpy(), gw.ToNumpy()
+        go.SetValue(float("nan"))
+        assert attention.fused_attention_forward(gq, gk, gv, go, None, batch=B, heads=H, tq=Tq, tkv=Tk, dk=d, dv=d,
+                                                 scale=scale, is_causal=causal, packed=packed)
+        assert np.array_equal(go.ToNumpy(), got_o)          # same kernel without its weight stores
+    finally:
+        w.set_math_mode(0)
+    assert np.max(np.abs(got_o - lay(o32, Tq))) <= 1e-2 * float(np.max(np.abs(v)))
+    assert np.max(np.abs(got_w - w32)) <= 1e-2 * float(np.max(w32)) + 3e-2 * float(np.max(w32))
+    assert np.max(np.abs(got_w - wbf)) <= 2e-6 + 1e-5 * float(np.max(wbf))
+    o_from_got_w = oracle.bmm(oracle.round_to_bf16(got_w), False, oracle.round_to_bf16(v), False)
+    assert np.max(np.abs(got_o - lay(o_from_got_w, Tq))) <= 2e-5 * float(np.max(np.abs(v)))
+    assert np.max(np.abs(got_o - lay(obf, Tq))) <= 2.0 ** -8 * float(np.max(np.abs(v)))
