@@ -221,7 +221,7 @@ int snhip_activation_backward(void* handle, int activation, float activation_par
  * `weights` the output may come from a single pass with a running maximum, which rounds differently), or
  * Tk <= 128 with dk, dv <= 128; anything else returns status 15 (NOT_SUPPORTED) and the caller issues the reference's
  * sequence of calls instead.  On a handle in the bf16-input math mode the two products use bf16 MFMAs where a kernel
- * for them exists (head dimension exactly 64, up to 256 keys), fp32 MFMAs otherwise. */
+ * for them exists (head dimension exactly 64; beyond 256 keys: a multiple of 4 keys), fp32 MFMAs otherwise. */
 typedef struct snhip_attention_desc {
     int struct_size;
     int batch, batch_inner; /* matrices; batch_inner as in snhip_gemm_desc (0: single level) */

@@ -1071,6 +1071,40 @@ struct Attn16BCfg {
     static constexpr int LDS_BYTES = (KEYS * KP + D * VP) * 2;
 };
 
+// The two products in bf16 MFMAs, shared by attention_fwd16_bf16_kernel and the long-key kernel's bf16 form.
+// qf[s] holds the lane's query floats 16 s + 4 g .. + 3 (fp32, rounded here).
+template <int NKT, int NS, int KP>
+__device__ __forceinline__ void attn16_score_product_bf16(const __bf16* Kb, int g, int l16, const f32x4 (&qf)[NS],
+                                                          f32x4 (&sacc)[NKT]) {
+#pragma unroll
+    for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const __bf16* kbase = Kb + l16 * KP + 4 * g;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const bf16x4_bits qb = round_to_bf16x4(qf[s]);
+        bf16x4_bits ka[NKT];
+#pragma unroll
+        for (int t = 0; t < NKT; ++t) ka[t] = *reinterpret_cast<const bf16x4_bits*>(kbase + t * 16 * KP + 16 * s);
+#pragma unroll
+        for (int t = 0; t < NKT; ++t) sacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[t], qb, sacc[t], 0, 0, 0);
+    }
+}
+
+template <int NKT, int NDT, int VP>
+__device__ __forceinline__ void attn16_second_product_bf16(const __bf16* Vt, int g, int l16, const f32x4 (&sacc)[NKT],
+                                                           f32x4 (&oacc)[NDT]) {
+    const __bf16* vbase = Vt + l16 * VP + 4 * g;
+#pragma unroll
+    for (int t = 0; t < NKT; ++t) {
+        const bf16x4_bits pb = round_to_bf16x4(sacc[t]);
+#pragma unroll
+        for (int mt = 0; mt < NDT; ++mt) {
+            const bf16x4_bits va = *reinterpret_cast<const bf16x4_bits*>(vbase + mt * 16 * VP + 16 * t);
+            oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb, oacc[mt], 0, 0, 0);
+        }
+    }
+}
+
 template <int KEYS>
 __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnParams p) {
     using CFG = Attn16BCfg<KEYS>;
@@ -1166,21 +1200,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
 
         // ---- S^T = K . Q^T ----
         f32x4 sacc[NKT];
-#pragma unroll
-        for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        {
-            const __bf16* kbase = Kb + l16 * KP + 4 * g;
-#pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                const bf16x4_bits qb = round_to_bf16x4(qf[s]);
-                bf16x4_bits ka[NKT];
-#pragma unroll
-                for (int t = 0; t < NKT; ++t) ka[t] = *reinterpret_cast<const bf16x4_bits*>(kbase + t * 16 * KP + 16 * s);
-#pragma unroll
-                for (int t = 0; t < NKT; ++t)
-                    sacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[t], qb, sacc[t], 0, 0, 0);
-            }
-        }
+        attn16_score_product_bf16<NKT, NS, KP>(Kb, g, l16, qf, sacc);
         // (behind the product: the wait in front of it covers every load in flight, see attention_fwd16_kernel)
         if (last_tile && has_next) load_kv(z_next);
         __builtin_amdgcn_sched_barrier(0);
@@ -1251,18 +1271,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
         f32x4 oacc[NDT];
 #pragma unroll
         for (int mt = 0; mt < NDT; ++mt) oacc[mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        {
-            const __bf16* vbase = Vt + l16 * VP + 4 * g;
-#pragma unroll
-            for (int t = 0; t < NKT; ++t) {
-                const bf16x4_bits pb = round_to_bf16x4(sacc[t]);
-#pragma unroll
-                for (int mt = 0; mt < NDT; ++mt) {
-                    const bf16x4_bits va = *reinterpret_cast<const bf16x4_bits*>(vbase + mt * 16 * VP + 16 * t);
-                    oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb, oacc[mt], 0, 0, 0);
-                }
-            }
-        }
+        attn16_second_product_bf16<NKT, NDT, VP>(Vt, g, l16, sacc, oacc);
         if (row_ok) {
             float* orow = Oz + (long long)row * p.ldo + 4 * g;
 #pragma unroll
@@ -1281,17 +1290,22 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
 // worked on, so that a block change costs the two barriers and the LDS stores but not the round trip to memory.
 // Same passes, same skipping of causal blocks and the same zero-fill of the skipped weights as
 // attention_fwd_long_kernel.  ONE_PASS is for callers that do not keep the weights (P == nullptr, inference): a single
-// walk over the key blocks with a running maximum and sum (two thirds of the MFMA work).
+// walk over the key blocks with a running maximum and sum (two thirds of the MFMA work).  BF16: both products in bf16
+// MFMAs as in attention_fwd16_bf16_kernel (operands rounded on their way into LDS, probabilities on their way into the
+// second product), for handles in the bf16-input math mode.
 // ---------------------------------------------------------------------------------------------------------------
-template <bool ONE_PASS>
+template <bool ONE_PASS, bool BF16 = false>
 __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnParams p) {
     constexpr int KEYS = 256;
     using CFG = Attn16Cfg<KEYS>;
+    using BCFG = Attn16BCfg<KEYS>;
     constexpr int D = CFG::D, KP = CFG::KP, VP = CFG::VP;
     constexpr int NKT = KEYS / 16, NDT = D / 16, NQ = D / 4;
     extern __shared__ __attribute__((aligned(16))) float smem[];
     float* const Ks = smem;            // [D][KP]
     float* const Vs = smem + D * KP;   // [KEYS][VP]
+    __bf16* const Kb = reinterpret_cast<__bf16*>(smem);  // BF16: [KEYS][BCFG::KP]
+    __bf16* const Vt = Kb + KEYS * BCFG::KP;              // BF16: [D][BCFG::VP]
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l16 = lane & 15, g = lane >> 4;
@@ -1304,14 +1318,20 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
     const bool row_ok = row < p.Tq;
 
     // qf[s] = Q[row][16 (lane / 16) + s]; rows past Tq read the last row (never stored)
+    // (BF16: qb[s] = Q[row][16 s + 4 g .. + 3], the k order of the bf16 MFMA)
     float qf[NQ];
+    f32x4 qb[NQ / 4];
     {
-        const float* qrow = p.Q + batch_offset(bi, p.sQ, p.sQ2) + (long long)(row_ok ? row : p.Tq - 1) * p.ldq + NQ * g;
+        const float* qrow = p.Q + batch_offset(bi, p.sQ, p.sQ2) + (long long)(row_ok ? row : p.Tq - 1) * p.ldq;
 #pragma unroll
         for (int j = 0; j < NQ / 4; ++j) {
-            f32x4 x;
-            __builtin_memcpy(&x, qrow + 4 * j, 16);
-            qf[4 * j] = x.x, qf[4 * j + 1] = x.y, qf[4 * j + 2] = x.z, qf[4 * j + 3] = x.w;
+            if constexpr (BF16) {
+                __builtin_memcpy(&qb[j], qrow + 16 * j + 4 * g, 16);
+            } else {
+                f32x4 x;
+                __builtin_memcpy(&x, qrow + NQ * g + 4 * j, 16);
+                qf[4 * j] = x.x, qf[4 * j + 1] = x.y, qf[4 * j + 2] = x.z, qf[4 * j + 3] = x.w;
+            }
         }
     }
 
@@ -1338,6 +1358,28 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
             __builtin_memcpy(&dst[it], base + (long long)(key < p.Tk ? key : p.Tk - 1) * ld + 4 * v, 16);
         }
     };
+    // BF16: V with the same four columns of two adjacent keys per thread (pairs of keys go into the transposed tile
+    // as whole words)
+    auto load_block_v_pairs = [&](int kb) {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+#pragma unroll
+        for (int it = 0; it < KIT / 2; ++it) {
+            const int idx = it * 512 + tid;
+            const int kp = idx % (KEYS / 2), v = idx / (KEYS / 2);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int key = kb * KEYS + 2 * kp + h;
+                __builtin_memcpy(&vx[2 * it + h], Vz + (long long)(key < p.Tk ? key : p.Tk - 1) * p.ldv + 4 * v, 16);
+            }
+        }
+    };
+    auto load_v = [&](int kb) {
+        if constexpr (BF16)
+            load_block_v_pairs(kb);
+        else
+            load_block(Vz, p.ldv, kb, vx);
+    };
     auto store_k = [&](int kb) {
         int tid = threadIdx.x;
         asm volatile("" : "+v"(tid));
@@ -1347,21 +1389,40 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
             const int idx = it * 512 + tid;
             const int key = idx / (D / 4), v = idx % (D / 4);
             const f32x4 x = kb * KEYS + key < p.Tk ? kx[it] : zero;
-            Ks[(4 * v + 0) * KP + key] = x.x;
-            Ks[(4 * v + 1) * KP + key] = x.y;
-            Ks[(4 * v + 2) * KP + key] = x.z;
-            Ks[(4 * v + 3) * KP + key] = x.w;
+            if constexpr (BF16) {
+                *reinterpret_cast<bf16x4_bits*>(Kb + key * BCFG::KP + 4 * v) = round_to_bf16x4(x);
+            } else {
+                Ks[(4 * v + 0) * KP + key] = x.x;
+                Ks[(4 * v + 1) * KP + key] = x.y;
+                Ks[(4 * v + 2) * KP + key] = x.z;
+                Ks[(4 * v + 3) * KP + key] = x.w;
+            }
         }
     };
     auto store_v = [&](int kb) {
         int tid = threadIdx.x;
         asm volatile("" : "+v"(tid));
         const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (BF16) {
 #pragma unroll
-        for (int it = 0; it < KIT; ++it) {
-            const int idx = it * 512 + tid;
-            const int key = idx / (D / 4), v = idx % (D / 4);
-            *reinterpret_cast<f32x4*>(Vs + key * VP + 4 * v) = kb * KEYS + key < p.Tk ? vx[it] : zero;
+            for (int it = 0; it < KIT / 2; ++it) {
+                const int idx = it * 512 + tid;
+                const int kp = idx % (KEYS / 2), v = idx / (KEYS / 2);
+                const bf16x4_bits lo = round_to_bf16x4(kb * KEYS + 2 * kp < p.Tk ? vx[2 * it] : zero);
+                const bf16x4_bits hi = round_to_bf16x4(kb * KEYS + 2 * kp + 1 < p.Tk ? vx[2 * it + 1] : zero);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const unsigned int w2 = (unsigned int)(unsigned short)lo[c] | ((unsigned int)(unsigned short)hi[c] << 16);
+                    *reinterpret_cast<unsigned int*>(Vt + (4 * v + c) * BCFG::VP + 2 * kp) = w2;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < KIT; ++it) {
+                const int idx = it * 512 + tid;
+                const int key = idx / (D / 4), v = idx % (D / 4);
+                *reinterpret_cast<f32x4*>(Vs + key * VP + 4 * v) = kb * KEYS + key < p.Tk ? vx[it] : zero;
+            }
         }
     };
 
@@ -1378,7 +1439,12 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
 
     // raw scores of the block in LDS: sacc[t][r] belongs to key kb * 256 + 16 t + 4 g + r
     f32x4 sacc[NKT];
-    auto score_product = [&]() { attn16_score_product<NKT, NQ, KP>(Ks, g, l16, qf, sacc); };
+    auto score_product = [&]() {
+        if constexpr (BF16)
+            attn16_score_product_bf16<NKT, NQ / 4, BCFG::KP>(Kb, g, l16, qb, sacc);
+        else
+            attn16_score_product<NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+    };
     // log2-domain scores with the mask (a key past Tk or above the diagonal becomes kMasked: its exponential is 0)
     auto scale_and_mask = [&](int kb) {
         int lim = p.Tk - 1;
@@ -1396,7 +1462,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
     // ---- pass 1: row maximum and row sum over all needed blocks ----
     float m = -3.402823466e+38f, l = 0.0f;
     load_block(Kz, p.ldk, 0, kx);
-    if constexpr (ONE_PASS) load_block(Vz, p.ldv, 0, vx);
+    if constexpr (ONE_PASS) load_v(0);
     product_priority();
     for (int kb = 0; !ONE_PASS && kb < nb_needed; ++kb) {
         __syncthreads();  // every wavefront is done with the previous block
@@ -1409,7 +1475,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
             load_block(Kz, p.ldk, kb + 1, kx);
         } else {
             load_block(Kz, p.ldk, 0, kx);
-            load_block(Vz, p.ldv, 0, vx);
+            load_v(0);
         }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(3);
@@ -1450,7 +1516,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         score_product();
         if (kb + 1 < nb_needed) {
             load_block(Kz, p.ldk, kb + 1, kx);
-            load_block(Vz, p.ldv, kb + 1, vx);
+            load_v(kb + 1);
         }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(3);
@@ -1490,14 +1556,16 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         product_priority();
 
         // P out: inside the second product when the whole block and the whole tile exist (uniform), else here
-        const bool p_inline = pbase != nullptr && (kb + 1) * KEYS <= p.Tk && q0 + AT_BQ <= p.Tq;
+        const bool p_inline = !BF16 && pbase != nullptr && (kb + 1) * KEYS <= p.Tk && q0 + AT_BQ <= p.Tq;
         if (pbase != nullptr && !p_inline && row_ok) {
             float* prow = pbase + kb * KEYS;
 #pragma unroll
             for (int t = 0; t < NKT; ++t)
                 if (kb * KEYS + t * 16 + 4 * g < p.Tk) *reinterpret_cast<f32x4*>(prow + t * 16) = sacc[t];
         }
-        if (p_inline)
+        if constexpr (BF16)
+            attn16_second_product_bf16<NKT, NDT, BCFG::VP>(Vt, g, l16, sacc, oacc);
+        else if (p_inline)
             attn16_second_product<NKT, NDT, VP, true>(Vs, g, l16, sacc, oacc, pbase + kb * KEYS);
         else
             attn16_second_product<NKT, NDT, VP, false>(Vs, g, l16, sacc, oacc, nullptr);

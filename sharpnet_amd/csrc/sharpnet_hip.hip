@@ -872,6 +872,12 @@ hipError_t prepare_kernels_once(int dev) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<256>::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<true, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<256>::LDS_BYTES);
+    if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd_long_kernel<32>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, AttnCfg<8, 32>::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -1044,10 +1050,16 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
         p.q_tiles = 1;
         constexpr int lds32 = AttnCfg<8, 32>::LDS_BYTES, lds64 = AttnCfg<8, 64>::LDS_BYTES;
         // head dimension exactly 64 and outputs that take 16-byte stores: the form with two wavefronts per SIMD
-        if (d->dk == 64 && d->dv == 64 && d->Tk % 4 == 0 && (p.flags & 1) && (d->weights == nullptr || (p.flags & 2)))
-            hipLaunchKernelGGL(d->weights == nullptr ? attention_fwd16_long_kernel<true> : attention_fwd16_long_kernel<false>,
-                               dim3((unsigned)d->batch, (unsigned)tiles), dim3(512), Attn16Cfg<256>::LDS_BYTES, h->stream, p);
-        else if (hd <= 32)
+        if (d->dk == 64 && d->dv == 64 && d->Tk % 4 == 0 && (p.flags & 1) && (d->weights == nullptr || (p.flags & 2))) {
+            const bool bf16 = h->math_mode == SNHIP_MATH_BF16_INPUT;  // bf16 MFMAs, as this handle's GEMMs
+            void (*fn)(const AttnParams);
+            if (d->weights == nullptr)
+                fn = bf16 ? attention_fwd16_long_kernel<true, true> : attention_fwd16_long_kernel<true, false>;
+            else
+                fn = bf16 ? attention_fwd16_long_kernel<false, true> : attention_fwd16_long_kernel<false, false>;
+            hipLaunchKernelGGL(fn, dim3((unsigned)d->batch, (unsigned)tiles), dim3(512),
+                               bf16 ? Attn16BCfg<256>::LDS_BYTES : Attn16Cfg<256>::LDS_BYTES, h->stream, p);
+        } else if (hd <= 32)
             hipLaunchKernelGGL(attention_fwd_long_kernel<32>, dim3((unsigned)d->batch, (unsigned)tiles), dim3(256), lds32,
                                h->stream, p);
         else

@@ -386,7 +386,9 @@ def test_bf16_streaming_kernels_strided_batches(oracle, gpu_wrapper, tA, tB):
 
 
 @pytest.mark.parametrize("B,H,Tq,Tk,causal,packed", [(2, 3, 256, 256, True, True), (3, 2, 200, 132, False, False),
-                                                       (2, 2, 130, 100, True, False), (70, 8, 130, 136, False, True)])
+                                                       (2, 2, 130, 100, True, False), (70, 8, 130, 136, False, True),
+                                                       # more than 256 keys: key blocks, two passes / one pass
+                                                       (2, 2, 300, 700, True, False), (1, 3, 650, 516, False, True)])
 def test_attention_forward_in_bf16_input_mode(oracle, gpu_wrapper, B, H, Tq, Tk, causal, packed):
     """snhip_attention_forward on a handle in the bf16-input math mode (head dimension 64, up to 256 keys): Q, K, V and
     the probabilities entering the second product are rounded to bf16, sums and softmax stay fp32.
@@ -429,7 +431,10 @@ def test_attention_forward_in_bf16_input_mode(oracle, gpu_wrapper, B, H, Tq, Tk,
         go.SetValue(float("nan"))
         assert attention.fused_attention_forward(gq, gk, gv, go, None, batch=B, heads=H, tq=Tq, tkv=Tk, dk=d, dv=d,
                                                  scale=scale, is_causal=causal, packed=packed)
-        assert np.array_equal(go.ToNumpy(), got_o)          # same kernel without its weight stores
+        if Tk <= 256:
+            assert np.array_equal(go.ToNumpy(), got_o)      # same kernel without its weight stores
+        else:                                               # a single pass with a running maximum instead of two
+            assert np.max(np.abs(go.ToNumpy() - lay(o32, Tq))) <= 1e-2 * float(np.max(np.abs(v)))
     finally:
         w.set_math_mode(0)
     assert np.max(np.abs(got_o - lay(o32, Tq))) <= 1e-2 * float(np.max(np.abs(v)))
