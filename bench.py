@@ -189,6 +189,21 @@ def main():
                 attention.fused_attention_forward(q, k, v, o, wts, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
                                                   scale=0.125, is_causal=causal, packed=False)
             w.synchronize()
+        for t in (q, k, v, o, wts):
+            t.Dispose()
+        # the handle in the bf16-input math mode: 512 x (256 x 64) with and without the weights, then 64 x 1024 keys
+        w.set_math_mode(1)
+        for Z, Tn in ((512, 256), (64, 1024)):
+            q, k, v = (GPUTensor([Z, Tn, d], rng.uniform(-1, 1, (Z, Tn, d)).astype(np.float32), w) for _ in range(3))
+            o, wts = GPUTensor([Z, Tn, d], None, w), GPUTensor([Z, Tn, Tn], None, w)
+            for keep in (wts, None):
+                for _ in range(20):
+                    attention.fused_attention_forward(q, k, v, o, keep, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
+                                                      scale=0.125, is_causal=False, packed=False)
+                w.synchronize()
+            for t in (q, k, v, o, wts):
+                t.Dispose()
+        w.set_math_mode(0)
         return
     if args.rnn_probe:
         from sharpnet_amd import recurrent

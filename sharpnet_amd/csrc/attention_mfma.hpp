@@ -1072,21 +1072,28 @@ struct Attn16BCfg {
 };
 
 // The two products in bf16 MFMAs, shared by attention_fwd16_bf16_kernel and the long-key kernel's bf16 form.
-// qf[s] holds the lane's query floats 16 s + 4 g .. + 3 (fp32, rounded here).
+// qb[s] holds the lane's query values 16 s + 4 g .. + 3, rounded.
 template <int NKT, int NS, int KP>
-__device__ __forceinline__ void attn16_score_product_bf16(const __bf16* Kb, int g, int l16, const f32x4 (&qf)[NS],
+__device__ __forceinline__ void attn16_score_product_bf16(const __bf16* Kb, int g, int l16, const bf16x4_bits (&qbits)[NS],
                                                           f32x4 (&sacc)[NKT]) {
 #pragma unroll
     for (int t = 0; t < NKT; ++t) sacc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     const __bf16* kbase = Kb + l16 * KP + 4 * g;
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-        const bf16x4_bits qb = round_to_bf16x4(qf[s]);
-        bf16x4_bits ka[NKT];
+        const bf16x4_bits qb = qbits[s];
+        constexpr int H = NKT / 2;  // operands of half the key tiles at a time (registers)
 #pragma unroll
-        for (int t = 0; t < NKT; ++t) ka[t] = *reinterpret_cast<const bf16x4_bits*>(kbase + t * 16 * KP + 16 * s);
+        for (int half = 0; half < 2; ++half) {
+            bf16x4_bits ka[H];
 #pragma unroll
-        for (int t = 0; t < NKT; ++t) sacc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[t], qb, sacc[t], 0, 0, 0);
+            for (int t = 0; t < H; ++t)
+                ka[t] = *reinterpret_cast<const bf16x4_bits*>(kbase + (half * H + t) * 16 * KP + 16 * s);
+#pragma unroll
+            for (int t = 0; t < H; ++t)
+                sacc[half * H + t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[t], qb, sacc[half * H + t], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 }
 
@@ -1102,6 +1109,9 @@ __device__ __forceinline__ void attn16_second_product_bf16(const __bf16* Vt, int
             const bf16x4_bits va = *reinterpret_cast<const bf16x4_bits*>(vbase + mt * 16 * VP + 16 * t);
             oacc[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb, oacc[mt], 0, 0, 0);
         }
+        // (keeps the scheduler from pulling every step's operand reads to the front: registers, not MFMA time, are
+        // what is short here)
+        if (t % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -1200,7 +1210,12 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
 
         // ---- S^T = K . Q^T ----
         f32x4 sacc[NKT];
-        attn16_score_product_bf16<NKT, NS, KP>(Kb, g, l16, qf, sacc);
+        {
+            bf16x4_bits qbits[NS];
+#pragma unroll
+            for (int s = 0; s < NS; ++s) qbits[s] = round_to_bf16x4(qf[s]);
+            attn16_score_product_bf16<NKT, NS, KP>(Kb, g, l16, qbits, sacc);
+        }
         // (behind the product: the wait in front of it covers every load in flight, see attention_fwd16_kernel)
         if (last_tile && has_next) load_kv(z_next);
         __builtin_amdgcn_sched_barrier(0);
@@ -1320,13 +1335,15 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
     // qf[s] = Q[row][16 (lane / 16) + s]; rows past Tq read the last row (never stored)
     // (BF16: qb[s] = Q[row][16 s + 4 g .. + 3], the k order of the bf16 MFMA)
     float qf[NQ];
-    f32x4 qb[NQ / 4];
+    bf16x4_bits qb[NQ / 4];
     {
         const float* qrow = p.Q + batch_offset(bi, p.sQ, p.sQ2) + (long long)(row_ok ? row : p.Tq - 1) * p.ldq;
 #pragma unroll
         for (int j = 0; j < NQ / 4; ++j) {
             if constexpr (BF16) {
-                __builtin_memcpy(&qb[j], qrow + 16 * j + 4 * g, 16);
+                f32x4 x;
+                __builtin_memcpy(&x, qrow + 16 * j + 4 * g, 16);
+                qb[j] = round_to_bf16x4(x);
             } else {
                 f32x4 x;
                 __builtin_memcpy(&x, qrow + NQ * g + 4 * j, 16);
