@@ -1115,7 +1115,8 @@ __device__ __forceinline__ void attn16_second_product_bf16(const __bf16* Vt, int
     }
 }
 
-template <int KEYS>
+// BWD: the backward instantiation, roles exchanged as in attention_fwd16_kernel (dP^T = V . dO^T, dS from the stored P, dQ = dS . K).
+template <int KEYS, bool BWD = false>
 __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnParams p) {
     using CFG = Attn16BCfg<KEYS>;
     constexpr int D = CFG::D, KP = CFG::KP, VP = CFG::VP;
@@ -1217,9 +1218,31 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
             attn16_score_product_bf16<NKT, NS, KP>(Kb, g, l16, qbits, sacc);
         }
         // (behind the product: the wait in front of it covers every load in flight, see attention_fwd16_kernel)
-        if (last_tile && has_next) load_kv(z_next);
+        if (!BWD && last_tile && has_next) load_kv(z_next);
         __builtin_amdgcn_sched_barrier(0);
 
+        if constexpr (BWD) {
+            // dS = scale * P * (dP - sum_keys dP * P), P read once (keys past Tk: dP is zero there, P taken as zero)
+            f32x4 pin[NKT];
+            {
+                const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + 4 * g;
+#pragma unroll
+                for (int t = 0; t < NKT; ++t)
+                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : 0), 16);
+            }
+            float rs = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NKT; ++t) {
+                if (p.Tk < KEYS && t * 16 + 4 * g >= p.Tk) pin[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                rs += sacc[t].x * pin[t].x + sacc[t].y * pin[t].y + sacc[t].z * pin[t].z + sacc[t].w * pin[t].w;
+            }
+            rs += __shfl_xor(rs, 16, 64);
+            rs += __shfl_xor(rs, 32, 64);
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sacc[t][r] = p.scale * pin[t][r] * (sacc[t][r] - rs);
+        } else {
         // ---- softmax over the keys, as in attention_fwd16_kernel ----
         constexpr float kLog2e = 1.44269504088896340736f;
         constexpr float kMasked = -1e12f * kLog2e;
@@ -1266,6 +1289,9 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
         for (int t = 0; t < NKT; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) sacc[t][r] *= inv;
+        }
+        if (BWD && last_tile && has_next) load_kv(z_next);  // (behind the stretch that holds P in registers)
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- P out (fp32, as computed) ----
         if (p.P != nullptr && row_ok) {

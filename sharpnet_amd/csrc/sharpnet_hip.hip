@@ -578,6 +578,20 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     if (g.D != nullptr && g.ldd < N) return SNHIP_STATUS_INVALID_VALUE;
     const int inner = (g.batch_inner > 0) ? g.batch_inner : batch;
     if (batch % inner != 0) return SNHIP_STATUS_INVALID_VALUE;
+    if (inner < batch) {
+        // A two-level batch that is really one level - a single matrix per outer step, or outer strides that continue
+        // the inner ones - is run as one: every kernel walks a single-level batch, only the extended fp32 ones a
+        // two-level one (the others would be launched once per outer step).
+        const bool has_d = g.D != nullptr && g.gamma != 0.0f;
+        GemmArgs one = g;
+        one.batch_inner = 0;
+        if (inner == 1) {
+            one.sA = g.sA2, one.sB = g.sB2, one.sC = g.sC2, one.sD = g.sD2;
+            return gemm_core(h, one);
+        }
+        if (g.sA2 == inner * g.sA && g.sB2 == inner * g.sB && g.sC2 == inner * g.sC && (!has_d || g.sD2 == inner * g.sD))
+            return gemm_core(h, one);
+    }
     if (batch > 65535) {
         // grid.y carries batch * splitk: a longer single-level batch goes out in slices (cuBLAS takes any batchCount)
         if (inner < batch) return SNHIP_STATUS_NOT_SUPPORTED;
@@ -864,6 +878,12 @@ hipError_t prepare_kernels_once(int dev) {
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_bf16_kernel<128>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<128>::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_bf16_kernel<256, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<256>::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_bf16_kernel<128, true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<128>::LDS_BYTES);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false>),
@@ -1162,7 +1182,14 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
             const int gx = ceil_div(tiles, p.q_tiles);
             int gy = h->num_cu / gx;
             gy = gy < 1 ? 1 : (gy > d->batch ? d->batch : gy);
-            hipLaunchKernelGGL(e16->fn, dim3((unsigned)gx, (unsigned)gy), dim3(512), e16->lds_bytes, h->stream, p);
+            if (h->math_mode == SNHIP_MATH_BF16_INPUT && e->hd == 64 && e->keys == 256)  // as this handle's GEMMs
+                hipLaunchKernelGGL((attention_fwd16_bf16_kernel<256, true>), dim3((unsigned)gx, (unsigned)gy), dim3(512),
+                                   Attn16BCfg<256>::LDS_BYTES, h->stream, p);
+            else if (h->math_mode == SNHIP_MATH_BF16_INPUT && e->hd == 64 && e->keys == 128)
+                hipLaunchKernelGGL((attention_fwd16_bf16_kernel<128, true>), dim3((unsigned)gx, (unsigned)gy), dim3(512),
+                                   Attn16BCfg<128>::LDS_BYTES, h->stream, p);
+            else
+                hipLaunchKernelGGL(e16->fn, dim3((unsigned)gx, (unsigned)gy), dim3(512), e16->lds_bytes, h->stream, p);
         } else {
             hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256),
                                e->lds_bytes, h->stream, p);

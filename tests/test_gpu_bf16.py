@@ -443,3 +443,43 @@ def test_attention_forward_in_bf16_input_mode(oracle, gpu_wrapper, B, H, Tq, Tk,
     o_from_got_w = oracle.bmm(oracle.round_to_bf16(got_w), False, oracle.round_to_bf16(v), False)
     assert np.max(np.abs(got_o - lay(o_from_got_w, Tq))) <= 2e-5 * float(np.max(np.abs(v)))
     assert np.max(np.abs(got_o - lay(obf, Tq))) <= 2.0 ** -8 * float(np.max(np.abs(v)))
+
+
+@pytest.mark.parametrize("B,H,Tq,Tk,packed", [(2, 3, 256, 256, True), (3, 2, 200, 132, False), (70, 8, 130, 100, False)])
+def test_attention_backward_in_bf16_input_mode(oracle, gpu_wrapper, B, H, Tq, Tk, packed):
+    """snhip_attention_backward on a handle in the bf16-input math mode (head dimension 64, up to 256 keys): the batched
+    products dV = P^T.dO and dK = dS^T.Q go through the bf16-input GEMMs as every product of such a handle does, and
+    the kernel between them (dP = dO.V^T, softmax gradient, dQ = dS.K) multiplies in bf16 as well; sums and the softmax
+    gradient stay fp32.  Bar: 1e-2 of the largest reference value of each output (the bf16-input bar of the GEMMs)."""
+    from sharpnet_amd import GPUTensor, attention
+    rng = np.random.default_rng(73)
+    Z, d = B * H, 64
+    q, k = random_tensor(rng, (Z, Tq, d), -1, 1), random_tensor(rng, (Z, Tk, d), -1, 1)
+    v, do = random_tensor(rng, (Z, Tk, d), -1, 1), random_tensor(rng, (Z, Tq, d), -1, 1)
+    wts = oracle.softmax_last_dim(random_tensor(rng, (Z, Tq, Tk), -3, 3))
+    scale = 0.37
+    dv_ref = oracle.bmm(wts, True, do, False)
+    ds_ref = oracle.softmax_last_dim_backward(wts, oracle.bmm(do, False, v, True, scale))
+    dq_ref = oracle.bmm(ds_ref, False, k, False)
+    dk_ref = oracle.bmm(ds_ref, True, q, False)
+
+    def lay(x, steps):
+        if not packed:
+            return x
+        return np.ascontiguousarray(x.reshape(B, H, steps, d).transpose(0, 2, 1, 3)).reshape(B, steps, H * d)
+    w = gpu_wrapper
+    gq, gk, gv, gdo = (GPUTensor(list(lay(x, t).shape), lay(x, t), w) for x, t in ((q, Tq), (k, Tk), (v, Tk), (do, Tq)))
+    gw, gds = GPUTensor(list(wts.shape), wts, w), GPUTensor([Z, Tq, Tk], None, w)
+    gdq, gdk, gdv = (GPUTensor(t.Shape, None, w) for t in (gq, gk, gv))
+    for t in (gds, gdq, gdk, gdv):
+        t.SetValue(float("nan"))
+    w.set_math_mode(1)
+    try:
+        attention.attention_backward(gdq, gdk, gdv, gq, gk, gv, gdo, gw, gds, batch=B, heads=H, tq=Tq, tkv=Tk, dk=d, dv=d,
+                                     scale=scale, packed=packed)
+        got = [t.ToNumpy() for t in (gds, gdv, gdq, gdk)]
+    finally:
+        w.set_math_mode(0)
+    for name, g, ref in zip(("dS", "dV", "dQ", "dK"), got, (ds_ref, lay(dv_ref, Tk), lay(dq_ref, Tq), lay(dk_ref, Tk))):
+        assert np.all(np.isfinite(g)), name
+        assert np.max(np.abs(g - ref)) <= 1e-2 * float(np.max(np.abs(ref))), name

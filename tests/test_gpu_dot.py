@@ -388,11 +388,17 @@ def test_limits_and_user_stream(oracle, gpu_wrapper):
     tiny2 = GPUTensor([70000, 1, 1], vals, gpu_wrapper)
     assert lib.snhip_bmm(h, tiny.Pointer, 1, 1, 0, 1, tiny2.Pointer, 1, 1, 0, 1, out.Pointer, 1, 70000, 2.0, 0.0) == 0
     assert np.array_equal(out.ToNumpy().reshape(-1), 2.0 * vals)
-    # a two-level batch that long is refused (status 15)
+    # a two-level batch whose outer strides continue the inner ones is one level to the library: also sliced
     from sharpnet_amd import hiplib
     import ctypes
+    out.ZeroMemory()
     d = hiplib.GemmDesc(M=1, N=1, K=1, A=tiny.Pointer, lda=1, strideA=1, strideA_outer=2, B=tiny2.Pointer, ldb=1, strideB=1,
                         strideB_outer=2, C=out.Pointer, ldc=1, strideC=1, strideC_outer=2, batch=70000, batch_inner=2)
+    assert lib.snhip_gemm_ex(h, ctypes.byref(d)) == 0
+    assert np.array_equal(out.ToNumpy().reshape(-1), vals)
+    # a genuine two-level batch that long is refused (status 15): inner stride 0, outer stride 1 for A and B
+    d = hiplib.GemmDesc(M=1, N=1, K=1, A=tiny.Pointer, lda=1, strideA=0, strideA_outer=1, B=tiny2.Pointer, ldb=1, strideB=0,
+                        strideB_outer=1, C=out.Pointer, ldc=1, strideC=1, strideC_outer=2, batch=70000, batch_inner=2)
     assert lib.snhip_gemm_ex(h, ctypes.byref(d)) == 15
     # K == 0 on a batch: C = beta * C
     c0 = random_tensor(rng, (4, 3, 5))
