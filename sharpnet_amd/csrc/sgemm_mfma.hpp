@@ -106,6 +106,9 @@ __device__ __host__ __forceinline__ long long batch_offset(BatchIndex b, long lo
     return (long long)b.outer * stride_outer + (long long)b.inner * stride_inner;
 }
 
+// "no offset given" for store_accumulators_plain's optional output offset
+constexpr long long kNoBatchOffset = -0x7fffffffffffffffLL - 1;
+
 struct GemmParams {
     const float* A;
     const float* B;
@@ -500,7 +503,8 @@ __device__ __forceinline__ void store_patch_fast(const f32x16 (&acc)[TM][TN], fl
 // ---------------------------------------------------------------------------
 template <int TM, int TN, bool PIN = (TM * TN >= 16)>
 __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM][TN], const GemmParams& p, int row_base,
-                                                   int col0, int lhi, int zb, int batch, int tile_index) {
+                                                   int col0, int lhi, int zb, int batch, int tile_index,
+                                                   long long c_offset = kNoBatchOffset) {
     const bool to_ws = (p.splitk > 1);
     float* out;
     long long ldo;
@@ -515,7 +519,7 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
         bias = nullptr;
         vec_ok = (p.flags & GEMM_FLAG_WS_VEC) && (col0 + TN <= p.N);
     } else {
-        out = p.C + (long long)batch * p.strideC;
+        out = p.C + (c_offset != kNoBatchOffset ? c_offset : (long long)batch * p.strideC);  // c_offset: the caller's own batch walk
         ldo = p.ldc;
         alpha = p.alpha;
         beta = p.beta;

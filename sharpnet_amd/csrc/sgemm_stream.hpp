@@ -81,8 +81,11 @@ __global__ void __launch_bounds__(256, stream_occupancy(TN, BK_)) sgemm_stream_k
     StageB sb;
     f32x4 ra[StageA::NV], rb[StageB::NV];
     auto fetch = [&](const Tile& t, int kp) {
-        sa.init(p.A + (long long)t.z * p.strideA, p.lda, t.m0, kp * BK, tid);
-        sb.init(p.B + (long long)t.z * p.strideB, p.ldb, t.n0, kp * BK, tid);
+        // (a two-level batch: entry z is matrix z % batch_inner of outer step z / batch_inner; with a single level
+        // batch_inner is the batch count and the outer term vanishes)
+        const BatchIndex bz = split_batch(t.z, p.batch_inner);
+        sa.init(p.A + batch_offset(bz, p.strideA, p.strideA2), p.lda, t.m0, kp * BK, tid);
+        sb.init(p.B + batch_offset(bz, p.strideB, p.strideB2), p.ldb, t.n0, kp * BK, tid);
         const int m_rem = p.M - t.m0, n_rem = p.N - t.n0, k_rem = p.K - kp * BK;
         if (m_rem >= BM && n_rem >= BN && k_rem >= BK) {
             sa.load_fast(ra);
@@ -144,7 +147,8 @@ __global__ void __launch_bounds__(256, stream_occupancy(TN, BK_)) sgemm_stream_k
             sb.store_lds(Bs, rb);
         }
         if (last_panel) {
-            store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
+            store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
+                                            batch_offset(split_batch(cur.z, p.batch_inner), p.strideC, p.strideC2));
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -220,8 +224,9 @@ __global__ void __launch_bounds__(256, bstream_occupancy(sizeof(TIN))) bgemm_str
     StageB sb;
     f32x4 ra[StageA::NV], rb[StageB::NV];
     auto fetch = [&](const Tile& t, int kp) {
-        sa.init(reinterpret_cast<const TIN*>(p.A) + (long long)t.z * p.strideA, p.lda, t.m0, kp * BK, tid);
-        sb.init(reinterpret_cast<const TIN*>(p.B) + (long long)t.z * p.strideB, p.ldb, t.n0, kp * BK, tid);
+        const BatchIndex bz = split_batch(t.z, p.batch_inner);
+        sa.init(reinterpret_cast<const TIN*>(p.A) + batch_offset(bz, p.strideA, p.strideA2), p.lda, t.m0, kp * BK, tid);
+        sb.init(reinterpret_cast<const TIN*>(p.B) + batch_offset(bz, p.strideB, p.strideB2), p.ldb, t.n0, kp * BK, tid);
         const int m_rem = p.M - t.m0, n_rem = p.N - t.n0, k_rem = p.K - kp * BK;
         if (m_rem >= BM && n_rem >= BN && k_rem >= BK) {
             sa.load_fast(ra);
@@ -277,7 +282,8 @@ __global__ void __launch_bounds__(256, bstream_occupancy(sizeof(TIN))) bgemm_str
             sb.store_lds(Bs, rb);
         }
         if (last_panel) {
-            store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
+            store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
+                                            batch_offset(split_batch(cur.z, p.batch_inner), p.strideC, p.strideC2));
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll

@@ -540,7 +540,8 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
 // strided batches of small matrices whose K fits a few 64-wide panels, where the tiled kernels' pipeline never
 // fills and every workgroup is prologue and write-out.
 int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, bool wants_ext) {
-    if (two_level || wants_ext) return -1;
+    (void)two_level;  // the streaming kernels walk a two-level batch themselves
+    if (wants_ext) return -1;
     const int first = math == SNHIP_MATH_FP32 ? kStreamConfig
                                               : (math == SNHIP_MATH_BF16_INPUT ? kBStreamConfig : kBStreamStoredConfig);
     const bool forced = h->force_cfg == first || h->force_cfg == first + 1;
@@ -689,7 +690,8 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     const bool relu_family = (ep.act == ACT_RELU || ep.act == ACT_LEAKY_RELU);
     const bool want_ext = ep.addend != nullptr || relu_family || two_level || g.colsum != nullptr;
     const bool use_ext = want_ext && fn_ext != nullptr;
-    if (two_level && !use_ext) {
+    const bool walks_two_levels = cfg.kind == 3 || cfg.kind == 5 || cfg.kind == 6;  // the streaming kernels
+    if (two_level && !use_ext && !walks_two_levels) {
         GemmArgs part = g;
         part.batch = inner;
         part.batch_inner = 0;

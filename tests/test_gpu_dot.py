@@ -753,3 +753,43 @@ def test_k_split_kernel_padded_pitches_fuzz(oracle, gpu_wrapper):
         assert used >= 50, used
     finally:
         gpu_wrapper.set_tuning(-1, 0)
+
+
+@pytest.mark.parametrize("math,configs", [(0, (16, 17)), (1, (22, 23))])
+@pytest.mark.parametrize("tA,tB", [(False, True), (False, False), (True, False)])
+def test_streaming_kernels_walk_a_two_level_batch(oracle, gpu_wrapper, math, configs, tA, tB):
+    """The persistent streaming kernels (fp32 and bf16-input) on heads addressed in place: entry z of the batch is head
+    z % heads of sample z / heads inside (batch, steps, heads * dim) activations, the output a contiguous stack or in
+    place as well.  Every product against the oracle (bf16: on rounded operands, the bound of the bf16 tests)."""
+    from sharpnet_amd import GPUTensor
+    rng = np.random.default_rng(83)
+    B, H, M, N, K = 5, 3, 130, 96, 64
+    w = gpu_wrapper
+    a_rows, a_cols = (K, M) if tA else (M, K)      # per-head operand shapes
+    b_rows, b_cols = (N, K) if tB else (K, N)
+    a = random_tensor(rng, (B, a_rows, H * a_cols), -1, 1)     # packed: head h is the column block [h*cols, (h+1)*cols)
+    b = random_tensor(rng, (B, b_rows, H * b_cols), -1, 1)
+    ga, gb = GPUTensor(list(a.shape), a, w), GPUTensor(list(b.shape), b, w)
+    want = np.empty((B, H, M, N), np.float32)
+    for z, h in itertools.product(range(B), range(H)):
+        ah, bh = a[z][:, h * a_cols:(h + 1) * a_cols], b[z][:, h * b_cols:(h + 1) * b_cols]
+        if math == 1:
+            ah, bh = oracle.round_to_bf16(ah), oracle.round_to_bf16(bh)
+        want[z, h] = oracle.dot(np.ascontiguousarray(ah), tA, np.ascontiguousarray(bh), tB, 0.5, 0.0)
+    w.set_math_mode(math)
+    try:
+        for cfg, c_packed in itertools.product(configs, (False, True)):
+            gc = GPUTensor([B, M, H * N] if c_packed else [B * H, M, N], None, w)
+            gc.SetValue(float("nan"))
+            w.set_tuning(cfg, 1)
+            gc.GemmEx(transA=int(tA), transB=int(tB), M=M, N=N, K=K, alpha=0.5, beta=0.0, A=ga, lda=H * a_cols, strideA=a_cols,
+                      strideA_outer=a_rows * H * a_cols, B=gb, ldb=H * b_cols, strideB=b_cols, strideB_outer=b_rows * H * b_cols,
+                      ldc=H * N if c_packed else N, strideC=N if c_packed else M * N,
+                      strideC_outer=M * H * N if c_packed else H * M * N, batch=B * H, batch_inner=H)
+            assert w.last_tuning() == (cfg, 1)
+            got = gc.ToNumpy()
+            got = got.reshape(B, M, H, N).transpose(0, 2, 1, 3) if c_packed else got.reshape(B, H, M, N)
+            assert np.max(np.abs(got - want)) <= 1e-4 * np.sqrt(K) * 0.5, (cfg, c_packed)
+    finally:
+        w.set_tuning(-1, 0)
+        w.set_math_mode(0)
