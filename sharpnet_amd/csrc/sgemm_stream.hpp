@@ -35,8 +35,11 @@ struct StreamCfg {
     static constexpr int LDS_BYTES = BK * (PA + PB) * 4;
 };
 
-template <int TN, bool TA, bool TB, int BK_ = 64>
-__global__ void __launch_bounds__(256, stream_occupancy(TN, BK_)) sgemm_stream_kernel(const GemmParams p) {
+// TWO_LEVEL: entry z of the batch is matrix z % batch_inner of outer step z / batch_inner (heads addressed in place);
+// a variant of its own because the extra address arithmetic does not fit the register budget of the single-level
+// kernel's occupancy (it runs with one workgroup fewer per compute unit).
+template <int TN, bool TA, bool TB, int BK_ = 64, bool TWO_LEVEL = false>
+__global__ void __launch_bounds__(256, stream_occupancy(TN, BK_) - (TWO_LEVEL ? 1 : 0)) sgemm_stream_kernel(const GemmParams p) {
     using CFG = StreamCfg<TN, BK_>;
     constexpr int BM = CFG::BM, BN = CFG::BN, BK = CFG::BK, NT = CFG::NT, PA = CFG::PA, PB = CFG::PB;
     using StageA = TileStage<BM, BK, NT, PA, !TA, true>;
@@ -81,11 +84,14 @@ __global__ void __launch_bounds__(256, stream_occupancy(TN, BK_)) sgemm_stream_k
     StageB sb;
     f32x4 ra[StageA::NV], rb[StageB::NV];
     auto fetch = [&](const Tile& t, int kp) {
-        // (a two-level batch: entry z is matrix z % batch_inner of outer step z / batch_inner; with a single level
-        // batch_inner is the batch count and the outer term vanishes)
-        const BatchIndex bz = split_batch(t.z, p.batch_inner);
-        sa.init(p.A + batch_offset(bz, p.strideA, p.strideA2), p.lda, t.m0, kp * BK, tid);
-        sb.init(p.B + batch_offset(bz, p.strideB, p.strideB2), p.ldb, t.n0, kp * BK, tid);
+        if constexpr (TWO_LEVEL) {
+            const BatchIndex bz = split_batch(t.z, p.batch_inner);
+            sa.init(p.A + batch_offset(bz, p.strideA, p.strideA2), p.lda, t.m0, kp * BK, tid);
+            sb.init(p.B + batch_offset(bz, p.strideB, p.strideB2), p.ldb, t.n0, kp * BK, tid);
+        } else {
+            sa.init(p.A + (long long)t.z * p.strideA, p.lda, t.m0, kp * BK, tid);
+            sb.init(p.B + (long long)t.z * p.strideB, p.ldb, t.n0, kp * BK, tid);
+        }
         const int m_rem = p.M - t.m0, n_rem = p.N - t.n0, k_rem = p.K - kp * BK;
         if (m_rem >= BM && n_rem >= BN && k_rem >= BK) {
             sa.load_fast(ra);
@@ -147,8 +153,11 @@ __global__ void __launch_bounds__(256, stream_occupancy(TN, BK_)) sgemm_stream_k
             sb.store_lds(Bs, rb);
         }
         if (last_panel) {
-            store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
-                                            batch_offset(split_batch(cur.z, p.batch_inner), p.strideC, p.strideC2));
+            if constexpr (TWO_LEVEL)
+                store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
+                                                batch_offset(split_batch(cur.z, p.batch_inner), p.strideC, p.strideC2));
+            else
+                store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -182,8 +191,8 @@ struct BStreamCfg {
 // workgroups per compute unit the register budget is set for: fp32 storage keeps twice the bytes in flight
 constexpr int bstream_occupancy(int bytes_per_element) { return bytes_per_element == 4 ? 2 : 3; }
 
-template <int TN, bool TA, bool TB, typename TIN>
-__global__ void __launch_bounds__(256, bstream_occupancy(sizeof(TIN))) bgemm_stream_kernel(const GemmParams p) {
+template <int TN, bool TA, bool TB, typename TIN, bool TWO_LEVEL = false>
+__global__ void __launch_bounds__(256, bstream_occupancy(sizeof(TIN)) - (TWO_LEVEL ? 1 : 0)) bgemm_stream_kernel(const GemmParams p) {
     using CFG = BStreamCfg<TN>;
     constexpr int BM = CFG::BM, BN = CFG::BN, BK = CFG::BK, NT = CFG::NT, PITCH = CFG::PITCH;
     using StageA = BStage<BM, BK, NT, PITCH, 1, !TA, TIN>;
@@ -224,9 +233,14 @@ __global__ void __launch_bounds__(256, bstream_occupancy(sizeof(TIN))) bgemm_str
     StageB sb;
     f32x4 ra[StageA::NV], rb[StageB::NV];
     auto fetch = [&](const Tile& t, int kp) {
-        const BatchIndex bz = split_batch(t.z, p.batch_inner);
-        sa.init(reinterpret_cast<const TIN*>(p.A) + batch_offset(bz, p.strideA, p.strideA2), p.lda, t.m0, kp * BK, tid);
-        sb.init(reinterpret_cast<const TIN*>(p.B) + batch_offset(bz, p.strideB, p.strideB2), p.ldb, t.n0, kp * BK, tid);
+        if constexpr (TWO_LEVEL) {
+            const BatchIndex bz = split_batch(t.z, p.batch_inner);
+            sa.init(reinterpret_cast<const TIN*>(p.A) + batch_offset(bz, p.strideA, p.strideA2), p.lda, t.m0, kp * BK, tid);
+            sb.init(reinterpret_cast<const TIN*>(p.B) + batch_offset(bz, p.strideB, p.strideB2), p.ldb, t.n0, kp * BK, tid);
+        } else {
+            sa.init(reinterpret_cast<const TIN*>(p.A) + (long long)t.z * p.strideA, p.lda, t.m0, kp * BK, tid);
+            sb.init(reinterpret_cast<const TIN*>(p.B) + (long long)t.z * p.strideB, p.ldb, t.n0, kp * BK, tid);
+        }
         const int m_rem = p.M - t.m0, n_rem = p.N - t.n0, k_rem = p.K - kp * BK;
         if (m_rem >= BM && n_rem >= BN && k_rem >= BK) {
             sa.load_fast(ra);
@@ -282,8 +296,11 @@ __global__ void __launch_bounds__(256, bstream_occupancy(sizeof(TIN))) bgemm_str
             sb.store_lds(Bs, rb);
         }
         if (last_panel) {
-            store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
-                                            batch_offset(split_batch(cur.z, p.batch_inner), p.strideC, p.strideC2));
+            if constexpr (TWO_LEVEL)
+                store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
+                                                batch_offset(split_batch(cur.z, p.batch_inner), p.strideC, p.strideC2));
+            else
+                store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll

@@ -188,12 +188,14 @@ const ConfigEntry kConfigs[] = {
     ConfigEntry{128, 128, 32, 256, StreamCfg<4, 32>::LDS_BYTES, 4, 3,
                 {{sgemm_stream_kernel<4, false, false, 32>, sgemm_stream_kernel<4, false, true, 32>},
                  {sgemm_stream_kernel<4, true, false, 32>, sgemm_stream_kernel<4, true, true, 32>}},
-                {{nullptr, nullptr}, {nullptr, nullptr}},
+                {{sgemm_stream_kernel<4, false, false, 32, true>, sgemm_stream_kernel<4, false, true, 32, true>},
+                 {sgemm_stream_kernel<4, true, false, 32, true>, sgemm_stream_kernel<4, true, true, 32, true>}},
                 3, 0.8, 0.9, 1.1},  // 16: 128 x 128, k panels of 32, three workgroups per compute unit
     ConfigEntry{128, 64, 32, 256, StreamCfg<2, 32>::LDS_BYTES, 2, 3,
                 {{sgemm_stream_kernel<2, false, false, 32>, sgemm_stream_kernel<2, false, true, 32>},
                  {sgemm_stream_kernel<2, true, false, 32>, sgemm_stream_kernel<2, true, true, 32>}},
-                {{nullptr, nullptr}, {nullptr, nullptr}},
+                {{sgemm_stream_kernel<2, false, false, 32, true>, sgemm_stream_kernel<2, false, true, 32, true>},
+                 {sgemm_stream_kernel<2, true, false, 32, true>, sgemm_stream_kernel<2, true, true, 32, true>}},
                 4, 0.7, 0.85, 1.1},  // 17: 128 x 64, k panels of 32, four workgroups per compute unit
     // bf16-input kernels on operands stored as bf16 (SNHIP_MATH_BF16_STORED)
     make_entry_bf16_stored<BTileCfg<4, 4, 2, 2, 64>>(1, 0.85, 0.85, 3.0),   // 18: 256 x 256, BK 64
@@ -210,23 +212,27 @@ const ConfigEntry kConfigs[] = {
     ConfigEntry{128, 128, 64, 256, BStreamCfg<4>::LDS_BYTES, 4, 5,
                 {{bgemm_stream_kernel<4, false, false, float>, bgemm_stream_kernel<4, false, true, float>},
                  {bgemm_stream_kernel<4, true, false, float>, bgemm_stream_kernel<4, true, true, float>}},
-                {{nullptr, nullptr}, {nullptr, nullptr}},
+                {{bgemm_stream_kernel<4, false, false, float, true>, bgemm_stream_kernel<4, false, true, float, true>},
+                 {bgemm_stream_kernel<4, true, false, float, true>, bgemm_stream_kernel<4, true, true, float, true>}},
                 2, 0.8, 0.9, 1.1},  // 22: 128 x 128, k panels of 64
     ConfigEntry{128, 64, 128, 256, BStreamCfg<2>::LDS_BYTES, 2, 5,
                 {{bgemm_stream_kernel<2, false, false, float>, bgemm_stream_kernel<2, false, true, float>},
                  {bgemm_stream_kernel<2, true, false, float>, bgemm_stream_kernel<2, true, true, float>}},
-                {{nullptr, nullptr}, {nullptr, nullptr}},
+                {{bgemm_stream_kernel<2, false, false, float, true>, bgemm_stream_kernel<2, false, true, float, true>},
+                 {bgemm_stream_kernel<2, true, false, float, true>, bgemm_stream_kernel<2, true, true, float, true>}},
                 2, 0.7, 0.85, 1.1},  // 23: 128 x 64, k panels of 128
     // ... and bf16 storage (kind 6)
     ConfigEntry{128, 128, 64, 256, BStreamCfg<4>::LDS_BYTES, 4, 6,
                 {{bgemm_stream_kernel<4, false, false, __bf16>, bgemm_stream_kernel<4, false, true, __bf16>},
                  {bgemm_stream_kernel<4, true, false, __bf16>, bgemm_stream_kernel<4, true, true, __bf16>}},
-                {{nullptr, nullptr}, {nullptr, nullptr}},
+                {{bgemm_stream_kernel<4, false, false, __bf16, true>, bgemm_stream_kernel<4, false, true, __bf16, true>},
+                 {bgemm_stream_kernel<4, true, false, __bf16, true>, bgemm_stream_kernel<4, true, true, __bf16, true>}},
                 3, 0.8, 0.9, 1.1},  // 24: 128 x 128, k panels of 64
     ConfigEntry{128, 64, 128, 256, BStreamCfg<2>::LDS_BYTES, 2, 6,
                 {{bgemm_stream_kernel<2, false, false, __bf16>, bgemm_stream_kernel<2, false, true, __bf16>},
                  {bgemm_stream_kernel<2, true, false, __bf16>, bgemm_stream_kernel<2, true, true, __bf16>}},
-                {{nullptr, nullptr}, {nullptr, nullptr}},
+                {{bgemm_stream_kernel<2, false, false, __bf16, true>, bgemm_stream_kernel<2, false, true, __bf16, true>},
+                 {bgemm_stream_kernel<2, true, false, __bf16, true>, bgemm_stream_kernel<2, true, true, __bf16, true>}},
                 3, 0.7, 0.85, 1.1},  // 25: 128 x 64, k panels of 128
     // 16 x 16 tiles (v_mfma_f32_16x16x4_f32), K split over eight wavefronts: see prefer_ksplit()
     ConfigEntry{16, 16, 32, 512, Ksplit16Cfg::LDS_BYTES, 1, 2,
@@ -540,7 +546,7 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
 // strided batches of small matrices whose K fits a few 64-wide panels, where the tiled kernels' pipeline never
 // fills and every workgroup is prologue and write-out.
 int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, bool wants_ext) {
-    (void)two_level;  // the streaming kernels walk a two-level batch themselves
+    (void)two_level;  // the streaming kernels have a variant that walks a two-level batch (their fn_ext entries)
     if (wants_ext) return -1;
     const int first = math == SNHIP_MATH_FP32 ? kStreamConfig
                                               : (math == SNHIP_MATH_BF16_INPUT ? kBStreamConfig : kBStreamStoredConfig);
@@ -690,8 +696,7 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     const bool relu_family = (ep.act == ACT_RELU || ep.act == ACT_LEAKY_RELU);
     const bool want_ext = ep.addend != nullptr || relu_family || two_level || g.colsum != nullptr;
     const bool use_ext = want_ext && fn_ext != nullptr;
-    const bool walks_two_levels = cfg.kind == 3 || cfg.kind == 5 || cfg.kind == 6;  // the streaming kernels
-    if (two_level && !use_ext && !walks_two_levels) {
+    if (two_level && !use_ext) {
         GemmArgs part = g;
         part.batch = inner;
         part.batch_inner = 0;
