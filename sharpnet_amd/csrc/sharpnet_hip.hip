@@ -275,10 +275,13 @@ const AttnEntry kAttnBwd[] = {attn_bwd_entry<2, 32>(), attn_bwd_entry<4, 32>(), 
 struct Attn16Entry {
     int keys, hd, lds_bytes;
     void (*fn)(const AttnParams);
+    int wgs_per_cu;  // resident workgroups per compute unit (registers, LDS): the persistent grid is that many times the CUs
 };
 template <int KEYS, int HD, bool BWD>
 constexpr Attn16Entry attn16_entry() {
-    return Attn16Entry{KEYS, HD, Attn16Cfg<KEYS, HD>::LDS_BYTES, attention_fwd16_kernel<KEYS, BWD, HD>};
+    // 128 keys x 32 forward: 104 registers and 35 KB of LDS, two workgroups fit; every other size: one
+    return Attn16Entry{KEYS, HD, Attn16Cfg<KEYS, HD>::LDS_BYTES, attention_fwd16_kernel<KEYS, BWD, HD>,
+                       (KEYS == 128 && HD == 32 && !BWD) ? 2 : 1};
 }
 const Attn16Entry kAttn16[] = {attn16_entry<128, 32, false>(), attn16_entry<256, 32, false>(),
                                attn16_entry<128, 64, false>(), attn16_entry<256, 64, false>()};
@@ -1106,7 +1109,9 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
         (d->weights == nullptr || (p.flags & 2))) {
         // one workgroup per compute unit, each walking through its share of the matrices
         const int gx = ceil_div(tiles, p.q_tiles);
-        int gy = h->num_cu / gx;
+        const bool bf16 = h->math_mode == SNHIP_MATH_BF16_INPUT && e->hd == 64;
+        const int per_cu = bf16 ? 1 : e16->wgs_per_cu;  // (a second resident workgroup measured no gain in bf16)
+        int gy = per_cu * h->num_cu / gx;
         gy = gy < 1 ? 1 : (gy > d->batch ? d->batch : gy);
         // a handle in the bf16-input math mode multiplies in bf16 here as it does in its GEMMs (head dimension 64)
         if (h->math_mode == SNHIP_MATH_BF16_INPUT && e->hd == 64 && e->keys == 256)
