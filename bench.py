@@ -624,6 +624,15 @@ def layer_timings(w, wl):
         res.append({"layer": "ScaledDotProductAttention forward + backward 512 x (256 x 64), causal",
                     "form": "one launch forward, three backward" if fused else "reference sequence (4 + 5 calls)",
                     "forward_ms": f, "backward_ms": round(fb - f, 4)})
+        if fused:
+            w.set_math_mode(1)
+            try:
+                f = timed(sdpa_f, 20, 10)
+                fb = timed(sdpa_fb, 20, 10)
+            finally:
+                w.set_math_mode(0)
+            res.append({"layer": "ScaledDotProductAttention forward + backward 512 x (256 x 64), causal, bf16-input math",
+                        "form": "one launch forward, three backward", "forward_ms": f, "backward_ms": round(fb - f, 4)})
     for t in (q, k, v, o, dq, dk_, dv_, do):
         t.Dispose()
     # more than 256 keys: 64 matrices of 1024 x 1024, head dimension 64 (key blocks of 256; two passes when the weights
