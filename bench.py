@@ -189,7 +189,15 @@ def main():
                 attention.fused_attention_forward(q, k, v, o, wts, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
                                                   scale=0.125, is_causal=causal, packed=False)
             w.synchronize()
-        for t in (q, k, v, o, wts):
+        # and the backward call at that size (dV, the two-pass kernel for dS and dQ, dK)
+        do, ds = GPUTensor([Z, Tn, d], None, w), GPUTensor([Z, Tn, Tn], None, w)
+        dq, dk_, dv_ = (GPUTensor([Z, Tn, d], None, w) for _ in range(3))
+        do.SetValue(0.01)
+        for _ in range(20):
+            attention.attention_backward(dq, dk_, dv_, q, k, v, do, wts, ds, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
+                                         scale=0.125, packed=False)
+        w.synchronize()
+        for t in (q, k, v, o, wts, do, ds, dq, dk_, dv_):
             t.Dispose()
         # the handle in the bf16-input math mode: 512 x (256 x 64) with and without the weights, then 64 x 1024 keys
         w.set_math_mode(1)
@@ -652,7 +660,21 @@ def layer_timings(w, wl):
                                      (", causal" if causal else "", "kept" if training else "not kept"),
                             "form": "one launch" if fused else "reference sequence (4 calls)", "forward_ms": ms,
                             "backward_ms": float("nan")})
-    for t in (q, k, v, o):
+    dq, dk_, dv_, do = (GPUTensor([Z, Tn, d], None, w) for _ in range(4))
+    do.SetValue(0.01)
+    for fused in (True, False):
+        def long_fb():
+            wts = attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, True, fused=fused)
+            attention.ScaledDotProductAttentionBackwardPropagation(dq, dk_, dv_, q, k, v, do, wts, True, fused=fused)
+
+        def long_f():
+            attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, True, fused=fused).Dispose()
+        f = timed(long_f, 10, 5)
+        fb = timed(long_fb, 10, 5)
+        res.append({"layer": "ScaledDotProductAttention forward + backward 64 x (1024 x 64), causal",
+                    "form": "one launch forward, three backward" if fused else "reference sequence (4 + 5 calls)",
+                    "forward_ms": f, "backward_ms": round(fb - f, 4)})
+    for t in (q, k, v, o, dq, dk_, dv_, do):
         t.Dispose()
     B, Tn, H, d = 64, 256, 8, 64
     E = H * d

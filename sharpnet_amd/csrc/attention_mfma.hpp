@@ -664,7 +664,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p
                 const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + 4 * g;
 #pragma unroll
                 for (int t = 0; t < NKT; ++t)
-                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : 0), 16);  // past Tk: any valid address
+                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : -4 * g), 16);  // past Tk: the row's first keys
             }
             float rs = 0.0f;
 #pragma unroll
@@ -1228,7 +1228,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
                 const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + 4 * g;
 #pragma unroll
                 for (int t = 0; t < NKT; ++t)
-                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : 0), 16);
+                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : -4 * g), 16);
             }
             float rs = 0.0f;
 #pragma unroll
@@ -1334,9 +1334,13 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
 // walk over the key blocks with a running maximum and sum (two thirds of the MFMA work).  BF16: both products in bf16
 // MFMAs as in attention_fwd16_bf16_kernel (operands rounded on their way into LDS, probabilities on their way into the
 // second product), for handles in the bf16-input math mode.
+// BWD: the first half of the backward pass with the roles exchanged as in attention_fwd16_kernel (Q <- dO, K <- V,
+// V <- K, Pin <- the stored weights, P <- dS out, O <- dQ): pass 1 gathers the row sums rs = sum_k P . dP over all key
+// blocks, pass 2 forms dS = scale . P . (dP - rs) block by block, writes it and accumulates dQ += dS . K.
 // ---------------------------------------------------------------------------------------------------------------
-template <bool ONE_PASS, bool BF16 = false>
+template <bool ONE_PASS, bool BF16 = false, bool BWD = false>
 __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnParams p) {
+    static_assert(!BWD || (!ONE_PASS && !BF16), "the backward instantiation is the two-pass fp32 one");
     constexpr int KEYS = 256;
     using CFG = Attn16Cfg<KEYS>;
     using BCFG = Attn16BCfg<KEYS>;
@@ -1502,8 +1506,26 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
             }
     };
 
-    // ---- pass 1: row maximum and row sum over all needed blocks ----
+    // BWD: the stored weights of this lane's keys in block kb (keys past Tk: the row's first key of the block is read
+    // instead and zero is taken)
+    f32x4 pin[BWD ? NKT : 1];
+    auto load_weights = [&](int kb) {
+        const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + kb * KEYS + 4 * g;
+#pragma unroll
+        for (int t = 0; t < (BWD ? NKT : 0); ++t)
+            __builtin_memcpy(&pin[t], prow + (kb * KEYS + t * 16 + 4 * g < p.Tk ? t * 16 : -4 * g), 16);
+    };
+    auto zero_weights_past_end = [&](int kb) {
+        if ((kb + 1) * KEYS > p.Tk) {  // uniform
+#pragma unroll
+            for (int t = 0; t < (BWD ? NKT : 0); ++t)
+                if (kb * KEYS + t * 16 + 4 * g >= p.Tk) pin[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    };
+
+    // ---- pass 1: row maximum and row sum over all needed blocks (BWD: the row sums of P . dP) ----
     float m = -3.402823466e+38f, l = 0.0f;
+    float rs = 0.0f;
     load_block(Kz, p.ldk, 0, kx);
     if constexpr (ONE_PASS) load_v(0);
     product_priority();
@@ -1512,16 +1534,37 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         store_k(kb);
         __syncthreads();
         score_product();
+        // BWD: the weights are asked for behind the product as well: carried across it, or from one block to the next,
+        // they do not fit into the registers beside the product's operands
+        if constexpr (BWD) load_weights(kb);
         // the next block is asked for behind the product (the wait in front of a loop body's first MFMA covers every
         // load in flight); after the last block of this pass that is the first block of the next one
-        if (kb + 1 < nb_needed) {
-            load_block(Kz, p.ldk, kb + 1, kx);
-        } else {
-            load_block(Kz, p.ldk, 0, kx);
-            load_v(0);
+        // (BWD: behind the stretch that holds the weights in registers)
+        if constexpr (!BWD) {
+            if (kb + 1 < nb_needed) {
+                load_block(Kz, p.ldk, kb + 1, kx);
+            } else {
+                load_block(Kz, p.ldk, 0, kx);
+                load_v(0);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(3);
+        if constexpr (BWD) {
+            zero_weights_past_end(kb);
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+                rs += sacc[t].x * pin[t].x + sacc[t].y * pin[t].y + sacc[t].z * pin[t].z + sacc[t].w * pin[t].w;
+            product_priority();
+            __builtin_amdgcn_sched_barrier(0);
+            if (kb + 1 < nb_needed) {
+                load_block(Kz, p.ldk, kb + 1, kx);
+            } else {
+                load_block(Kz, p.ldk, 0, kx);
+                load_v(0);
+            }
+            continue;
+        }
         scale_and_mask(kb);
         float bm = -3.402823466e+38f;
 #pragma unroll
@@ -1542,7 +1585,11 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         m = m_new;
         product_priority();
     }
-    const float inv = ONE_PASS ? 1.0f : 1.0f / l;
+    const float inv = (ONE_PASS || BWD) ? 1.0f : 1.0f / l;
+    if constexpr (BWD) {
+        rs += __shfl_xor(rs, 16, 64);
+        rs += __shfl_xor(rs, 32, 64);
+    }
 
     // ---- pass 2: probabilities, P out, O += P . V.  ONE_PASS (no weights kept): this is the only pass; maximum and
     //      sum run along with the blocks, the output is rescaled whenever the maximum moves (a multiplication by
@@ -1557,14 +1604,21 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         store_v(kb);
         __syncthreads();
         score_product();
-        if (kb + 1 < nb_needed) {
+        if constexpr (BWD) load_weights(kb);
+        if (!BWD && kb + 1 < nb_needed) {
             load_block(Kz, p.ldk, kb + 1, kx);
             load_v(kb + 1);
         }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_setprio(3);
-        scale_and_mask(kb);
-        if constexpr (ONE_PASS) {
+        if constexpr (!BWD) scale_and_mask(kb);
+        if constexpr (BWD) {
+            zero_weights_past_end(kb);
+#pragma unroll
+            for (int t = 0; t < NKT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sacc[t][r] = p.scale * pin[t][r] * (sacc[t][r] - rs);
+        } else if constexpr (ONE_PASS) {
             float bm = -3.402823466e+38f;
 #pragma unroll
             for (int t = 0; t < NKT; ++t)
@@ -1597,6 +1651,11 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
                 for (int r = 0; r < 4; ++r) sacc[t][r] = __builtin_amdgcn_exp2f(sacc[t][r] - m) * inv;
         }
         product_priority();
+        if (BWD && kb + 1 < nb_needed) {  // behind the stretch that holds the weights in registers
+            load_block(Kz, p.ldk, kb + 1, kx);
+            load_v(kb + 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
 
         // P out: inside the second product when the whole block and the whole tile exist (uniform), else here
         const bool p_inline = !BF16 && pbase != nullptr && (kb + 1) * KEYS <= p.Tk && q0 + AT_BQ <= p.Tq;

@@ -902,6 +902,9 @@ hipError_t prepare_kernels_once(int dev) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false, false, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
+    if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false, true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -1165,7 +1168,8 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
             e = &c;
             break;
         }
-    if (e != nullptr && d->dk > 0 && d->dv > 0) {
+    bool fused = false;
+    if (d->dk > 0 && d->dv > 0 && (e != nullptr || (d->dk == 64 && d->dv == 64))) {
         AttnParams p;
         p.Q = d->dO, p.K = d->V, p.V = d->K, p.O = d->dQ, p.P = d->scores_gradients, p.Pin = d->weights;
         p.Tq = d->Tq, p.Tk = d->Tk, p.dk = d->dv, p.dv = d->dk;  // first product contracts over dv, second produces dk
@@ -1187,8 +1191,19 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
         int groups = 1;
         while (groups < tiles && (long long)d->batch * groups < 2LL * h->num_cu) ++groups;
         p.q_tiles = ceil_div(tiles, groups);
-        const Attn16Entry* e16 = find_attn16(kAttn16Bwd, e->keys, e->hd);
-        if (e16 != nullptr && d->dk == e->hd && d->dv == e->hd && (p.flags & 7) == 7) {
+        const Attn16Entry* e16 = e != nullptr ? find_attn16(kAttn16Bwd, e->keys, e->hd) : nullptr;
+        if (e == nullptr) {
+            // more than 256 keys, head dimension exactly 64: the two-pass kernel over key blocks (fp32 in every math
+            // mode); anything else takes the three calls below
+            if ((p.flags & 7) == 7 && tiles <= 65535) {
+                p.q_tiles = 1;
+                hipLaunchKernelGGL((attention_fwd16_long_kernel<false, false, true>),
+                                   dim3((unsigned)d->batch, (unsigned)tiles), dim3(512), Attn16Cfg<256>::LDS_BYTES,
+                                   h->stream, p);
+                fused = true;
+            }
+        } else if (e16 != nullptr && d->dk == e->hd && d->dv == e->hd && (p.flags & 7) == 7) {
+            fused = true;
             // head dimension exactly 32 or 64, as in the forward call: two wavefronts per SIMD, one workgroup per
             // compute unit
             const int gx = ceil_div(tiles, p.q_tiles);
@@ -1203,12 +1218,16 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
             else
                 hipLaunchKernelGGL(e16->fn, dim3((unsigned)gx, (unsigned)gy), dim3(512), e16->lds_bytes, h->stream, p);
         } else {
+            fused = true;
             hipLaunchKernelGGL(e->fn, dim3((unsigned)ceil_div(tiles, p.q_tiles), (unsigned)d->batch), dim3(256),
                                e->lds_bytes, h->stream, p);
         }
-        st = hip_to_status(hipGetLastError());
-        if (st != SNHIP_STATUS_SUCCESS) return st;
-    } else {
+        if (fused) {
+            st = hip_to_status(hipGetLastError());
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
+    }
+    if (!fused) {
         GemmArgs s1;
         s1.tB = true;
         s1.M = d->Tq, s1.N = d->Tk, s1.K = d->dv, s1.alpha = d->scale;

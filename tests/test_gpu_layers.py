@@ -600,6 +600,11 @@ def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
     (2, 1, 384, 200, 64, 64, True), (2, 3, 128, 128, 64, 64, True), (3, 2, 100, 68, 64, 64, False),
     (2, 2, 256, 256, 32, 32, True), (3, 1, 200, 132, 32, 32, False), (2, 2, 130, 100, 32, 32, False),
     (75, 8, 130, 132, 64, 64, True), (700, 1, 100, 100, 64, 64, False), (90, 7, 140, 136, 32, 32, False),
+    # beyond 256 keys with head dimension exactly 64: the two-pass kernel over key blocks (a last block of 4 keys,
+    # ragged query tiles, whole blocks, many matrices); 1002 keys and head dimension 32: the five-launch sequence
+    (2, 2, 300, 520, 64, 64, False), (1, 3, 130, 1024, 64, 64, True), (2, 1, 257, 260, 64, 64, False),
+    (1, 2, 100, 1000, 64, 64, True), (40, 8, 128, 512, 64, 64, True), (1, 2, 100, 1002, 64, 64, False),
+    (1, 2, 100, 512, 32, 32, False),
 ])
 def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, packed):
     """snhip_attention_backward (dV, score gradient through the softmax, dQ, dK; the middle two from one kernel when
