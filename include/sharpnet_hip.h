@@ -247,7 +247,7 @@ int snhip_sizeof_attention_desc(void);
  * the reference takes from its memory pool for dS (:121) and must be supplied.  Q / dQ, K / dK and V / dV share their
  * row pitch and batch strides; dO has its own.  `scale` is the factor the reference applies here (1/sqrt(dV.Shape[2])
  * with use_scale, :113-119).  Three launches when Tk <= 256 and both dimensions <= 64, or up to 128 keys with
- * dimensions up to 128, or any multiple of 4 keys with both dimensions exactly 64 and 16-byte aligned buffers (dS and
+ * dimensions up to 128, or any multiple of 4 keys with both dimensions exactly 32 or exactly 64 and 16-byte aligned buffers (dS and
  * dQ come from one kernel); otherwise five, the reference's own sequence. */
 typedef struct snhip_attention_bwd_desc {
     int struct_size;

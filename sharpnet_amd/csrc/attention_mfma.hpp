@@ -1325,8 +1325,8 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// The two-pass kernel for any number of keys in the layout of attention_fwd16_kernel (head dimension exactly 64 on
-// both sides, a multiple of 4 keys, aligned outputs): eight wavefronts of 16 queries, 16x16x4 MFMAs, two wavefronts per
+// The two-pass kernel for any number of keys in the layout of attention_fwd16_kernel (head dimension exactly HD = 32
+// or 64 on both sides, a multiple of 4 keys, aligned outputs): eight wavefronts of 16 queries, 16x16x4 MFMAs, two wavefronts per
 // SIMD, and the next key block's K (pass 1) or K and V (pass 2) travelling in registers while the current block is
 // worked on, so that a block change costs the two barriers and the LDS stores but not the round trip to memory.
 // Same passes, same skipping of causal blocks and the same zero-fill of the skipped weights as
@@ -1338,11 +1338,12 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
 // V <- K, Pin <- the stored weights, P <- dS out, O <- dQ): pass 1 gathers the row sums rs = sum_k P . dP over all key
 // blocks, pass 2 forms dS = scale . P . (dP - rs) block by block, writes it and accumulates dQ += dS . K.
 // ---------------------------------------------------------------------------------------------------------------
-template <bool ONE_PASS, bool BF16 = false, bool BWD = false>
+template <bool ONE_PASS, bool BF16 = false, bool BWD = false, int HD = 64>
 __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnParams p) {
     static_assert(!BWD || (!ONE_PASS && !BF16), "the backward instantiation is the two-pass fp32 one");
+    static_assert(!BF16 || HD == 64, "the bf16 form is written for head dimension 64");
     constexpr int KEYS = 256;
-    using CFG = Attn16Cfg<KEYS>;
+    using CFG = Attn16Cfg<KEYS, HD>;
     using BCFG = Attn16BCfg<KEYS>;
     constexpr int D = CFG::D, KP = CFG::KP, VP = CFG::VP;
     constexpr int NKT = KEYS / 16, NDT = D / 16, NQ = D / 4;
@@ -1362,7 +1363,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
     const int row = q0 + wave * 16 + l16;
     const bool row_ok = row < p.Tq;
 
-    // qf[s] = Q[row][16 (lane / 16) + s]; rows past Tq read the last row (never stored)
+    // qf[s] = Q[row][(HD / 4) (lane / 16) + s]; rows past Tq read the last row (never stored)
     // (BF16: qb[s] = Q[row][16 s + 4 g .. + 3], the k order of the bf16 MFMA)
     float qf[NQ];
     bf16x4_bits qb[NQ / 4];

@@ -905,6 +905,15 @@ hipError_t prepare_kernels_once(int dev) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false, false, true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false, false, false, 32>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256, 32>::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<true, false, false, 32>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256, 32>::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false, false, true, 32>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, Attn16Cfg<256, 32>::LDS_BYTES);
+    if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd16_long_kernel<false, true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, Attn16BCfg<256>::LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -1082,8 +1091,14 @@ int snhip_attention_forward(void* handle, const snhip_attention_desc* d) {
         if (tiles > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
         p.q_tiles = 1;
         constexpr int lds32 = AttnCfg<8, 32>::LDS_BYTES, lds64 = AttnCfg<8, 64>::LDS_BYTES;
-        // head dimension exactly 64 and outputs that take 16-byte stores: the form with two wavefronts per SIMD
-        if (d->dk == 64 && d->dv == 64 && d->Tk % 4 == 0 && (p.flags & 1) && (d->weights == nullptr || (p.flags & 2))) {
+        // head dimension exactly 32 or 64 and outputs that take 16-byte stores: the form with two wavefronts per SIMD
+        if (d->dk == 32 && d->dv == 32 && d->Tk % 4 == 0 && (p.flags & 1) && (d->weights == nullptr || (p.flags & 2))) {
+            void (*fn)(const AttnParams) = d->weights == nullptr ? attention_fwd16_long_kernel<true, false, false, 32>
+                                                                 : attention_fwd16_long_kernel<false, false, false, 32>;
+            hipLaunchKernelGGL(fn, dim3((unsigned)d->batch, (unsigned)tiles), dim3(512), (Attn16Cfg<256, 32>::LDS_BYTES),
+                               h->stream, p);
+        } else if (d->dk == 64 && d->dv == 64 && d->Tk % 4 == 0 && (p.flags & 1) &&
+                   (d->weights == nullptr || (p.flags & 2))) {
             const bool bf16 = h->math_mode == SNHIP_MATH_BF16_INPUT;  // bf16 MFMAs, as this handle's GEMMs
             void (*fn)(const AttnParams);
             if (d->weights == nullptr)
@@ -1169,7 +1184,7 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
             break;
         }
     bool fused = false;
-    if (d->dk > 0 && d->dv > 0 && (e != nullptr || (d->dk == 64 && d->dv == 64))) {
+    if (d->dk > 0 && d->dv > 0 && (e != nullptr || (d->dk == d->dv && (d->dk == 64 || d->dk == 32)))) {
         AttnParams p;
         p.Q = d->dO, p.K = d->V, p.V = d->K, p.O = d->dQ, p.P = d->scores_gradients, p.Pin = d->weights;
         p.Tq = d->Tq, p.Tk = d->Tk, p.dk = d->dv, p.dv = d->dk;  // first product contracts over dv, second produces dk
@@ -1193,13 +1208,18 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
         p.q_tiles = ceil_div(tiles, groups);
         const Attn16Entry* e16 = e != nullptr ? find_attn16(kAttn16Bwd, e->keys, e->hd) : nullptr;
         if (e == nullptr) {
-            // more than 256 keys, head dimension exactly 64: the two-pass kernel over key blocks (fp32 in every math
-            // mode); anything else takes the three calls below
+            // more than 256 keys, head dimension exactly 32 or 64: the two-pass kernel over key blocks (fp32 in every
+            // math mode); anything else takes the three calls below
             if ((p.flags & 7) == 7 && tiles <= 65535) {
                 p.q_tiles = 1;
-                hipLaunchKernelGGL((attention_fwd16_long_kernel<false, false, true>),
-                                   dim3((unsigned)d->batch, (unsigned)tiles), dim3(512), Attn16Cfg<256>::LDS_BYTES,
-                                   h->stream, p);
+                if (d->dk == 64)
+                    hipLaunchKernelGGL((attention_fwd16_long_kernel<false, false, true, 64>),
+                                       dim3((unsigned)d->batch, (unsigned)tiles), dim3(512),
+                                       (Attn16Cfg<256, 64>::LDS_BYTES), h->stream, p);
+                else
+                    hipLaunchKernelGGL((attention_fwd16_long_kernel<false, false, true, 32>),
+                                       dim3((unsigned)d->batch, (unsigned)tiles), dim3(512),
+                                       (Attn16Cfg<256, 32>::LDS_BYTES), h->stream, p);
                 fused = true;
             }
         } else if (e16 != nullptr && d->dk == e->hd && d->dv == e->hd && (p.flags & 7) == 7) {

@@ -445,12 +445,14 @@ def test_attention_forward_in_bf16_input_mode(oracle, gpu_wrapper, B, H, Tq, Tk,
     assert np.max(np.abs(got_o - lay(obf, Tq))) <= 2.0 ** -8 * float(np.max(np.abs(v)))
 
 
-@pytest.mark.parametrize("B,H,Tq,Tk,packed", [(2, 3, 256, 256, True), (3, 2, 200, 132, False), (70, 8, 130, 100, False)])
+@pytest.mark.parametrize("B,H,Tq,Tk,packed", [(2, 3, 256, 256, True), (3, 2, 200, 132, False), (70, 8, 130, 100, False),
+                                              (2, 2, 200, 520, True)])
 def test_attention_backward_in_bf16_input_mode(oracle, gpu_wrapper, B, H, Tq, Tk, packed):
-    """snhip_attention_backward on a handle in the bf16-input math mode (head dimension 64, up to 256 keys): the batched
+    """snhip_attention_backward on a handle in the bf16-input math mode (head dimension 64): the batched
     products dV = P^T.dO and dK = dS^T.Q go through the bf16-input GEMMs as every product of such a handle does, and
-    the kernel between them (dP = dO.V^T, softmax gradient, dQ = dS.K) multiplies in bf16 as well; sums and the softmax
-    gradient stay fp32.  Bar: 1e-2 of the largest reference value of each output (the bf16-input bar of the GEMMs)."""
+    up to 256 keys the kernel between them (dP = dO.V^T, softmax gradient, dQ = dS.K) multiplies in bf16 as well (beyond
+    256 keys it stays fp32); sums and the softmax gradient stay fp32.  Bar: 1e-2 of the largest reference value of each
+    output (the bf16-input bar of the GEMMs)."""
     from sharpnet_amd import GPUTensor, attention
     rng = np.random.default_rng(73)
     Z, d = B * H, 64

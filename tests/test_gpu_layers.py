@@ -407,6 +407,9 @@ def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrap
     # ... head dimension exactly 64 (two wavefronts per SIMD): ragged query tiles and a last key block short of 256,
     # with and without the mask; 770 keys (not a multiple of 4) stay on the general two-pass kernel
     (2, 2, 300, 700, 64, 64, True, False), (1, 3, 650, 516, 64, 64, False, True), (1, 1, 130, 770, 64, 64, True, True),
+    # ... and head dimension exactly 32
+    (2, 2, 300, 700, 32, 32, True, False), (1, 3, 650, 516, 32, 32, False, True), (40, 8, 128, 512, 32, 32, True, True),
+    (1, 2, 260, 260, 32, 32, False, False),
 ])
 def test_fused_attention_forward(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, causal, packed):
     """snhip_attention_forward (scores, mask, softmax and P.V in one launch) against the oracle's
@@ -600,11 +603,12 @@ def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
     (2, 1, 384, 200, 64, 64, True), (2, 3, 128, 128, 64, 64, True), (3, 2, 100, 68, 64, 64, False),
     (2, 2, 256, 256, 32, 32, True), (3, 1, 200, 132, 32, 32, False), (2, 2, 130, 100, 32, 32, False),
     (75, 8, 130, 132, 64, 64, True), (700, 1, 100, 100, 64, 64, False), (90, 7, 140, 136, 32, 32, False),
-    # beyond 256 keys with head dimension exactly 64: the two-pass kernel over key blocks (a last block of 4 keys,
-    # ragged query tiles, whole blocks, many matrices); 1002 keys and head dimension 32: the five-launch sequence
+    # beyond 256 keys with head dimension exactly 64 or 32: the two-pass kernel over key blocks (a last block of 4 keys,
+    # ragged query tiles, whole blocks, many matrices); 1002 keys and head dimension 48: the five-launch sequence
     (2, 2, 300, 520, 64, 64, False), (1, 3, 130, 1024, 64, 64, True), (2, 1, 257, 260, 64, 64, False),
     (1, 2, 100, 1000, 64, 64, True), (40, 8, 128, 512, 64, 64, True), (1, 2, 100, 1002, 64, 64, False),
-    (1, 2, 100, 512, 32, 32, False),
+    (1, 2, 100, 512, 32, 32, False), (2, 2, 300, 520, 32, 32, True), (30, 8, 130, 772, 32, 32, False),
+    (1, 2, 100, 512, 48, 48, False),
 ])
 def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, packed):
     """snhip_attention_backward (dV, score gradient through the softmax, dQ, dK; the middle two from one kernel when
