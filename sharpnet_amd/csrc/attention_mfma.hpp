@@ -502,6 +502,31 @@ __device__ __forceinline__ void attn16_score_product(const float* Ks, int g, int
     }
 }
 
+// The same product for the key tiles T0 .. T0 + NT_ - 1 only (the other accumulators are left alone).
+template <int T0, int NT_, int NKT, int NQ, int KP>
+__device__ __forceinline__ void attn16_score_product_part(const float* Ks, int g, int l16, const float (&qf)[NQ],
+                                                          f32x4 (&sacc)[NKT]) {
+    static_assert(T0 + NT_ <= NKT, "tile range");
+#pragma unroll
+    for (int t = 0; t < NT_; ++t) sacc[T0 + t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const float* kbase = Ks + (NQ * g) * KP + l16 + T0 * 16;
+    float ka[2][NT_];
+#pragma unroll
+    for (int t = 0; t < NT_; ++t) ka[0][t] = kbase[t * 16];
+#pragma unroll
+    for (int s = 0; s < NQ; ++s) {
+        if (s + 1 < NQ) {
+#pragma unroll
+            for (int t = 0; t < NT_; ++t) ka[(s + 1) & 1][t] = kbase[(s + 1) * KP + t * 16];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < NT_; ++t)
+            sacc[T0 + t] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[s & 1][t], qf[s], sacc[T0 + t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // O^T += V^T . P^T for one wavefront: k step (t, r) takes the score register sacc[t][r] as the B operand as it lies and
 // A[i = dv][k = g] = Vs[16 t + 4 g + r][16 mt + lane % 16] (pitch VP), read LOOK steps ahead.  STORE_P: the lane's
 // probabilities go out on the way, one 16-byte store (four consecutive keys, at prow + 16 t) every four k steps.
@@ -1509,18 +1534,43 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
 
     // BWD: the stored weights of this lane's keys in block kb (keys past Tk: the row's first key of the block is read
     // instead and zero is taken)
+    // The product runs in two halves of NKT / 2 key tiles: the weights of a half are asked for in front of that
+    // half's MFMAs and used behind them, so their way from memory is covered by the product, and only one half's
+    // weights wait in registers at a time (all of them across the whole product do not fit beside its operands).
+    constexpr int HALF = NKT / 2;
     f32x4 pin[BWD ? NKT : 1];
-    auto load_weights = [&](int kb) {
+    auto load_weights = [&](int kb, int t0) {
         const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + kb * KEYS + 4 * g;
 #pragma unroll
-        for (int t = 0; t < (BWD ? NKT : 0); ++t)
+        for (int i = 0; i < (BWD ? HALF : 0); ++i) {
+            const int t = t0 + i;
             __builtin_memcpy(&pin[t], prow + (kb * KEYS + t * 16 + 4 * g < p.Tk ? t * 16 : -4 * g), 16);
+        }
     };
-    auto zero_weights_past_end = [&](int kb) {
+    auto zero_weights_past_end = [&](int kb, int t0) {
         if ((kb + 1) * KEYS > p.Tk) {  // uniform
 #pragma unroll
-            for (int t = 0; t < (BWD ? NKT : 0); ++t)
+            for (int i = 0; i < (BWD ? HALF : 0); ++i) {
+                const int t = t0 + i;
                 if (kb * KEYS + t * 16 + 4 * g >= p.Tk) pin[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+    };
+    auto row_sum_part = [&](int kb, int t0, float& rs) {
+        zero_weights_past_end(kb, t0);
+#pragma unroll
+        for (int i = 0; i < (BWD ? HALF : 0); ++i) {
+            const int t = t0 + i;
+            rs += sacc[t].x * pin[t].x + sacc[t].y * pin[t].y + sacc[t].z * pin[t].z + sacc[t].w * pin[t].w;
+        }
+    };
+    auto gradient_part = [&](int kb, int t0, float rs) {
+        zero_weights_past_end(kb, t0);
+#pragma unroll
+        for (int i = 0; i < (BWD ? HALF : 0); ++i) {
+            const int t = t0 + i;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sacc[t][r] = p.scale * pin[t][r] * (sacc[t][r] - rs);
         }
     };
 
@@ -1534,29 +1584,16 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         __syncthreads();  // every wavefront is done with the previous block
         store_k(kb);
         __syncthreads();
-        score_product();
-        // BWD: the weights are asked for behind the product as well: carried across it, or from one block to the next,
-        // they do not fit into the registers beside the product's operands
-        if constexpr (BWD) load_weights(kb);
-        // the next block is asked for behind the product (the wait in front of a loop body's first MFMA covers every
-        // load in flight); after the last block of this pass that is the first block of the next one
-        // (BWD: behind the stretch that holds the weights in registers)
-        if constexpr (!BWD) {
-            if (kb + 1 < nb_needed) {
-                load_block(Kz, p.ldk, kb + 1, kx);
-            } else {
-                load_block(Kz, p.ldk, 0, kx);
-                load_v(0);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_setprio(3);
         if constexpr (BWD) {
-            zero_weights_past_end(kb);
-#pragma unroll
-            for (int t = 0; t < NKT; ++t)
-                rs += sacc[t].x * pin[t].x + sacc[t].y * pin[t].y + sacc[t].z * pin[t].z + sacc[t].w * pin[t].w;
-            product_priority();
+            load_weights(kb, 0);
+            attn16_score_product_part<0, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+            load_weights(kb, HALF);
+            __builtin_amdgcn_sched_barrier(0);
+            row_sum_part(kb, 0, rs);
+            __builtin_amdgcn_sched_barrier(0);
+            attn16_score_product_part<HALF, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+            __builtin_amdgcn_sched_barrier(0);
+            row_sum_part(kb, HALF, rs);
             __builtin_amdgcn_sched_barrier(0);
             if (kb + 1 < nb_needed) {
                 load_block(Kz, p.ldk, kb + 1, kx);
@@ -1566,6 +1603,17 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
             }
             continue;
         }
+        score_product();
+        // the next block is asked for behind the product (the wait in front of a loop body's first MFMA covers every
+        // load in flight); after the last block of this pass that is the first block of the next one
+        if (kb + 1 < nb_needed) {
+            load_block(Kz, p.ldk, kb + 1, kx);
+        } else {
+            load_block(Kz, p.ldk, 0, kx);
+            load_v(0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_setprio(3);
         scale_and_mask(kb);
         float bm = -3.402823466e+38f;
 #pragma unroll
@@ -1604,8 +1652,19 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         store_k(kb);
         store_v(kb);
         __syncthreads();
-        score_product();
-        if constexpr (BWD) load_weights(kb);
+        if constexpr (BWD) {
+            load_weights(kb, 0);
+            attn16_score_product_part<0, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+            load_weights(kb, HALF);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(3);
+            gradient_part(kb, 0, rs);
+            product_priority();
+            __builtin_amdgcn_sched_barrier(0);
+            attn16_score_product_part<HALF, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+        } else {
+            score_product();
+        }
         if (!BWD && kb + 1 < nb_needed) {
             load_block(Kz, p.ldk, kb + 1, kx);
             load_v(kb + 1);
@@ -1614,11 +1673,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         __builtin_amdgcn_s_setprio(3);
         if constexpr (!BWD) scale_and_mask(kb);
         if constexpr (BWD) {
-            zero_weights_past_end(kb);
-#pragma unroll
-            for (int t = 0; t < NKT; ++t)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) sacc[t][r] = p.scale * pin[t][r] * (sacc[t][r] - rs);
+            gradient_part(kb, HALF, rs);
         } else if constexpr (ONE_PASS) {
             float bm = -3.402823466e+38f;
 #pragma unroll
