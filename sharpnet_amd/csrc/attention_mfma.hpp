@@ -670,7 +670,28 @@ __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p
 
         // ---- S^T = K . Q^T ----
         f32x4 sacc[NKT];
-        attn16_score_product<NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+        f32x4 pin[BWD ? NKT : 1];
+        // BWD: the product in two halves of NKT / 2 key tiles, the stored weights of a half asked for in front of that
+        // half's MFMAs, so that they arrive behind the product instead of being waited for after it (keys past Tk:
+        // dP is zero there, zero rows of the staged operand, and the lane's first keys are read in their place: this kernel
+        // is given more than 64 keys, so those exist).
+        // 256 keys x 64 do not have the registers for that (66 spilled, measured slower): there the weights are
+        // asked for behind the whole product.
+        constexpr bool SPLIT = BWD && !(KEYS == 256 && HD == 64);
+        if constexpr (SPLIT) {
+            constexpr int HALF = NKT / 2;
+            const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + 4 * g;
+#pragma unroll
+            for (int t = 0; t < HALF; ++t)
+                __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : 0), 16);
+            attn16_score_product_part<0, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+#pragma unroll
+            for (int t = HALF; t < NKT; ++t)
+                __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : 0), 16);
+            attn16_score_product_part<HALF, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+        } else {
+            attn16_score_product<NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+        }
         // The next matrix is asked for here, behind the score product: the wait the compiler puts in front of that
         // product's first MFMA (for the queries) covers every load in flight, and these should not be among them.
         if (!BWD && last_tile && has_next) load_kv(z_next);
@@ -684,12 +705,11 @@ __global__ void __launch_bounds__(512) attention_fwd16_kernel(const AttnParams p
         __builtin_amdgcn_s_setprio(3);
         if constexpr (BWD) {
             // keys past Tk: dP is zero there (zero rows of the staged operand) and so is what is taken for P
-            f32x4 pin[NKT];
-            {
+            if constexpr (!SPLIT) {
                 const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + 4 * g;
 #pragma unroll
                 for (int t = 0; t < NKT; ++t)
-                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : -4 * g), 16);  // past Tk: the row's first keys
+                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : 0), 16);
             }
             float rs = 0.0f;
 #pragma unroll
@@ -1253,7 +1273,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
                 const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + 4 * g;
 #pragma unroll
                 for (int t = 0; t < NKT; ++t)
-                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : -4 * g), 16);
+                    __builtin_memcpy(&pin[t], prow + (t * 16 + 4 * g < p.Tk ? t * 16 : 0), 16);
             }
             float rs = 0.0f;
 #pragma unroll
@@ -1532,8 +1552,8 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
             }
     };
 
-    // BWD: the stored weights of this lane's keys in block kb (keys past Tk: the row's first key of the block is read
-    // instead and zero is taken)
+    // BWD: the stored weights of this lane's keys in block kb (keys past Tk: the lane's keys of block 0 are read
+    // instead - they exist, this kernel is given more than 256 keys - and zero is taken)
     // The product runs in two halves of NKT / 2 key tiles: the weights of a half are asked for in front of that
     // half's MFMAs and used behind them, so their way from memory is covered by the product, and only one half's
     // weights wait in registers at a time (all of them across the whole product do not fit beside its operands).
@@ -1544,7 +1564,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
 #pragma unroll
         for (int i = 0; i < (BWD ? HALF : 0); ++i) {
             const int t = t0 + i;
-            __builtin_memcpy(&pin[t], prow + (kb * KEYS + t * 16 + 4 * g < p.Tk ? t * 16 : -4 * g), 16);
+            __builtin_memcpy(&pin[t], prow + (kb * KEYS + t * 16 + 4 * g < p.Tk ? t * 16 : -kb * KEYS), 16);
         }
     };
     auto zero_weights_past_end = [&](int kb, int t0) {
