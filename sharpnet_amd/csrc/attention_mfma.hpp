@@ -1554,10 +1554,12 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
 
     // BWD: the stored weights of this lane's keys in block kb (keys past Tk: the lane's keys of block 0 are read
     // instead - they exist, this kernel is given more than 256 keys - and zero is taken)
-    // The product runs in two halves of NKT / 2 key tiles: the weights of a half are asked for in front of that
-    // half's MFMAs and used behind them, so their way from memory is covered by the product, and only one half's
-    // weights wait in registers at a time (all of them across the whole product do not fit beside its operands).
-    constexpr int HALF = NKT / 2;
+    // The product runs in PARTS parts of NKT / PARTS key tiles: the weights of a part are asked for in front of that
+    // part's MFMAs and used behind them, so their way from memory is covered by the product, and only two parts'
+    // weights are in registers at a time (all of them across the whole product do not fit beside its operands; at
+    // head dimension 64 halves still had the compiler move the output accumulators to scratch and back per block).
+    constexpr int PARTS = HD == 64 ? 4 : 2;
+    constexpr int HALF = NKT / PARTS;  // key tiles per part
     f32x4 pin[BWD ? NKT : 1];
     auto load_weights = [&](int kb, int t0) {
         const float* prow = p.Pin + ((long long)z * p.Tq + (row_ok ? row : p.Tq - 1)) * p.Tk + kb * KEYS + 4 * g;
@@ -1594,6 +1596,25 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         }
     };
 
+    // one part of the first product of a block and what follows it (behind_part(first key tile of the part))
+    auto bwd_part = [&](auto ic, int kb, auto&& behind_part) {
+        constexpr int I = decltype(ic)::value;
+        attn16_score_product_part<I * HALF, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+        if constexpr (I + 1 < PARTS) load_weights(kb, (I + 1) * HALF);
+        __builtin_amdgcn_sched_barrier(0);
+        behind_part(I * HALF);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto bwd_parts = [&](int kb, auto&& behind_part) {
+        load_weights(kb, 0);
+        bwd_part(std::integral_constant<int, 0>{}, kb, behind_part);
+        bwd_part(std::integral_constant<int, 1>{}, kb, behind_part);
+        if constexpr (PARTS == 4) {
+            bwd_part(std::integral_constant<int, 2>{}, kb, behind_part);
+            bwd_part(std::integral_constant<int, 3>{}, kb, behind_part);
+        }
+    };
+
     // ---- pass 1: row maximum and row sum over all needed blocks (BWD: the row sums of P . dP) ----
     float m = -3.402823466e+38f, l = 0.0f;
     float rs = 0.0f;
@@ -1605,22 +1626,10 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         store_k(kb);
         __syncthreads();
         if constexpr (BWD) {
-            load_weights(kb, 0);
-            attn16_score_product_part<0, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
-            load_weights(kb, HALF);
-            __builtin_amdgcn_sched_barrier(0);
-            row_sum_part(kb, 0, rs);
-            __builtin_amdgcn_sched_barrier(0);
-            attn16_score_product_part<HALF, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
-            __builtin_amdgcn_sched_barrier(0);
-            row_sum_part(kb, HALF, rs);
-            __builtin_amdgcn_sched_barrier(0);
-            if (kb + 1 < nb_needed) {
-                load_block(Kz, p.ldk, kb + 1, kx);
-            } else {
-                load_block(Kz, p.ldk, 0, kx);
-                load_v(0);
-            }
+            bwd_parts(kb, [&](int t0) { row_sum_part(kb, t0, rs); });
+            // (the second operand of pass 2 is asked for behind this loop: asked for in its last round it would be
+            // carried around the loop in registers that the rounds before need)
+            load_block(Kz, p.ldk, kb + 1 < nb_needed ? kb + 1 : 0, kx);
             continue;
         }
         score_product();
@@ -1656,6 +1665,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
     }
     const float inv = (ONE_PASS || BWD) ? 1.0f : 1.0f / l;
     if constexpr (BWD) {
+        load_v(0);
         rs += __shfl_xor(rs, 16, 64);
         rs += __shfl_xor(rs, 32, 64);
     }
@@ -1673,15 +1683,11 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         store_v(kb);
         __syncthreads();
         if constexpr (BWD) {
-            load_weights(kb, 0);
-            attn16_score_product_part<0, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
-            load_weights(kb, HALF);
-            __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_setprio(3);
-            gradient_part(kb, 0, rs);
-            product_priority();
-            __builtin_amdgcn_sched_barrier(0);
-            attn16_score_product_part<HALF, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
+            bwd_parts(kb, [&](int t0) {
+                __builtin_amdgcn_s_setprio(3);
+                gradient_part(kb, t0, rs);
+                product_priority();
+            });
         } else {
             score_product();
         }
@@ -1693,7 +1699,7 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
         __builtin_amdgcn_s_setprio(3);
         if constexpr (!BWD) scale_and_mask(kb);
         if constexpr (BWD) {
-            gradient_part(kb, HALF, rs);
+            // (the gradient is formed part by part behind the product above)
         } else if constexpr (ONE_PASS) {
             float bm = -3.402823466e+38f;
 #pragma unroll
