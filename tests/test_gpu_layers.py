@@ -657,3 +657,34 @@ def test_bias_gradient_tall_matrices(gpu_wrapper, rows, cols):
     T(gpu_wrapper, dy).Compute_BiasGradient_from_dy(g)
     ref = dy.astype(np.float64).sum(axis=0)
     assert np.max(np.abs(g.ToNumpy() - ref)) <= 1e-5 * np.sqrt(rows) + 1e-6 * rows ** 0.5
+
+
+def test_fused_attention_agrees_with_the_call_sequence_on_seeded_random_sizes(gpu_wrapper):
+    """ScaledDotProductAttention forward (weights kept) and backward through the fused entry points against the
+    reference's own sequence of calls (ScaledDotProductAttentionLayer.cs:46-91, 97-135) issued through the same library,
+    on 28 seeded random sizes: 1-9 matrices, 1-900 positions, head dimensions 4-64, with and without the mask.  Both
+    sides compute in fp32; the bar is the sum of two rounding bounds."""
+    from sharpnet_amd import GPUTensor, attention
+    rng = np.random.default_rng(2024)
+    w = gpu_wrapper
+    for case in range(28):
+        Z = int(rng.integers(1, 10))
+        steps = int(rng.integers(1, 901)) if case % 4 else int(rng.choice([64, 128, 256, 260, 512, 772]))
+        d = int(rng.choice([4, 8, 16, 24, 32, 40, 64]))
+        causal = bool(rng.integers(0, 2))
+        host = [random_tensor(rng, (Z, steps, d), -1, 1) for _ in range(4)]
+        results = []
+        for fused in (True, False):
+            q, k, v, dy = (T(w, x) for x in host)
+            y, dq, dk, dv = (GPUTensor([Z, steps, d], None, w) for _ in range(4))
+            wts = attention.ScaledDotProductAttentionForwardPropagation(q, k, v, y, True, True, causal, fused=fused)
+            out = [y.ToNumpy(), wts.ToNumpy()]
+            attention.ScaledDotProductAttentionBackwardPropagation(dq, dk, dv, q, k, v, dy, wts, True, fused=fused)
+            out += [dq.ToNumpy(), dk.ToNumpy(), dv.ToNumpy()]
+            results.append(out)
+            for t in (q, k, v, dy, y, dq, dk, dv):
+                t.Dispose()
+        tol = 4e-5 * np.sqrt(max(steps, d))
+        for name, a, b in zip(("y", "weights", "dQ", "dK", "dV"), results[0], results[1]):
+            assert np.all(np.isfinite(a)), (case, Z, steps, d, causal, name)
+            assert np.max(np.abs(a - b)) <= tol, (case, Z, steps, d, causal, name, float(np.max(np.abs(a - b))))
