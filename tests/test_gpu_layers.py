@@ -368,6 +368,31 @@ def test_multi_head_attention_forward_backward(oracle, gpu_wrapper, heads_in_pla
         assert err <= 3e-4 * max(float(np.max(np.abs(ref))), 1.0), (k, err)
 
 
+@pytest.mark.parametrize("B,Tn,H,d,is_causal", [(2, 256, 4, 64, True), (3, 300, 2, 32, False), (2, 130, 8, 64, True),
+                                                 (1, 520, 2, 64, False), (2, 516, 3, 32, True)])
+def test_multi_head_attention_heads_in_place_against_transposition_copies(gpu_wrapper, B, Tn, H, d, is_causal):
+    """MultiheadAttention forward and backward at sizes that take the 16-query attention kernels and the two-level
+    batches of the streaming GEMM kernels (heads multiplied in place in the (batch, steps, heads * dim) activations)
+    against the same layer run the reference's way, with its transposition copies (MultiheadAttention.cs:178-292); both
+    on the device, both fp32."""
+    rng = np.random.default_rng(33)
+    E = H * d
+    Q, K, V, dy = (random_tensor(rng, (B, Tn, E), -1, 1) for _ in range(4))
+    w_Q, w_K, w_V, w_O = (random_tensor(rng, (E, E), -0.1, 0.1) for _ in range(4))
+    b_Q, b_K, b_V, b_O = (random_tensor(rng, (E,), -0.5, 0.5) for _ in range(4))
+    res = []
+    for heads_in_place in (True, False):
+        fwd, bwd = _gpu_mha(gpu_wrapper, heads_in_place)
+        y, g = fwd(Q, K, V, w_Q, w_K, w_V, w_O, H, d, d, b_Q, b_K, b_V, b_O, is_causal=is_causal)
+        got = bwd(dy, g)
+        got["y"] = y
+        res.append(got)
+    for k, ref in res[1].items():
+        assert np.all(np.isfinite(res[0][k])), k
+        err = float(np.max(np.abs(res[0][k] - ref)))
+        assert err <= 1e-4 * max(float(np.max(np.abs(ref))), 1.0), (k, err)
+
+
 @pytest.mark.parametrize("variant,is_causal", [("no_bias", False), ("no_bias", True), ("with_bias", False),
                                                ("with_bias", True)])
 def test_multi_head_attention_training_losses_on_device(golden, oracle, gpu_wrapper, variant, is_causal):
