@@ -633,7 +633,7 @@ def test_gemm_ex_features_under_bf16_input_math(oracle, gpu_wrapper):
     (2, 2, 300, 520, 64, 64, False), (1, 3, 130, 1024, 64, 64, True), (2, 1, 257, 260, 64, 64, False),
     (1, 2, 100, 1000, 64, 64, True), (40, 8, 128, 512, 64, 64, True), (1, 2, 100, 1002, 64, 64, False),
     (1, 2, 100, 512, 32, 32, False), (2, 2, 300, 520, 32, 32, True), (30, 8, 130, 772, 32, 32, False),
-    (1, 2, 100, 512, 48, 48, False),
+    (1, 2, 100, 512, 48, 48, False), (1, 1, 300, 2048, 64, 64, False), (1, 2, 130, 1540, 32, 32, True),
 ])
 def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, packed):
     """snhip_attention_backward (dV, score gradient through the softmax, dQ, dK; the middle two from one kernel when
