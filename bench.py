@@ -11,11 +11,15 @@ in HBM before the timed region.  Prints ONE JSON line on stdout:
              HIP events on the stream the kernel runs on, against the 157.3 TFLOP/s fp32 MFMA peak;
   cpu_baseline  the reference's CPU route (MKL cblas_sgemm RowMajor, the call of
              Prod/Data/BlasServices.cs:20) timed on this box's host cores on a bounded sample;
-  extra      GPU TFLOP/s and roofline fraction of the other benchmark configurations
-             (dense layer, sweep, MLP step, LSTM projections, attention matmuls).
-Everything but the JSON line goes to stderr.
+  summary    a handful of figures of the other benchmark configurations.
+The line is strict JSON (no NaN tokens) and short (under 4000 characters): it is the LAST line of
+stdout.  The per-product figures of the other configurations (dense layer, sweep, MLP step, LSTM
+projections, attention matmuls, whole-layer calls) go to stderr and to --extra-out (a JSON file,
+default gpurun_out/bench_extra.json).  Every timed product is checked against the oracle on sampled
+rows of the timed result; a miss ends the run with an error.
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -27,8 +31,52 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 
+MAX_LINE_CHARS = 4000     # the line must fit well inside what a harness keeps of stdout
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def _no_constants(token):
+    raise ValueError("non-JSON constant %r in the bench line" % token)
+
+
+def headline_line(out):
+    """The one stdout line: strict JSON (NaN / Infinity refused), short, parsed back before it is returned."""
+    line = json.dumps(out, allow_nan=False, separators=(", ", ": "))
+    if len(line) >= MAX_LINE_CHARS:
+        raise ValueError("bench line has %d characters (limit %d): move detail into the extra file"
+                         % (len(line), MAX_LINE_CHARS))
+    json.loads(line, parse_constant=_no_constants)
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "dtype", "config", "roofline"):
+        if key not in out:
+            raise ValueError("bench line lacks %r" % key)
+    return line
+
+
+def source_hash(path):
+    """sha256 (first 16 hex digits) of a source file, to tell whether a stored counter figure is still the kernel's."""
+    with open(path, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def traffic_record(root):
+    """HBM bytes per launch of the headline kernel: a counter figure from two rocprofv3 --pmc runs, stored under
+    profiles/ together with a hash of the kernel source it was measured on.  Returns (bytes or None, source dict)."""
+    tpath = os.path.join(root, "profiles", "sgemm_8192_hbm_traffic.json")
+    if not os.path.exists(tpath):
+        return None, None
+    with open(tpath) as f:
+        tj = json.load(f)
+    kernel_file = tj.get("kernel_source_file", "sharpnet_amd/csrc/sgemm_mfma.hpp")
+    kpath = os.path.join(root, kernel_file)
+    now = source_hash(kpath) if os.path.exists(kpath) else None
+    stale = (tj.get("kernel_source_sha256_16") is None) or (now != tj.get("kernel_source_sha256_16"))
+    return tj.get("hbm_bytes_per_launch"), {"file": "profiles/sgemm_8192_hbm_traffic.json",
+                                            "measured_in_this_run": False, "stale": bool(stale),
+                                            "kernel_source_sha256_16": tj.get("kernel_source_sha256_16"),
+                                            "summary": tj.get("source")}
 
 
 def main():
@@ -39,6 +87,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--extra-out", default=os.path.join("gpurun_out", "bench_extra.json"), metavar="PATH",
+                    help="where the per-product figures of the other configurations are written (JSON)")
     ap.add_argument("--table", default=None, metavar="PATH",
                     help="also write the per-configuration figures of `extra` as a markdown table to PATH")
     ap.add_argument("--pcie", action="store_true",
@@ -89,6 +139,9 @@ def main():
                 for _ in range(10):
                     launch()
                 w.synchronize()
+        if c is not None:
+            # beta != 0: the timed launches start from the seeded C again, so that the timed result has a closed form
+            gc.InitializeFromHostMemory(c)
         e0, e1 = w.new_event(), w.new_event()
         w.synchronize()
         t0 = time.perf_counter()
@@ -106,6 +159,35 @@ def main():
         if gbias is not None:
             gbias.Dispose()
         return wall_ms, ev_ms, gc
+
+    def check_timed_result(gm, aa, bb, cc, got, steps, bias=None, bf16=False, nrows=6):
+        """Sampled rows of a timed result against the oracle.  `got` is C after `steps` launches that started from
+        the seeded C (beta is 0 or 1 in every benchmark product: C = steps*alpha*op(A)op(B) + C0 for beta = 1).
+        bf16: the oracle multiplies the operands rounded to bf16 (what the reduced-precision kernels compute)."""
+        from oracle import dot_oracle
+        assert gm.beta in (0.0, 1.0)
+        pick = np.random.default_rng(4242)
+        reps = steps if gm.beta != 0 else 1
+        mats = [None] if gm.batch == 1 else list(np.sort(pick.choice(gm.batch, min(3, gm.batch), replace=False)))
+        worst, bound = 0.0, 0.0
+        for z in mats:
+            a2, b2 = (aa, bb) if z is None else (aa[z], bb[z])
+            g2 = got if z is None else got[z]
+            rows = np.sort(pick.choice(gm.M, min(nrows, gm.M), replace=False))
+            a_sub = np.ascontiguousarray(a2[:, rows] if gm.tA else a2[rows])
+            if bf16:
+                a_sub, b2 = dot_oracle.round_to_bf16(a_sub), dot_oracle.round_to_bf16(b2)
+            ref = dot_oracle.dot_f64(a_sub, gm.tA, b2, gm.tB, gm.alpha) * reps
+            if gm.beta != 0:
+                ref = ref + (cc if z is None else cc[z])[rows].astype(np.float64)
+            if bias is not None:
+                ref = ref + bias.reshape(1, -1).astype(np.float64) * reps
+            worst = max(worst, float(np.max(np.abs(g2[rows].astype(np.float64) - ref))))
+            bound = max(bound, dot_oracle.tolerance(gm.K, a_sub, b2) * abs(gm.alpha) * reps)
+        if not worst <= bound:
+            sys.exit("bench.py: timed result of %s is outside the parity bound (max|d| = %.3e, bound %.3e)"
+                     % (gm.label(), worst, bound))
+        return worst, bound
 
     def run_stored(gm, seed, steps, warmup, to_nt=False):
         """One product with operands stored as bf16.  to_nt (single matrices only): a transposed A / a plain B is
@@ -155,12 +237,14 @@ def main():
             return ms
         conv_ms = timed(convert, 5, 2)
         ms = timed(launch, steps, warmup)
+        err, bound = check_timed_result(gm, aa, bb, None, gcs.ToNumpy(), steps, bf16=True)
         by = gm.batch * (2.0 * (gm.M * gm.K + gm.K * gm.N) + 4.0 * gm.M * gm.N)
         roof_s = max(gm.flops / (wl.BF16_MFMA_PEAK_TFLOPS * 1e12), by / (wl.HBM_PEAK_GBS * 1e9))
         r = {"gemm": gm.label() + (" (bf16 storage, operands transposed to the NT form by the conversion)" if to_nt
                                  else " (bf16 storage)"), "ms": round(ms, 4), "tflops": round(gm.flops / (ms * 1e-3) / 1e12, 2),
              "frac_of_roofline": round(roof_s * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
-             "splitk": w.last_tuning()[1], "algorithmic_bytes": by, "convert_both_operands_ms": round(conv_ms, 4)}
+             "splitk": w.last_tuning()[1], "algorithmic_bytes": by, "convert_both_operands_ms": round(conv_ms, 4),
+             "max_abs_err": err, "parity_bound": bound}
         w.release(pa, 2 * ga.Count)
         w.release(pb, 2 * gb.Count)
         for t in (ga, gb, gcs):
@@ -303,15 +387,7 @@ def main():
 
     # HBM traffic per launch is a counter figure (two rocprofv3 --pmc runs); it cannot be collected from inside
     # this process, so the line carries the stored figure together with where and when it was measured.
-    traffic, traffic_source = None, None
-    tpath = os.path.join(ROOT, "profiles", "sgemm_8192_hbm_traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            tj = json.load(f)
-        traffic = tj.get("hbm_bytes_per_launch")
-        traffic_source = {"file": "profiles/sgemm_8192_hbm_traffic.json", "measured_in_this_run": False,
-                          "kernel": tj.get("workload"), "kernel_source_commit": tj.get("kernel_source_commit"),
-                          "summary": tj.get("source")}
+    traffic, traffic_source = traffic_record(ROOT)
 
     out = {
         "metric": "fp32 GEMM throughput, Tensor.Dot M=N=K=8192 (GEMM TFLOP/s + % of fp32 MFMA peak at 1 GPU)",
@@ -324,7 +400,9 @@ def main():
                    "device": {"cu": info["compute_units"], "clock_mhz": info["clock_khz"] / 1000.0}},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": wl.FP32_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / wl.FP32_MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
-                     "traffic_source": traffic_source, "flops_per_launch": g.flops, "ms_per_launch_hip_events": round(ev_ms, 4)},
+                     "traffic_source": traffic_source, "flops_per_launch": g.flops,
+                     "ms_per_launch_hip_events": round(ev_ms, 4),
+                     "kernel": "sgemm_mfma_kernel<TileCfg<4,4,2,2,16>, NN> (256x256x16 tiles)"},
         "parity": {"max_abs_err": err, "bound": bound, "rows_checked": 16},
     }
 
@@ -387,6 +465,7 @@ def main():
         cpu_on = not args.no_cpu
         cpu_cores = dot_oracle.mkl_threads() if cpu_on else 0
         cpu_spent = [0.0]
+        bf16_math = [False]       # set while the handle multiplies in the bf16-input math mode
 
         def cpu_ms(gm, aa, bb, cc, reps, bias=None):
             """Median ms of the product through MKL after one warm-up call."""
@@ -409,11 +488,12 @@ def main():
         def run(gm, seed, steps=10, warmup=3, bias=None, cpu_reps=0):
             aa, bb, cc = wl.uniform_operands(gm, seed)
             _, ms, gcx = time_gemm(gm, aa, bb, cc, steps, warmup, bias=bias, min_warm_ms=40.0)
+            err, bound = check_timed_result(gm, aa, bb, cc, gcx.ToNumpy(), steps, bias=bias, bf16=bf16_math[0])
             gcx.Dispose()
             tf = gm.flops / (ms * 1e-3) / 1e12
             r = {"gemm": gm.label(), "ms": round(ms, 4), "tflops": round(tf, 2),
                  "frac_of_roofline": round(gm.roofline_seconds() * 1e3 / ms, 4), "tile_config": w.last_tuning()[0],
-                 "splitk": w.last_tuning()[1]}
+                 "splitk": w.last_tuning()[1], "max_abs_err": err, "parity_bound": bound}
             if cpu_on and cpu_reps > 0:
                 cms = cpu_ms(gm, aa, bb, cc, cpu_reps, bias=bias)
                 r["cpu_mkl_ms"] = round(cms, 4)
@@ -510,6 +590,7 @@ def main():
                                         "(CpuTensor.BatchMatrixMultiplication), median of 3 passes after a warm-up")}
         # bf16-input / fp32-accumulate variant (operands stay fp32 in HBM, rounded on the way into LDS)
         w.set_math_mode(w.MATH_BF16_INPUT)
+        bf16_math[0] = True
         try:
             bf = [run(gm, 5, 50, 10) for gm in att_g]
             for r, gm in zip(bf, att_g):   # HBM-bound: roofline = bytes / 8 TB/s vs bf16 MFMA peak
@@ -522,6 +603,7 @@ def main():
             extra["config2_8192_bf16_input_TN"] = hb
         finally:
             w.set_math_mode(w.MATH_FP32)
+            bf16_math[0] = False
 
         # The same arithmetic on operands STORED as bf16 (2 bytes per element in HBM; algorithmic bytes use s_in = 2).
         # Operands are converted once by the library's own pass (timed separately: it is not part of the product).
@@ -538,13 +620,65 @@ def main():
             extra["cpu_leg_seconds"] = round(cpu_spent[0], 1)
             log("[bench] CPU side of the other configurations took %.1f s" % cpu_spent[0])
         extra["layers_fused_vs_reference_sequence"] = layer_timings(w, wl)
-        out["extra"] = extra
         for k, v in extra.items():
-            log("[bench]", k, json.dumps(v))
+            log("[bench]", k, json.dumps(v, allow_nan=False))
+        out["summary"] = summarize(extra)
+        full = dict(out)
+        full["extra"] = extra
+        try:
+            d = os.path.dirname(args.extra_out)
+            if d:
+                os.makedirs(d, exist_ok=True)
+            with open(args.extra_out, "w") as f:
+                json.dump(full, f, allow_nan=False, indent=1)
+            out["summary"]["per_product_figures"] = args.extra_out
+        except OSError as e:
+            log("[bench] could not write %s: %s" % (args.extra_out, e))
+        if args.table:
+            write_table(args.table, full)
 
-    if args.table and "extra" in out:
-        write_table(args.table, out)
-    print(json.dumps(out), flush=True)
+    print(headline_line(out), flush=True)
+
+
+def summarize(extra):
+    """A few figures of the other configurations for the stdout line (the rest is in the extra file)."""
+    def best(rows, key="tflops"):
+        return max(r[key] for r in rows)
+
+    def pick(rows, label):
+        for r in rows:
+            if r["gemm"].startswith(label) or label in r["gemm"]:
+                return r
+        return None
+    s = {}
+    fb = extra.get("config1_dense_layer_fwd_bwd")
+    if fb:
+        s["config1_dense_fwd_bwd_ms"] = {"gpu": fb["gpu_ms"], "cpu_mkl": fb["cpu_mkl_ms"], "cpu_cores": fb["cpu_cores"]}
+    else:
+        s["config1_dense_fwd_bwd_ms"] = {"gpu": round(sum(r["ms"] for r in extra["config1_dense_layer"]["gemms"]), 4)}
+    for r in extra.get("layers_fused_vs_reference_sequence", []):
+        if r["layer"].startswith("Linear 128x784->256") and r["form"] == "fused":
+            s["config1_dense_fused_calls_ms"] = {"forward": r["forward_ms"], "backward": r["backward_ms"]}
+    sw = extra["config2_sweep"]["gemms"]
+    fr = {}
+    for r in sw:
+        size = r["gemm"].split(")")[0] + ")"
+        fr.setdefault(size, []).append(r["frac_of_roofline"])
+    s["config2_frac_of_roofline_min_max"] = {k: [min(v), max(v)] for k, v in fr.items()}
+    s["config3_mlp_step"] = {"ms": extra["config3_mlp_step"]["total_ms"], "tflops": extra["config3_mlp_step"]["tflops"]}
+    s["config4_lstm"] = {"input_projection_frac": extra["config4_lstm"]["input_projection"]["frac_of_roofline"],
+                         "recurrent_step_ms": extra["config4_lstm"]["recurrent_step"]["ms"]}
+    s["config5_attention_ms"] = {"fp32": [r["ms"] for r in extra["config5_attention_fp32"]["gemms"]],
+                                 "bf16_input": [r["ms"] for r in extra["config5_attention_bf16_input"]["gemms"]],
+                                 "bf16_stored": [r["ms"] for r in extra["config5_attention_bf16_stored"]["gemms"]]}
+    s["bf16_8192_tflops"] = {"input_TN": extra["config2_8192_bf16_input_TN"]["tflops"],
+                             "stored_best": best(extra["config2_8192_bf16_stored"])}
+    rows = 0
+    for v in extra.values():
+        items = v if isinstance(v, list) else (v.get("gemms") or [v]) if isinstance(v, dict) else []
+        rows += sum(1 for r in items if isinstance(r, dict) and "max_abs_err" in r)
+    s["timed_products_checked_against_oracle"] = rows
+    return s
 
 
 def layer_timings(w, wl):
@@ -603,7 +737,7 @@ def layer_timings(w, wl):
             res.append({"layer": "ScaledDotProductAttention forward 512 x (256 x 64)%s, weights kept" %
                                  (", causal" if causal else ""),
                         "form": "one launch" if fused else "reference sequence (4 calls)", "forward_ms": ms,
-                        "backward_ms": float("nan")})
+                        "backward_ms": None})
     # the same launch on a handle in the bf16-input math mode (Q, K, V and the probabilities rounded to bf16 for the MFMAs)
     w.set_math_mode(1)
     try:
@@ -615,7 +749,7 @@ def layer_timings(w, wl):
             ms = timed(sdpa_bf16, 20, 10)
             res.append({"layer": "ScaledDotProductAttention forward 512 x (256 x 64), bf16-input math, weights %s" %
                                  ("kept" if training else "not kept"),
-                        "form": "one launch", "forward_ms": ms, "backward_ms": float("nan")})
+                        "form": "one launch", "forward_ms": ms, "backward_ms": None})
     finally:
         w.set_math_mode(0)
     dq, dk_, dv_, do = (GPUTensor([Z, Tn, d], None, w) for _ in range(4))
@@ -659,7 +793,7 @@ def layer_timings(w, wl):
                 res.append({"layer": "ScaledDotProductAttention forward 64 x (1024 x 64)%s, weights %s" %
                                      (", causal" if causal else "", "kept" if training else "not kept"),
                             "form": "one launch" if fused else "reference sequence (4 calls)", "forward_ms": ms,
-                            "backward_ms": float("nan")})
+                            "backward_ms": None})
     dq, dk_, dv_, do = (GPUTensor([Z, Tn, d], None, w) for _ in range(4))
     do.SetValue(0.01)
     for fused in (True, False):
@@ -791,7 +925,7 @@ def write_table(path, out):
                     "| layer | form | forward ms | backward ms |\n|---|---|---|---|\n")
             for r in layers:
                 f.write("| %s | %s | %.4f | %s |\n" % (r["layer"], r["form"], r["forward_ms"],
-                                                         "" if r["backward_ms"] != r["backward_ms"] else "%.4f" % r["backward_ms"]))
+                                                         "" if r["backward_ms"] is None else "%.4f" % r["backward_ms"]))
             f.write("\n")
         f.write("Headline line of the same run: %.2f TFLOP/s (%.1f %% of fp32 MFMA peak)" %
                 (out["value"], 100.0 * out["roofline"]["frac"]))

@@ -90,16 +90,19 @@ int snhip_dot(void* handle, const float* A, int aH, int aW, int transposeA, cons
  * of tile configuration and split-K factor, bit-identical results; the difference is where split-K partial sums
  * go: into a fixed array of snhip_static_scratch_bytes() (32 MiB) that is part of the library's code object on
  * every GPU, instead of the handle's lazily grown workspace.  The call never allocates, frees or synchronises.
- * A product whose partial sums need more than the array holds is refused with status 15 (NOT_SUPPORTED) before
- * anything is launched; snhip_get_last_error_message then says how many bytes were needed.  Products that run
- * without split-K use no scratch and are never refused.  All handles of one GPU share that GPU's array: calls that
+ * A split-K factor the library chose by itself is halved until the partial sums fit the array (down to no split):
+ * results are then within the same bound but bit-identical to snhip_dot's only while the factor is unchanged
+ * (snhip_get_last_tuning reports it).  A factor forced with snhip_set_tuning whose partial sums need more than the
+ * array holds is refused with status 15 (NOT_SUPPORTED) before anything is launched; snhip_get_last_error_message
+ * then says how many bytes were needed.  Products that run without split-K use no scratch and are never refused.  All handles of one GPU share that GPU's array: calls that
  * overlap in time on one GPU (two handles on two streams) race on it. */
 int snhip_dot_noalloc(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
                       int transposeB, float* C, float alpha, float beta);
 /* Size in bytes of the static scratch array (returns the size, not a status). */
 int snhip_static_scratch_bytes(void);
-/* Copies the text of the handle's last refusal that carries detail beyond its status code (empty if none) into
- * buffer as a NUL-terminated string of at most capacity bytes. */
+/* Copies the detail text of the handle's most recent product call into buffer as a NUL-terminated string of at
+ * most capacity bytes: empty unless that call was refused with more to say than its status code (every product call
+ * clears the text on entry, so it never describes an older call). */
 int snhip_get_last_error_message(void* handle, char* buffer, int capacity);
 
 /* snhip_dot followed by C[m][n] += bias[n], in one kernel.  Replaces the pair
@@ -342,6 +345,10 @@ int snhip_rnn_backward_weights(void* handle, const snhip_rnn_desc* desc, int bat
 /* Selects the arithmetic used by every GEMM entry point of this handle
  * (the role cublasSetMathMode plays for cuBLAS handles). Default SNHIP_MATH_FP32. */
 int snhip_set_math_mode(void* handle, int mode);
+/* Bytes one element of A or B takes in device memory under a math mode: 2 for SNHIP_MATH_BF16_STORED, 4 for the
+ * other two, 0 for a value that is no mode (returns that size, not a status).  Strides and pitches of such operands
+ * count elements, and this is the factor the library itself applies wherever it offsets an operand on the host. */
+int snhip_operand_element_bytes(int math_mode);
 /* snhip_dot_bias / snhip_bmm in bf16-input arithmetic regardless of the handle's mode. */
 int snhip_dot_bf16(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,
                    int transposeB, float* C, float alpha, float beta, const float* bias);

@@ -201,7 +201,8 @@ const ConfigEntry kConfigs[] = {
     make_entry_bf16_stored<BTileCfg<4, 4, 2, 2, 64>>(1, 0.85, 0.85, 3.0),   // 18: 256 x 256, BK 64
     make_entry_bf16_stored<BTileCfg<2, 2, 2, 2, 64>>(2, 0.65, 0.80, 1.3),   // 19: 128 x 128, BK 64
     make_entry_bf16_stored<BTileCfg<1, 1, 2, 2, 128>>(2, 0.45, 0.60, 1.1),  // 20: 64 x 64, BK 128
-    // K split eight ways over a workgroup of eight wavefronts: see prefer_ksplit()
+    // K split eight ways over a workgroup of eight wavefronts.  No product takes it by default (configuration 26,
+    // 16 x 16 tiles, superseded it); it runs only when forced with snhip_set_tuning(21, 1)
     ConfigEntry{32, 32, 32, 512, KsplitCfg<1, 8>::LDS_BYTES, 1, 2,
                 {{sgemm_ksplit_kernel<false, false, 1, 8>, sgemm_ksplit_kernel<false, true, 1, 8>},
                  {sgemm_ksplit_kernel<true, false, 1, 8>, sgemm_ksplit_kernel<true, true, 1, 8>}},
@@ -566,9 +567,18 @@ int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, 
     return cfg;
 }
 
+// Operand pointers travel as const float* whatever the storage; A and B of SNHIP_MATH_BF16_STORED hold 2-byte
+// elements and their strides count those, so host-side offsets are applied in bytes.
+inline const float* advance_operand(const float* base, long long elements, int math) {
+    if (base == nullptr) return nullptr;
+    const long long elem_bytes = snhip_operand_element_bytes(math);
+    return reinterpret_cast<const float*>(reinterpret_cast<const char*>(base) + elements * elem_bytes);
+}
+
 int gemm_core(Handle* h, const GemmArgs& g) {
     if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     const int math = (g.math < 0) ? h->math_mode : g.math;
+    h->last_error[0] = 0;  // the text belongs to the call that set it
     {
         // The handle belongs to one device (GPUWrapper.AssociateCurrentThreadWithDevice, GPUWrapper.cs:782-788);
         // a caller thread whose current device differs is switched to it, as cudaSetDevice would have been.
@@ -609,8 +619,8 @@ int gemm_core(Handle* h, const GemmArgs& g) {
         part.batch_inner = 0;
         for (int z0 = 0; z0 < batch; z0 += 65535) {
             part.batch = (batch - z0 < 65535) ? (batch - z0) : 65535;
-            part.A = (g.A != nullptr) ? g.A + (long long)z0 * g.sA : nullptr;
-            part.B = (g.B != nullptr) ? g.B + (long long)z0 * g.sB : nullptr;
+            part.A = advance_operand(g.A, (long long)z0 * g.sA, math);
+            part.B = advance_operand(g.B, (long long)z0 * g.sB, math);
             part.C = g.C + (long long)z0 * g.sC;
             part.D = (g.D != nullptr) ? g.D + (long long)z0 * g.sD : nullptr;
             part.colsum = (g.colsum != nullptr) ? g.colsum + (long long)z0 * M : nullptr;
@@ -690,6 +700,11 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     }
     const ConfigEntry& cfg = kConfigs[ch.cfg];
     if ((long long)batch * ch.splitk > 65535) ch.splitk = 1;
+    if (g.no_alloc && h->force_splitk <= 0) {
+        // an automatically chosen split is halved until its partial sums fit the static scratch (a forced one is refused
+        // below if it does not): the product then runs with fewer K slices than the allocating entry point would use
+        while (ch.splitk > 1 && (size_t)M * N * batch * ch.splitk * sizeof(float) > kStaticScratchBytes) ch.splitk /= 2;
+    }
 
     // The extended kernels apply gamma * D and the (leaky) ReLU while writing C, walk a two-level batch, and -
     // transposed A, plain B, no split-K - add up the column sum on the side.  They are used only when one of
@@ -704,8 +719,8 @@ int gemm_core(Handle* h, const GemmArgs& g) {
         part.batch = inner;
         part.batch_inner = 0;
         for (int zo = 0; zo < batch / inner; ++zo) {
-            part.A = g.A + (long long)zo * g.sA2;
-            part.B = g.B + (long long)zo * g.sB2;
+            part.A = advance_operand(g.A, (long long)zo * g.sA2, math);
+            part.B = advance_operand(g.B, (long long)zo * g.sB2, math);
             part.C = g.C + (long long)zo * g.sC2;
             part.D = (g.D != nullptr) ? g.D + (long long)zo * g.sD2 : nullptr;
             part.colsum = (g.colsum != nullptr) ? g.colsum + (long long)zo * inner * M : nullptr;
@@ -1282,6 +1297,10 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
 }
 
 int snhip_sizeof_gemm_desc(void) { return (int)sizeof(snhip_gemm_desc); }
+int snhip_operand_element_bytes(int math_mode) {
+    if (math_mode == SNHIP_MATH_BF16_STORED) return 2;
+    return (math_mode == SNHIP_MATH_FP32 || math_mode == SNHIP_MATH_BF16_INPUT) ? 4 : 0;
+}
 
 int snhip_gemm_ex(void* handle, const snhip_gemm_desc* d) {
     if (d == nullptr || d->struct_size != (int)sizeof(snhip_gemm_desc)) return SNHIP_STATUS_INVALID_VALUE;

@@ -178,6 +178,7 @@ SIGNATURES = {
     "snhip_convert_f32_to_bf16_2d": [_vp, _vp, _i, _i, _ll, _i, _vp, _ll],
     "snhip_gemm_ex": [_vp, ctypes.POINTER(GemmDesc)],
     "snhip_sizeof_gemm_desc": [],
+    "snhip_operand_element_bytes": [_i],
     "snhip_attention_forward": [_vp, ctypes.POINTER(AttentionDesc)],
     "snhip_sizeof_attention_desc": [],
     "snhip_attention_backward": [_vp, ctypes.POINTER(AttentionBwdDesc)],

@@ -75,6 +75,8 @@ def test_gemm_descriptor_layout_matches_the_library():
     assert lib.snhip_gemm_ex(None, None) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
     d = hiplib.GemmDesc(M=1, N=1, K=1)
     assert lib.snhip_gemm_ex(None, ctypes.byref(d)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
+    # host-side operand offsets are taken in bytes of the storage type: bf16-stored operands advance 2 bytes an element
+    assert [lib.snhip_operand_element_bytes(m) for m in (0, 1, 2, 3, -1)] == [4, 4, 2, 0, 0]
     assert lib.snhip_sizeof_attention_desc() == ctypes.sizeof(hiplib.AttentionDesc)
     a = hiplib.AttentionDesc(batch=1, Tq=1, Tk=1, dk=1, dv=1)
     assert lib.snhip_attention_forward(None, ctypes.byref(a)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED

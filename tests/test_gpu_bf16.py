@@ -311,6 +311,50 @@ def test_bf16_stored_batched_bias_and_refusals(oracle, gpu_wrapper):
     assert np.isnan(go.ToNumpy()).all()
 
 
+@pytest.mark.parametrize("B,H,T,d,K_long", [(3, 2, 96, 64, False), (4, 4, 128, 320, True), (2, 3, 40, 48, False)])
+def test_bf16_stored_two_level_batch_through_gemm_ex(oracle, gpu_wrapper, B, H, T, d, K_long):
+    """snhip_gemm_ex with math = SNHIP_MATH_BF16_STORED on heads addressed in place: a two-level batch whose outer
+    strides do not continue the inner ones, with too few matrices (or too long a K) for the streaming kernels, so the
+    library walks the outer level on the host and must offset the 2-byte operands in bytes.  S[b][h] = Q[b][:, h] .
+    K[b][:, h]^T; compared with the same call in bf16-input arithmetic on the fp32 originals and with the oracle on
+    rounded inputs."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    rng = np.random.default_rng(4300 + B * 7 + H)
+    E = H * d
+    q, k = random_tensor(rng, (B, T, E), -1, 1), random_tensor(rng, (B, T, E), -1, 1)
+    gq, gk = GPUTensor(q.shape, q, w), GPUTensor(k.shape, k, w)
+    pq, pk = to_bf16_on_device(w, gq), to_bf16_on_device(w, gk)
+    print("two-level bf16-stored", B, H, T, d, K_long, flush=True)
+    fields = dict(transA=0, transB=1, M=T, N=T, K=d, alpha=0.125, beta=0.0, lda=E, ldb=E, ldc=T, batch=B * H,
+                  batch_inner=H, strideA=d, strideB=d, strideC=T * T, strideA_outer=T * E, strideB_outer=T * E,
+                  strideC_outer=H * T * T)
+    got = {}
+    for math, a_ptr, b_ptr in ((2, pq, pk), (1, gq.Pointer, gk.Pointer)):
+        gs = GPUTensor([B, H, T, T], None, w)
+        gs.SetValue(float("nan"))
+        gs.GemmEx(A=a_ptr, B=b_ptr, math=math, **fields)
+        got[math] = gs.ToNumpy()
+        if math == 2:
+            # the path under test: not the streaming kernels (which walk both levels themselves)
+            kinds = {c["id"]: c["kind"] for c in w.configs()}
+            assert kinds[w.last_tuning()[0]] == "bf16-stored", kinds[w.last_tuning()[0]]
+        gs.Dispose()
+    qr, kr = oracle.round_to_bf16(q).reshape(B, T, H, d), oracle.round_to_bf16(k).reshape(B, T, H, d)
+    ref = np.empty((B, H, T, T), np.float32)
+    for b in range(B):
+        for h in range(H):
+            ref[b, h] = oracle.dot(np.ascontiguousarray(qr[b, :, h]), False, np.ascontiguousarray(kr[b, :, h]), True, 0.125)
+    bound = 1e-4 * np.sqrt(d) * 0.125
+    assert np.all(np.isfinite(got[2]))
+    assert float(np.max(np.abs(got[2] - ref))) <= bound
+    assert float(np.max(np.abs(got[2] - got[1]))) <= bound
+    w.release(pq, max(2 * gq.Count, 8))
+    w.release(pk, max(2 * gk.Count, 8))
+    gq.Dispose()
+    gk.Dispose()
+
+
 @pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
 def test_bf16_streaming_kernels_strided_batches(oracle, gpu_wrapper, tA, tB):
     """The persistent streaming kernels in bf16-input arithmetic, fp32 storage and bf16 storage: more tiles than

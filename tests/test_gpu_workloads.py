@@ -102,15 +102,18 @@ def test_config4_lstm_projections(oracle, gpu_wrapper):
     d = wl.lstm_inputs(seed=4)
     proj, rec, _ = wl.lstm_gemms()
     sampled_rows_check(oracle, w, proj, d["x"], d["w"], None, nrows=8)
-    steps = 6
+    _, _, steps = wl.lstm_gemms()
+    assert steps == 128                         # the whole chain of sequential beta = 1 products
     rng = np.random.default_rng(44)
     hs = [np.tanh(rng.normal(0, 1, d["h"].shape)).astype(np.float32) for _ in range(steps)]
     gates0 = rng.normal(0, 1, (rec.M, rec.N)).astype(np.float32)
     gg, gu = GPUTensor([rec.M, rec.N], gates0, w), GPUTensor(list(d["u"].shape), d["u"], w)
-    ref = gates0.copy()
+    ref = gates0.astype(np.float64)
     for h in hs:
-        gg.Dot(GPUTensor(list(h.shape), h, w), False, gu, False, 1.0, 1.0)
-        ref = oracle.dot(h, False, d["u"], False, 1.0, 1.0, ref)
+        gh = GPUTensor(list(h.shape), h, w)
+        gg.Dot(gh, False, gu, False, 1.0, 1.0)
+        gh.Dispose()
+        ref = oracle.dot_f64(h, False, d["u"], False, 1.0, 1.0, ref)
     assert np.max(np.abs(gg.ToNumpy() - ref)) <= steps * bound(rec.K, hs[0], d["u"], 1e-6)
 
 
