@@ -29,6 +29,84 @@ def test_library_exports_every_declared_symbol():
     assert sorted(hiplib.SIGNATURES) == declared_symbols()
 
 
+def _c_prototypes():
+    """name -> list of C parameter type classes, from include/sharpnet_hip.h."""
+    text = open(os.path.join(ROOT, "include", "sharpnet_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    protos = {}
+    for name, args in re.findall(r"\bint\s+(snhip_\w+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        params = [a.strip() for a in args.replace("\n", " ").split(",")]
+        if params == ["void"] or params == [""]:
+            params = []
+        kinds = []
+        for prm in params:
+            if "*" in prm:
+                kinds.append("ptr")
+            elif re.match(r"(unsigned\s+)?long long\b", prm):
+                kinds.append("i64")
+            elif prm.startswith("size_t"):
+                kinds.append("size")
+            elif prm.startswith("float"):
+                kinds.append("f32")
+            elif re.match(r"(unsigned(\s+int)?|int)\b", prm):
+                kinds.append("i32")
+            else:
+                raise AssertionError("unclassified C parameter %r of %s" % (prm, name))
+        protos[name] = kinds
+    return protos
+
+
+def _csharp_prototypes():
+    """name -> list of parameter type classes, from the DllImport declarations of integration/SharpNetHipWrapper.cs."""
+    text = open(os.path.join(ROOT, "integration", "SharpNetHipWrapper.cs")).read()
+    text = re.sub(r"//[^\n]*", "", text)
+    protos = {}
+    for ret, name, args in re.findall(r"\[DllImport\(DLL_NAME\)\]\s*public static extern (\w+) (snhip_\w+)\(([^;]*?)\);",
+                                      text, flags=re.S):
+        assert ret in ("cublasStatus_t", "int"), (name, ret)
+        params = [a.strip() for a in args.replace("\n", " ").split(",") if a.strip()]
+        kinds = []
+        for prm in params:
+            words = prm.split()
+            if words[0] in ("ref", "out") or words[0] in ("IntPtr", "System.Text.StringBuilder"):
+                kinds.append("ptr")
+            elif words[0] == "long":
+                kinds.append("i64")
+            elif words[0] in ("UIntPtr", "size_t"):
+                kinds.append("size")
+            elif words[0] == "float":
+                kinds.append("f32")
+            elif words[0] in ("int", "uint", "cublasOperation_t", "cublasSideMode_t"):
+                kinds.append("i32")
+            else:
+                raise AssertionError("unclassified C# parameter %r of %s" % (prm, name))
+        protos[name] = kinds
+    return protos
+
+
+def test_csharp_shim_matches_the_header():
+    """The P/Invoke declarations a SharpNet maintainer would add (the counterpart of Prod/GPU/CublasWrapper.cs:219-252)
+    name only functions the header declares, with the same number of arguments and the same class of type in every
+    position, and cover the entry points GPUTensor.Dot / BatchMatrixMultiplication and GPUWrapper need."""
+    c, cs = _c_prototypes(), _csharp_prototypes()
+    assert len(cs) >= 50
+    for name, kinds in cs.items():
+        assert name in c, name + " is bound in the C# shim but not declared in the header"
+        assert kinds == c[name], (name, kinds, c[name])
+    for required in ("snhip_create", "snhip_destroy", "snhip_sgemm", "snhip_sgemm_strided_batched", "snhip_sgeam",
+                     "snhip_sdgmm", "snhip_dot", "snhip_dot_bias", "snhip_bmm", "snhip_gemm_ex", "snhip_dense_forward",
+                     "snhip_dense_backward", "snhip_attention_forward", "snhip_attention_backward", "snhip_rnn_forward",
+                     "snhip_dot_noalloc"):
+        assert required in cs, required
+    # the two cuBLAS-shaped calls keep cuBLAS's argument order (CublasWrapper.cs:229-244)
+    assert cs["snhip_sgemm"] == ["ptr", "i32", "i32", "i32", "i32", "i32", "ptr", "ptr", "i32", "ptr", "i32", "ptr", "ptr", "i32"]
+    assert cs["snhip_sgemm_strided_batched"] == ["ptr", "i32", "i32", "i32", "i32", "i32", "ptr", "ptr", "i32", "i64", "ptr",
+                                                 "i32", "i64", "ptr", "ptr", "i32", "i64", "i32"]
+    patch = open(os.path.join(ROOT, "integration", "call_sites.patch")).read()
+    for callee in ("snhip_sgemm(", "snhip_sgemm_strided_batched(", "snhip_create(", "snhip_destroy("):
+        assert "SharpNetHipWrapper." + callee in patch
+
+
 def test_no_compute_symbols_from_vendor_blas():
     # the library must not link a vendor GEMM (hipBLAS / rocBLAS / hipBLASLt)
     import subprocess
