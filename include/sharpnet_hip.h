@@ -194,7 +194,9 @@ int snhip_sizeof_gemm_desc(void);
 int snhip_dense_forward(void* handle, float* y, const float* x, const float* weights, const float* bias, int rows,
                         int in_features, int out_features, int activation, float activation_param);
 
-/* Linear.DenseBackwardPropagation (Prod/Layers/Linear.cs:143-191) in at most two launches:
+/* Linear.DenseBackwardPropagation (Prod/Layers/Linear.cs:143-191) in at most two launches - one when dW and dx are
+ * both a handful of 32 x 32 tiles (a layer on a small batch, e.g. 128 x 784 -> 256: the two products and the bias
+ * gradient then share one grid; not while a tile configuration is forced with snhip_set_tuning):
  *   weight_gradients = multiplier * dy^T . x + weight_decay_alpha * weights   (Linear.cs:151-158,168-178)
  *   bias_gradients   = column sums of dy, or NULL to skip                    (Linear.cs:160-165)
  *   dx               = dy . weights, or NULL when the previous layer is the input (Linear.cs:184-190)
@@ -202,6 +204,12 @@ int snhip_dense_forward(void* handle, float* y, const float* x, const float* wei
 int snhip_dense_backward(void* handle, float* dx, float* weight_gradients, float* bias_gradients, const float* x,
                          const float* dy, const float* weights, int rows, int in_features, int out_features,
                          float multiplier, float weight_decay_alpha);
+/* The same with the weight decay the reference applies to the bias gradient in its PyTorch compatibility mode
+ * (Linear.cs:178-181):  bias_gradients += bias_decay_alpha * bias  (bias of length out_features; ignored when
+ * bias_decay_alpha is 0 or bias_gradients is NULL).  In the one-launch form this rides in the column-sum workgroups. */
+int snhip_dense_backward_ex(void* handle, float* dx, float* weight_gradients, float* bias_gradients, const float* x,
+                            const float* dy, const float* weights, int rows, int in_features, int out_features,
+                            float multiplier, float weight_decay_alpha, const float* bias, float bias_decay_alpha);
 
 /* y = act(x) and dx = dy * act'(x) expressed through y, element-wise over n floats (in place allowed):
  * Tensor.ActivationForward / ActivationBackward for the modes above (Prod/GPU/GpuTensor.cs ActivationForward,

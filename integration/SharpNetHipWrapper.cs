@@ -92,6 +92,8 @@ namespace SharpNet.GPU
         // Linear layer in one / two launches; activation: 0 none, 1 relu, 2 leaky relu (param = slope), 3 sigmoid, 4 tanh
         [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_dense_forward(IntPtr handle, IntPtr y, IntPtr x, IntPtr weights, IntPtr bias, int rows, int inFeatures, int outFeatures, int activation, float activationParam);
         [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_dense_backward(IntPtr handle, IntPtr dx, IntPtr weightGradients, IntPtr biasGradients, IntPtr x, IntPtr dy, IntPtr weights, int rows, int inFeatures, int outFeatures, float multiplier, float weightDecayAlpha);
+        // ... with the PyTorch-mode weight decay on the bias gradient (Linear.cs:178-181): biasGradients += biasDecayAlpha * bias
+        [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_dense_backward_ex(IntPtr handle, IntPtr dx, IntPtr weightGradients, IntPtr biasGradients, IntPtr x, IntPtr dy, IntPtr weights, int rows, int inFeatures, int outFeatures, float multiplier, float weightDecayAlpha, IntPtr bias, float biasDecayAlpha);
         [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_activation_forward(IntPtr handle, int activation, float activationParam, IntPtr x, IntPtr y, long n);
         [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_activation_backward(IntPtr handle, int activation, float activationParam, IntPtr y, IntPtr dy, IntPtr dx, long n);
 

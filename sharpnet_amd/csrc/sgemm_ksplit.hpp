@@ -98,11 +98,12 @@ struct KsplitOperand {
     }
 };
 
-template <bool TA, bool TB, int NT = 1, int NW = 4>
-__global__ void __launch_bounds__(64 * NW) sgemm_ksplit_kernel(const GemmParams p) {
+// One workgroup's share of the product: tile `tile_index` (of p.tiles_m * p.tiles_n) of matrix z.  `smem` is the
+// workgroup's dynamic LDS (KsplitCfg<NT, NW>::LDS_BYTES).
+template <bool TA, bool TB, int NT, int NW>
+__device__ __forceinline__ void ksplit_tile(const GemmParams& p, int tile_index, int z, float* smem) {
     using C = KsplitCfg<NT, NW>;
     constexpr int KS = C::KS, D = C::DEPTH, P = C::PITCH;
-    extern __shared__ __attribute__((aligned(16))) float smem[];
     float(*const part)[NT][32][33] = reinterpret_cast<float(*)[NT][32][33]>(smem);  // [KS][NT][32][33], after the k loop
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lhi = lane >> 5;
     const int nt = wave % NT, kg = wave / NT;
@@ -110,10 +111,9 @@ __global__ void __launch_bounds__(64 * NW) sgemm_ksplit_kernel(const GemmParams 
     // the XCDs, the other one stays put (when the fast count is a multiple of 8): the dispatcher lets the tiles of
     // the smaller operand run fastest, so that each XCD's L2 fetches its own part of the larger operand only once.
     const bool n_fastest = (p.flags & GEMM_FLAG_TILE_N_FASTEST) != 0;
-    const int tile_m = n_fastest ? blockIdx.x / p.tiles_n : blockIdx.x % p.tiles_m;
-    const int tile_n = n_fastest ? blockIdx.x % p.tiles_n : blockIdx.x / p.tiles_m;
+    const int tile_m = n_fastest ? tile_index / p.tiles_n : tile_index % p.tiles_m;
+    const int tile_n = n_fastest ? tile_index % p.tiles_n : tile_index / p.tiles_m;
     const int m0 = tile_m * 32, n0 = tile_n * (32 * NT) + 32 * nt;
-    const int z = blockIdx.y;
     const float* Ab = p.A + (long long)z * p.strideA;
     const float* Bb = p.B + (long long)z * p.strideB;
     float* Cb = p.C + (long long)z * p.strideC;
@@ -228,6 +228,65 @@ __global__ void __launch_bounds__(64 * NW) sgemm_ksplit_kernel(const GemmParams 
         if (p.ep.addend != nullptr) v += p.ep.gamma * p.ep.addend[(long long)z * p.ep.strideD + (long long)row * p.ep.ldd + col];
         if (p.ep.act == ACT_RELU || p.ep.act == ACT_LEAKY_RELU) v = leaky_relu(v, p.ep.act_param);
         *c = v;
+    }
+}
+
+template <bool TA, bool TB, int NT = 1, int NW = 4>
+__global__ void __launch_bounds__(64 * NW) sgemm_ksplit_kernel(const GemmParams p) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    ksplit_tile<TA, TB, NT, NW>(p, blockIdx.x, blockIdx.y, smem);
+}
+
+// The backward pass of a Dense layer on a small batch in ONE launch (Linear.DenseBackwardPropagation,
+// Prod/Layers/Linear.cs:142-191): the three results come from the same dy,
+//     dW = multiplier * dy^T . x + gamma * W     (pw: transposed A = dy, plain B = x, addend W)
+//     dx = dy . W                                (px: plain A = dy, plain B = W)
+//     db[c] = sum over rows of dy[r][c] + bias_alpha * bias[c]     (64 columns per workgroup; the second term is
+//                                                the weight decay on the bias of Linear.cs:178-181, bias may be nullptr)
+// and each alone is a handful of 32 x 32 tiles that costs a launch more than its arithmetic.  The grid is the
+// concatenation of the three jobs' workgroups: [0, blocks_w) tiles of dW, then blocks_x tiles of dx, then the column
+// blocks of db; every workgroup runs exactly the code its job would run in a launch of its own, so results are
+// bit-identical to the separate launches.
+struct DenseBackwardSmallParams {
+    GemmParams pw, px;
+    int blocks_w, blocks_x;
+    const float* dy;   // rows x cols, row pitch ld; db may be nullptr (no column blocks in the grid then)
+    float* db;
+    const float* bias;
+    float bias_alpha;
+    int rows, cols;
+    long long ld;
+};
+__global__ void __launch_bounds__(256) dense_backward_small_kernel(const DenseBackwardSmallParams q) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    const int b = blockIdx.x;  // uniform: the three branches never diverge inside a workgroup
+    if (b < q.blocks_w) {
+        ksplit_tile<true, false, 1, 4>(q.pw, b, 0, smem);
+    } else if (b < q.blocks_w + q.blocks_x) {
+        ksplit_tile<false, false, 1, 4>(q.px, b - q.blocks_w, 0, smem);
+    } else {
+        // wavefront w adds rows w, w + 4, ... of its 64 columns; the four partial sums meet in LDS in a fixed order
+        float(*const part)[64] = reinterpret_cast<float(*)[64]>(smem);
+        const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+        const int c = (b - q.blocks_w - q.blocks_x) * 64 + lane;
+        float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+        if (c < q.cols) {
+            int r = w;
+            for (; r + 12 < q.rows; r += 16) {
+                s0 += q.dy[(long long)r * q.ld + c];
+                s1 += q.dy[(long long)(r + 4) * q.ld + c];
+                s2 += q.dy[(long long)(r + 8) * q.ld + c];
+                s3 += q.dy[(long long)(r + 12) * q.ld + c];
+            }
+            for (; r < q.rows; r += 4) s0 += q.dy[(long long)r * q.ld + c];
+        }
+        part[w][lane] = (s0 + s1) + (s2 + s3);
+        __syncthreads();
+        if (w == 0 && c < q.cols) {
+            float v = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+            if (q.bias != nullptr) v += q.bias_alpha * q.bias[c];
+            q.db[c] = v;
+        }
     }
 }
 

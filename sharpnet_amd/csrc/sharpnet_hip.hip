@@ -949,6 +949,73 @@ hipError_t prepare_kernels_once(int dev) {
 
 }  // namespace
 
+// Dense-layer backward on a small batch: when dW and dx are each a product that prefer_ksplit() would give 32 x 32
+// tiles with K split over four wavefronts, the two products and the bias gradient go out as ONE launch
+// (dense_backward_small_kernel).  Returns kNotTaken when the layer does not qualify (the caller then issues the
+// products one by one), else the status of the launch.
+constexpr int kNotTaken = -1;
+int dense_backward_small(Handle* h, float* dx, float* dW, float* db, const float* x, const float* dy, const float* W,
+                         int rows, int in_features, int out_features, float multiplier, float weight_decay_alpha,
+                         const float* bias, float bias_decay_alpha) {
+    if (h->math_mode != SNHIP_MATH_FP32 || h->force_cfg >= 0 || h->force_splitk > 0) return kNotTaken;
+    if (rows <= 0 || in_features <= 0 || out_features <= 0 || x == nullptr || dy == nullptr || W == nullptr) return kNotTaken;
+    if (multiplier == 0.0f) return kNotTaken;  // alpha == 0: A and B are not referenced, another path
+    GemmArgs gw;  // dW = multiplier * dy^T . x + weight_decay_alpha * W
+    gw.tA = true;
+    gw.M = out_features, gw.N = in_features, gw.K = rows;
+    gw.alpha = multiplier;
+    gw.A = dy, gw.lda = out_features, gw.B = x, gw.ldb = in_features, gw.C = dW, gw.ldc = in_features;
+    gw.D = W, gw.ldd = in_features, gw.gamma = weight_decay_alpha;
+    GemmArgs gx;  // dx = dy . W
+    gx.M = rows, gx.N = in_features, gx.K = out_features;
+    gx.A = dy, gx.lda = out_features, gx.B = W, gx.ldb = in_features, gx.C = dx, gx.ldc = in_features;
+    if (prefer_ksplit(h, gw, SNHIP_MATH_FP32, false) != kKsplitConfig) return kNotTaken;
+    if (prefer_ksplit(h, gx, SNHIP_MATH_FP32, false) != kKsplitConfig) return kNotTaken;
+    {
+        int cur = -1;
+        if (hipGetDevice(&cur) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+        if (cur != h->device && hipSetDevice(h->device) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;
+    }
+    h->last_error[0] = 0;
+    auto fill = [](const GemmArgs& g, GemmParams& p) {
+        p = GemmParams{};
+        p.A = g.A, p.B = g.B, p.C = g.C;
+        p.ep.bias = nullptr;
+        p.ep.addend = (g.gamma != 0.0f) ? g.D : nullptr;
+        p.ep.ldd = g.ldd;
+        p.ep.strideD = 0, p.ep.strideD2 = 0;
+        p.ep.gamma = g.gamma;
+        p.ep.act = ACT_NONE;
+        p.ep.act_param = 0.0f;
+        p.M = g.M, p.N = g.N, p.K = g.K;
+        p.lda = g.lda, p.ldb = g.ldb, p.ldc = g.ldc;
+        p.batch_inner = 1;
+        p.tiles_m = ceil_div(g.M, 32);
+        p.tiles_n = ceil_div(g.N, 32);
+        p.splitk = 1;
+        p.kchunk = g.K;
+        p.alpha = g.alpha, p.beta = 0.0f;
+        p.group_m = 8;
+        p.nz = 1;
+        p.flags = (g.M <= g.N) ? GEMM_FLAG_TILE_N_FASTEST : 0;
+    };
+    DenseBackwardSmallParams q;
+    fill(gw, q.pw);
+    fill(gx, q.px);
+    q.blocks_w = q.pw.tiles_m * q.pw.tiles_n;
+    q.blocks_x = q.px.tiles_m * q.px.tiles_n;
+    q.dy = dy, q.db = db, q.rows = rows, q.cols = out_features, q.ld = out_features;
+    q.bias = (bias_decay_alpha != 0.0f) ? bias : nullptr;
+    q.bias_alpha = bias_decay_alpha;
+    const int blocks_b = (db != nullptr) ? ceil_div(out_features, 64) : 0;
+    constexpr int kLdsBytes = KsplitCfg<1, 4>::LDS_BYTES;
+    hipLaunchKernelGGL(dense_backward_small_kernel, dim3((unsigned)(q.blocks_w + q.blocks_x + blocks_b)), dim3(256),
+                       kLdsBytes, h->stream, q);
+    h->last_cfg = kKsplitConfig;
+    h->last_splitk = 1;
+    return hip_to_status(hipGetLastError());
+}
+
 extern "C" {
 
 int snhip_create(void** handle) {
@@ -1330,10 +1397,16 @@ int snhip_dense_forward(void* handle, float* y, const float* x, const float* wei
     return gemm_core(static_cast<Handle*>(handle), g);
 }
 
-int snhip_dense_backward(void* handle, float* dx, float* weight_gradients, float* bias_gradients, const float* x,
-                         const float* dy, const float* weights, int rows, int in_features, int out_features,
-                         float multiplier, float weight_decay_alpha) {
+int snhip_dense_backward_ex(void* handle, float* dx, float* weight_gradients, float* bias_gradients, const float* x,
+                            const float* dy, const float* weights, int rows, int in_features, int out_features,
+                            float multiplier, float weight_decay_alpha, const float* bias, float bias_decay_alpha) {
     Handle* h = static_cast<Handle*>(handle);
+    if (bias_decay_alpha != 0.0f && bias_gradients != nullptr && bias == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    if (h != nullptr && dx != nullptr && weight_gradients != nullptr) {
+        const int st = dense_backward_small(h, dx, weight_gradients, bias_gradients, x, dy, weights, rows, in_features,
+                                            out_features, multiplier, weight_decay_alpha, bias, bias_decay_alpha);
+        if (st != kNotTaken) return st;
+    }
     if (weight_gradients != nullptr || bias_gradients != nullptr) {
         if (weight_gradients == nullptr) {
             const int st = snhip_bias_gradient(handle, dy, rows, out_features, bias_gradients);
@@ -1349,12 +1422,23 @@ int snhip_dense_backward(void* handle, float* dx, float* weight_gradients, float
             const int st = gemm_core(h, g);
             if (st != SNHIP_STATUS_SUCCESS) return st;
         }
+        if (bias_gradients != nullptr && bias_decay_alpha != 0.0f) {  // Linear.cs:178-181
+            const int st = snhip_axpy(handle, out_features, bias_decay_alpha, bias, bias_gradients);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
     }
     if (dx == nullptr) return SNHIP_STATUS_SUCCESS;
     GemmArgs g;  // dx = dy . W
     g.M = rows, g.N = in_features, g.K = out_features;
     g.A = dy, g.lda = out_features, g.B = weights, g.ldb = in_features, g.C = dx, g.ldc = in_features;
     return gemm_core(h, g);
+}
+
+int snhip_dense_backward(void* handle, float* dx, float* weight_gradients, float* bias_gradients, const float* x,
+                         const float* dy, const float* weights, int rows, int in_features, int out_features,
+                         float multiplier, float weight_decay_alpha) {
+    return snhip_dense_backward_ex(handle, dx, weight_gradients, bias_gradients, x, dy, weights, rows, in_features,
+                                   out_features, multiplier, weight_decay_alpha, nullptr, 0.0f);
 }
 
 int snhip_dot_bias(void* handle, const float* A, int aH, int aW, int transposeA, const float* B, int bH, int bW,

@@ -195,6 +195,7 @@ SIGNATURES = {
     "snhip_rnn_backward_weights": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz],
     "snhip_dense_forward": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f],
     "snhip_dense_backward": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f],
+    "snhip_dense_backward_ex": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _vp, _f],
     "snhip_activation_forward": [_vp, _i, _f, _vp, _vp, _ll],
     "snhip_activation_backward": [_vp, _i, _f, _vp, _vp, _vp, _ll],
     "snhip_sgeam": [_vp, _i, _i, _i, _i, _c_float_p, _vp, _i, _c_float_p, _vp, _i, _vp, _i],

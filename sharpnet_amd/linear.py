@@ -55,13 +55,13 @@ def DenseBackwardPropagation(dx, weightGradients, biasGradients_1D, x, dy, weigh
         rows, in_features = xAs2DMatrix.Shape
         out_features = weights.Shape[0]
         assert dyAs2DMatrix.Shape == [rows, out_features] and weightGradients.Shape == [out_features, in_features]
-        check_status(dy._lib.snhip_dense_backward(
+        # weight decay on the bias gradient as well in the PyTorch mode (Linear.cs:178-181)
+        bias_alpha = alpha if (alpha and compatibility_mode == "PyTorch" and biasGradients_1D is not None) else 0.0
+        check_status(dy._lib.snhip_dense_backward_ex(
             dy.Wrapper.handle, None if prevLayerIsInputLayer else dx.As2DTensor(flattenInputTensorOnLastDimension).Pointer,
             weightGradients.Pointer, biasGradients_1D.Pointer if biasGradients_1D is not None else None,
-            xAs2DMatrix.Pointer, dyAs2DMatrix.Pointer, weights.Pointer, rows, in_features, out_features, multiplier, alpha),
-            "snhip_dense_backward")
-        if alpha and compatibility_mode == "PyTorch" and biasGradients_1D is not None:
-            biasGradients_1D.Update_Adding_Alpha_X(alpha, bias_1D)
+            xAs2DMatrix.Pointer, dyAs2DMatrix.Pointer, weights.Pointer, rows, in_features, out_features, multiplier, alpha,
+            bias_1D.Pointer if bias_alpha else None, bias_alpha), "snhip_dense_backward_ex")
         return
     weightGradients.Dot(dyAs2DMatrix, True, xAs2DMatrix, False, multiplier, 0.0)
     if biasGradients_1D is not None:

@@ -163,6 +163,58 @@ def test_bias_gradient_rides_along_with_dW_for_every_tile_configuration(oracle, 
         gc.GemmEx(transA=0, M=4, N=4, K=4, A=gdy, lda=4, B=gx, ldb=4, ldc=4, colsum=gcs)
 
 
+@pytest.mark.parametrize("rows,in_f,out_f,with_db,wd", [(128, 784, 256, True, 1e-2), (36, 100, 64, False, 0.0),
+                                                         (96, 132, 68, True, 0.5), (32, 32, 32, True, 0.0),
+                                                         (64, 1000, 128, True, 0.0)])
+def test_dense_backward_small_layer_in_one_launch(oracle, gpu_wrapper, rows, in_f, out_f, with_db, wd):
+    """snhip_dense_backward on a layer whose dW and dx are each a handful of 32 x 32 tiles (benchmark configuration 1:
+    128 x 784 -> 256): both products and the bias gradient leave as one launch.  Checked against the oracle's
+    Linear.DenseBackwardPropagation restatement and, bit for bit, against the same call with the tile configuration
+    forced (which takes the products one by one through the same 32 x 32 K-split kernel)."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    rng = np.random.default_rng(rows + in_f + out_f)
+    x, dy = random_tensor(rng, (rows, in_f), 0, 1), random_tensor(rng, (rows, out_f), -0.1, 0.1)
+    W = random_tensor(rng, (out_f, in_f), -0.07, 0.07)
+    gx, gdy, gW = T(w, x), T(w, dy), T(w, W)
+    bias = random_tensor(rng, (out_f,), -1, 1)
+    gbias = T(w, bias)
+    bias_wd = wd if with_db else 0.0          # the PyTorch-mode decay on the bias gradient (Linear.cs:178-181)
+    mult = 1.0 / rows
+    ksplit = [c["id"] for c in w.configs() if c["kind"] == "fp32-ksplit"][0]
+    got = {}
+    for form in ("one launch", "forced"):
+        gdx, gdW, gdb = (GPUTensor(sh, None, w) for sh in ([rows, in_f], [out_f, in_f], [out_f]))
+        for t in (gdx, gdW, gdb):
+            t.SetValue(float("nan"))
+        print("dense backward", rows, in_f, out_f, with_db, wd, form, flush=True)
+        if form == "forced":
+            w.set_tuning(ksplit, 1)
+        try:
+            check_status(w.lib.snhip_dense_backward_ex(w.handle, gdx.Pointer, gdW.Pointer, gdb.Pointer if with_db else None,
+                                                       gx.Pointer, gdy.Pointer, gW.Pointer, rows, in_f, out_f, mult, wd,
+                                                       gbias.Pointer if bias_wd else None, bias_wd))
+        finally:
+            w.set_tuning(-1, 0)
+        got[form] = (gdx.ToNumpy(), gdW.ToNumpy(), gdb.ToNumpy())
+        assert w.last_tuning() == (ksplit, 1)
+    dx, dW, db = got["one launch"]
+    ref_dW = oracle.dot_f64(dy, True, x, False, mult) + wd * W.astype(np.float64)
+    ref_dx = oracle.dot_f64(dy, False, W, False)
+    assert np.max(np.abs(dW - ref_dW)) <= bound(rows, dy, x, 1e-6) * mult + 1e-6 * wd
+    assert np.max(np.abs(dx - ref_dx)) <= bound(out_f, dy, W, 1e-7)
+    if with_db:
+        ref_db = dy.astype(np.float64).sum(axis=0) + bias_wd * bias.astype(np.float64)
+        assert np.max(np.abs(db - ref_db)) <= 1e-5 * np.sqrt(rows) * 0.1 + 1e-6 * bias_wd + 1e-7
+    else:
+        assert np.isnan(db).all()
+    for a, b in zip(got["one launch"][:2], got["forced"][:2]):
+        assert np.array_equal(a, b, equal_nan=True)
+    # db: the same column sums; the decay term is one fused multiply-add here and a separate pass there
+    assert np.allclose(got["one launch"][2], got["forced"][2], rtol=0, atol=1e-6, equal_nan=True)
+
+
 def test_linear_sigmoid_predictions_on_device(golden, gpu_wrapper):
     """Tests/NonReg/TestNetworkPropagation.cs:36-105 predictions through the GPU Dot."""
     from sharpnet_amd import GPUTensor, linear
