@@ -466,7 +466,9 @@ int snhip_config_count(void);
  * tiles, never part of a split-K launch, used only when the operands can be read in 16-byte pieces; 3 fp32 kernel
  * with persistent workgroups and 32-wide k panels: chosen by itself for strided batches of small matrices with a
  * short K, never part of a split-K launch; 4 tiled kernel for operands stored as bf16 (SNHIP_MATH_BF16_STORED);
- * 5 / 6 the persistent kernel of kind 3 with bf16 arithmetic on fp32-stored / bf16-stored operands) */
+ * 5 / 6 the persistent kernel of kind 3 with bf16 arithmetic on fp32-stored / bf16-stored operands; 7 the kernel
+ * for bf16-stored operands that are both contiguous along k (A plain, B transposed) and whole 256 x 256 x 32 tiles,
+ * fed by global -> LDS direct loads: chosen by itself when the shape allows) */
 int snhip_config_desc(int config, int desc[6]);
 
 #ifdef __cplusplus

@@ -19,7 +19,7 @@ MAIN_SOURCE = os.path.join(CSRC, "sharpnet_hip.hip")       # C ABI, dispatch, sm
 KERNEL_SOURCE = os.path.join(CSRC, "gemm_kernels.hip")     # GEMM kernels, compiled once per group of kernel_list.hpp
 KERNEL_GROUPS = 10                                         # SNHIP_NUM_KERNEL_GROUPS
 SOURCES = [MAIN_SOURCE, KERNEL_SOURCE]
-HEADERS = [os.path.join(CSRC, n) for n in ("sgemm_mfma.hpp", "bgemm_mfma.hpp", "rowops.hpp", "kernel_list.hpp", "attention_mfma.hpp", "rnn_cells.hpp", "rnn_layers.hpp", "sgemm_ksplit.hpp", "sgemm_stream.hpp")] + \
+HEADERS = [os.path.join(CSRC, n) for n in ("sgemm_mfma.hpp", "bgemm_mfma.hpp", "rowops.hpp", "kernel_list.hpp", "attention_mfma.hpp", "rnn_cells.hpp", "rnn_layers.hpp", "sgemm_ksplit.hpp", "sgemm_stream.hpp", "bgemm_dtl.hpp")] + \
           [os.path.join(REPO, "include", "sharpnet_hip.h")]
 # what gemm_kernels.hip includes; the other headers belong to the translation unit with the C ABI
 KERNEL_HEADERS = [os.path.join(CSRC, n) for n in ("sgemm_mfma.hpp", "bgemm_mfma.hpp", "kernel_list.hpp")]

@@ -92,7 +92,7 @@ class GPUWrapper:
             check_status(self.lib.snhip_config_desc(i, d))
             out.append({"id": i, "BM": d[0], "BN": d[1], "BK": d[2], "threads": d[3], "lds_bytes": d[4],
                         "kind": {0: "fp32", 1: "bf16", 2: "fp32-ksplit", 3: "fp32-stream", 4: "bf16-stored", 5: "bf16-stream",
-                                 6: "bf16-stored-stream"}[d[5]]})
+                                 6: "bf16-stored-stream", 7: "bf16-stored-dtl"}[d[5]]})
         return out
 
     # -- device memory -------------------------------------------------------

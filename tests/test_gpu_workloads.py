@@ -57,19 +57,46 @@ def test_config2_sweep_all_sizes_transposes_betas(oracle, gpu_wrapper):
 
 
 def test_config2_headline_bf16(oracle, gpu_wrapper):
-    from sharpnet_amd import workloads as wl
+    """The headline size (8192^3) in bf16-input arithmetic, all four transposes with fp32 storage, and the NT form
+    with operands stored as bf16 (the kernel fed by global -> LDS direct loads): sampled rows against the oracle on
+    bf16-rounded inputs (fp32 bound) and against the fp32 result (1e-2 relative)."""
+    from sharpnet_amd import GPUTensor, workloads as wl
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    S = 8192
     rng = np.random.default_rng(22)
-    a, b = rng.uniform(-1, 1, (4096, 4096)).astype(np.float32), rng.uniform(-1, 1, (4096, 4096)).astype(np.float32)
+    a, b = rng.uniform(-1, 1, (S, S)).astype(np.float32), rng.uniform(-1, 1, (S, S)).astype(np.float32)
     try:
-        gpu_wrapper.set_math_mode(gpu_wrapper.MATH_BF16_INPUT)
+        w.set_math_mode(w.MATH_BF16_INPUT)
         for tA, tB in [(False, False), (False, True), (True, False), (True, True)]:
-            got = sampled_rows_check(oracle, gpu_wrapper, wl.Gemm(4096, 4096, 4096, tA, tB), a, b, None, bf16=True)
+            print("bf16-input 8192^3", tA, tB, flush=True)
+            got = sampled_rows_check(oracle, w, wl.Gemm(S, S, S, tA, tB), a, b, None, nrows=6, bf16=True)
             # 1e-2 relative to the fp32 result as well
             rows = slice(0, 4)
             ref32 = oracle.dot(np.ascontiguousarray(a[:, rows].T if tA else a[rows]), False, b, tB)
             assert np.max(np.abs(got[rows] - ref32)) / np.max(np.abs(ref32)) <= 1e-2
+            del got
     finally:
-        gpu_wrapper.set_math_mode(gpu_wrapper.MATH_FP32)
+        w.set_math_mode(w.MATH_FP32)
+    # operands stored as bf16, A plain and B transposed
+    print("bf16-stored 8192^3 NT", flush=True)
+    ga, gb, gc = GPUTensor([S, S], a, w), GPUTensor([S, S], b, w), GPUTensor([S, S], None, w)
+    pa, pb = w.allocate(2 * S * S), w.allocate(2 * S * S)
+    check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, ga.Pointer, pa, S * S))
+    check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, gb.Pointer, pb, S * S))
+    gc.SetValue(float("nan"))
+    check_status(w.lib.snhip_dot_bf16_stored(w.handle, pa, S, S, 0, pb, S, S, 1, gc.Pointer, 1.0, 0.0, None))
+    kinds = {c["id"]: c["kind"] for c in w.configs()}
+    assert kinds[w.last_tuning()[0]] == "bf16-stored-dtl"
+    got = gc.ToNumpy()
+    assert np.all(np.isfinite(got))
+    rows = np.sort(rng.choice(S, 6, replace=False))
+    ref = oracle.dot(oracle.round_to_bf16(a[rows]), False, oracle.round_to_bf16(b), True)
+    assert np.max(np.abs(got[rows] - ref)) <= bound(S, a, b)
+    w.release(pa, 2 * S * S)
+    w.release(pb, 2 * S * S)
+    for t in (ga, gb, gc):
+        t.Dispose()
 
 
 def test_config3_mlp_step_gemms(oracle, gpu_wrapper):
