@@ -244,12 +244,15 @@ __global__ void __launch_bounds__(64 * NW) sgemm_ksplit_kernel(const GemmParams 
 //     db[c] = sum over rows of dy[r][c] + bias_alpha * bias[c]     (64 columns per workgroup; the second term is
 //                                                the weight decay on the bias of Linear.cs:178-181, bias may be nullptr)
 // and each alone is a handful of 32 x 32 tiles that costs a launch more than its arithmetic.  The grid is the
-// concatenation of the three jobs' workgroups: [0, blocks_w) tiles of dW, then blocks_x tiles of dx, then the column
-// blocks of db; every workgroup runs exactly the code its job would run in a launch of its own, so results are
-// bit-identical to the separate launches.
+// concatenation of the three jobs' workgroups: [0, blocks_x) tiles of dx, then blocks_w tiles of dW, then the column
+// blocks of db; every workgroup runs exactly the code its job would run in a launch of its own (32 x 32 tiles with
+// four K slices, or 32 x 64 tiles with two: the order of summation inside a K slice and across slices is the same
+// ascending one either way).
 struct DenseBackwardSmallParams {
     GemmParams pw, px;
     int blocks_w, blocks_x;
+    int nt_w, nt_x;    // 32-column tiles per workgroup (1: four K slices, 2: two) of the dW / dx product: the host
+                       // picks them so that the whole grid is resident at once when it can be
     const float* dy;   // rows x cols, row pitch ld; db may be nullptr (no column blocks in the grid then)
     float* db;
     const float* bias;
@@ -260,10 +263,16 @@ struct DenseBackwardSmallParams {
 __global__ void __launch_bounds__(256) dense_backward_small_kernel(const DenseBackwardSmallParams q) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int b = blockIdx.x;  // uniform: the three branches never diverge inside a workgroup
-    if (b < q.blocks_w) {
-        ksplit_tile<true, false, 1, 4>(q.pw, b, 0, smem);
-    } else if (b < q.blocks_w + q.blocks_x) {
-        ksplit_tile<false, false, 1, 4>(q.px, b - q.blocks_w, 0, smem);
+    if (b < q.blocks_x) {  // the longer K first
+        if (q.nt_x == 2)
+            ksplit_tile<false, false, 2, 4>(q.px, b, 0, smem);
+        else
+            ksplit_tile<false, false, 1, 4>(q.px, b, 0, smem);
+    } else if (b < q.blocks_x + q.blocks_w) {
+        if (q.nt_w == 2)
+            ksplit_tile<true, false, 2, 4>(q.pw, b - q.blocks_x, 0, smem);
+        else
+            ksplit_tile<true, false, 1, 4>(q.pw, b - q.blocks_x, 0, smem);
     } else {
         // wavefront w adds rows w, w + 4, ... of its 64 columns; the four partial sums meet in LDS in a fixed order
         float(*const part)[64] = reinterpret_cast<float(*)[64]>(smem);

@@ -1034,13 +1034,25 @@ int dense_backward_small(Handle* h, float* dx, float* dW, float* db, const float
     DenseBackwardSmallParams q;
     fill(gw, q.pw);
     fill(gx, q.px);
+    // One workgroup per compute unit is resident (the kernel uses more than half of the register file), so a grid
+    // beyond the number of compute units runs in two rounds: give the product with more tiles 32 x 64 tiles (two K
+    // slices instead of four), then the other one, while that brings the grid under one round.
+    q.nt_w = q.nt_x = 1;
+    const int blocks_b = (db != nullptr) ? ceil_div(out_features, 64) : 0;
+    auto blocks = [&](const GemmParams& p, int nt) { return p.tiles_m * ceil_div(p.N, 32 * nt); };
+    if (blocks(q.pw, 1) + blocks(q.px, 1) + blocks_b > h->num_cu) {
+        (blocks(q.pw, 1) >= blocks(q.px, 1) ? q.nt_w : q.nt_x) = 2;
+        if (blocks(q.pw, q.nt_w) + blocks(q.px, q.nt_x) + blocks_b > h->num_cu) q.nt_w = q.nt_x = 2;
+    }
+    q.pw.tiles_n = ceil_div(q.pw.N, 32 * q.nt_w);
+    q.px.tiles_n = ceil_div(q.px.N, 32 * q.nt_x);
     q.blocks_w = q.pw.tiles_m * q.pw.tiles_n;
     q.blocks_x = q.px.tiles_m * q.px.tiles_n;
     q.dy = dy, q.db = db, q.rows = rows, q.cols = out_features, q.ld = out_features;
     q.bias = (bias_decay_alpha != 0.0f) ? bias : nullptr;
     q.bias_alpha = bias_decay_alpha;
-    const int blocks_b = (db != nullptr) ? ceil_div(out_features, 64) : 0;
     constexpr int kLdsBytes = KsplitCfg<1, 4>::LDS_BYTES;
+    static_assert(KsplitCfg<2, 4>::LDS_BYTES == kLdsBytes, "both tile forms share one LDS size");
     hipLaunchKernelGGL(dense_backward_small_kernel, dim3((unsigned)(q.blocks_w + q.blocks_x + blocks_b)), dim3(256),
                        kLdsBytes, h->stream, q);
     h->last_cfg = kKsplitConfig;

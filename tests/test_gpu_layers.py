@@ -169,8 +169,8 @@ def test_bias_gradient_rides_along_with_dW_for_every_tile_configuration(oracle, 
 def test_dense_backward_small_layer_in_one_launch(oracle, gpu_wrapper, rows, in_f, out_f, with_db, wd):
     """snhip_dense_backward on a layer whose dW and dx are each a handful of 32 x 32 tiles (benchmark configuration 1:
     128 x 784 -> 256): both products and the bias gradient leave as one launch.  Checked against the oracle's
-    Linear.DenseBackwardPropagation restatement and, bit for bit, against the same call with the tile configuration
-    forced (which takes the products one by one through the same 32 x 32 K-split kernel)."""
+    Linear.DenseBackwardPropagation restatement and against the same call with the tile configuration forced (which
+    takes the products one by one through the 32 x 32 K-split kernel)."""
     from sharpnet_amd import GPUTensor
     from sharpnet_amd.hiplib import check_status
     w = gpu_wrapper
@@ -209,9 +209,11 @@ def test_dense_backward_small_layer_in_one_launch(oracle, gpu_wrapper, rows, in_
         assert np.max(np.abs(db - ref_db)) <= 1e-5 * np.sqrt(rows) * 0.1 + 1e-6 * bias_wd + 1e-7
     else:
         assert np.isnan(db).all()
-    for a, b in zip(got["one launch"][:2], got["forced"][:2]):
-        assert np.array_equal(a, b, equal_nan=True)
-    # db: the same column sums; the decay term is one fused multiply-add here and a separate pass there
+    # against the products issued one by one: the same kernel code per tile, but the one-launch form may give a product
+    # 32 x 64 tiles with two K slices where the forced configuration has 32 x 32 tiles with four (another grouping of
+    # the same partial sums), and the bias decay is one multiply-add here and a separate pass there
+    assert np.allclose(got["one launch"][0], got["forced"][0], rtol=0, atol=bound(out_f, dy, W) / 10)
+    assert np.allclose(got["one launch"][1], got["forced"][1], rtol=0, atol=bound(rows, dy, x) * mult / 10 + 1e-7)
     assert np.allclose(got["one launch"][2], got["forced"][2], rtol=0, atol=1e-6, equal_nan=True)
 
 
