@@ -285,6 +285,11 @@ def main():
             attention.attention_backward(dq, dk_, dv_, q, k, v, do, wts, ds, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
                                          scale=0.125, packed=False)
         w.synchronize()
+        # ... and with the causal hint, on the weights of the causal forward call just above
+        for _ in range(20):
+            attention.attention_backward(dq, dk_, dv_, q, k, v, do, wts, ds, batch=Z, heads=1, tq=Tn, tkv=Tn, dk=d, dv=d,
+                                         scale=0.125, packed=False, is_causal=True)
+        w.synchronize()
         for t in (q, k, v, o, wts, do, ds, dq, dk_, dv_):
             t.Dispose()
         # the handle in the bf16-input math mode: 512 x (256 x 64) with and without the weights, then 64 x 1024 keys
@@ -761,7 +766,8 @@ def layer_timings(w, wl):
     for fused in (True, False):
         def sdpa_fb():
             wts = attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, True, fused=fused)
-            attention.ScaledDotProductAttentionBackwardPropagation(dq, dk_, dv_, q, k, v, do, wts, True, fused=fused)
+            attention.ScaledDotProductAttentionBackwardPropagation(dq, dk_, dv_, q, k, v, do, wts, True, fused=fused,
+                                                                   is_causal=True)
 
         def sdpa_f():
             attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, True, fused=fused).Dispose()
@@ -803,7 +809,8 @@ def layer_timings(w, wl):
     for fused in (True, False):
         def long_fb():
             wts = attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, True, fused=fused)
-            attention.ScaledDotProductAttentionBackwardPropagation(dq, dk_, dv_, q, k, v, do, wts, True, fused=fused)
+            attention.ScaledDotProductAttentionBackwardPropagation(dq, dk_, dv_, q, k, v, do, wts, True, fused=fused,
+                                                                   is_causal=True)
 
         def long_f():
             attention.ScaledDotProductAttentionForwardPropagation(q, k, v, o, True, True, True, fused=fused).Dispose()

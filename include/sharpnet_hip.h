@@ -277,6 +277,10 @@ typedef struct snhip_attention_bwd_desc {
     int ldq, ldk, ldv, ldo;
     long long strideQ, strideK, strideV, strideO;
     long long strideQ_outer, strideK_outer, strideV_outer, strideO_outer;
+    int causal; /* 0 / 1: `weights` come from a causally masked forward call (zero above the diagonal).  A hint that
+                 * never changes the result for such weights: key blocks above the diagonal are skipped and the sums
+                 * over queries of dV and dK start at the first query that sees the key.  A descriptor without this
+                 * field (struct_size = its offset) is accepted and means 0. */
 } snhip_attention_bwd_desc;
 int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* desc);
 int snhip_sizeof_attention_bwd_desc(void);

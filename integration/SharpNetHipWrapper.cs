@@ -136,6 +136,7 @@ namespace SharpNet.GPU
             public IntPtr Q, K, V, dO, weights, scores_gradients, dQ, dK, dV;
             public int ldq, ldk, ldv, ldo;   // dQ, dK, dV use the pitch and strides of Q, K, V
             public long strideQ, strideK, strideV, strideO, strideQ_outer, strideK_outer, strideV_outer, strideO_outer;
+            public int causal;               // weights come from a causally masked forward call: lets the library skip the zeros
         }
         [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_attention_backward(IntPtr handle, ref AttentionBwdDesc desc);
         [DllImport(DLL_NAME)] public static extern int snhip_sizeof_attention_bwd_desc();

@@ -51,10 +51,12 @@ def fused_attention_forward(Q, K, V, O, weights, *, batch, heads, tq, tkv, dk, d
     return True
 
 
-def attention_backward(dQ, dK, dV, Q, K, V, dO, weights, scores_gradients, *, batch, heads, tq, tkv, dk, dv, scale, packed):
+def attention_backward(dQ, dK, dV, Q, K, V, dO, weights, scores_gradients, *, batch, heads, tq, tkv, dk, dv, scale, packed,
+                       is_causal=False):
     """snhip_attention_backward: dV, dS (into scores_gradients), dQ, dK in three launches (five beyond the one-kernel
     limits).  Layout conventions as in fused_attention_forward; weights and scores_gradients are contiguous
-    (batch*heads, tq, tkv) stacks."""
+    (batch*heads, tq, tkv) stacks.  is_causal: the weights come from a causally masked forward call (the layer's own
+    flag, ScaledDotProductAttentionLayer.cs:25): the library then skips what the mask zeroed."""
     def strides(steps, dim):
         if packed:
             return heads * dim, dim, steps * heads * dim
@@ -67,7 +69,8 @@ def attention_backward(dQ, dK, dV, Q, K, V, dO, weights, scores_gradients, *, ba
                                 Q=Q.Pointer, K=K.Pointer, V=V.Pointer, dO=dO.Pointer, weights=weights.Pointer,
                                 scores_gradients=scores_gradients.Pointer, dQ=dQ.Pointer, dK=dK.Pointer, dV=dV.Pointer,
                                 ldq=ldq, ldk=ldk, ldv=ldv, ldo=ldo, strideQ=sq, strideK=sk, strideV=sv, strideO=so,
-                                strideQ_outer=sq2, strideK_outer=sk2, strideV_outer=sv2, strideO_outer=so2)
+                                strideQ_outer=sq2, strideK_outer=sk2, strideV_outer=sv2, strideO_outer=so2,
+                                causal=int(bool(is_causal)))
     check_status(Q._lib.snhip_attention_backward(Q.Wrapper.handle, ctypes.byref(d)), "snhip_attention_backward")
 
 
@@ -106,15 +109,18 @@ def ScaledDotProductAttentionForwardPropagation(Q, K, V, y, isTraining, use_scal
     return weights_buffer
 
 
-def ScaledDotProductAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, weights_buffer, use_scale, fused=True):
+def ScaledDotProductAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, weights_buffer, use_scale, fused=True,
+                                                 is_causal=False):
     """fused=True: one library call (the score gradient and dQ come out of one kernel when the sizes allow it);
-    False: the reference's five calls one by one."""
+    False: the reference's five calls one by one.  is_causal (the layer's flag; the reference's static method does not
+    take it) only lets the fused call skip what the mask zeroed."""
     embedding_dim = dV.Shape[2]
     if fused:
         scaling = 1.0 / math.sqrt(embedding_dim) if use_scale else 1.0
         scores_gradients_buffer = GPUTensor(weights_buffer.Shape, None, Q.Wrapper)
         attention_backward(dQ, dK, dV, Q, K, V, dy, weights_buffer, scores_gradients_buffer, batch=K.Shape[0], heads=1,
-                           tq=Q.Shape[1], tkv=V.Shape[1], dk=K.Shape[2], dv=V.Shape[2], scale=scaling, packed=False)
+                           tq=Q.Shape[1], tkv=V.Shape[1], dk=K.Shape[2], dv=V.Shape[2], scale=scaling, packed=False,
+                           is_causal=is_causal)
         scores_gradients_buffer.Dispose()
         weights_buffer.Dispose()
         return
@@ -141,6 +147,7 @@ class MultiheadAttentionState:
         self.attention_heads_T = None   # place, (batch*heads, T, dim) copies in the reference's sequence
         self.dims = None
         self.heads_in_place = True
+        self.is_causal = False          # the layer's mask flag: backward may skip what it zeroed
 
 
 def _heads_gemm(c, a, b, *, transA, transB, M, N, K, alpha, batch, heads, a_packed, b_packed, c_packed,
@@ -188,6 +195,7 @@ def MultiheadAttentionForwardPropagation(Q, K, V, y, w_Q, w_K, w_V, out_proj_wei
     st = MultiheadAttentionState()
     st.dims = (batch_size, tq, tkv, H, dk, dv)
     st.heads_in_place = heads_in_place
+    st.is_causal = bool(is_causal)
     Q_heads = GPUTensor([batch_size * tq, H * dk], None, w)
     K_heads = GPUTensor([batch_size * tkv, H * dk], None, w)
     V_heads = GPUTensor([batch_size * tkv, H * dv], None, w)
@@ -266,7 +274,8 @@ def MultiheadAttentionBackwardPropagation(dQ, dK, dV, Q, K, V, dy, st, w_Q, w_K,
         dS = GPUTensor(P.Shape, None, w)
         if fused_attention:
             attention_backward(dQ_p, dK_p, dV_p, st.Q_heads, st.K_heads, st.V_heads, d_attention_heads_T, P, dS,
-                               batch=batch_size, heads=H, tq=tq, tkv=tkv, dk=dk, dv=dv, scale=scaling, packed=True)
+                               batch=batch_size, heads=H, tq=tq, tkv=tkv, dk=dk, dv=dv, scale=scaling, packed=True,
+                               is_causal=st.is_causal)
         else:
             common = dict(batch=batch_size, heads=H)
             # dV = P^T . dO                                                          (ScaledDotProductAttentionLayer.cs:117)

@@ -49,6 +49,10 @@ enum : int {
     GEMM_FLAG_C_VEC = 1,   // C (and the addend D, if any) rows may be accessed as aligned vectors of up to 16 bytes
                            // (pointer, pitch, batch strides)
     GEMM_FLAG_WS_VEC = 2,  // split-K workspace rows may be accessed as aligned 16-byte vectors (N % 4 == 0)
+    // (4: GEMM_FLAG_TILE_N_FASTEST of sgemm_ksplit.hpp)
+    GEMM_FLAG_K_FROM_M = 8,  // a hint, honoured by the extended fp32 kernels: op(A)[m][k] is zero for k < m (the
+                             // transposed softmax weights of a causally masked attention layer), so the tile whose
+                             // first row is m0 starts its k loop at m0 rounded down to a whole k tile
 };
 
 // Element-wise function applied last in the epilogue (the layer that follows a
@@ -884,11 +888,17 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         split = zb - batch * p.splitk;
     }
 
-    const int kbeg = split * p.kchunk;
+    int kbeg = split * p.kchunk;
     const int kend = (kbeg + p.kchunk < p.K) ? (kbeg + p.kchunk) : p.K;
+    if constexpr (EXT) {
+        if (p.flags & GEMM_FLAG_K_FROM_M) {  // uniform
+            const int k0 = (m0 / BK) * BK;
+            if (k0 > kbeg) kbeg = k0;
+        }
+    }
     const int klen = kend - kbeg;  // may be <= 0 for a trailing empty split
     const int nk = (klen + BK - 1) / BK;
-    const int nk_full = klen / BK;
+    const int nk_full = klen > 0 ? klen / BK : 0;
 
     BatchIndex bi = {0, batch};
     if constexpr (EXT) bi = split_batch(batch, p.batch_inner);

@@ -523,6 +523,7 @@ struct GemmArgs {
     float* colsum = nullptr;
     int math = -1;  // -1: the handle's math mode
     bool no_alloc = false;  // split-K partial sums go to the static scratch array; nothing is allocated or freed
+    bool k_from_m = false;  // hint: op(A)[m][k] == 0 for k < m (see GEMM_FLAG_K_FROM_M); kernels without it multiply the zeros
 };
 
 // Whether the product goes to sgemm_ksplit_kernel (32 x 32 tiles, K split inside the workgroup) instead of the
@@ -743,7 +744,9 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     // plain kernel plus passes over C / A, and one launch per outer batch step.
     const KernelFn fn_ext = cfg.fn_ext[g.tA ? 1 : 0][g.tB ? 1 : 0];
     const bool relu_family = (ep.act == ACT_RELU || ep.act == ACT_LEAKY_RELU);
-    const bool want_ext = ep.addend != nullptr || relu_family || two_level || g.colsum != nullptr;
+    // (the k-range hint is worth an extended kernel only for a K long enough to have whole tiles to skip)
+    const bool want_ext = ep.addend != nullptr || relu_family || two_level || g.colsum != nullptr ||
+                          (g.k_from_m && g.tA && K >= 4 * cfg.BK && cfg.kind == 0);
     const bool use_ext = want_ext && fn_ext != nullptr;
     if (two_level && !use_ext) {
         GemmArgs part = g;
@@ -806,6 +809,7 @@ int gemm_core(Handle* h, const GemmArgs& g) {
                         ((uintptr_t)ep_kernel.addend % 16 == 0 && g.ldd % 4 == 0 && (!multi || g.sD % 4 == 0) &&
                          (!two_level || g.sD2 % 4 == 0)));
     if (c_vec) p.flags |= GEMM_FLAG_C_VEC;
+    if (g.k_from_m && g.tA && use_ext && cfg.kind == 0) p.flags |= GEMM_FLAG_K_FROM_M;
     if (cfg.kind == 2 && M <= N) p.flags |= GEMM_FLAG_TILE_N_FASTEST;  // the K-split kernel keeps B's column blocks per XCD
     bool fused_reduce = false;
     if (ch.splitk > 1) {
@@ -1276,7 +1280,11 @@ int snhip_sizeof_attention_bwd_desc(void) { return (int)sizeof(snhip_attention_b
 
 int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
     Handle* h = static_cast<Handle*>(handle);
-    if (d == nullptr || d->struct_size != (int)sizeof(snhip_attention_bwd_desc)) return SNHIP_STATUS_INVALID_VALUE;
+    // the descriptor grew by one field (causal); a caller built against the shorter one says so through struct_size
+    constexpr int kSizeWithoutCausal = (int)offsetof(snhip_attention_bwd_desc, causal);
+    if (d == nullptr || (d->struct_size != (int)sizeof(snhip_attention_bwd_desc) && d->struct_size != kSizeWithoutCausal))
+        return SNHIP_STATUS_INVALID_VALUE;
+    const bool causal = d->struct_size == (int)sizeof(snhip_attention_bwd_desc) && d->causal != 0;
     if (h == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
     if (d->batch < 0 || d->batch_inner < 0 || d->Tq < 0 || d->Tk < 0 || d->dk < 0 || d->dv < 0)
         return SNHIP_STATUS_INVALID_VALUE;
@@ -1298,6 +1306,7 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
     g.B = d->dO, g.ldb = d->ldo, g.sB = d->strideO, g.sB2 = d->strideO_outer;
     g.C = d->dV, g.ldc = d->ldv, g.sC = d->strideV, g.sC2 = d->strideV_outer;
     g.batch = d->batch, g.batch_inner = d->batch_inner;
+    g.k_from_m = causal;  // P[query][key] == 0 for key > query: a tile of keys starts its sum at its first query
     int st = gemm_core(h, g);
     if (st != SNHIP_STATUS_SUCCESS) return st;
 
@@ -1320,7 +1329,7 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
         p.batch_inner = inner;
         p.batch = d->batch;
         p.scale = d->scale;
-        p.causal = 0;
+        p.causal = 0;  // (set below for the kernel that walks key blocks: the others see one block of keys)
         p.flags = 0;
         const bool multi = d->batch > 1, two_level = multi && inner < d->batch;
         if ((uintptr_t)d->dQ % 16 == 0 && d->ldq % 4 == 0 && (!multi || d->strideQ % 4 == 0) &&
@@ -1338,6 +1347,7 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
             // math mode); anything else takes the three calls below
             if ((p.flags & 7) == 7 && tiles <= 65535) {
                 p.q_tiles = 1;
+                p.causal = causal ? 1 : 0;  // key blocks wholly above the diagonal are skipped, their dS zero-filled
                 if (d->dk == 64)
                     hipLaunchKernelGGL((attention_fwd16_long_kernel<false, false, true, 64>),
                                        dim3((unsigned)d->batch, (unsigned)tiles), dim3(512),
@@ -1404,6 +1414,7 @@ int snhip_attention_backward(void* handle, const snhip_attention_bwd_desc* d) {
     k.B = d->Q, k.ldb = d->ldq, k.sB = d->strideQ, k.sB2 = d->strideQ_outer;
     k.C = d->dK, k.ldc = d->ldk, k.sC = d->strideK, k.sC2 = d->strideK_outer;
     k.batch = d->batch, k.batch_inner = d->batch_inner;
+    k.k_from_m = causal;  // dS[query][key] == 0 for key > query, like the weights it was formed from
     return gemm_core(h, k);
 }
 

@@ -105,7 +105,7 @@ class AttentionBwdDesc(ctypes.Structure):
         ("scale", _f), ("Q", _vp), ("K", _vp), ("V", _vp), ("dO", _vp), ("weights", _vp), ("scores_gradients", _vp),
         ("dQ", _vp), ("dK", _vp), ("dV", _vp), ("ldq", _i), ("ldk", _i), ("ldv", _i), ("ldo", _i),
         ("strideQ", _ll), ("strideK", _ll), ("strideV", _ll), ("strideO", _ll), ("strideQ_outer", _ll),
-        ("strideK_outer", _ll), ("strideV_outer", _ll), ("strideO_outer", _ll),
+        ("strideK_outer", _ll), ("strideV_outer", _ll), ("strideO_outer", _ll), ("causal", _i),
     ]
 
     def __init__(self, **kw):

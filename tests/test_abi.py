@@ -163,8 +163,11 @@ def test_gemm_descriptor_layout_matches_the_library():
     assert lib.snhip_sizeof_attention_bwd_desc() == ctypes.sizeof(hiplib.AttentionBwdDesc)
     g = hiplib.AttentionBwdDesc(batch=1, Tq=1, Tk=1, dk=1, dv=1)
     assert lib.snhip_attention_backward(None, ctypes.byref(g)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
-    g.struct_size -= 8
+    g.struct_size -= 4
     assert lib.snhip_attention_backward(None, ctypes.byref(g)) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
+    # the descriptor as it was before the `causal` field (its offset as struct_size) is still taken, and means 0
+    g.struct_size = hiplib.AttentionBwdDesc.causal.offset
+    assert lib.snhip_attention_backward(None, ctypes.byref(g)) == hiplib.CublasStatus.CUBLAS_STATUS_NOT_INITIALIZED
     assert lib.snhip_attention_backward(None, None) == hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
     assert lib.snhip_sizeof_rnn_desc() == ctypes.sizeof(hiplib.RnnDesc)
     r = hiplib.RnnDesc(cell_mode=2, bias_mode=1, bidirectional=1, num_layers=2, input_size=3, hidden_size=5)

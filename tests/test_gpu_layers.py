@@ -725,6 +725,62 @@ def test_attention_backward_call(oracle, gpu_wrapper, B, H, Tq, Tk, dk, dv, pack
     assert np.max(np.abs(gdk.ToNumpy() - lay(dk_ref, Tk, dk))) <= tol
 
 
+@pytest.mark.parametrize("B,H,Tq,Tk,d,packed", [
+    (2, 2, 1024, 1024, 64, False), (1, 3, 700, 900, 64, True), (2, 1, 1030, 520, 32, False), (1, 2, 300, 1540, 32, True),
+    (3, 2, 256, 256, 64, False), (1, 2, 200, 132, 32, True), (1, 1, 520, 516, 48, False)])
+def test_attention_backward_with_the_causal_hint(oracle, gpu_wrapper, B, H, Tq, Tk, d, packed):
+    """snhip_attention_backward with `causal` set, on weights that a causally masked forward pass produced (zero above
+    the diagonal): beyond 256 keys the key blocks above the diagonal are skipped and their score gradients
+    zero-filled, and the sums over queries of dV and dK start at the first query that sees a key.  Every output
+    against the oracle's ScaledDotProductAttentionBackwardPropagation on the same weights, and against the same call
+    without the hint (the hint must not change what comes out).  Sizes: square and ragged, more queries than keys
+    and the reverse, both 16-query head dimensions, <= 256 keys (nothing to skip in the kernel), and a head dimension
+    that takes the call sequence."""
+    from sharpnet_amd import GPUTensor, attention
+    rng = np.random.default_rng(6100 + Tq + Tk + d)
+    Z = B * H
+    q, k = random_tensor(rng, (Z, Tq, d), -1, 1), random_tensor(rng, (Z, Tk, d), -1, 1)
+    v, do = random_tensor(rng, (Z, Tk, d), -1, 1), random_tensor(rng, (Z, Tq, d), -1, 1)
+    scores = random_tensor(rng, (Z, Tq, Tk), -3, 3)
+    scores[:, np.triu_indices(Tq, 1, Tk)[0], np.triu_indices(Tq, 1, Tk)[1]] = -1e12     # SetAllElementsAboveMainDiagonal
+    wts = oracle.softmax_last_dim(scores)
+    assert np.all(wts[:, np.triu_indices(Tq, 1, Tk)[0], np.triu_indices(Tq, 1, Tk)[1]] == 0.0)
+    scale = 0.37
+    dv_ref = oracle.bmm(wts, True, do, False)
+    ds_ref = oracle.softmax_last_dim_backward(wts, oracle.bmm(do, False, v, True, scale))
+    dq_ref = oracle.bmm(ds_ref, False, k, False)
+    dk_ref = oracle.bmm(ds_ref, True, q, False)
+
+    def lay(x, steps, dim):
+        if not packed:
+            return x
+        return np.ascontiguousarray(x.reshape(B, H, steps, dim).transpose(0, 2, 1, 3)).reshape(B, steps, H * dim)
+    w = gpu_wrapper
+    gq, gk, gv, gdo = T(w, lay(q, Tq, d)), T(w, lay(k, Tk, d)), T(w, lay(v, Tk, d)), T(w, lay(do, Tq, d))
+    gw = T(w, wts)
+    outs = {}
+    for causal in (True, False):
+        gds = GPUTensor([Z, Tq, Tk], None, w)
+        gdq, gdk, gdv = (GPUTensor(t.Shape, None, w) for t in (gq, gk, gv))
+        for t in (gds, gdq, gdk, gdv):
+            t.SetValue(float("nan"))
+        print("attention backward", B, H, Tq, Tk, d, packed, "causal hint", causal, flush=True)
+        attention.attention_backward(gdq, gdk, gdv, gq, gk, gv, gdo, gw, gds, batch=B, heads=H, tq=Tq, tkv=Tk, dk=d, dv=d,
+                                     scale=scale, packed=packed, is_causal=causal)
+        outs[causal] = [t.ToNumpy() for t in (gds, gdv, gdq, gdk)]
+        for t in (gds, gdq, gdk, gdv):
+            t.Dispose()
+    tol = 2e-5 * np.sqrt(max(Tq, Tk, d))
+    for got in outs.values():
+        assert np.max(np.abs(got[0] - ds_ref)) <= tol
+        assert np.max(np.abs(got[1] - lay(dv_ref, Tk, d))) <= tol
+        assert np.max(np.abs(got[2] - lay(dq_ref, Tq, d))) <= tol
+        assert np.max(np.abs(got[3] - lay(dk_ref, Tk, d))) <= tol
+    # the score gradient and dQ come from the same arithmetic with or without the hint; dV and dK leave out exact zeros
+    assert np.array_equal(outs[True][0], outs[False][0]) and np.array_equal(outs[True][2], outs[False][2])
+    assert np.max(np.abs(outs[True][1] - outs[False][1])) <= tol and np.max(np.abs(outs[True][3] - outs[False][3])) <= tol
+
+
 @pytest.mark.parametrize("rows,cols", [(33333, 130), (512, 64), (511, 3), (100000, 1), (4096, 4096)])
 def test_bias_gradient_tall_matrices(gpu_wrapper, rows, cols):
     """Column sums of matrices much taller than wide are cut into row chunks (two kernels); same result as one pass."""
