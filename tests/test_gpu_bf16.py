@@ -385,6 +385,56 @@ def test_bf16_stored_direct_to_lds_kernel(oracle, gpu_wrapper):
     assert float(np.max(np.abs(got[0][rows] - ref))) <= 1e-4 * np.sqrt(K)
 
 
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_bf16_input_large_products_go_through_one_conversion(oracle, gpu_wrapper, tA, tB):
+    """bf16-input arithmetic on a product of whole 256 x 256 tiles with a tile per compute unit: the library rounds both
+    fp32 operands to bf16 once (into its workspace, in the k-contiguous form) and multiplies them with the bf16-storage
+    kernel - except for transposed A with plain B, which the fp32-storage kernel takes directly.  Sampled rows against
+    the oracle on rounded inputs (fp32 bound), alpha / beta / bias, contiguous operands and operands with padded rows
+    (snhip_gemm_rm), and the same product again after a smaller one (the workspace is reused)."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    lib, h = w.lib, w.handle
+    kinds = {c["id"]: c["kind"] for c in w.configs()}
+    rng = np.random.default_rng(880 + 2 * tA + tB)
+    M, N, K = 4096, 4096, 256
+    want_kind = "bf16" if (tA and not tB) else "bf16-stored-dtl"
+    for pad in (0, 8):
+        a = random_tensor(rng, (K, M + pad) if tA else (M, K + pad), -1, 1)
+        b = random_tensor(rng, (N, K + pad) if tB else (K, N + pad), -1, 1)
+        c0, bias = random_tensor(rng, (M, N), -1, 1), random_tensor(rng, (N,), -1, 1)
+        ga, gb, gc, gbias = T(w, a), T(w, b), T(w, c0), T(w, bias)
+        print("bf16-input via conversion", tA, tB, "padding", pad, flush=True)
+        check_status(lib.snhip_gemm_rm(h, int(tA), int(tB), M, N, K, 0.5, ga.Pointer, a.shape[1], 0, gb.Pointer, b.shape[1],
+                                       0, -1.0, gc.Pointer, N, 0, 1, gbias.Pointer))     # handle in fp32 mode: reference
+        ref32 = gc.ToNumpy()
+        gc.InitializeFromHostMemory(c0)
+        w.set_math_mode(w.MATH_BF16_INPUT)
+        try:
+            check_status(lib.snhip_gemm_rm(h, int(tA), int(tB), M, N, K, 0.5, ga.Pointer, a.shape[1], 0, gb.Pointer,
+                                           b.shape[1], 0, -1.0, gc.Pointer, N, 0, 1, gbias.Pointer))
+        finally:
+            w.set_math_mode(w.MATH_FP32)
+        assert kinds[w.last_tuning()[0]] == want_kind, (kinds[w.last_tuning()[0]], want_kind)
+        got = gc.ToNumpy()
+        assert np.all(np.isfinite(got))
+        rows = np.sort(rng.choice(M, 6, replace=False))
+        opa = np.ascontiguousarray((a[:, :M].T if tA else a[:, :K])[rows])
+        opb = np.ascontiguousarray(b[:, :K] if tB else b[:, :N])
+        ref = oracle.dot(oracle.round_to_bf16(opa), False, oracle.round_to_bf16(opb), tB, 0.5, -1.0, c0[rows]) + bias
+        assert float(np.max(np.abs(got[rows] - ref))) <= 1e-4 * np.sqrt(K) * 0.5 + 2e-6
+        assert float(np.max(np.abs(got - ref32))) / float(np.max(np.abs(ref32))) <= 1e-2
+        for t in (ga, gb, gc, gbias):
+            t.Dispose()
+
+
+def T(w, a):
+    from sharpnet_amd import GPUTensor
+    a = np.asarray(a, np.float32)
+    return GPUTensor(list(a.shape), a, w)
+
+
 @pytest.mark.parametrize("B,H,T,d,K_long", [(3, 2, 96, 64, False), (4, 4, 128, 320, True), (2, 3, 40, 48, False)])
 def test_bf16_stored_two_level_batch_through_gemm_ex(oracle, gpu_wrapper, B, H, T, d, K_long):
     """snhip_gemm_ex with math = SNHIP_MATH_BF16_STORED on heads addressed in place: a two-level batch whose outer
