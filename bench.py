@@ -102,6 +102,14 @@ def main():
     ap.add_argument("--shapes-probe", action="store_true",
                     help="30 launches each of the skinny, small-M and batched shapes (and the bf16-input headline), in "
                          "the order printed, for profilers")
+    ap.add_argument("--bf16-data-probe", action="store_true",
+                    help="the bf16-storage product of the headline size (8192^3, A plain, B transposed) on operands of "
+                         "different bit activity - U(-1,1), small integers, all ones - 20 launches each through the "
+                         "direct-load kernel, then U(-1,1) through the register-staged one: for profilers (the engine "
+                         "clock under each load = GRBM_GUI_ACTIVE / duration)")
+    ap.add_argument("--dense-probe", action="store_true",
+                    help="2000 calls each of the Dense layer of configuration 1 (128 x 784 -> 256) forward (bias + ReLU) "
+                         "and backward (bias gradient + weight decay) through the one-launch entry points, for profilers")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: 3 plain copies of 1 GiB, then 3 headline GEMMs")
     args = ap.parse_args()
@@ -255,6 +263,65 @@ def main():
             t.Dispose()
         return r
 
+    if args.bf16_data_probe:
+        from sharpnet_amd.hiplib import check_status
+        S = 8192
+        rng = np.random.default_rng(2)
+        fills = [("U(-1,1)", lambda: rng.uniform(-1, 1, (S, S)).astype(np.float32)),
+                 ("integers -2..2", lambda: rng.integers(-2, 3, (S, S)).astype(np.float32)),
+                 ("all ones", lambda: np.ones((S, S), np.float32))]
+        dtl = [c["id"] for c in w.configs() if c["kind"] == "bf16-stored-dtl"][0]
+        staged = [c["id"] for c in w.configs() if c["kind"] == "bf16-stored"][0]
+        pa, pb = w.allocate(2 * S * S), w.allocate(2 * S * S)
+        gc = GPUTensor([S, S], None, w)
+        for name, make, cfg in [(n, m, dtl) for n, m in fills] + [(fills[0][0], fills[0][1], staged)]:
+            for host, dst in ((make(), pa), (make(), pb)):
+                g = upload(host)
+                check_status(w.lib.snhip_convert_f32_to_bf16(w.handle, g.Pointer, dst, S * S))
+                g.Dispose()
+            w.set_tuning(cfg, 1)
+            try:
+                def launch():
+                    check_status(w.lib.snhip_dot_bf16_stored(w.handle, pa, S, S, 0, pb, S, S, 1, gc.Pointer, 1.0, 0.0, None))
+                for _ in range(10):
+                    launch()
+                e0, e1 = w.new_event(), w.new_event()
+                w.synchronize()
+                w.record(e0)
+                for _ in range(20):
+                    launch()
+                w.record(e1)
+                w.synchronize()
+                ms = w.elapsed_ms(e0, e1) / 20
+            finally:
+                w.set_tuning(-1, 0)
+            print(json.dumps({"operands": name, "tile_config": w.last_tuning()[0], "launches": 30, "event_ms": round(ms, 4),
+                              "tflops": round(2.0 * S ** 3 / (ms * 1e-3) / 1e12, 1)}), flush=True)
+        return
+    if args.dense_probe:
+        from sharpnet_amd.hiplib import check_status
+        d = wl.dense_layer_inputs(seed=1)
+        rows, fin = d["x"].shape
+        fout = d["w_out_in"].shape[0]
+        x, W, b, dy = upload(d["x"]), upload(d["w_out_in"]), upload(d["bias"]), upload(d["dy"])
+        y, dx, dW, db = (GPUTensor(sh, None, w) for sh in ([rows, fout], [rows, fin], [fout, fin], [fout]))
+        for name, call in (("forward", lambda: w.lib.snhip_dense_forward(w.handle, y.Pointer, x.Pointer, W.Pointer, b.Pointer,
+                                                                         rows, fin, fout, 1, 0.0)),
+                           ("backward", lambda: w.lib.snhip_dense_backward_ex(w.handle, dx.Pointer, dW.Pointer, db.Pointer,
+                                                                             x.Pointer, dy.Pointer, W.Pointer, rows, fin,
+                                                                             fout, 1.0, 0.0128, b.Pointer, 0.0128))):
+            for _ in range(500):
+                check_status(call())
+            e0, e1 = w.new_event(), w.new_event()
+            w.synchronize()
+            w.record(e0)
+            for _ in range(2000):
+                check_status(call())
+            w.record(e1)
+            w.synchronize()
+            print(json.dumps({"call": "Dense 128x784->256 " + name, "calls": 2500,
+                              "event_us_per_call": round(w.elapsed_ms(e0, e1) / 2, 3)}), flush=True)
+        return
     if args.attention_probe:
         from sharpnet_amd import attention
         rng = np.random.default_rng(5)
@@ -331,6 +398,7 @@ def main():
         shapes += [("lstm input projection", proj, 0), ("lstm recurrent step (beta=1)", rec, 0)]
         shapes += [("attention " + gm.name, gm, 0) for gm in wl.attention_gemms()]
         shapes += [("bf16-input 8192^3 TN", wl.Gemm(8192, 8192, 8192, True, False), 1),
+                   ("bf16-input 8192^3 NN", wl.Gemm(8192, 8192, 8192), 1),
                    ("bf16-input 4096^3 NN", wl.Gemm(4096, 4096, 4096), 1)]
         shapes += [("bf16-input attention " + gm.name, gm, 1) for gm in wl.attention_gemms()]
         shapes += [("square %d^3 NN" % n, wl.Gemm(n, n, n), 0) for n in (1024, 2048, 4096)]
@@ -607,9 +675,15 @@ def main():
             extra["config5_attention_bf16_input"] = {
                 "gemms": bf, "cpu_baseline": extra["config5_attention_fp32"]["cpu_baseline"],
                 "note": "the reference has no reduced-precision CPU route: the CPU figure is the fp32 one"}
-            hb = run(wl.Gemm(8192, 8192, 8192, True, False, 1.0, 0.0), 2, 10, 5)
-            hb["frac_of_roofline"] = round(hb["tflops"] / wl.BF16_MFMA_PEAK_TFLOPS, 4)
-            extra["config2_8192_bf16_input_TN"] = hb
+            # the headline size, all four forms: transposed A with plain B runs on the fp32-storage kernel, the others
+            # through one rounding pass into the workspace and the bf16-storage kernel (the pass is inside the time)
+            hbs = []
+            for (tA, tB) in ((True, False), (False, False), (False, True), (True, True)):
+                hb = run(wl.Gemm(8192, 8192, 8192, tA, tB, 1.0, 0.0), 2, 10, 5)
+                hb["frac_of_roofline"] = round(hb["tflops"] / wl.BF16_MFMA_PEAK_TFLOPS, 4)
+                hb["gemm"] += " (bf16-input arithmetic, fp32 storage)"
+                hbs.append(hb)
+            extra["config2_8192_bf16_input"] = hbs
         finally:
             w.set_math_mode(w.MATH_FP32)
             bf16_math[0] = False
@@ -680,7 +754,8 @@ def summarize(extra):
     s["config5_attention_ms"] = {"fp32": [r["ms"] for r in extra["config5_attention_fp32"]["gemms"]],
                                  "bf16_input": [r["ms"] for r in extra["config5_attention_bf16_input"]["gemms"]],
                                  "bf16_stored": [r["ms"] for r in extra["config5_attention_bf16_stored"]["gemms"]]}
-    s["bf16_8192_tflops"] = {"input_TN": extra["config2_8192_bf16_input_TN"]["tflops"],
+    s["bf16_8192_tflops"] = {"input_TN": extra["config2_8192_bf16_input"][0]["tflops"],
+                             "input_best": best(extra["config2_8192_bf16_input"]),
                              "stored_best": best(extra["config2_8192_bf16_stored"])}
     rows = 0
     for v in extra.values():

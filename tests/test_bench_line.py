@@ -40,7 +40,7 @@ def _fake_extra():
         "config5_attention_fp32": {"gemms": att, "cpu_baseline": None},
         "config5_attention_bf16_input": {"gemms": att, "cpu_baseline": None},
         "config5_attention_bf16_stored": {"gemms": att, "cpu_baseline": None},
-        "config2_8192_bf16_input_TN": _fake_gemm_row("(8192,8192,8192) TN beta=0", 0.37),
+        "config2_8192_bf16_input": [_fake_gemm_row("(8192,8192,8192) TN beta=0", 0.37)] * 4,
         "config2_8192_bf16_stored": [_fake_gemm_row("(8192,8192,8192) NT beta=0 (bf16 storage)", 0.46)] * 5,
         "layers_fused_vs_reference_sequence": layers,
     }
