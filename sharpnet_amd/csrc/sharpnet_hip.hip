@@ -243,11 +243,10 @@ const ConfigEntry kConfigs[] = {
                 {{sgemm_ksplit16_kernel<false, false>, sgemm_ksplit16_kernel<false, true>},
                  {sgemm_ksplit16_kernel<true, false>, sgemm_ksplit16_kernel<true, true>}},
                 4, 0.5, 0.5, 1.0},  // 26: 16 x 16, eight K slices
-    // bf16 storage, tiles through global -> LDS direct loads (bgemm_dtl.hpp): shapes that are whole tiles; see
-    // prefer_dtl()
+    // bf16 storage, both operands k-contiguous, tiles through global -> LDS direct loads (bgemm_dtl.hpp): one form
+    // only (A plain, B transposed), shapes that are whole tiles; see prefer_dtl()
     ConfigEntry{BDtlCfg::BM, BDtlCfg::BN, BDtlCfg::BK, BDtlCfg::NT, BDtlCfg::LDS_BYTES, 16, 7,
-                {{bgemm_dtl_kernel<false, false>, bgemm_dtl_kernel<false, true>},
-                 {bgemm_dtl_kernel<true, false>, bgemm_dtl_kernel<true, true>}},
+                {{nullptr, bgemm_nt_dtl_kernel}, {nullptr, nullptr}},
                 {{nullptr, nullptr}, {nullptr, nullptr}},
                 1, 0.9, 0.9, 1.0},  // 27: 256 x 256, k panels of 32, four LDS stages
 };
@@ -577,13 +576,13 @@ int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, 
     return cfg;
 }
 
-// Whether a product on operands stored as bf16 goes to bgemm_dtl_kernel (configuration 27) instead of what the cost
-// model chose: M and N whole 256-wide tiles, K whole 32-wide panels, rows and matrices on 16-byte boundaries, a plain
-// epilogue (alpha, beta, bias), and enough tiles that the 256 x 256 tile is what the cost model would have picked
-// anyway (at least one per compute unit).  Measured on MI355X, 8192^3, U(-1, 1) operands: the four transpose forms
-// within a few percent of one another (the register-staged kernel: NT 1.12-1.21, NN 0.97, TN 0.78 PFLOP/s).
+// Whether a product on operands stored as bf16 goes to bgemm_nt_dtl_kernel (configuration 27) instead of what the
+// cost model chose: both operands k-contiguous (A plain, B transposed), M and N whole 256-wide tiles, K whole 32-wide
+// panels, rows and matrices on 16-byte boundaries, a plain epilogue (alpha, beta, bias), and enough tiles that the
+// 256 x 256 tile is what the cost model would have picked anyway (at least one per compute unit).  Measured on
+// MI355X, 8192^3, U(-1, 1) operands: 1.19-1.21 PFLOP/s against 1.12-1.15 for the register-staged 256 x 256 kernel.
 int prefer_dtl(const Handle* h, const GemmArgs& g, int math, bool wants_ext) {
-    if (math != SNHIP_MATH_BF16_STORED || wants_ext) return -1;
+    if (math != SNHIP_MATH_BF16_STORED || g.tA || !g.tB || wants_ext) return -1;
     if (h->force_cfg >= 0 && h->force_cfg != kBDtlConfig) return -1;
     if (h->force_splitk > 1) return -1;
     if (g.M % BDtlCfg::BM != 0 || g.N % BDtlCfg::BN != 0 || g.K % BDtlCfg::BK != 0 || g.K < BDtlCfg::BK) return -1;
@@ -718,12 +717,14 @@ int gemm_core(Handle* h, const GemmArgs& g) {
             (multi && (g.sA % 2 != 0 || g.sB % 2 != 0)) || (two_level && (g.sA2 % 2 != 0 || g.sB2 % 2 != 0)))
             return SNHIP_STATUS_NOT_SUPPORTED;
     }
-    // bf16-input arithmetic on a large product of whole tiles: round both operands to bf16 once, into the workspace
-    // (same shape, rows packed), and multiply them with the bf16-storage kernel fed by direct loads.  Each fp32 element
-    // is then read once by a streaming pass instead of once per tile that needs it, which is what bounds the
-    // fp32-storage kernels.  Same rounding, same products; the sums may be grouped differently.
+    // bf16-input arithmetic on a large product of whole tiles: round both operands to bf16 once, into the workspace and
+    // into the k-contiguous form (A plain, B transposed), and multiply them with the bf16-storage kernel fed by direct
+    // loads.  Each fp32 element is then read once by a streaming pass instead of once per tile that needs it, which is
+    // what bounds the fp32-storage kernels (8192^3 on MI355X: NN 1.59 -> 1.16 ms, NT 1.43 -> 1.10 ms, the conversion
+    // included).  Same rounding, same products; the sums may be grouped differently.  Not for transposed A with plain B:
+    // both operands would have to be transposed on the way, and the direct kernel is as fast there.
     if (math == SNHIP_MATH_BF16_INPUT && !g.no_alloc && batch == 1 && h->force_cfg < 0 && h->force_splitk <= 0 &&
-        ep.addend == nullptr && ep.act == ACT_NONE && g.colsum == nullptr &&
+        !(g.tA && !g.tB) && ep.addend == nullptr && ep.act == ACT_NONE && g.colsum == nullptr &&
         M % BDtlCfg::BM == 0 && N % BDtlCfg::BN == 0 && K % BDtlCfg::BK == 0 && K >= 8 * BDtlCfg::BK &&
         (long long)(M / BDtlCfg::BM) * (N / BDtlCfg::BN) >= h->num_cu &&
         2 * ((size_t)M + N) * K <= kMaxWorkspaceBytes) {
@@ -732,18 +733,26 @@ int gemm_core(Handle* h, const GemmArgs& g) {
         if (st != SNHIP_STATUS_SUCCESS) return st;
         __bf16* wa = reinterpret_cast<__bf16*>(h->ws);
         __bf16* wb = wa + a_elems;
-        const int a_rows = g.tA ? K : M, a_cols = g.tA ? M : K, b_rows = g.tB ? N : K, b_cols = g.tB ? K : N;
         GemmArgs s = g;
         s.math = SNHIP_MATH_BF16_STORED;
-        s.A = reinterpret_cast<const float*>(wa), s.lda = a_cols;
-        s.B = reinterpret_cast<const float*>(wb), s.ldb = b_cols;
+        s.tA = false, s.tB = true;
+        s.A = reinterpret_cast<const float*>(wa), s.lda = K;
+        s.B = reinterpret_cast<const float*>(wb), s.ldb = K;
         if (prefer_dtl(h, s, SNHIP_MATH_BF16_STORED, false) == kBDtlConfig) {
-            // (an operand without row padding takes the one-dimensional pass: 16-byte pieces)
-            st = (g.lda == a_cols) ? snhip_convert_f32_to_bf16(h, g.A, wa, (long long)a_elems)
-                                   : snhip_convert_f32_to_bf16_2d(h, g.A, a_rows, a_cols, g.lda, 0, wa, a_cols);
+            // (an operand that is already k-contiguous without padding takes the one-dimensional pass: 16-byte pieces)
+            if (g.tA)
+                st = snhip_convert_f32_to_bf16_2d(h, g.A, K, M, g.lda, 1, wa, K);
+            else if (g.lda == K)
+                st = snhip_convert_f32_to_bf16(h, g.A, wa, (long long)a_elems);
+            else
+                st = snhip_convert_f32_to_bf16_2d(h, g.A, M, K, g.lda, 0, wa, K);
             if (st != SNHIP_STATUS_SUCCESS) return st;
-            st = (g.ldb == b_cols) ? snhip_convert_f32_to_bf16(h, g.B, wb, (long long)b_elems)
-                                   : snhip_convert_f32_to_bf16_2d(h, g.B, b_rows, b_cols, g.ldb, 0, wb, b_cols);
+            if (!g.tB)
+                st = snhip_convert_f32_to_bf16_2d(h, g.B, K, N, g.ldb, 1, wb, K);
+            else if (g.ldb == K)
+                st = snhip_convert_f32_to_bf16(h, g.B, wb, (long long)b_elems);
+            else
+                st = snhip_convert_f32_to_bf16_2d(h, g.B, N, K, g.ldb, 0, wb, K);
             if (st != SNHIP_STATUS_SUCCESS) return st;
             return gemm_core(h, s);
         }
