@@ -53,6 +53,8 @@ enum : int {
     GEMM_FLAG_K_FROM_M = 8,  // a hint, honoured by the extended fp32 kernels: op(A)[m][k] is zero for k < m (the
                              // transposed softmax weights of a causally masked attention layer), so the tile whose
                              // first row is m0 starts its k loop at m0 rounded down to a whole k tile
+    GEMM_FLAG_LONGEST_FIRST = 16,  // with K_FROM_M: tiles are dealt out by work_coords_longest_first (group_m then
+                                   // carries the number of compute units per XCD)
 };
 
 // Element-wise function applied last in the epilogue (the layer that follows a
@@ -376,6 +378,28 @@ __device__ __forceinline__ WorkCoords work_coords(unsigned lin, int tiles_m, int
     const int in_g = logical - g * per_group;
     w.tile_m = first_m + in_g % gsz;
     w.tile_n = in_g / gsz;
+    return w;
+}
+
+// The order for products whose tiles do unequal work because their k loops start at their first row
+// (GEMM_FLAG_K_FROM_M): tile row 0 sums over all of K, the last one over a sliver.  Every XCD owns nz / 8 whole matrices
+// (the host checks that the counts divide and that there is one tile column).  Inside an XCD the (tile row, matrix)
+// pairs are taken longest first, and the rounds of `cu_per_xcd` workgroups alternate direction, so that the compute
+// unit that got the longest item of one round gets the shortest of the next (workgroups of one XCD go to its compute
+// units in turn): co-resident workgroups then add up to about the same work everywhere.
+__device__ __forceinline__ WorkCoords work_coords_longest_first(unsigned lin, int tiles_m, int nz, int cu_per_xcd) {
+    constexpr unsigned NXCD = 8;
+    const unsigned xcd = lin % NXCD, local = lin / NXCD;
+    const unsigned nm = (unsigned)nz / NXCD;               // matrices per XCD
+    const unsigned q = nm * (unsigned)tiles_m;             // items per XCD
+    const unsigned round = local / (unsigned)cu_per_xcd, pos = local % (unsigned)cu_per_xcd;
+    const unsigned left = q - round * (unsigned)cu_per_xcd;
+    const unsigned len = left < (unsigned)cu_per_xcd ? left : (unsigned)cu_per_xcd;
+    const unsigned item = round * (unsigned)cu_per_xcd + ((round & 1u) ? len - 1u - pos : pos);
+    WorkCoords w;
+    w.tile_m = (int)(item / nm);
+    w.tile_n = 0;
+    w.zb = (int)(xcd * nm + item % nm);
     return w;
 }
 
@@ -878,7 +902,10 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, lhi = lane >> 5;
 
-    const WorkCoords wc = work_coords(blockIdx.x, p.tiles_m, p.tiles_n, p.nz, p.group_m);
+    WorkCoords wc = work_coords(blockIdx.x, p.tiles_m, p.tiles_n, p.nz, p.group_m);
+    if constexpr (EXT) {
+        if (p.flags & GEMM_FLAG_LONGEST_FIRST) wc = work_coords_longest_first(blockIdx.x, p.tiles_m, p.nz, p.group_m);
+    }
     const int tile_m = wc.tile_m, tile_n = wc.tile_n;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int zb = wc.zb;  // batch * splitk + split

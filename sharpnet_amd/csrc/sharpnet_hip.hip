@@ -849,7 +849,15 @@ int gemm_core(Handle* h, const GemmArgs& g) {
                         ((uintptr_t)ep_kernel.addend % 16 == 0 && g.ldd % 4 == 0 && (!multi || g.sD % 4 == 0) &&
                          (!two_level || g.sD2 % 4 == 0)));
     if (c_vec) p.flags |= GEMM_FLAG_C_VEC;
-    if (g.k_from_m && g.tA && use_ext && cfg.kind == 0) p.flags |= GEMM_FLAG_K_FROM_M;
+    if (g.k_from_m && g.tA && use_ext && cfg.kind == 0) {
+        p.flags |= GEMM_FLAG_K_FROM_M;
+        // tiles then do unequal work: deal them out longest first when the grid has the regular shape that order is
+        // written for (one tile column, no split, whole matrices per XCD)
+        if (p.tiles_n == 1 && ch.splitk == 1 && batch % 8 == 0 && h->num_cu % 8 == 0 && p.tiles_m > 1) {
+            p.flags |= GEMM_FLAG_LONGEST_FIRST;
+            p.group_m = h->num_cu / 8;
+        }
+    }
     if (cfg.kind == 2 && M <= N) p.flags |= GEMM_FLAG_TILE_N_FASTEST;  // the K-split kernel keeps B's column blocks per XCD
     bool fused_reduce = false;
     if (ch.splitk > 1) {
