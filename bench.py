@@ -299,28 +299,8 @@ def main():
                               "tflops": round(2.0 * S ** 3 / (ms * 1e-3) / 1e12, 1)}), flush=True)
         return
     if args.dense_probe:
-        from sharpnet_amd.hiplib import check_status
-        d = wl.dense_layer_inputs(seed=1)
-        rows, fin = d["x"].shape
-        fout = d["w_out_in"].shape[0]
-        x, W, b, dy = upload(d["x"]), upload(d["w_out_in"]), upload(d["bias"]), upload(d["dy"])
-        y, dx, dW, db = (GPUTensor(sh, None, w) for sh in ([rows, fout], [rows, fin], [fout, fin], [fout]))
-        for name, call in (("forward", lambda: w.lib.snhip_dense_forward(w.handle, y.Pointer, x.Pointer, W.Pointer, b.Pointer,
-                                                                         rows, fin, fout, 1, 0.0)),
-                           ("backward", lambda: w.lib.snhip_dense_backward_ex(w.handle, dx.Pointer, dW.Pointer, db.Pointer,
-                                                                             x.Pointer, dy.Pointer, W.Pointer, rows, fin,
-                                                                             fout, 1.0, 0.0128, b.Pointer, 0.0128))):
-            for _ in range(500):
-                check_status(call())
-            e0, e1 = w.new_event(), w.new_event()
-            w.synchronize()
-            w.record(e0)
-            for _ in range(2000):
-                check_status(call())
-            w.record(e1)
-            w.synchronize()
-            print(json.dumps({"call": "Dense 128x784->256 " + name, "calls": 2500,
-                              "event_us_per_call": round(w.elapsed_ms(e0, e1) / 2, 3)}), flush=True)
+        for r in dense_layer_calls(w, wl, upload, timed_calls=2000)["calls"]:
+            print(json.dumps(r), flush=True)
         return
     if args.attention_probe:
         from sharpnet_amd import attention
@@ -594,6 +574,7 @@ def main():
             "gemms": rows,
             "cpu_baseline": cpu_summary(rows, dense, "forward (cblas_sgemm NT + bias pass), dW (TN), dx (NN) of the "
                                         "128 x 784 -> 256 layer, each the median of 200 calls after a warm-up")}
+        extra["config1_dense_layer_calls"] = dense_layer_calls(w, wl, upload)
         if cpu_on:
             # the same three products (and the bias add) back to back on the host, as a layer step runs them
             d = wl.dense_layer_inputs(seed=1)
@@ -613,11 +594,15 @@ def main():
                 cpu_layer()
             cpu_layer_ms = (time.perf_counter() - t0) * 1e3 / 200
             cpu_spent[0] += time.perf_counter() - t0
-            gpu_ms = sum(r["ms"] for r in rows)
+            lc = extra["config1_dense_layer_calls"]
             extra["config1_dense_layer_fwd_bwd"] = {
-                "gpu_ms": round(gpu_ms, 4), "cpu_mkl_ms": round(cpu_layer_ms, 4), "cpu_cores": cpu_cores,
-                "note": "forward + dW + dx of the 128 x 784 -> 256 layer; GPU = sum of the three launches above, "
-                        "CPU = cblas_sgemm x 3 + bias add, 200 repetitions"}
+                "gpu_ms": round(lc["forward_ms"] + lc["backward_ms"], 4),
+                "gpu_forward_ms": lc["forward_ms"], "gpu_backward_ms": lc["backward_ms"],
+                "gpu_three_separate_products_ms": round(sum(r["ms"] for r in rows), 4),
+                "cpu_mkl_ms": round(cpu_layer_ms, 4), "cpu_cores": cpu_cores,
+                "note": "forward + backward of the 128 x 784 -> 256 layer; GPU = snhip_dense_forward + "
+                        "snhip_dense_backward_ex (one launch each: dx, dW and db share a grid), beside the sum of the "
+                        "three products as separate launches; CPU = cblas_sgemm x 3 + bias add, 200 repetitions"}
         sweep, sweep_gemms = [], []
         for (M, N, K) in wl.SWEEP_SIZES:
             steps, warm = (5, 3) if M * N * K > 1e11 else (50, 20)
@@ -736,12 +721,14 @@ def summarize(extra):
     s = {}
     fb = extra.get("config1_dense_layer_fwd_bwd")
     if fb:
-        s["config1_dense_fwd_bwd_ms"] = {"gpu": fb["gpu_ms"], "cpu_mkl": fb["cpu_mkl_ms"], "cpu_cores": fb["cpu_cores"]}
+        s["config1_dense_fwd_bwd_ms"] = {"gpu": fb["gpu_ms"], "gpu_forward": fb["gpu_forward_ms"],
+                                         "gpu_backward": fb["gpu_backward_ms"],
+                                         "gpu_three_separate_products": fb["gpu_three_separate_products_ms"],
+                                         "cpu_mkl": fb["cpu_mkl_ms"], "cpu_cores": fb["cpu_cores"]}
     else:
-        s["config1_dense_fwd_bwd_ms"] = {"gpu": round(sum(r["ms"] for r in extra["config1_dense_layer"]["gemms"]), 4)}
-    for r in extra.get("layers_fused_vs_reference_sequence", []):
-        if r["layer"].startswith("Linear 128x784->256") and r["form"] == "fused":
-            s["config1_dense_fused_calls_ms"] = {"forward": r["forward_ms"], "backward": r["backward_ms"]}
+        lc = extra["config1_dense_layer_calls"]
+        s["config1_dense_fwd_bwd_ms"] = {"gpu": round(lc["forward_ms"] + lc["backward_ms"], 4),
+                                         "gpu_forward": lc["forward_ms"], "gpu_backward": lc["backward_ms"]}
     sw = extra["config2_sweep"]["gemms"]
     fr = {}
     for r in sw:
@@ -754,15 +741,72 @@ def summarize(extra):
     s["config5_attention_ms"] = {"fp32": [r["ms"] for r in extra["config5_attention_fp32"]["gemms"]],
                                  "bf16_input": [r["ms"] for r in extra["config5_attention_bf16_input"]["gemms"]],
                                  "bf16_stored": [r["ms"] for r in extra["config5_attention_bf16_stored"]["gemms"]]}
-    s["bf16_8192_tflops"] = {"input_TN": extra["config2_8192_bf16_input"][0]["tflops"],
-                             "input_best": best(extra["config2_8192_bf16_input"]),
-                             "stored_best": best(extra["config2_8192_bf16_stored"])}
+    def form(r):
+        return r["gemm"].split(")")[1].split()[0]      # "(M,N,K) NT beta=0 ..." -> "NT"
+    # fp32 operands rounded on the way (all four forms) and operands stored as bf16 (the first three rows: the operands
+    # as the caller laid them out; the rows after them repeat NN / TN with the caller transposing while converting)
+    s["bf16_8192_tflops"] = {"input": {form(r): r["tflops"] for r in extra["config2_8192_bf16_input"]},
+                             "stored": {form(r): r["tflops"] for r in extra["config2_8192_bf16_stored"][:3]}}
     rows = 0
     for v in extra.values():
         items = v if isinstance(v, list) else (v.get("gemms") or [v]) if isinstance(v, dict) else []
         rows += sum(1 for r in items if isinstance(r, dict) and "max_abs_err" in r)
     s["timed_products_checked_against_oracle"] = rows
     return s
+
+
+def dense_layer_calls(w, wl, upload, timed_calls=1000):
+    """The 128 x 784 -> 256 layer of configuration 1 as the two library calls a Linear layer makes per step
+    (Linear.cs:125-132 and :143-191): snhip_dense_forward (bias + ReLU in the write-out) and snhip_dense_backward_ex
+    (dx, dW + decay * W and db + decay * bias).  Called straight through the C ABI, HIP events around `timed_calls`
+    calls issued back to back (dependent launches: each reads what the one before wrote), and every output of the
+    timed calls compared with the float64 result."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    d = wl.dense_layer_inputs(seed=1)
+    xs, ws, dys = d["x"], d["w_out_in"], d["dy"]
+    bs = np.random.default_rng(11).uniform(-0.1, 0.1, ws.shape[0]).astype(np.float32)  # the workload's bias is all zeros
+    rows, fin = xs.shape
+    fout = ws.shape[0]
+    decay = 0.0128
+    x, W, b, dy = upload(xs), upload(ws), upload(bs), upload(dys)
+    y, dx, dW, db = (GPUTensor(sh, None, w) for sh in ([rows, fout], [rows, fin], [fout, fin], [fout]))
+    calls = (("forward", lambda: w.lib.snhip_dense_forward(w.handle, y.Pointer, x.Pointer, W.Pointer, b.Pointer,
+                                                           rows, fin, fout, 1, 0.0)),
+             ("backward", lambda: w.lib.snhip_dense_backward_ex(w.handle, dx.Pointer, dW.Pointer, db.Pointer, x.Pointer,
+                                                                dy.Pointer, W.Pointer, rows, fin, fout, 1.0, decay,
+                                                                b.Pointer, decay)))
+    res = []
+    for name, call in calls:
+        for _ in range(500):
+            check_status(call())
+        e0, e1 = w.new_event(), w.new_event()
+        w.synchronize()
+        w.record(e0)
+        for _ in range(timed_calls):
+            check_status(call())
+        w.record(e1)
+        w.synchronize()
+        res.append({"call": "Dense 128x784->256 " + name, "calls": 500 + timed_calls,
+                    "event_us_per_call": round(w.elapsed_ms(e0, e1) * 1e3 / timed_calls, 3)})
+        w.destroy_event(e0)
+        w.destroy_event(e1)
+    x64, w64, b64, dy64 = (a.astype(np.float64) for a in (xs, ws, bs, dys))
+    want = {"y": np.maximum(x64 @ w64.T + b64, 0.0), "dx": dy64 @ w64, "dW": dy64.T @ x64 + decay * w64,
+            "db": dy64.sum(axis=0) + decay * b64}
+    got = {"y": y.ToNumpy(), "dx": dx.ToNumpy(), "dW": dW.ToNumpy(), "db": db.ToNumpy()}
+    scale = {"y": np.sqrt(fin), "dx": np.sqrt(fout), "dW": np.sqrt(rows), "db": np.sqrt(rows)}
+    parity = {}
+    for k in want:
+        err = float(np.max(np.abs(got[k].reshape(want[k].shape) - want[k])))
+        bound = 1e-4 * float(scale[k]) * max(1.0, float(np.max(np.abs(want[k]))))
+        parity[k] = {"max_abs_err": err, "bound": bound}
+        if not err <= bound:
+            raise RuntimeError("dense layer %s: max|d| = %.3e beyond %.3e" % (k, err, bound))
+    for t in (x, W, b, dy, y, dx, dW, db):
+        t.Dispose()
+    return {"calls": res, "parity": parity,
+            "forward_ms": round(res[0]["event_us_per_call"] * 1e-3, 5), "backward_ms": round(res[1]["event_us_per_call"] * 1e-3, 5)}
 
 
 def layer_timings(w, wl):
@@ -978,7 +1022,7 @@ def write_table(path, out):
     rows = []
     layers = out["extra"].get("layers_fused_vs_reference_sequence", [])
     for name, v in out["extra"].items():
-        if name in ("layers_fused_vs_reference_sequence", "config1_dense_layer_fwd_bwd") or not isinstance(v, (list, dict)):
+        if name in ("layers_fused_vs_reference_sequence", "config1_dense_layer_fwd_bwd", "config1_dense_layer_calls") or not isinstance(v, (list, dict)):
             continue
         items = v if isinstance(v, list) else v.get("gemms") or [v]
         for r in items:
@@ -1004,8 +1048,10 @@ def write_table(path, out):
         f.write("\n".join(rows) + "\n\n")
         fb = out["extra"].get("config1_dense_layer_fwd_bwd")
         if fb:
-            f.write("Dense layer forward + backward (configuration 1): %.4f ms on the GPU (three launches) against %.4f ms "
-                    "through MKL on %d host threads.\n\n" % (fb["gpu_ms"], fb["cpu_mkl_ms"], fb["cpu_cores"]))
+            f.write("Dense layer forward + backward (configuration 1): %.4f ms on the GPU (forward call %.4f + backward call "
+                    "%.4f, one launch each; the three products as separate launches: %.4f) against %.4f ms through MKL on "
+                    "%d host threads.\n\n" % (fb["gpu_ms"], fb["gpu_forward_ms"], fb["gpu_backward_ms"],
+                                              fb["gpu_three_separate_products_ms"], fb["cpu_mkl_ms"], fb["cpu_cores"]))
         if layers:
             f.write("Whole layer calls through the host mirrors (HIP events around repeated calls, host launch time included):\n\n"
                     "| layer | form | forward ms | backward ms |\n|---|---|---|---|\n")

@@ -356,4 +356,44 @@ __global__ void __launch_bounds__(256) convert_f32_to_bf16_2d_kernel(const float
     }
 }
 
+// dst[c][r] (bf16) = src[r][c] for matrices of whole 64-row blocks whose rows start on 16-byte boundaries on both
+// sides: no LDS.  A thread owns 8 rows x CW columns (CW = 4 fp32 or 8 bf16 source elements: one 16-byte load per
+// row), turns them in registers and writes CW rows of the transpose, 16 bytes (8 bf16) each.  Lanes 0-7 of a
+// wavefront run along the rows, lanes / 8 along the columns: a load instruction reads 128 contiguous bytes from each
+// of 8 source rows per row step, a store instruction writes 128 contiguous bytes to each of 8 destination rows.
+// Requirements (checked by the host): rows % 64 == 0, cols % (8 * CW) == 0, 16-byte aligned bases and row pitches.
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+template <bool SRC_BF16>
+__global__ void __launch_bounds__(256) transpose_to_bf16_kernel(const void* __restrict__ src, long long ld_src, int rows,
+                                                                int cols, __bf16* __restrict__ dst, long long ld_dst) {
+    constexpr int CW = SRC_BF16 ? 8 : 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long long r0 = (long long)blockIdx.y * 64 + (lane & 7) * 8;
+    const long long cw0 = ((long long)blockIdx.x * 4 + wave) * (8 * CW);  // first column of this wavefront
+    if (cw0 >= cols) return;                                              // uniform over the wavefront
+    const long long c0 = cw0 + (lane >> 3) * CW;
+    u16x8 out[CW];
+    if constexpr (SRC_BF16) {
+        const unsigned short* s = static_cast<const unsigned short*>(src) + r0 * ld_src + c0;
+        u16x8 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const u16x8*>(s + j * ld_src);
+#pragma unroll
+        for (int i = 0; i < CW; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) out[i][j] = v[j][i];
+    } else {
+        const float* s = static_cast<const float*>(src) + r0 * ld_src + c0;
+        f32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const f32x4*>(s + j * ld_src);
+#pragma unroll
+        for (int i = 0; i < CW; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) out[i][j] = __builtin_bit_cast(unsigned short, (__bf16)v[j][i]);
+    }
+#pragma unroll
+    for (int i = 0; i < CW; ++i) *reinterpret_cast<u16x8*>(dst + (c0 + i) * ld_dst + r0) = out[i];
+}
+
 }  // namespace snhip

@@ -419,6 +419,21 @@ Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
     return best;
 }
 
+// what transpose_to_bf16_kernel asks of its operands (elem_bytes: 4 for an fp32 source, 2 for a bf16 one)
+bool wide_transpose_ok(const void* src, int rows, int cols, long long ld_src, int elem_bytes, const void* dst,
+                       long long ld_dst) {
+    const int cw = 16 / elem_bytes;
+    return rows % 64 == 0 && cols % (8 * cw) == 0 && rows / 64 <= 65535 && (uintptr_t)src % 16 == 0 &&
+           (uintptr_t)dst % 16 == 0 && (ld_src * elem_bytes) % 16 == 0 && (ld_dst * 2) % 16 == 0;
+}
+
+// dst[c][r] = src[r][c], both bf16 (the caller has checked wide_transpose_ok)
+int transpose_bf16(Handle* h, const void* src, int rows, int cols, long long ld_src, void* dst, long long ld_dst) {
+    hipLaunchKernelGGL(transpose_to_bf16_kernel<true>, dim3((unsigned)ceil_div(cols, 256), (unsigned)(rows / 64)), dim3(256),
+                       0, h->stream, src, ld_src, rows, cols, static_cast<__bf16*>(dst), ld_dst);
+    return hip_to_status(hipGetLastError());
+}
+
 int ensure_workspace(Handle* h, size_t bytes) {
     if (bytes <= h->ws_bytes) return SNHIP_STATUS_SUCCESS;
     if (h->ws != nullptr) {
@@ -720,11 +735,11 @@ int gemm_core(Handle* h, const GemmArgs& g) {
     // bf16-input arithmetic on a large product of whole tiles: round both operands to bf16 once, into the workspace and
     // into the k-contiguous form (A plain, B transposed), and multiply them with the bf16-storage kernel fed by direct
     // loads.  Each fp32 element is then read once by a streaming pass instead of once per tile that needs it, which is
-    // what bounds the fp32-storage kernels (8192^3 on MI355X: NN 1.59 -> 1.16 ms, NT 1.43 -> 1.10 ms, the conversion
-    // included).  Same rounding, same products; the sums may be grouped differently.  Not for transposed A with plain B:
-    // both operands would have to be transposed on the way, and the direct kernel is as fast there.
+    // what bounds the fp32-storage kernels (8192^3 on MI355X: NN 1.59 -> 1.00 ms, NT 1.43 -> 0.99 ms, TN 1.18 -> 1.01 ms,
+    // the conversion included; a transposing pass over an 8192^2 operand takes 0.085 ms, a plain one 0.07 ms).  Same
+    // rounding, same products; the sums may be grouped differently.
     if (math == SNHIP_MATH_BF16_INPUT && !g.no_alloc && batch == 1 && h->force_cfg < 0 && h->force_splitk <= 0 &&
-        !(g.tA && !g.tB) && ep.addend == nullptr && ep.act == ACT_NONE && g.colsum == nullptr &&
+        ep.addend == nullptr && ep.act == ACT_NONE && g.colsum == nullptr &&
         M % BDtlCfg::BM == 0 && N % BDtlCfg::BN == 0 && K % BDtlCfg::BK == 0 && K >= 8 * BDtlCfg::BK &&
         (long long)(M / BDtlCfg::BM) * (N / BDtlCfg::BN) >= h->num_cu &&
         2 * ((size_t)M + N) * K <= kMaxWorkspaceBytes) {
@@ -754,6 +769,43 @@ int gemm_core(Handle* h, const GemmArgs& g) {
             else
                 st = snhip_convert_f32_to_bf16_2d(h, g.B, N, K, g.ldb, 0, wb, K);
             if (st != SNHIP_STATUS_SUCCESS) return st;
+            return gemm_core(h, s);
+        }
+    }
+    // Operands stored as bf16, a large product of whole tiles, but not in the k-contiguous form: the operand(s) lying the
+    // other way are transposed once into the workspace (2 bytes read and written per element) and the product runs in
+    // the direct-load kernel.  The register-transposing kernels lose more than the pass costs (8192^3: NN 1.13 ms, TN
+    // 1.41 ms against 0.95 ms in the k-contiguous form).  Same values multiplied; the sums may be grouped differently.
+    if (math == SNHIP_MATH_BF16_STORED && !g.no_alloc && batch == 1 && h->force_cfg < 0 && h->force_splitk <= 0 &&
+        (g.tA || !g.tB) && ep.addend == nullptr && ep.act == ACT_NONE && g.colsum == nullptr && M % BDtlCfg::BM == 0 &&
+        N % BDtlCfg::BN == 0 && K % BDtlCfg::BK == 0 && K >= 8 * BDtlCfg::BK &&
+        (long long)(M / BDtlCfg::BM) * (N / BDtlCfg::BN) >= h->num_cu && 2 * ((size_t)M + N) * K <= kMaxWorkspaceBytes) {
+        const size_t a_elems = g.tA ? (size_t)M * K : 0, b_elems = !g.tB ? (size_t)N * K : 0;
+        // (checked against the caller's pointers and a 256-byte aligned stand-in for the workspace, which may not
+        // exist yet)
+        const void* const aligned = reinterpret_cast<const void*>(uintptr_t(256));
+        const bool ok_a = !g.tA || wide_transpose_ok(g.A, K, M, g.lda, 2, aligned, K);
+        const bool ok_b = g.tB || wide_transpose_ok(g.B, K, N, g.ldb, 2, aligned, K);
+        GemmArgs s = g;
+        s.math = SNHIP_MATH_BF16_STORED;
+        s.tA = false, s.tB = true;
+        if (g.tA) s.A = reinterpret_cast<const float*>(uintptr_t(256)), s.lda = K;
+        if (!g.tB) s.B = reinterpret_cast<const float*>(uintptr_t(256)), s.ldb = K;
+        if (ok_a && ok_b && prefer_dtl(h, s, SNHIP_MATH_BF16_STORED, false) == kBDtlConfig) {
+            int st = ensure_workspace(h, 2 * (a_elems + b_elems));
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+            __bf16* wa = reinterpret_cast<__bf16*>(h->ws);
+            __bf16* wb = wa + a_elems;
+            if (g.tA) {
+                st = transpose_bf16(h, g.A, K, M, g.lda, wa, K);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+                s.A = reinterpret_cast<const float*>(wa);
+            }
+            if (!g.tB) {
+                st = transpose_bf16(h, g.B, K, N, g.ldb, wb, K);
+                if (st != SNHIP_STATUS_SUCCESS) return st;
+                s.B = reinterpret_cast<const float*>(wb);
+            }
             return gemm_core(h, s);
         }
     }
@@ -1650,6 +1702,12 @@ int snhip_convert_f32_to_bf16_2d(void* handle, const float* src, int rows, int c
     if (rows == 0 || cols == 0) return SNHIP_STATUS_SUCCESS;
     if (src == nullptr || dst == nullptr || (uintptr_t)dst % 2 != 0 || ld_src < cols || ld_dst < (transpose ? rows : cols))
         return SNHIP_STATUS_INVALID_VALUE;
+    if (transpose != 0 && wide_transpose_ok(src, rows, cols, ld_src, 4, dst, ld_dst)) {
+        hipLaunchKernelGGL(transpose_to_bf16_kernel<false>, dim3((unsigned)ceil_div(cols, 128), (unsigned)(rows / 64)),
+                           dim3(256), 0, static_cast<Handle*>(handle)->stream, static_cast<const void*>(src), ld_src, rows,
+                           cols, static_cast<__bf16*>(dst), ld_dst);
+        return hip_to_status(hipGetLastError());
+    }
     if (ceil_div(rows, 32) > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
     hipLaunchKernelGGL(convert_f32_to_bf16_2d_kernel, dim3((unsigned)ceil_div(cols, 32), (unsigned)ceil_div(rows, 32)),
                        dim3(256), 0, static_cast<Handle*>(handle)->stream, src, ld_src, rows, cols, transpose != 0,

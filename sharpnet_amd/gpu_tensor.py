@@ -67,6 +67,7 @@ class GPUWrapper:
     # -- arithmetic ----------------------------------------------------------
     MATH_FP32 = 0
     MATH_BF16_INPUT = 1
+    MATH_BF16_STORED = 2
 
     def set_math_mode(self, mode):
         """fp32 MFMA (default) or bf16-input / fp32-accumulate MFMA for every GEMM of this handle."""

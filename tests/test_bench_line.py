@@ -30,7 +30,10 @@ def _fake_extra():
                "forward_ms": 0.085, "backward_ms": None}]
     return {
         "config1_dense_layer": {"gemms": [_fake_gemm_row("fwd y=x.Wt+b (128,256,784) NT beta=0", 0.06)] * 3, "cpu_baseline": None},
-        "config1_dense_layer_fwd_bwd": {"gpu_ms": 0.0154, "cpu_mkl_ms": 0.2, "cpu_cores": 16, "note": "x" * 300},
+        "config1_dense_layer_calls": {"calls": [], "parity": {}, "forward_ms": 0.0049, "backward_ms": 0.0067},
+        "config1_dense_layer_fwd_bwd": {"gpu_ms": 0.0116, "gpu_forward_ms": 0.0049, "gpu_backward_ms": 0.0067,
+                                        "gpu_three_separate_products_ms": 0.0154, "cpu_mkl_ms": 0.2, "cpu_cores": 16,
+                                        "note": "x" * 300},
         "config2_sweep": {"gemms": sweep, "cpu_baseline": None},
         "config3_mlp_step": {"gemms": [_fake_gemm_row("fwd0 (4096,4096,3072) NT beta=0", 0.9)] * 9, "total_ms": 5.9,
                              "tflops": 139.0, "cpu_baseline": None},

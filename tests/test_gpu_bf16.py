@@ -159,7 +159,10 @@ def test_convert_2d_with_pitches_and_transpose(oracle, gpu_wrapper):
     from sharpnet_amd.hiplib import check_status
     w = gpu_wrapper
     rng = np.random.default_rng(44)
-    for rows, cols, pad_s, pad_d in [(1, 1, 0, 0), (33, 65, 3, 2), (100, 31, 0, 5), (256, 128, 4, 0)]:
+    # (the last four: whole 64-row blocks, 16-byte aligned rows on both sides - the wide transposing kernel - with
+    # one, several and partly filled column groups of four wavefronts, padded pitches)
+    for rows, cols, pad_s, pad_d in [(1, 1, 0, 0), (33, 65, 3, 2), (100, 31, 0, 5), (256, 128, 4, 0), (64, 32, 0, 0),
+                                     (192, 160, 4, 8), (128, 416, 0, 0), (64, 96, 8, 0)]:
         src = random_tensor(rng, (rows, cols + pad_s), -2, 2)
         gs = GPUTensor(src.shape, src, w)
         for transpose in (0, 1):
@@ -389,7 +392,7 @@ def test_bf16_stored_direct_to_lds_kernel(oracle, gpu_wrapper):
 def test_bf16_input_large_products_go_through_one_conversion(oracle, gpu_wrapper, tA, tB):
     """bf16-input arithmetic on a product of whole 256 x 256 tiles with a tile per compute unit: the library rounds both
     fp32 operands to bf16 once (into its workspace, in the k-contiguous form) and multiplies them with the bf16-storage
-    kernel - except for transposed A with plain B, which the fp32-storage kernel takes directly.  Sampled rows against
+    kernel, in all four transpose forms.  Sampled rows against
     the oracle on rounded inputs (fp32 bound), alpha / beta / bias, contiguous operands and operands with padded rows
     (snhip_gemm_rm), and the same product again after a smaller one (the workspace is reused)."""
     from sharpnet_amd import GPUTensor
@@ -399,7 +402,7 @@ def test_bf16_input_large_products_go_through_one_conversion(oracle, gpu_wrapper
     kinds = {c["id"]: c["kind"] for c in w.configs()}
     rng = np.random.default_rng(880 + 2 * tA + tB)
     M, N, K = 4096, 4096, 256
-    want_kind = "bf16" if (tA and not tB) else "bf16-stored-dtl"
+    want_kind = "bf16-stored-dtl"
     for pad in (0, 8):
         a = random_tensor(rng, (K, M + pad) if tA else (M, K + pad), -1, 1)
         b = random_tensor(rng, (N, K + pad) if tB else (K, N + pad), -1, 1)
@@ -426,6 +429,62 @@ def test_bf16_input_large_products_go_through_one_conversion(oracle, gpu_wrapper
         assert float(np.max(np.abs(got[rows] - ref))) <= 1e-4 * np.sqrt(K) * 0.5 + 2e-6
         assert float(np.max(np.abs(got - ref32))) / float(np.max(np.abs(ref32))) <= 1e-2
         for t in (ga, gb, gc, gbias):
+            t.Dispose()
+
+
+@pytest.mark.parametrize("tA,tB", [(False, False), (True, False), (True, True)])
+def test_bf16_stored_large_products_are_brought_into_the_k_contiguous_form(oracle, gpu_wrapper, tA, tB):
+    """Operands stored as bf16, a product of whole 256 x 256 tiles with a tile per compute unit, in a form other than
+    plain A with transposed B: the library transposes the operand(s) lying the other way once into its workspace
+    (bf16 to bf16) and runs the direct-load kernel.  Sampled rows against the oracle on the rounded inputs (fp32
+    bound), alpha / beta / bias, contiguous operands and padded rows (snhip_gemm_ex), agreement with the
+    register-transposing kernel forced through the tuning hook, and a smaller product of the same form afterwards."""
+    from sharpnet_amd.hiplib import check_status, GemmDesc
+    import ctypes
+    w = gpu_wrapper
+    lib, h = w.lib, w.handle
+    kinds = {c["id"]: c["kind"] for c in w.configs()}
+    staged = [c["id"] for c in w.configs() if c["kind"] == "bf16-stored"][0]
+    rng = np.random.default_rng(990 + 2 * tA + tB)
+    for (M, N, K, pad) in ((4096, 4096, 256, 0), (4096, 4096, 320, 8), (2048, 8192, 512, 0)):
+        a = random_tensor(rng, (K, M + pad) if tA else (M, K + pad), -1, 1)
+        b = random_tensor(rng, (N, K + pad) if tB else (K, N + pad), -1, 1)
+        c0, bias = random_tensor(rng, (M, N), -1, 1), random_tensor(rng, (N,), -1, 1)
+        ga, gb, gbias = T(w, a), T(w, b), T(w, bias)
+        pa, pb = to_bf16_on_device(w, ga), to_bf16_on_device(w, gb)
+        outs = {}
+        for force in (-1, staged):
+            gc = T(w, c0)
+            d = GemmDesc()
+            d.struct_size = ctypes.sizeof(GemmDesc)
+            d.transA, d.transB, d.M, d.N, d.K = int(tA), int(tB), M, N, K
+            d.alpha, d.beta = 0.5, -1.0
+            d.A, d.lda, d.B, d.ldb = pa, a.shape[1], pb, b.shape[1]
+            d.C, d.ldc, d.batch = gc.Pointer, N, 1
+            d.bias = gbias.Pointer
+            d.math = w.MATH_BF16_STORED
+            print("bf16-stored via transposition", tA, tB, (M, N, K), "padding", pad, "forced", force, flush=True)
+            w.set_tuning(force, 1 if force >= 0 else 0)
+            try:
+                check_status(lib.snhip_gemm_ex(h, ctypes.byref(d)))
+            finally:
+                w.set_tuning(-1, 0)
+            want_kind = "bf16-stored-dtl" if force < 0 else "bf16-stored"
+            assert kinds[w.last_tuning()[0]] == want_kind, (kinds[w.last_tuning()[0]], want_kind)
+            outs[force] = gc.ToNumpy()
+            gc.Dispose()
+        got = outs[-1]
+        assert np.all(np.isfinite(got))
+        rows = np.sort(rng.choice(M, 6, replace=False))
+        opa = np.ascontiguousarray((a[:, :M].T if tA else a[:, :K])[rows])
+        opb = np.ascontiguousarray(b[:, :K] if tB else b[:, :N])
+        ref = oracle.dot(oracle.round_to_bf16(opa), False, oracle.round_to_bf16(opb), tB, 0.5, -1.0, c0[rows]) + bias
+        bound = 1e-4 * np.sqrt(K) * 0.5 + 2e-6
+        assert float(np.max(np.abs(got[rows] - ref))) <= bound
+        assert float(np.max(np.abs(got - outs[staged]))) <= bound
+        w.release(pa, 2 * ga.Count)
+        w.release(pb, 2 * gb.Count)
+        for t in (ga, gb, gbias):
             t.Dispose()
 
 
