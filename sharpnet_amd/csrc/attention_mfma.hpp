@@ -1383,6 +1383,12 @@ __global__ void __launch_bounds__(512) attention_fwd16_bf16_kernel(const AttnPar
 // V <- K, Pin <- the stored weights, P <- dS out, O <- dQ): pass 1 gathers the row sums rs = sum_k P . dP over all key
 // blocks, pass 2 forms dS = scale . P . (dP - rs) block by block, writes it and accumulates dQ += dS . K.
 // ---------------------------------------------------------------------------------------------------------------
+// f(integral_constant<int, 0>), f(integral_constant<int, 1>), ... in order
+template <class F, int... I>
+__device__ __forceinline__ void for_each_index(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+
 template <bool ONE_PASS, bool BF16 = false, bool BWD = false, int HD = 64>
 __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnParams p) {
     static_assert(!BWD || (!ONE_PASS && !BF16), "the backward instantiation is the two-pass fp32 one");
@@ -1554,11 +1560,14 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
 
     // BWD: the stored weights of this lane's keys in block kb (keys past Tk: the lane's keys of block 0 are read
     // instead - they exist, this kernel is given more than 256 keys - and zero is taken)
-    // The product runs in PARTS parts of NKT / PARTS key tiles: the weights of a part are asked for in front of that
-    // part's MFMAs and used behind them, so their way from memory is covered by the product, and only two parts'
-    // weights are in registers at a time (all of them across the whole product do not fit beside its operands; at
-    // head dimension 64 halves still had the compiler move the output accumulators to scratch and back per block).
-    constexpr int PARTS = HD == 64 ? 4 : 2;
+    // The product runs in PARTS parts of NKT / PARTS key tiles: the weights of a part are asked for LA parts ahead of
+    // its MFMAs and used behind them, so their way from memory is covered by the product, and only LA + 1 parts'
+    // weights are in registers at a time (all of them across the whole product do not fit beside its operands).  At
+    // head dimension 64 a part is a single key tile, asked for four tiles ahead: with halves or quarters of the block
+    // (32 registers of weights in flight) the compiler moved half of the output accumulators to scratch and back in
+    // every block (48 bytes per lane); single tiles need 252 registers and no scratch, at the same speed.
+    constexpr int PARTS = HD == 64 ? 16 : 2;
+    constexpr int LA = HD == 64 ? 4 : 1;  // parts asked for ahead
     constexpr int HALF = NKT / PARTS;  // key tiles per part
     f32x4 pin[BWD ? NKT : 1];
     auto load_weights = [&](int kb, int t0) {
@@ -1600,19 +1609,15 @@ __global__ void __launch_bounds__(512) attention_fwd16_long_kernel(const AttnPar
     auto bwd_part = [&](auto ic, int kb, auto&& behind_part) {
         constexpr int I = decltype(ic)::value;
         attn16_score_product_part<I * HALF, HALF, NKT, NQ, KP>(Ks, g, l16, qf, sacc);
-        if constexpr (I + 1 < PARTS) load_weights(kb, (I + 1) * HALF);
+        if constexpr (I + LA < PARTS) load_weights(kb, (I + LA) * HALF);
         __builtin_amdgcn_sched_barrier(0);
         behind_part(I * HALF);
         __builtin_amdgcn_sched_barrier(0);
     };
     auto bwd_parts = [&](int kb, auto&& behind_part) {
-        load_weights(kb, 0);
-        bwd_part(std::integral_constant<int, 0>{}, kb, behind_part);
-        bwd_part(std::integral_constant<int, 1>{}, kb, behind_part);
-        if constexpr (PARTS == 4) {
-            bwd_part(std::integral_constant<int, 2>{}, kb, behind_part);
-            bwd_part(std::integral_constant<int, 3>{}, kb, behind_part);
-        }
+#pragma unroll
+        for (int i = 0; i < LA; ++i) load_weights(kb, i * HALF);
+        for_each_index([&](auto ic) { bwd_part(ic, kb, behind_part); }, std::make_integer_sequence<int, PARTS>{});
     };
 
     // ---- pass 1: row maximum and row sum over all needed blocks (BWD: the row sums of P . dP) ----
