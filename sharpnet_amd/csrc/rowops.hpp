@@ -396,4 +396,27 @@ __global__ void __launch_bounds__(256) transpose_to_bf16_kernel(const void* __re
     for (int i = 0; i < CW; ++i) *reinterpret_cast<u16x8*>(dst + (c0 + i) * ld_dst + r0) = out[i];
 }
 
+// dst[r][c] (bf16) = src[r][c] (fp32) for padded matrices whose rows start on 16-byte boundaries on both sides and
+// hold a multiple of 8 columns: a thread rounds 8 consecutive values of a row (two 16-byte loads, one 16-byte store),
+// consecutive threads walk along the row and on into the next one.
+__global__ void __launch_bounds__(256) convert_rows_to_bf16_kernel(const float* __restrict__ src, long long ld_src, int rows,
+                                                                   int cols, __bf16* __restrict__ dst, long long ld_dst) {
+    const int chunks = cols / 8;  // per row
+    const long long total = (long long)rows * chunks;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
+        const long long r = i / chunks;
+        const int c = (int)(i - r * chunks);
+        const float* s = src + r * ld_src + 8 * c;
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(s);
+        const f32x4 hi = *reinterpret_cast<const f32x4*>(s + 4);
+        u16x8 o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            o[j] = __builtin_bit_cast(unsigned short, (__bf16)lo[j]);
+            o[4 + j] = __builtin_bit_cast(unsigned short, (__bf16)hi[j]);
+        }
+        *reinterpret_cast<u16x8*>(dst + r * ld_dst + 8 * c) = o;
+    }
+}
+
 }  // namespace snhip

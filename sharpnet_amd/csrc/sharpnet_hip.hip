@@ -744,16 +744,20 @@ int gemm_core(Handle* h, const GemmArgs& g) {
         (long long)(M / BDtlCfg::BM) * (N / BDtlCfg::BN) >= h->num_cu &&
         2 * ((size_t)M + N) * K <= kMaxWorkspaceBytes) {
         const size_t a_elems = (size_t)M * K, b_elems = (size_t)N * K;
-        int st = ensure_workspace(h, 2 * (a_elems + b_elems));
-        if (st != SNHIP_STATUS_SUCCESS) return st;
-        __bf16* wa = reinterpret_cast<__bf16*>(h->ws);
-        __bf16* wb = wa + a_elems;
         GemmArgs s = g;
         s.math = SNHIP_MATH_BF16_STORED;
         s.tA = false, s.tB = true;
-        s.A = reinterpret_cast<const float*>(wa), s.lda = K;
-        s.B = reinterpret_cast<const float*>(wb), s.ldb = K;
+        // (the kernel's conditions are checked on a 256-byte aligned stand-in for the workspace, which is not grown
+        // before the route is known to be taken)
+        s.A = s.B = reinterpret_cast<const float*>(uintptr_t(256));
+        s.lda = s.ldb = K;
         if (prefer_dtl(h, s, SNHIP_MATH_BF16_STORED, false) == kBDtlConfig) {
+            int st = ensure_workspace(h, 2 * (a_elems + b_elems));
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+            __bf16* wa = reinterpret_cast<__bf16*>(h->ws);
+            __bf16* wb = wa + a_elems;
+            s.A = reinterpret_cast<const float*>(wa);
+            s.B = reinterpret_cast<const float*>(wb);
             // (an operand that is already k-contiguous without padding takes the one-dimensional pass: 16-byte pieces)
             if (g.tA)
                 st = snhip_convert_f32_to_bf16_2d(h, g.A, K, M, g.lda, 1, wa, K);
@@ -1706,6 +1710,13 @@ int snhip_convert_f32_to_bf16_2d(void* handle, const float* src, int rows, int c
         hipLaunchKernelGGL(transpose_to_bf16_kernel<false>, dim3((unsigned)ceil_div(cols, 128), (unsigned)(rows / 64)),
                            dim3(256), 0, static_cast<Handle*>(handle)->stream, static_cast<const void*>(src), ld_src, rows,
                            cols, static_cast<__bf16*>(dst), ld_dst);
+        return hip_to_status(hipGetLastError());
+    }
+    if (transpose == 0 && cols % 8 == 0 && (uintptr_t)src % 16 == 0 && (uintptr_t)dst % 16 == 0 && ld_src % 4 == 0 &&
+        ld_dst % 8 == 0) {
+        const long long blocks = ((long long)rows * (cols / 8) + 255) / 256;
+        hipLaunchKernelGGL(convert_rows_to_bf16_kernel, dim3((unsigned)(blocks < 16384 ? blocks : 16384)), dim3(256), 0,
+                           static_cast<Handle*>(handle)->stream, src, ld_src, rows, cols, static_cast<__bf16*>(dst), ld_dst);
         return hip_to_status(hipGetLastError());
     }
     if (ceil_div(rows, 32) > 65535) return SNHIP_STATUS_NOT_SUPPORTED;
