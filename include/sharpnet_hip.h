@@ -294,8 +294,9 @@ int snhip_sizeof_attention_bwd_desc(void);
  * (batch, steps, dirs * hidden_size) with the reverse direction in the second half of a row; hx, hy, cx, cy and their
  * gradients are (dirs * num_layers, batch, hidden_size), any of them may be NULL (zeros in, nothing out).
  * Each time step is one GEMM with the recurrent matrix plus one element-wise kernel; the input projections of all
- * steps, dx and both weight gradients are one GEMM each per layer and direction.  Dropout between stacked layers is
- * not implemented: a descriptor that asks for it is refused in training (status 15), never silently ignored. */
+ * steps, dx and both weight gradients are one GEMM each per layer and direction.  Dropout between stacked layers
+ * (training only, as in cuDNN) draws its masks from the library's own counter-based generator, see
+ * snhip_rnn_set_dropout_seed below: cuDNN's stream cannot be reproduced, the semantics are the same. */
 #define SNHIP_RNN_RELU 0 /* cudnnRNNMode_t, Prod/GPU/CudnnWrapper.cs:313-327 */
 #define SNHIP_RNN_TANH 1
 #define SNHIP_RNN_LSTM 2
@@ -310,9 +311,10 @@ typedef struct snhip_rnn_desc { /* the fields of Prod/Layers/RNNDescriptor.cs th
     int bidirectional;          /* 0 / 1 */
     int num_layers;
     int input_size, hidden_size;
-    float dropout;              /* RNNDescriptor.dropoutRate (Prod/Layers/RNNDescriptor.cs:21): applied by cuDNN between stacked
-                                   layers in training.  Not implemented: snhip_rnn_forward returns status 15 when it is
-                                   non-zero in training with num_layers > 1 (it has no effect otherwise, as in cuDNN). */
+    float dropout;              /* RNNDescriptor.dropoutRate (Prod/Layers/RNNDescriptor.cs:21), in [0, 1): in training the
+                                   outputs of every layer but the last are multiplied, on their way into the next layer,
+                                   by a mask of zeros (probability dropout) and 1 / (1 - dropout); no effect at inference
+                                   or with one layer, as in cuDNN. */
 } snhip_rnn_desc;
 int snhip_sizeof_rnn_desc(void);
 /* Bytes of the weight space.  Layout: all matrices (pseudo-layer by pseudo-layer = layer * dirs + direction: the
@@ -330,6 +332,20 @@ int snhip_rnn_temp_space_sizes(const snhip_rnn_desc* desc, int training, int bat
 int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, int batch, int steps, const float* x,
                       float* y, const float* hx, float* hy, const float* cx, float* cy, const float* weights,
                       void* workspace, size_t workspace_bytes, void* reserve, size_t reserve_bytes);
+/* Dropout masks.  The reference seeds cuDNN's dropout states once with 0 and lets every call advance them
+ * (GPUWrapper.DropoutDesc, Prod/GPU/GPUWrapper.cs:460-474); here a handle counts its training-mode forward calls that drop
+ * units (from 0; snhip_rnn_set_dropout_seed sets the seed and resets the count) and the mask is a pure function of
+ * (seed, call, boundary, element): Philox4x32-10 with key {seed & 0xffffffff, seed >> 32} and counter
+ * {e / 4 (low word), e / 4 (high word), boundary, call}; element e - numbered in (step, sample, unit) order over the
+ * (steps, batch, dirs * hidden) outputs of layer `boundary` - takes output word e % 4 and is dropped when
+ * (word >> 8) / 2^24 < dropout.  The forward call stores seed and call number in its reserve buffer, so the backward calls
+ * of a layer use the masks of that layer's own forward call whatever ran in between.
+ * snhip_rnn_dropout_mask writes the mask of one boundary (0 .. num_layers - 2) of call number `call` under the handle's
+ * current seed, values 0 or 1 / (1 - dropout), laid out like y: (batch, steps, dirs * hidden). */
+int snhip_rnn_set_dropout_seed(void* handle, unsigned long long seed);
+int snhip_rnn_get_dropout_calls(void* handle, unsigned long long* calls);
+int snhip_rnn_dropout_mask(void* handle, const snhip_rnn_desc* desc, int batch, int steps, unsigned long long call,
+                           int boundary, float* mask);
 /* Tuning hook: 0 (default) runs a time step, forward or backward, as one launch - the product with the recurrent
  * matrix and the cell arithmetic in one kernel - whenever hidden_size is a multiple of 4 and at least 32; 1 always
  * issues the GEMM and the cell kernel separately (what other hidden sizes get).  Same results within rounding

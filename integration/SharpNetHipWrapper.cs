@@ -144,7 +144,7 @@ namespace SharpNet.GPU
         public struct RnnDesc   // RNNDescriptor.cs: cellMode, biasMode, dirMode, numLayers, inputSize, hiddenSize
         {
             public int struct_size, cell_mode, bias_mode, bidirectional, num_layers, input_size, hidden_size;
-            public float dropout;   // RNNDescriptor.dropoutRate; non-zero with num_layers > 1 in training: status 15
+            public float dropout;   // RNNDescriptor.dropoutRate: between stacked layers, in training
         }
         [DllImport(DLL_NAME)] public static extern int snhip_sizeof_rnn_desc();
         [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_rnn_weight_space_size(ref RnnDesc desc, out size_t bytes);   // size_t: the reference's own struct (Prod/GPU/size_t.cs)
@@ -160,6 +160,11 @@ namespace SharpNet.GPU
             IntPtr workspace, size_t workspaceBytes, IntPtr reserve, size_t reserveBytes);
         [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_rnn_backward_weights(IntPtr handle, ref RnnDesc desc, int batch, int steps,
             IntPtr x, IntPtr hx, IntPtr y, IntPtr weightGradients, IntPtr workspace, size_t workspaceBytes, IntPtr reserve, size_t reserveBytes);
+        // dropout masks come from the library's own generator (the reference seeds cuDNN's with 0, GPUWrapper.cs:472)
+        [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_rnn_set_dropout_seed(IntPtr handle, ulong seed);
+        [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_rnn_get_dropout_calls(IntPtr handle, out ulong calls);
+        [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_rnn_dropout_mask(IntPtr handle, ref RnnDesc desc, int batch, int steps,
+            ulong call, int boundary, IntPtr mask);
         [DllImport(DLL_NAME)] public static extern cublasStatus_t snhip_gemm_ex(IntPtr handle, ref GemmDesc desc);
         [DllImport(DLL_NAME)] public static extern int snhip_sizeof_gemm_desc();
 

@@ -42,6 +42,14 @@ rnn_backward               cudnnRNNBackwardData_v8 +               the same 13 s
                                                                    10 epochs ParallelRunWithPyTorch.cs:951
                                                                    (0.2722862660884857); torch autograd through the
                                                                    same modules
+masks= of rnn_forward /    dropout between stacked layers as       the mask values are an input, so what is pinned is
+rnn_backward               cuDNN applies it in training            where they act: a two-layer call with a mask equals
+                           (RNNDescriptor.dropoutRate,             torch.nn.LSTM / GRU / RNN modules of one layer each
+                           RecurrentLayer.cs:69,123; states        with the mask multiplied in between, values and all
+                           seeded with 0, GPUWrapper.cs:460-474)   gradients through autograd (tests/test_oracle_rnn.py)
+philox4x32_10 /            the generator the library documents     the three known-answer vectors of the Random123
+dropout_mask               for its masks (cuDNN's own stream is    distribution (kat_vectors: zeros, all ones, digits of
+                           not reproducible)                       pi); the mask's layout by construction from them
 layer_forward /            RecurrentLayer.ForwardPropagation /     the same stored predictions and losses (last-step
 layer_backward             BackwardPropagation :305-520            outputs of uni- and bidirectional layers; a 2-layer
                            (returnSequences == false: last step    bidirectional sequence layer feeding a last-step
@@ -177,14 +185,46 @@ def _cell_backward(cell, H, dh, dc, saved):
     return (np.concatenate([dr_pre, dz_pre, dn_pre], 1), np.concatenate([dr_pre, dz_pre, dn_pre * r], 1), dh * z, dc)
 
 
-def rnn_forward(desc, x, weights, hx=None, cx=None):
-    """x (B, T, input) -> y (B, T, dirs*H), hy (pseudo_layers, B, H), cy (same, LSTM only), cache."""
+def philox4x32_10(counter, key):
+    """Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11): four arrays of
+    32-bit counter words and two key words -> four arrays of 32-bit output words."""
+    c0, c1, c2, c3 = (np.asarray(c, np.uint64) for c in counter)
+    k0, k1 = (np.uint64(k) for k in key)
+    m0, m1, w0, w1 = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57), np.uint64(0x9E3779B9), np.uint64(0xBB67AE85)
+    lo, sh = np.uint64(0xFFFFFFFF), np.uint64(32)
+    for _ in range(10):
+        p0, p1 = m0 * c0, m1 * c2
+        c0, c1, c2, c3 = ((p1 >> sh) ^ c1 ^ k0) & lo, p1 & lo, ((p0 >> sh) ^ c3 ^ k1) & lo, p0 & lo
+        k0, k1 = (k0 + w0) & lo, (k1 + w1) & lo
+    return [c.astype(np.uint32) for c in (c0, c1, c2, c3)]
+
+
+def dropout_mask(seed, call, boundary, rate, batch, steps, width):
+    """The mask the library documents for the activations between layers `boundary` and `boundary + 1` in its
+    training-mode forward call number `call`: element e, numbered in (step, sample, unit) order, takes word e % 4 of
+    philox(counter = {e // 4 low, e // 4 high, boundary, call}, key = {seed low, seed high}) and is dropped when
+    (word >> 8) / 2^24 < rate.  Returned as (batch, steps, width) float32 with values 0 and 1 / (1 - rate)."""
+    count = batch * steps * width
+    chunk = np.arange((count + 3) // 4, dtype=np.uint64)
+    words = philox4x32_10([chunk & np.uint64(0xFFFFFFFF), chunk >> np.uint64(32), np.full_like(chunk, boundary),
+                           np.full_like(chunk, call & 0xFFFFFFFF)], [seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF])
+    bits = np.stack(words, axis=1).reshape(-1)[:count]
+    u = (bits >> np.uint32(8)).astype(np.float32) * np.float32(1.0 / 16777216.0)
+    scale = np.float32(1.0) / (np.float32(1.0) - np.float32(rate))
+    step_major = np.where(u < np.float32(rate), np.float32(0.0), scale).astype(np.float32).reshape(steps, batch, width)
+    return np.ascontiguousarray(step_major.transpose(1, 0, 2))
+
+
+def rnn_forward(desc, x, weights, hx=None, cx=None, masks=None):
+    """x (B, T, input) -> y (B, T, dirs*H), hy (pseudo_layers, B, H), cy (same, LSTM only), cache.
+    masks (training with dropout): one (B, T, dirs*H) array per layer but the last, multiplied onto that layer's
+    outputs on their way into the next layer (values 0 and 1 / (1 - rate)); y, hy, cy are never masked."""
     B, T, _ = x.shape
     H, K = desc.hidden_size, desc.dirs
     inp = x.astype(np.float64)
     hy = np.zeros((desc.pseudo_layers, B, H))
     cy = np.zeros((desc.pseudo_layers, B, H))
-    cache = {"desc": desc, "weights": weights, "layers": []}
+    cache = {"desc": desc, "weights": weights, "layers": [], "masks": masks}
     for layer in range(desc.num_layers):
         out = np.zeros((B, T, K * H))
         per_dir = []
@@ -204,7 +244,9 @@ def rnn_forward(desc, x, weights, hx=None, cx=None):
             per_dir.append({"saved": saved, "h_in": h_in, "h0": h0})
         cache["layers"].append({"input": inp, "dirs": per_dir})
         inp = out
-    return inp.astype(np.float32), hy.astype(np.float32), cy.astype(np.float32), cache
+        if masks is not None and layer < desc.num_layers - 1:
+            inp = out * masks[layer].astype(np.float64)
+    return out.astype(np.float32), hy.astype(np.float32), cy.astype(np.float32), cache
 
 
 def rnn_backward(desc, dy, cache, dhy=None, dcy=None):
@@ -245,7 +287,9 @@ def rnn_backward(desc, dy, cache, dhy=None, dcy=None):
             if c0 is not None:
                 dw[c0:c0 + G * H] = dbR
         dout = dinp
-    return dout.astype(np.float32), dw.astype(np.float32), dhx.astype(np.float32), dcx.astype(np.float32)
+        if cache.get("masks") is not None and layer > 0:
+            dout = dinp * cache["masks"][layer - 1].astype(np.float64)   # gradient of the outputs of the layer below
+    return dinp.astype(np.float32), dw.astype(np.float32), dhx.astype(np.float32), dcx.astype(np.float32)
 
 
 def layer_forward(desc, x, weights, return_sequences):

@@ -550,4 +550,66 @@ __global__ void __launch_bounds__(256) set_rows_kernel(float* dst, long long ld_
     dst[r * ld_dst + c] = src ? src[r * ld_src + c] : 0.0f;
 }
 
+// ---------------------------------------------------------------------------
+// Dropout between stacked layers.  The mask is a pure function of (seed, call, boundary, element), so the backward
+// pass and a caller's own check can regenerate it instead of storing it:
+//   Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11) with
+//   key = {seed low word, seed high word} and counter = {e / 4 low word, e / 4 high word, boundary, call};
+//   element e takes output word e % 4; it is dropped when (word >> 8) * 2^-24 < rate, else multiplied by 1 / (1 - rate).
+// e numbers the elements of the (steps, batch, dirs * hidden) activations between layers `boundary` and `boundary + 1`
+// in that (step-major) order.
+// ---------------------------------------------------------------------------
+struct Philox4 {
+    unsigned int v[4];
+};
+__device__ __host__ __forceinline__ Philox4 philox4x32_10(unsigned int c0, unsigned int c1, unsigned int c2, unsigned int c3,
+                                                          unsigned int k0, unsigned int k1) {
+    constexpr unsigned int M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+#pragma unroll
+    for (int round = 0; round < 10; ++round) {
+        const unsigned long long p0 = (unsigned long long)M0 * c0, p1 = (unsigned long long)M1 * c2;
+        const unsigned int n0 = (unsigned int)(p1 >> 32) ^ c1 ^ k0, n1 = (unsigned int)p1;
+        const unsigned int n2 = (unsigned int)(p0 >> 32) ^ c3 ^ k1, n3 = (unsigned int)p0;
+        c0 = n0, c1 = n1, c2 = n2, c3 = n3;
+        k0 += W0, k1 += W1;
+    }
+    return Philox4{{c0, c1, c2, c3}};
+}
+
+struct RnnDropout {
+    unsigned long long seed;
+    unsigned int call, boundary;
+    float rate, scale;  // scale = 1 / (1 - rate)
+    // when not null: {seed low word, seed high word, call} as the forward call left them in its reserve buffer; they
+    // replace the three values above (the backward pass of a layer may run after other layers have drawn their masks)
+    const unsigned int* stored;
+};
+
+// dst[e] = src[e] * mask[e] over `count` step-major elements (count % 4 == 0 is not required); src == nullptr writes the
+// mask itself.  to_batch_major != 0: dst is laid out (batch, steps, width) and e is translated (the mask as a caller
+// sees it beside y).
+__global__ void __launch_bounds__(256) rnn_dropout_kernel(float* dst, const float* src, long long count, RnnDropout d,
+                                                          int to_batch_major, int batch, int steps, int width) {
+    const long long chunks = (count + 3) / 4;
+    unsigned int k0 = (unsigned int)d.seed, k1 = (unsigned int)(d.seed >> 32), call = d.call;
+    if (d.stored != nullptr) k0 = d.stored[0], k1 = d.stored[1], call = d.stored[2];
+    for (long long c = (long long)blockIdx.x * 256 + threadIdx.x; c < chunks; c += (long long)gridDim.x * 256) {
+        const Philox4 r = philox4x32_10((unsigned int)c, (unsigned int)(c >> 32), d.boundary, call, k0, k1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const long long e = 4 * c + j;
+            if (e >= count) break;
+            const float u = (float)(r.v[j] >> 8) * (1.0f / 16777216.0f);
+            const float m = u < d.rate ? 0.0f : d.scale;
+            long long o = e;
+            if (to_batch_major) {
+                const long long row = e / width;  // step * batch + sample
+                const long long t = row / batch, b = row - t * batch;
+                o = (b * steps + t) * width + (e - row * width);
+            }
+            dst[o] = src == nullptr ? m : (m != 0.0f ? src[e] * m : 0.0f);
+        }
+    }
+}
+
 }  // namespace snhip

@@ -30,6 +30,9 @@ struct RnnDims {
     long long gates_off, hprev_off, cells_off, gh_off;   // inside a pseudo-layer's region
     long long out_off;                // start of the stacked layers' outputs, after all regions
     long long xt_off;                 // step-major copy of x
+    bool dropout;                     // units are dropped between the stacked layers in training
+    long long drop_off;               // the stacked layers' outputs after dropout (what the next layer reads), if any
+    long long rng_off;                // {seed low, seed high, call} of the forward call's masks, as three 32-bit words
     long long total;                  // floats carried from forward to backward
     long long rt_off;                 // inside the backward scratch: the transposed recurrent matrix of direction 0
     long long dir1_off;               // ... dh, dc and the transposed recurrent matrix of direction 1
@@ -48,11 +51,11 @@ int rnn_check_desc(const snhip_rnn_desc* d) {
     return SNHIP_STATUS_SUCCESS;
 }
 
-// cuDNN drops units of the outputs that feed the next stacked layer, in training only; that is not implemented, so
-// the one combination in which the rate would change results is refused rather than computed without dropout.
-bool rnn_dropout_would_apply(const snhip_rnn_desc* d, int training) {
-    return training != 0 && d->dropout > 0.0f && d->num_layers > 1;
-}
+// cuDNN drops units of the outputs that feed the next stacked layer (RNNDescriptor.dropoutRate, handed to
+// cudnnSetRNNDescriptor_v8 through GPUWrapper.DropoutDesc, Prod/GPU/GPUWrapper.cs:460-474), in training only; a single
+// layer has nothing to drop.  The buffers are sized from the descriptor alone, so an inference call with such a
+// descriptor reserves the room and does not use it.
+bool rnn_has_dropout(const snhip_rnn_desc* d) { return d->dropout > 0.0f && d->num_layers > 1; }
 
 RnnDims rnn_dims(const snhip_rnn_desc* d, int batch, int steps) {
     RnnDims r;
@@ -75,7 +78,10 @@ RnnDims rnn_dims(const snhip_rnn_desc* d, int batch, int steps) {
     r.per_p = r.gh_off + (r.cell == RNN_GRU ? r.n * 3 * r.H : 0);
     r.out_off = r.per_p * r.P;
     r.xt_off = r.out_off + (long long)(r.L - 1) * r.n * r.K * r.H;
-    r.total = r.xt_off + r.n * r.I;
+    r.dropout = rnn_has_dropout(d);
+    r.drop_off = r.xt_off + r.n * r.I;
+    r.rng_off = r.drop_off + (r.dropout ? (long long)(r.L - 1) * r.n * r.K * r.H : 0);
+    r.total = r.rng_off + (r.dropout ? 4 : 0);
     // dh, dc, one bias gradient, two buffers for the gradients that travel between stacked layers, and R^T
     r.rt_off = 2LL * batch * r.H + (long long)r.G * r.H + (r.L > 1 ? 2 * r.n * r.K * r.H : 0);
     r.dir1_off = r.rt_off + (long long)r.G * r.H * r.H;
@@ -123,6 +129,21 @@ int rnn_set_rows(Handle* h, float* dst, long long ld_dst, const float* src, long
     const long long total = (long long)rows * cols;
     hipLaunchKernelGGL(set_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, h->stream, dst, ld_dst, src,
                        ld_src, rows, cols);
+    return hip_to_status(hipGetLastError());
+}
+
+// dst = src * mask (src == nullptr: the mask itself) over the (steps, batch, dirs * hidden) activations behind layer
+// `boundary`; see rnn_dropout_kernel for how the mask is drawn.
+int rnn_apply_dropout(Handle* h, const RnnDims& r, float rate, float* dst, const float* src, int boundary,
+                      unsigned long long seed, unsigned int call, const unsigned int* stored, bool to_batch_major) {
+    const long long count = r.n * r.K * r.H;
+    RnnDropout d;
+    d.seed = seed, d.call = call, d.boundary = (unsigned int)boundary;
+    d.rate = rate, d.scale = 1.0f / (1.0f - rate);
+    d.stored = stored;
+    const long long blocks = ((count + 3) / 4 + 255) / 256;
+    hipLaunchKernelGGL(rnn_dropout_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536)), dim3(256), 0, h->stream, dst,
+                       src, count, d, to_batch_major ? 1 : 0, r.batch, r.steps, r.K * r.H);
     return hip_to_status(hipGetLastError());
 }
 
@@ -221,7 +242,6 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
     Handle* h = static_cast<Handle*>(handle);
     int st = rnn_check_desc(desc);
     if (st != SNHIP_STATUS_SUCCESS) return st;
-    if (rnn_dropout_would_apply(desc, training)) return SNHIP_STATUS_NOT_SUPPORTED;
     st = rnn_common_checks(h, desc, batch, steps);
     if (st != SNHIP_STATUS_SUCCESS) return st;
     if (batch == 0 || steps == 0) return SNHIP_STATUS_SUCCESS;
@@ -237,8 +257,25 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
     st = snhip_transpose_second_and_third_dimension(handle, x, keep + r.xt_off, 1, B, T, r.I);
     if (st != SNHIP_STATUS_SUCCESS) return st;
 
+    // dropout between the stacked layers, training only: this call's masks are numbered by the handle's count of such
+    // calls; seed and count go into the reserve buffer for the backward calls
+    const bool drop = training != 0 && r.dropout;
+    const unsigned long long seed = h->rnn_dropout_seed;
+    const unsigned int call = (unsigned int)h->rnn_dropout_calls;
+    if (drop) {
+        ++h->rnn_dropout_calls;
+        const unsigned int words[3] = {(unsigned int)seed, (unsigned int)(seed >> 32), call};
+        for (int i = 0; i < 3; ++i) {
+            hipLaunchKernelGGL(fill32_kernel, dim3(1), dim3(256), 0, h->stream,
+                               reinterpret_cast<unsigned int*>(keep + r.rng_off) + i, words[i], 1LL);
+            st = hip_to_status(hipGetLastError());
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
+    }
+
     for (int layer = 0; layer < r.L; ++layer) {
-        const float* inp = layer == 0 ? keep + r.xt_off : keep + r.out_off + (long long)(layer - 1) * r.n * KH;
+        const float* inp = layer == 0 ? keep + r.xt_off
+                                      : keep + (drop ? r.drop_off : r.out_off) + (long long)(layer - 1) * r.n * KH;
         const bool top = layer == r.L - 1;
         float* out = top ? y : keep + r.out_off + (long long)layer * r.n * KH;
         // rows of step t: the caller's y is batch-major, the stacked layers' outputs are step-major
@@ -326,6 +363,11 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
                 if (st != SNHIP_STATUS_SUCCESS) return st;
             }
         }
+        if (drop && !top) {  // what the next layer reads: this layer's outputs with units dropped
+            st = rnn_apply_dropout(h, r, desc->dropout, keep + r.drop_off + (long long)layer * r.n * KH, out, layer, seed, call,
+                                   nullptr, false);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
     }
     return SNHIP_STATUS_SUCCESS;
 }
@@ -355,6 +397,14 @@ int snhip_rnn_backward_data(void* handle, const snhip_rnn_desc* desc, int batch,
         const float* dout = top ? dy : between[layer & 1];
         const long long out_step = top ? KH : (long long)B * KH, out_ld = top ? (long long)T * KH : KH;
         float* dinp = layer == 0 ? dx : between[(layer - 1) & 1];
+        if (r.dropout && !top) {
+            // the layer above produced the gradient of what it read, this layer's outputs after dropout: the same
+            // mask (regenerated from the seed and call number the forward call left in reserve) takes it to the
+            // gradient of the outputs themselves
+            st = rnn_apply_dropout(h, r, desc->dropout, between[layer & 1], between[layer & 1], layer, 0, 0,
+                                   reinterpret_cast<const unsigned int*>(keep + r.rng_off), false);
+            if (st != SNHIP_STATUS_SUCCESS) return st;
+        }
         const long long I = rnn_layer_inputs(r, layer);
         struct Dir {
             RnnWeights w;
@@ -499,7 +549,8 @@ int snhip_rnn_backward_weights(void* handle, const snhip_rnn_desc* desc, int bat
     float* colsum = ws + 2LL * batch * H;
 
     for (int layer = 0; layer < r.L; ++layer) {
-        const float* inp = layer == 0 ? keep + r.xt_off : keep + r.out_off + (long long)(layer - 1) * r.n * K * H;
+        const float* inp = layer == 0 ? keep + r.xt_off
+                                      : keep + (r.dropout ? r.drop_off : r.out_off) + (long long)(layer - 1) * r.n * K * H;
         const long long I = rnn_layer_inputs(r, layer);
         for (int d = 0; d < K; ++d) {
             const int p = layer * K + d;
@@ -541,6 +592,34 @@ int snhip_rnn_backward_weights(void* handle, const snhip_rnn_desc* desc, int bat
         }
     }
     return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_rnn_set_dropout_seed(void* handle, unsigned long long seed) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    Handle* h = static_cast<Handle*>(handle);
+    h->rnn_dropout_seed = seed;
+    h->rnn_dropout_calls = 0;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_rnn_get_dropout_calls(void* handle, unsigned long long* calls) {
+    if (handle == nullptr) return SNHIP_STATUS_NOT_INITIALIZED;
+    if (calls == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    *calls = static_cast<Handle*>(handle)->rnn_dropout_calls;
+    return SNHIP_STATUS_SUCCESS;
+}
+
+int snhip_rnn_dropout_mask(void* handle, const snhip_rnn_desc* desc, int batch, int steps, unsigned long long call,
+                           int boundary, float* mask) {
+    Handle* h = static_cast<Handle*>(handle);
+    const int st = rnn_common_checks(h, desc, batch, steps);
+    if (st != SNHIP_STATUS_SUCCESS) return st;
+    if (boundary < 0 || boundary >= desc->num_layers - 1) return SNHIP_STATUS_INVALID_VALUE;
+    if (batch == 0 || steps == 0) return SNHIP_STATUS_SUCCESS;
+    if (mask == nullptr) return SNHIP_STATUS_INVALID_VALUE;
+    const RnnDims r = rnn_dims(desc, batch, steps);
+    return rnn_apply_dropout(h, r, desc->dropout, mask, nullptr, boundary, h->rnn_dropout_seed, (unsigned int)call, nullptr,
+                             true);
 }
 
 }  // extern "C"

@@ -68,6 +68,8 @@ struct Handle {
     int last_cfg = -1;
     int last_splitk = 0;
     int rnn_step_mode = 0;  // 0: recurrent forward steps as one launch when the shape allows, 1: always GEMM + cell kernel
+    unsigned long long rnn_dropout_seed = 0;   // the reference seeds cuDNN's dropout states with 0 (GPUWrapper.cs:472)
+    unsigned long long rnn_dropout_calls = 0;  // training-mode forward calls that drew masks so far
     float* static_scratch = nullptr;  // this device's copy of `scratch` (kStaticScratchBytes), never freed
     char last_error[192] = {0};       // text of the last refusal that has more to say than its status code
 };

@@ -190,6 +190,9 @@ SIGNATURES = {
     "snhip_rnn_temp_space_sizes": [ctypes.POINTER(RnnDesc), _i, _i, _i, ctypes.POINTER(_sz), ctypes.POINTER(_sz)],
     "snhip_rnn_forward": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz],
     "snhip_rnn_set_step_mode": [_vp, _i],
+    "snhip_rnn_set_dropout_seed": [_vp, ctypes.c_ulonglong],
+    "snhip_rnn_get_dropout_calls": [_vp, ctypes.POINTER(ctypes.c_ulonglong)],
+    "snhip_rnn_dropout_mask": [_vp, ctypes.POINTER(RnnDesc), _i, _i, ctypes.c_ulonglong, _i, _vp],
     "snhip_rnn_backward_data": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                 _vp, _sz, _vp, _sz],
     "snhip_rnn_backward_weights": [_vp, ctypes.POINTER(RnnDesc), _i, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz],

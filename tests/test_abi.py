@@ -70,7 +70,7 @@ def _csharp_prototypes():
             words = prm.split()
             if words[0] in ("ref", "out") or words[0] in ("IntPtr", "System.Text.StringBuilder"):
                 kinds.append("ptr")
-            elif words[0] == "long":
+            elif words[0] in ("long", "ulong"):
                 kinds.append("i64")
             elif words[0] in ("UIntPtr", "size_t"):
                 kinds.append("size")
@@ -182,9 +182,9 @@ def test_gemm_descriptor_layout_matches_the_library():
         hiplib.CublasStatus.CUBLAS_STATUS_INVALID_VALUE
 
 
-def test_rnn_dropout_is_refused_not_ignored():
-    """RNNDescriptor.dropoutRate (Prod/Layers/RNNDescriptor.cs:21) travels in snhip_rnn_desc; the one combination in
-    which cuDNN would apply it (training, more than one layer) is refused, everything else is unaffected by it."""
+def test_rnn_dropout_rate_is_validated():
+    """RNNDescriptor.dropoutRate (Prod/Layers/RNNDescriptor.cs:21) travels in snhip_rnn_desc: a rate inside [0, 1) passes
+    the descriptor check in every mode (the calls below then stop at the missing handle), anything else is refused."""
     import ctypes
     from sharpnet_amd import hiplib
     lib = hiplib.load_library()
@@ -194,10 +194,16 @@ def test_rnn_dropout_is_refused_not_ignored():
         return lib.snhip_rnn_forward(None, ctypes.byref(desc), training, 1, 1, None, None, None, None, None, None, None,
                                      None, 0, None, 0)
     d = hiplib.RnnDesc(cell_mode=2, bias_mode=2, num_layers=2, input_size=3, hidden_size=5, dropout=0.25)
-    assert fwd(d, 1) == S.CUBLAS_STATUS_NOT_SUPPORTED
-    assert fwd(d, 0) == S.CUBLAS_STATUS_NOT_INITIALIZED          # inference: no dropout, goes on to the handle check
+    assert fwd(d, 1) == S.CUBLAS_STATUS_NOT_INITIALIZED
+    assert fwd(d, 0) == S.CUBLAS_STATUS_NOT_INITIALIZED
     d1 = hiplib.RnnDesc(cell_mode=2, bias_mode=2, num_layers=1, input_size=3, hidden_size=5, dropout=0.25)
-    assert fwd(d1, 1) == S.CUBLAS_STATUS_NOT_INITIALIZED         # one layer: nothing to drop between layers
+    assert fwd(d1, 1) == S.CUBLAS_STATUS_NOT_INITIALIZED
+    # the reserve buffer grows by the dropped copies of the inter-layer activations (and the generator's position)
+    ws, rs, rs0 = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    d0 = hiplib.RnnDesc(cell_mode=2, bias_mode=2, num_layers=2, input_size=3, hidden_size=5, dropout=0.0)
+    assert lib.snhip_rnn_temp_space_sizes(ctypes.byref(d), 1, 4, 6, ctypes.byref(ws), ctypes.byref(rs)) == 0
+    assert lib.snhip_rnn_temp_space_sizes(ctypes.byref(d0), 1, 4, 6, ctypes.byref(ws), ctypes.byref(rs0)) == 0
+    assert rs.value == rs0.value + 4 * (4 * 6 * 5 + 4)
     for bad in (-0.1, 1.0, float("nan")):
         db = hiplib.RnnDesc(cell_mode=2, bias_mode=2, num_layers=2, input_size=3, hidden_size=5, dropout=bad)
         assert fwd(db, 0) == S.CUBLAS_STATUS_INVALID_VALUE

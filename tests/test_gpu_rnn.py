@@ -18,10 +18,10 @@ def T(w, a):
     return GPUTensor(list(a.shape), a, w)
 
 
-def lib_desc(desc):
+def lib_desc(desc, dropout=0.0):
     from sharpnet_amd.hiplib import RnnDesc
     return RnnDesc(cell_mode=desc.cell, bias_mode=desc.bias_mode, bidirectional=desc.bidirectional,
-                   num_layers=desc.num_layers, input_size=desc.input_size, hidden_size=desc.hidden_size)
+                   num_layers=desc.num_layers, input_size=desc.input_size, hidden_size=desc.hidden_size, dropout=dropout)
 
 
 def check(st, what):
@@ -29,10 +29,12 @@ def check(st, what):
     check_status(st, what)
 
 
-def run_gpu(w, desc, x, weights, dy, hx=None, cx=None, dhy=None, dcy=None, training=True, want_dstate=True):
-    """Forward (+ backward when training) through the C ABI; returns dict of numpy arrays."""
+def run_gpu(w, desc, x, weights, dy, hx=None, cx=None, dhy=None, dcy=None, training=True, want_dstate=True, dropout=0.0,
+            between=None):
+    """Forward (+ backward when training) through the C ABI; returns dict of numpy arrays.  between: called after the
+    forward call and before the backward ones (other work on the same handle)."""
     from sharpnet_amd import GPUTensor
-    lib, d = w.lib, lib_desc(desc)
+    lib, d = w.lib, lib_desc(desc, dropout)
     B, Tn, _ = x.shape
     H, K, P = desc.hidden_size, desc.dirs, desc.pseudo_layers
     ws, rs = ctypes.c_size_t(), ctypes.c_size_t()
@@ -55,6 +57,8 @@ def run_gpu(w, desc, x, weights, dy, hx=None, cx=None, dhy=None, dcy=None, train
     out = {"y": gy.ToNumpy(), "hy": ghy.ToNumpy(), "cy": gcy.ToNumpy()}
     if not training:
         return out
+    if between is not None:
+        between()
     gdy = T(w, dy)
     gdx = GPUTensor(list(x.shape), None, w)
     gdhx, gdcx = GPUTensor([P, B, H], None, w), GPUTensor([P, B, H], None, w)
@@ -74,8 +78,8 @@ def run_gpu(w, desc, x, weights, dy, hx=None, cx=None, dhy=None, dcy=None, train
     return out
 
 
-def compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, tol):
-    y, hy, cy, cache = ro.rnn_forward(desc, x, weights, hx, cx)
+def compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, tol, masks=None):
+    y, hy, cy, cache = ro.rnn_forward(desc, x, weights, hx, cx, masks=masks)
     assert np.max(np.abs(got["y"] - y)) <= tol, "y"
     assert np.max(np.abs(got["hy"] - hy)) <= tol, "hy"
     if desc.cell == ro.LSTM:
@@ -369,3 +373,94 @@ def test_encoder_decoder_pair(gpu_wrapper, cell):
     assert np.max(np.abs(dec._weightsAndBiasesGradients.ToNumpy() - dw2)) <= 5e-5 * max(1.0, float(np.max(np.abs(dw2))))
     assert np.max(np.abs(gdx1.ToNumpy() - dx1)) <= 5e-5 * max(1.0, float(np.max(np.abs(dx1))))
     assert np.max(np.abs(enc._weightsAndBiasesGradients.ToNumpy() - dw1)) <= 5e-5 * max(1.0, float(np.max(np.abs(dw1))))
+
+
+def dropout_calls(w):
+    n = ctypes.c_ulonglong()
+    check(w.lib.snhip_rnn_get_dropout_calls(w.handle, ctypes.byref(n)), "snhip_rnn_get_dropout_calls")
+    return n.value
+
+
+@pytest.mark.parametrize("batch,steps,hidden,bidirectional,layers", [(3, 5, 6, False, 2), (4, 3, 5, True, 3), (1, 1, 3, False, 2),
+                                                                     (7, 9, 33, True, 2)])
+def test_dropout_mask_is_the_documented_generator(gpu_wrapper, batch, steps, hidden, bidirectional, layers):
+    """snhip_rnn_dropout_mask against the oracle's restatement of the documented stream (Philox4x32-10, itself pinned
+    by the published known-answer vectors): bit for bit, for several seeds, call numbers and boundaries, element counts
+    that are and are not multiples of four."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    desc = ro.RnnDesc(ro.LSTM, input_size=4, hidden_size=hidden, num_layers=layers, bidirectional=bidirectional)
+    width = desc.dirs * hidden
+    out = GPUTensor([batch, steps, width], None, w)
+    try:
+        for seed, call, rate in [(0, 0, 0.5), (12345678901234567, 3, 0.2), (2 ** 63 + 5, 2 ** 32 - 1, 0.9)]:
+            check(w.lib.snhip_rnn_set_dropout_seed(w.handle, seed), "seed")
+            d = lib_desc(desc, rate)
+            for boundary in range(layers - 1):
+                out.SetValue(float("nan"))
+                check(w.lib.snhip_rnn_dropout_mask(w.handle, ctypes.byref(d), batch, steps, call, boundary, out.Pointer), "mask")
+                want = ro.dropout_mask(seed, call, boundary, rate, batch, steps, width)
+                assert np.array_equal(out.ToNumpy(), want), (seed, call, boundary)
+        d = lib_desc(desc, 0.5)
+        assert w.lib.snhip_rnn_dropout_mask(w.handle, ctypes.byref(d), batch, steps, 0, layers - 1, out.Pointer) == 7
+        assert w.lib.snhip_rnn_dropout_mask(w.handle, ctypes.byref(d), batch, steps, 0, -1, out.Pointer) == 7
+    finally:
+        check(w.lib.snhip_rnn_set_dropout_seed(w.handle, 0), "seed")
+        out.Dispose()
+
+
+@pytest.mark.parametrize("cell", [ro.TANH, ro.LSTM, ro.GRU])
+@pytest.mark.parametrize("bidirectional,layers,hidden", [(False, 2, 5), (True, 3, 4), (False, 3, 32), (True, 2, 36)])
+def test_dropout_between_stacked_layers(gpu_wrapper, cell, bidirectional, layers, hidden):
+    """Training with RNNDescriptor.dropoutRate > 0 and more than one layer: the call draws the masks numbered by the
+    handle's call count; with those masks (regenerated on the host from the documented stream) the oracle gives the same
+    outputs, final states and gradients.  The masks belong to the forward call: another layer's training call between
+    this layer's forward and backward calls changes nothing.  Inference ignores the rate; so does a repeat of the
+    call not ignore the count: the second call draws other masks."""
+    w = gpu_wrapper
+    rng = np.random.default_rng(5000 + cell * 37 + layers * 5 + hidden + int(bidirectional))
+    rate, seed = 0.35, 77
+    desc = ro.RnnDesc(cell, input_size=6, hidden_size=hidden, num_layers=layers, bidirectional=bidirectional)
+    B, Tn = 5, 7
+    width = desc.dirs * hidden
+    weights = rng.uniform(-0.5, 0.5, ro.weight_space_size(desc)).astype(np.float32)
+    x = rng.uniform(-1, 1, (B, Tn, 6)).astype(np.float32)
+    dy = rng.uniform(-1, 1, (B, Tn, width)).astype(np.float32)
+    st = lambda: rng.uniform(-1, 1, (desc.pseudo_layers, B, hidden)).astype(np.float32)
+    hx, cx, dhy, dcy = st(), st(), st(), st()
+    if cell != ro.LSTM:
+        cx = dcy = None
+    other = ro.RnnDesc(ro.GRU, input_size=3, hidden_size=4, num_layers=2)
+    other_w = rng.uniform(-0.5, 0.5, ro.weight_space_size(other)).astype(np.float32)
+
+    def another_layers_training_call():
+        run_gpu(w, other, rng.uniform(-1, 1, (2, 3, 3)).astype(np.float32), other_w,
+                rng.uniform(-1, 1, (2, 3, 4)).astype(np.float32), dropout=0.5)
+    try:
+        check(w.lib.snhip_rnn_set_dropout_seed(w.handle, seed), "seed")
+        assert dropout_calls(w) == 0
+        first = None
+        for call in range(2):
+            print("rnn dropout", cell, bidirectional, layers, hidden, "call", call, flush=True)
+            got = run_gpu(w, desc, x, weights, dy, hx, cx, dhy, dcy, dropout=rate,
+                          between=another_layers_training_call if call == 1 else None)
+            masks = [ro.dropout_mask(seed, call, b, rate, B, Tn, width) for b in range(layers - 1)]
+            compare(desc, got, x, weights, dy, hx, cx, dhy, dcy, 3e-5, masks=masks)
+            if first is None:
+                first = got
+            else:
+                assert np.max(np.abs(first["y"] - got["y"])) > 1e-4           # other masks
+        assert dropout_calls(w) == 3                                           # two calls here, one of the other layer
+        # the masks act: the result without dropout is another one; inference with the same descriptor is that one
+        plain = run_gpu(w, desc, x, weights, dy, hx, cx, dhy, dcy)
+        assert np.max(np.abs(plain["y"] - first["y"])) > 1e-4
+        infer = run_gpu(w, desc, x, weights, dy, hx, cx, training=False, dropout=rate)
+        assert np.array_equal(infer["y"], plain["y"]) and np.array_equal(infer["hy"], plain["hy"])
+        assert dropout_calls(w) == 3
+        # same seed, same call number: the same masks again
+        check(w.lib.snhip_rnn_set_dropout_seed(w.handle, seed), "seed")
+        again = run_gpu(w, desc, x, weights, dy, hx, cx, dhy, dcy, dropout=rate)
+        for k in ("y", "hy", "dx", "dw"):
+            assert np.array_equal(again[k], first[k]), k
+    finally:
+        check(w.lib.snhip_rnn_set_dropout_seed(w.handle, 0), "seed")
