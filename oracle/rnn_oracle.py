@@ -49,7 +49,9 @@ rnn_backward               cuDNN applies it in training            where they ac
                            seeded with 0, GPUWrapper.cs:460-474)   gradients through autograd (tests/test_oracle_rnn.py)
 philox4x32_10 /            the generator the library documents     the three known-answer vectors of the Random123
 dropout_mask               for its masks (cuDNN's own stream is    distribution (kat_vectors: zeros, all ones, digits of
-                           not reproducible)                       pi); the mask's layout by construction from them
+                           not reproducible: which units cuDNN     pi); the mask's layout by construction from them
+                           would drop is "parity unpinned", and
+                           no reference fixture uses a rate > 0)
 layer_forward /            RecurrentLayer.ForwardPropagation /     the same stored predictions and losses (last-step
 layer_backward             BackwardPropagation :305-520            outputs of uni- and bidirectional layers; a 2-layer
                            (returnSequences == false: last step    bidirectional sequence layer feeding a last-step
