@@ -559,14 +559,18 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
     const int row_w = __builtin_amdgcn_readfirstlane(row_base);
     const int col_w = __builtin_amdgcn_readfirstlane(col0);  // lane 0 owns the wavefront's first column
     const bool ws_or_c_vec = to_ws ? ((p.flags & GEMM_FLAG_WS_VEC) != 0) : ((p.flags & GEMM_FLAG_C_VEC) != 0);
-    if (ws_or_c_vec && row_w + 32 * TM <= p.M && col_w + 32 * TN <= p.N) {
-        float bv[TN];
+    // (... and so does a patch that only sticks out over the right edge, with the lanes beyond the edge switched
+    // off, when the width is a multiple of a lane's TN columns: a lane is then either wholly inside or wholly outside)
+    if (ws_or_c_vec && row_w + 32 * TM <= p.M && (col_w + 32 * TN <= p.N || p.N % TN == 0)) {
+        if (col0 + TN <= p.N) {
+            float bv[TN];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) bv[j] = 0.0f;
-        if (bias != nullptr) load_row_vec<TN>(bias + col0, bv);
-        store_patch_fast<TM, TN, false, PIN>(acc, out + (long long)(row_base + TM * 4 * lhi) * ldo + col0, ldo, nullptr, 0, alpha,
-                                        beta, 0.0f, bv, ACT_NONE, 0.0f);
-    } else {
+            for (int j = 0; j < TN; ++j) bv[j] = 0.0f;
+            if (bias != nullptr) load_row_vec<TN>(bias + col0, bv);
+            store_patch_fast<TM, TN, false, PIN>(acc, out + (long long)(row_base + TM * 4 * lhi) * ldo + col0, ldo, nullptr, 0,
+                                                 alpha, beta, 0.0f, bv, ACT_NONE, 0.0f);
+        }
+    } else if (row_w < p.M && col_w < p.N) {  // (a wavefront whose patch lies wholly outside the matrix writes nothing)
         float bv[TN];
 #pragma unroll
         for (int j = 0; j < TN; ++j) bv[j] = (bias != nullptr && col0 + j < p.N) ? bias[col0 + j] : 0.0f;
@@ -575,49 +579,62 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
 #pragma unroll
         for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bv[j]));
 
-        // Old values (beta != 0) are asked for four rows at a time, from addresses clamped into the matrix and outside
-        // the per-row conditions, before any of the four rows is stored: one wait per four rows instead of a
-        // load - wait - store round trip per row (the compiler may not move a load across the store of the row
-        // before it: for all it knows they alias).
+        // Two copies of the loop, chosen by a uniform branch: one for beta == 0 that contains no load at all, one
+        // that asks for the old values four rows at a time, from addresses clamped into the matrix and outside the
+        // per-row conditions, before any of the four rows is stored.  Stores count like loads in the memory wait
+        // counter, so wherever a load's result is awaited the stores issued before it are awaited too: with the load of
+        // the old value inside a row's own condition, or merely present under an `if (beta != 0)` that is not
+        // taken, a ragged right edge cost a store round trip per row (measured: 1.5 us for the 16 rows of a
+        // 64 x 64 tile, against 0.4 us for the branch-free write-out of a whole patch).
+        auto rows = [&](auto with_old) {
+        constexpr bool OLD = decltype(with_old)::value;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
             for (int rc = 0; rc < 4; ++rc) {
                 float cold[4][TN];
-                if (vec_ok && beta != 0.0f) {
+                if constexpr (OLD) {
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const int rq = row_base + TM * (8 * rc + 4 * lhi + q) + i;
-                        load_row_vec<TN>(out + (long long)(rq < p.M ? rq : p.M - 1) * ldo + col0, cold[q]);
+                        const float* src = out + (long long)(rq < p.M ? rq : p.M - 1) * ldo;
+                        if (vec_ok) {
+                            load_row_vec<TN>(src + col0, cold[q]);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) cold[q][j] = src[col0 + j < p.N ? col0 + j : p.N - 1];
+                        }
                     }
                 }
+                // (one address product per block of four rows; the rows of a block lie TM * ldo apart)
+                const int row0 = row_base + TM * (8 * rc + 4 * lhi) + i;
+                float* const crow0 = out + (long long)row0 * ldo + col0;
 #pragma unroll
                 for (int r = 4 * rc; r < 4 * rc + 4; ++r) {
-                    const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
-                    if (row >= p.M) continue;
-                    float* crow = out + (long long)row * ldo + col0;
+                    if (row0 + TM * (r % 4) >= p.M) continue;
+                    float* crow = crow0 + (long long)(TM * (r % 4)) * ldo;
                     float v[TN];
 #pragma unroll
                     for (int j = 0; j < TN; ++j) v[j] = alpha * acc_value<PIN>(acc[i][j][r]) + bv[j];
-                    if (vec_ok) {
-                        if (beta != 0.0f) {
+                    if constexpr (OLD) {
 #pragma unroll
-                            for (int j = 0; j < TN; ++j) v[j] += beta * cold[r % 4][j];
-                        }
+                        for (int j = 0; j < TN; ++j) v[j] += beta * cold[r % 4][j];
+                    }
+                    if (vec_ok) {
                         store_row_vec<TN>(crow, v);
                     } else {
 #pragma unroll
-                        for (int j = 0; j < TN; ++j) {
-                            if (col0 + j < p.N) {
-                                float o = v[j];
-                                if (beta != 0.0f) o += beta * crow[j];
-                                crow[j] = o;
-                            }
-                        }
+                        for (int j = 0; j < TN; ++j)
+                            if (col0 + j < p.N) crow[j] = v[j];
                     }
                 }
             }
         }
+        };  // rows
+        if (beta != 0.0f)  // uniform
+            rows(std::true_type{});
+        else
+            rows(std::false_type{});
     }
 
     if (!to_ws || p.counters == nullptr) return;
@@ -784,27 +801,77 @@ __device__ __forceinline__ void store_accumulators_ext(const f32x16 (&acc)[TM][T
     const int row_w = __builtin_amdgcn_readfirstlane(row_base);
     const int col_w = __builtin_amdgcn_readfirstlane(col0);  // lane 0 owns the wavefront's first column
     const bool ws_or_c_vec = to_ws ? ((p.flags & GEMM_FLAG_WS_VEC) != 0) : ((p.flags & GEMM_FLAG_C_VEC) != 0);
-    if (ws_or_c_vec && row_w + 32 * TM <= p.M && col_w + 32 * TN <= p.N) {
-        // the wavefront's patch lies inside the matrix: branch-free write-out
-        const long long first = (long long)(row_base + TM * 4 * lhi);
-        store_patch_fast<TM, TN, true>(acc, out + first * ldo + col0, ldo, has_d ? dsrc + first * ldd + col0 : nullptr, ldd,
-                                       alpha, beta, gamma, bv, act, p.ep.act_param);
-    } else {
+    if (ws_or_c_vec && row_w + 32 * TM <= p.M && (col_w + 32 * TN <= p.N || p.N % TN == 0)) {
+        // the wavefront's patch lies inside the matrix, or sticks out over the right edge only, with every lane wholly
+        // inside or wholly outside: branch-free write-out (lanes beyond the edge switched off)
+        if (col0 + TN <= p.N) {
+            const long long first = (long long)(row_base + TM * 4 * lhi);
+            store_patch_fast<TM, TN, true>(acc, out + first * ldo + col0, ldo, has_d ? dsrc + first * ldd + col0 : nullptr,
+                                           ldd, alpha, beta, gamma, bv, act, p.ep.act_param);
+        }
+    } else if (row_w < p.M && col_w < p.N) {  // (a wavefront whose patch lies wholly outside the matrix writes nothing)
+        // as in store_accumulators_plain: a copy of the loop without any load for beta == 0 and no addend, and one that
+        // asks for the old values of C and the addend four rows at a time, outside the per-row conditions and from
+        // addresses clamped into the matrix, so that no load stands between the stores
+        auto rows = [&](auto with_old) {
+        constexpr bool OLD = decltype(with_old)::value;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
-                if (row >= p.M) continue;
-                float v[TN];
+            for (int rc = 0; rc < 4; ++rc) {
+                float cold[4][TN], dold[4][TN];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) v[j] = alpha * acc_value<(TM * TN >= 16)>(acc[i][j][r]);
-                const float* drow = nullptr;
-                if (has_d) drow = dsrc + (long long)row * ldd + col0;
-                finish_row<TN>(v, out + (long long)row * ldo + col0, drow, has_d, bv, beta, gamma, act, p.ep.act_param,
-                               vec_ok, p.N - col0);
+                for (int q = 0; q < (OLD ? 4 : 0); ++q) {
+                    const int rq = row_base + TM * (8 * rc + 4 * lhi + q) + i;
+                    const long long rcl = rq < p.M ? rq : p.M - 1;
+                    if (beta != 0.0f) {  // uniform
+                        if (vec_ok) {
+                            load_row_vec<TN>(out + rcl * ldo + col0, cold[q]);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) cold[q][j] = out[rcl * ldo + (col0 + j < p.N ? col0 + j : p.N - 1)];
+                        }
+                    }
+                    if (has_d) {  // uniform
+                        if (vec_ok) {
+                            load_row_vec<TN>(dsrc + rcl * ldd + col0, dold[q]);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) dold[q][j] = dsrc[rcl * ldd + (col0 + j < p.N ? col0 + j : p.N - 1)];
+                        }
+                    }
+                }
+                const int row0 = row_base + TM * (8 * rc + 4 * lhi) + i;
+                float* const crow0 = out + (long long)row0 * ldo + col0;
+#pragma unroll
+                for (int r = 4 * rc; r < 4 * rc + 4; ++r) {
+                    if (row0 + TM * (r % 4) >= p.M) continue;
+                    float* crow = crow0 + (long long)(TM * (r % 4)) * ldo;
+                    float v[TN];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        v[j] = alpha * acc_value<(TM * TN >= 16)>(acc[i][j][r]) + bv[j];
+                        if constexpr (OLD) {
+                            if (beta != 0.0f) v[j] += beta * cold[r % 4][j];
+                            if (has_d) v[j] += gamma * dold[r % 4][j];
+                        }
+                        if (act != ACT_NONE) v[j] = leaky_relu(v[j], p.ep.act_param);
+                    }
+                    if (vec_ok) {
+                        store_row_vec<TN>(crow, v);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+                            if (col0 + j < p.N) crow[j] = v[j];
+                    }
+                }
             }
         }
+        };  // rows
+        if (beta != 0.0f || has_d)  // uniform
+            rows(std::true_type{});
+        else
+            rows(std::false_type{});
     }
 
     if (!to_ws) return;
