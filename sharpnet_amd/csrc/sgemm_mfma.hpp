@@ -529,7 +529,9 @@ __device__ __forceinline__ void store_patch_fast(const f32x16 (&acc)[TM][TN], fl
 // uses, and the extended one (also gamma * D, (leaky) ReLU, two-level batch) compiled only into the kernels
 // instantiated with EXT, so that the extra tests and registers cost the plain product nothing.
 // ---------------------------------------------------------------------------
-template <int TM, int TN, bool PIN = (TM * TN >= 16)>
+// LEAN: for callers that hold many registers across the call (the streaming kernels keep the next panel in flight):
+// the path for patches that stick out of the matrix then takes its compact form.
+template <int TM, int TN, bool PIN = (TM * TN >= 16), bool LEAN = false>
 __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM][TN], const GemmParams& p, int row_base,
                                                    int col0, int lhi, int zb, int batch, int tile_index,
                                                    long long c_offset = kNoBatchOffset) {
@@ -559,9 +561,18 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
     const int row_w = __builtin_amdgcn_readfirstlane(row_base);
     const int col_w = __builtin_amdgcn_readfirstlane(col0);  // lane 0 owns the wavefront's first column
     const bool ws_or_c_vec = to_ws ? ((p.flags & GEMM_FLAG_WS_VEC) != 0) : ((p.flags & GEMM_FLAG_C_VEC) != 0);
-    // (... and so does a patch that only sticks out over the right edge, with the lanes beyond the edge switched
-    // off, when the width is a multiple of a lane's TN columns: a lane is then either wholly inside or wholly outside)
-    if (ws_or_c_vec && row_w + 32 * TM <= p.M && (col_w + 32 * TN <= p.N || p.N % TN == 0)) {
+    if (ws_or_c_vec && row_w + 32 * TM <= p.M && col_w + 32 * TN <= p.N) {
+        float bv[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bv[j] = 0.0f;
+        if (bias != nullptr) load_row_vec<TN>(bias + col0, bv);
+        store_patch_fast<TM, TN, false, PIN>(acc, out + (long long)(row_base + TM * 4 * lhi) * ldo + col0, ldo, nullptr, 0, alpha,
+                                        beta, 0.0f, bv, ACT_NONE, 0.0f);
+    } else if (!LEAN && ws_or_c_vec && row_w + 32 * TM <= p.M && p.N % TN == 0) {
+        // A patch that only sticks out over the right edge of a matrix whose width is a multiple of a lane's TN
+        // columns (a lane is then wholly inside or wholly outside): the same write-out with the outside lanes switched
+        // off.  A copy of its own: under a lane condition the whole-patch case above measured 3 % slower on products
+        // without any edge (2048^3).
         if (col0 + TN <= p.N) {
             float bv[TN];
 #pragma unroll
@@ -569,6 +580,60 @@ __device__ __forceinline__ void store_accumulators_plain(const f32x16 (&acc)[TM]
             if (bias != nullptr) load_row_vec<TN>(bias + col0, bv);
             store_patch_fast<TM, TN, false, PIN>(acc, out + (long long)(row_base + TM * 4 * lhi) * ldo + col0, ldo, nullptr, 0,
                                                  alpha, beta, 0.0f, bv, ACT_NONE, 0.0f);
+        }
+    } else if constexpr (LEAN) {
+        // the compact form: old values asked for on the vector path only, element-wise stores with their loads inside
+        // the row's condition (a store round trip per row at a ragged right edge, few registers)
+        float bv[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bv[j] = (bias != nullptr && col0 + j < p.N) ? bias[col0 + j] : 0.0f;
+        // the bias values are needed (and waited for) here, on every path: otherwise each row's block below
+        // would wait for "a load that may still be pending" and with it for the previous row's store
+#pragma unroll
+        for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(bv[j]));
+
+        // Old values (beta != 0) are asked for four rows at a time, from addresses clamped into the matrix and outside
+        // the per-row conditions, before any of the four rows is stored: one wait per four rows instead of a
+        // load - wait - store round trip per row (the compiler may not move a load across the store of the row
+        // before it: for all it knows they alias).
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int rc = 0; rc < 4; ++rc) {
+                float cold[4][TN];
+                if (vec_ok && beta != 0.0f) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int rq = row_base + TM * (8 * rc + 4 * lhi + q) + i;
+                        load_row_vec<TN>(out + (long long)(rq < p.M ? rq : p.M - 1) * ldo + col0, cold[q]);
+                    }
+                }
+#pragma unroll
+                for (int r = 4 * rc; r < 4 * rc + 4; ++r) {
+                    const int row = row_base + TM * (8 * (r / 4) + 4 * lhi + (r % 4)) + i;
+                    if (row >= p.M) continue;
+                    float* crow = out + (long long)row * ldo + col0;
+                    float v[TN];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) v[j] = alpha * acc_value<PIN>(acc[i][j][r]) + bv[j];
+                    if (vec_ok) {
+                        if (beta != 0.0f) {
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) v[j] += beta * cold[r % 4][j];
+                        }
+                        store_row_vec<TN>(crow, v);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) {
+                            if (col0 + j < p.N) {
+                                float o = v[j];
+                                if (beta != 0.0f) o += beta * crow[j];
+                                crow[j] = o;
+                            }
+                        }
+                    }
+                }
+            }
         }
     } else if (row_w < p.M && col_w < p.N) {  // (a wavefront whose patch lies wholly outside the matrix writes nothing)
         float bv[TN];
@@ -801,9 +866,14 @@ __device__ __forceinline__ void store_accumulators_ext(const f32x16 (&acc)[TM][T
     const int row_w = __builtin_amdgcn_readfirstlane(row_base);
     const int col_w = __builtin_amdgcn_readfirstlane(col0);  // lane 0 owns the wavefront's first column
     const bool ws_or_c_vec = to_ws ? ((p.flags & GEMM_FLAG_WS_VEC) != 0) : ((p.flags & GEMM_FLAG_C_VEC) != 0);
-    if (ws_or_c_vec && row_w + 32 * TM <= p.M && (col_w + 32 * TN <= p.N || p.N % TN == 0)) {
-        // the wavefront's patch lies inside the matrix, or sticks out over the right edge only, with every lane wholly
-        // inside or wholly outside: branch-free write-out (lanes beyond the edge switched off)
+    if (ws_or_c_vec && row_w + 32 * TM <= p.M && col_w + 32 * TN <= p.N) {
+        // the wavefront's patch lies inside the matrix: branch-free write-out
+        const long long first = (long long)(row_base + TM * 4 * lhi);
+        store_patch_fast<TM, TN, true>(acc, out + first * ldo + col0, ldo, has_d ? dsrc + first * ldd + col0 : nullptr, ldd,
+                                       alpha, beta, gamma, bv, act, p.ep.act_param);
+    } else if (ws_or_c_vec && row_w + 32 * TM <= p.M && p.N % TN == 0) {
+        // it sticks out over the right edge only, with every lane wholly inside or wholly outside: the same write-out
+        // with the outside lanes switched off (a copy of its own, see store_accumulators_plain)
         if (col0 + TN <= p.N) {
             const long long first = (long long)(row_base + TM * 4 * lhi);
             store_patch_fast<TM, TN, true>(acc, out + first * ldo + col0, ldo, has_d ? dsrc + first * ldd + col0 : nullptr,

@@ -154,10 +154,10 @@ __global__ void __launch_bounds__(256, stream_occupancy(TN, BK_) - (TWO_LEVEL ? 
         }
         if (last_panel) {
             if constexpr (TWO_LEVEL)
-                store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
+                store_accumulators_plain<1, TN, false, true>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
                                                 batch_offset(split_batch(cur.z, p.batch_inner), p.strideC, p.strideC2));
             else
-                store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
+                store_accumulators_plain<1, TN, false, true>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -297,10 +297,10 @@ __global__ void __launch_bounds__(256, bstream_occupancy(sizeof(TIN)) - (TWO_LEV
         }
         if (last_panel) {
             if constexpr (TWO_LEVEL)
-                store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
+                store_accumulators_plain<1, TN, false, true>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0,
                                                 batch_offset(split_batch(cur.z, p.batch_inner), p.strideC, p.strideC2));
             else
-                store_accumulators_plain<1, TN>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
+                store_accumulators_plain<1, TN, false, true>(acc, p, cur.m0 + wave * 32, cur.n0 + TN * l32, lhi, cur.z, cur.z, 0);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
