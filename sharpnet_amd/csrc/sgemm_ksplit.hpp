@@ -118,6 +118,25 @@ __device__ __forceinline__ void ksplit_tile(const GemmParams& p, int tile_index,
     const float* Bb = p.B + (long long)z * p.strideB;
     float* Cb = p.C + (long long)z * p.strideC;
 
+    // What the write-out reads from memory - bias, old C, addend - is asked for here, in front of the k loop, for all
+    // of a thread's elements and from addresses clamped into the matrix: in a kernel that lasts a few microseconds the
+    // way of these values from memory would otherwise come on top of the operands' (the three conditions are uniform).
+    constexpr int Q = (16 * NT) / NW;
+    float bval[Q], cold[Q], dold[Q];
+    {
+        const int nbase = tile_n * (32 * NT);
+#pragma unroll
+        for (int q = 0; q < Q; ++q) {
+            const int e = threadIdx.x + (64 * NW) * q;
+            const int lr = e / (32 * NT), lc = e % (32 * NT);
+            const int row = m0 + lr < p.M ? m0 + lr : p.M - 1, col = nbase + lc < p.N ? nbase + lc : p.N - 1;
+            bval[q] = cold[q] = dold[q] = 0.0f;
+            if (p.ep.bias != nullptr) bval[q] = p.ep.bias[col];
+            if (p.beta != 0.0f) cold[q] = Cb[(long long)row * p.ldc + col];
+            if (p.ep.addend != nullptr) dold[q] = p.ep.addend[(long long)z * p.ep.strideD + (long long)row * p.ep.ldd + col];
+        }
+    }
+
     KsplitOperand<TA> oa;     // A transposed: stored K x M, contiguous along m
     KsplitOperand<!TB> ob;    // B not transposed: stored K x N, contiguous along n
     oa.init(Ab, p.lda, m0, p.M, lane);
@@ -213,7 +232,7 @@ __device__ __forceinline__ void ksplit_tile(const GemmParams& p, int tile_index,
 
     const int nbase = tile_n * (32 * NT);
 #pragma unroll
-    for (int q = 0; q < (16 * NT) / NW; ++q) {
+    for (int q = 0; q < Q; ++q) {
         const int e = threadIdx.x + (64 * NW) * q;
         const int lr = e / (32 * NT), lc = e % (32 * NT);
         const int row = m0 + lr, col = nbase + lc;
@@ -222,12 +241,11 @@ __device__ __forceinline__ void ksplit_tile(const GemmParams& p, int tile_index,
 #pragma unroll
         for (int k = 0; k < KS; ++k) v += part[k][lc / 32][lr][lc % 32];
         v *= p.alpha;
-        if (p.ep.bias != nullptr) v += p.ep.bias[col];
-        float* c = Cb + (long long)row * p.ldc + col;
-        if (p.beta != 0.0f) v += p.beta * *c;
-        if (p.ep.addend != nullptr) v += p.ep.gamma * p.ep.addend[(long long)z * p.ep.strideD + (long long)row * p.ep.ldd + col];
+        v += bval[q];
+        if (p.beta != 0.0f) v += p.beta * cold[q];
+        if (p.ep.addend != nullptr) v += p.ep.gamma * dold[q];
         if (p.ep.act == ACT_RELU || p.ep.act == ACT_LEAKY_RELU) v = leaky_relu(v, p.ep.act_param);
-        *c = v;
+        Cb[(long long)row * p.ldc + col] = v;
     }
 }
 
@@ -390,6 +408,16 @@ __global__ void __launch_bounds__(512) sgemm_ksplit16_kernel(const GemmParams p)
     const float* Bb = p.B + (long long)z * p.strideB;
     float* Cb = p.C + (long long)z * p.strideC;
 
+    // bias, old C and addend of this thread's element, asked for in front of the k loop (see ksplit_tile)
+    float bval = 0.0f, cold = 0.0f, dold = 0.0f;
+    if (threadIdx.x < 256) {
+        const int lr = threadIdx.x / 16, lc = threadIdx.x % 16;
+        const int row = m0 + lr < p.M ? m0 + lr : p.M - 1, col = n0 + lc < p.N ? n0 + lc : p.N - 1;
+        if (p.ep.bias != nullptr) bval = p.ep.bias[col];
+        if (p.beta != 0.0f) cold = Cb[(long long)row * p.ldc + col];
+        if (p.ep.addend != nullptr) dold = p.ep.addend[(long long)z * p.ep.strideD + (long long)row * p.ep.ldd + col];
+    }
+
     KsplitOperand16<TA> oa;
     KsplitOperand16<!TB> ob;
     oa.init(Ab, p.lda, m0, p.M, lane);
@@ -457,13 +485,11 @@ __global__ void __launch_bounds__(512) sgemm_ksplit16_kernel(const GemmParams p)
 #pragma unroll
             for (int k = 0; k < NW; ++k) v += part[k][lr][lc];
             v *= p.alpha;
-            if (p.ep.bias != nullptr) v += p.ep.bias[col];
-            float* c = Cb + (long long)row * p.ldc + col;
-            if (p.beta != 0.0f) v += p.beta * *c;
-            if (p.ep.addend != nullptr)
-                v += p.ep.gamma * p.ep.addend[(long long)z * p.ep.strideD + (long long)row * p.ep.ldd + col];
+            v += bval;
+            if (p.beta != 0.0f) v += p.beta * cold;
+            if (p.ep.addend != nullptr) v += p.ep.gamma * dold;
             if (p.ep.act == ACT_RELU || p.ep.act == ACT_LEAKY_RELU) v = leaky_relu(v, p.ep.act_param);
-            *c = v;
+            Cb[(long long)row * p.ldc + col] = v;
         }
     }
 }
