@@ -576,6 +576,11 @@ __device__ __host__ __forceinline__ Philox4 philox4x32_10(unsigned int c0, unsig
     return Philox4{{c0, c1, c2, c3}};
 }
 
+// {seed low word, seed high word, call} into a forward call's reserve buffer, for its backward calls
+__global__ void rnn_dropout_note_kernel(unsigned int* dst, unsigned int seed_lo, unsigned int seed_hi, unsigned int call) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) dst[0] = seed_lo, dst[1] = seed_hi, dst[2] = call;
+}
+
 struct RnnDropout {
     unsigned long long seed;
     unsigned int call, boundary;

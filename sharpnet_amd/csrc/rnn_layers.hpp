@@ -264,13 +264,10 @@ int snhip_rnn_forward(void* handle, const snhip_rnn_desc* desc, int training, in
     const unsigned int call = (unsigned int)h->rnn_dropout_calls;
     if (drop) {
         ++h->rnn_dropout_calls;
-        const unsigned int words[3] = {(unsigned int)seed, (unsigned int)(seed >> 32), call};
-        for (int i = 0; i < 3; ++i) {
-            hipLaunchKernelGGL(fill32_kernel, dim3(1), dim3(256), 0, h->stream,
-                               reinterpret_cast<unsigned int*>(keep + r.rng_off) + i, words[i], 1LL);
-            st = hip_to_status(hipGetLastError());
-            if (st != SNHIP_STATUS_SUCCESS) return st;
-        }
+        hipLaunchKernelGGL(rnn_dropout_note_kernel, dim3(1), dim3(64), 0, h->stream,
+                           reinterpret_cast<unsigned int*>(keep + r.rng_off), (unsigned int)seed, (unsigned int)(seed >> 32), call);
+        st = hip_to_status(hipGetLastError());
+        if (st != SNHIP_STATUS_SUCCESS) return st;
     }
 
     for (int layer = 0; layer < r.L; ++layer) {
