@@ -1212,10 +1212,15 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     // MODE 1: a full-k tile of an edge block (branch-free loads through the precomputed edge facts ea / eb);
     // MODE 2: the last tiles of an interior block (each fetch decides between unchecked loads and, at or past the
     //         end of K, checked ones);
+    // MODE 7: tile `fetch` is the tile of zeros that completes a pair of tiles (no loads: the stage is cleared);
     // MODE 3: the last tiles of an edge block (edge loads for full-k tiles, fully checked loads otherwise);
     // MODE 4: MODE 1 for a block none of whose vectors arrives shifted (M and N multiples of 4, or the operand is
     //         k-contiguous): plain LDS stores.  The element selects of the shifted store, executed for nothing, made
     //         the 64-wide-tile kernels VALU-bound in edge blocks (12 instructions per MFMA).
+    // MODE 5 / 6: the last tiles of an interior / edge block, when no tile that is still to be multiplied remains to be
+    //         fetched: the register stage is stored to LDS and not refilled.  Without any load in it the pair costs what
+    //         a pair of the main loop costs (1361 cycles with 64 x 64 tiles); as a pair of MODE 2, whose every slot
+    //         chooses between two kinds of load (of tiles beyond the end: zeros), it took 2361.
     // R: the register stage that holds the next tile (it is stored to LDS buffer P ^ 1 and refilled).
     auto k_tile = [&](auto parity, auto stage, auto mode, const typename StageA::Edge& ea,
                       const typename StageB::Edge& eb) {
@@ -1227,6 +1232,9 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         // the tail of an edge block: a full-k tile still takes the branch-free edge loads
         const bool edge_fast = (MODE == 3) && edge_ok && (fetch < nk_full);
         const int k_rem = klen - fetch * BK;
+        // The stage stored in this tile holds the tile after this one.  Behind the last tile there is none: the tiles
+        // that fetch nothing (MODE 5 / 6) left the stage as it was, and what it holds must not be summed again.
+        const bool sum_stored = (MODE != 5 && MODE != 6) || (fetch - NS < nk);
         const float* as = a_rd + P * (BK * PA);
         const float* bs = b_rd + P * (BK * PB);
         float* const as_next = As + Q * (BK * PA);
@@ -1274,14 +1282,22 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                             if (q < StageA::NV) {
                                 const int v = q < StageA::NV ? q : 0;
                                 if (is_store) {
-                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4) {
+                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4 || MODE == 5 || MODE == 7) {
                                         sa.store_lds_vec(as_next, ra[R][v], v);
-                                        if constexpr (COLSUM) cs += ra[R][v];
+                                        if constexpr (COLSUM) {
+                                            if (sum_stored) cs += ra[R][v];
+                                        }
                                     } else {
                                         const f32x4 stored =
                                             sa.store_lds_vec_shifted(as_next, ra[R][v], v, sh_a[R], any_rot_a);
-                                        if constexpr (COLSUM) cs += stored;
+                                        if constexpr (COLSUM) {
+                                            if (sum_stored) cs += stored;
+                                        }
                                     }
+                                } else if constexpr (MODE == 5 || MODE == 6) {
+                                    // nothing left to fetch
+                                } else if constexpr (MODE == 7) {
+                                    ra[R][v] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
                                 } else if (MODE == 1 || MODE == 4 || edge_fast)
                                     sa.load_edge_vec(ra[R][v], v, ea);
                                 else if (fast)
@@ -1291,12 +1307,15 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                             } else {
                                 const int v = q >= StageA::NV ? q - StageA::NV : 0;
                                 if (is_store) {
-                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4)
+                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4 || MODE == 5 || MODE == 7)
                                         sb.store_lds_vec(bs_next, rb[R][v], v);
                                     else
                                         sb.store_lds_vec_shifted(bs_next, rb[R][v], v, sh_b[R], any_rot_b);
-                                }
-                                else if (MODE == 1 || MODE == 4 || edge_fast)
+                                } else if constexpr (MODE == 5 || MODE == 6) {
+                                    // nothing left to fetch
+                                } else if constexpr (MODE == 7) {
+                                    rb[R][v] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                                } else if (MODE == 1 || MODE == 4 || edge_fast)
                                     sb.load_edge_vec(rb[R][v], v, eb);
                                 else if (fast)
                                     sb.load_fast_vec(rb[R][v], v);
@@ -1319,12 +1338,13 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
 
     // NS tiles in a row, starting at a tile index that is a multiple of NS (tile kt reads LDS buffer kt & 1, the
     // next tile sits in stage (kt + 1) % NS).  `limit`: tiles at or past it are skipped, in pairs (NS = 4 only).
-    auto tiles = [&](auto mode, int first, int limit) {
+    auto tiles = [&](auto mode, int first, int limit, auto mode_of_second) {
         using M = decltype(mode);
+        using M2 = decltype(mode_of_second);
         using I0 = std::integral_constant<int, 0>;
         using I1 = std::integral_constant<int, 1>;
         k_tile(I0{}, std::integral_constant<int, 1 % NS>{}, M{}, ea, eb);
-        k_tile(I1{}, std::integral_constant<int, 2 % NS>{}, M{}, ea, eb);
+        k_tile(I1{}, std::integral_constant<int, 2 % NS>{}, M2{}, ea, eb);
         if constexpr (NS == 4) {
             if (first + 2 >= limit) return;  // uniform
             k_tile(I0{}, std::integral_constant<int, 3>{}, M{}, ea, eb);
@@ -1332,6 +1352,15 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         }
     };
     constexpr int kNoLimit = 0x7fffffff;
+    // a pair of tiles fetches the tiles NS + 1 and NS + 2 ahead of its first one; the loop multiplies nk tiles rounded up
+    // to a whole pair: once the first of those fetches lies beyond that, nothing needs fetching any more
+    const int nk_even = nk + (nk & 1);
+    static_assert(NS == 2, "the tail loops are written for pairs of tiles");
+    // The 256 x 256 tiles, which use every register there is, keep one kind of pair for the whole tail (MODE 2 / 3): with
+    // more kinds of pair the compiler spilled 1.2 KB per lane there.  (For the smaller tiles, too, the kinds of pair are
+    // kept to a few ifs and loops in a row: chosen in nested branches, one case per shape of the end of K, they doubled
+    // the accumulator registers and halved the number of blocks per CU.)
+    constexpr bool SPLIT_TAIL = (TM * TN < 16);
     int kt = 0;
     // branch-free groups of NS tiles while all their fetches (tiles kt+NS+1 .. kt+2*NS) are full k tiles,
     // then the last few tiles (K tail included): same body, each fetch chooses checked or unchecked loads
@@ -1343,16 +1372,44 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         // ran at one memory latency per pair of tiles (64 x 64 tiles: 885 cycles per tile for 512 cycles of MFMAs).
         // With nothing in flight at the entry the counts are exact (all but the newest NS * NP - 1 loads).
         wait_for_all_loads();
-        for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 0>{}, kt, kNoLimit);
-        for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 2>{}, kt, nk);
+        for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 0>{}, kt, kNoLimit, std::integral_constant<int, 0>{});
+        if constexpr (SPLIT_TAIL) {
+            // The pairs whose fetches reach the end of K.  An even number of full tiles: the last tile is fetched by
+            // the first tile of a pair whose second tile fetches nothing.
+            if (kt + NS + 1 < nk_full && kt + 2 * NS >= nk_even) {
+                tiles(std::integral_constant<int, 0>{}, kt, kNoLimit, std::integral_constant<int, 5>{});
+                kt += NS;
+            }
+            // a partial tile at the end of K, fetched by the second tile of a pair (which chooses per fetch) ...
+            for (; kt + NS + 2 < nk; kt += NS) tiles(std::integral_constant<int, 2>{}, kt, nk, std::integral_constant<int, 2>{});
+            // ... or by the first tile of a pair
+            if (kt + NS + 1 < nk) {
+                tiles(std::integral_constant<int, 2>{}, kt, nk, std::integral_constant<int, 5>{});
+                kt += NS;
+            }
+            // an odd number of tiles: the tile of zeros that completes the last pair
+            if (kt + NS + 1 < nk_even) {
+                tiles(std::integral_constant<int, 7>{}, kt, nk, std::integral_constant<int, 5>{});
+                kt += NS;
+            }
+            // what is left has nothing to fetch
+            for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 5>{}, kt, nk, std::integral_constant<int, 5>{});
+        } else {
+            for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 2>{}, kt, nk, std::integral_constant<int, 2>{});
+        }
     } else {
         if (edge_ok && (any_rot_a || any_rot_b)) {  // uniform
-            for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 1>{}, kt, kNoLimit);
+            for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 1>{}, kt, kNoLimit, std::integral_constant<int, 1>{});
         } else if (edge_ok) {
             wait_for_all_loads();  // exact wait counts inside the loop, as for interior blocks
-            for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 4>{}, kt, kNoLimit);
+            for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 4>{}, kt, kNoLimit, std::integral_constant<int, 4>{});
         }
-        for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 3>{}, kt, nk);
+        if constexpr (SPLIT_TAIL) {
+            for (; kt + NS + 1 < nk_even; kt += NS) tiles(std::integral_constant<int, 3>{}, kt, nk, std::integral_constant<int, 3>{});
+            for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 6>{}, kt, nk, std::integral_constant<int, 6>{});
+        } else {
+            for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 3>{}, kt, nk, std::integral_constant<int, 3>{});
+        }
     }
     };  // run
     if (full_mn)

@@ -163,6 +163,40 @@ def test_bias_gradient_rides_along_with_dW_for_every_tile_configuration(oracle, 
         gc.GemmEx(transA=0, M=4, N=4, K=4, A=gdy, lda=4, B=gx, ldb=4, ldc=4, colsum=gcs)
 
 
+def test_every_shape_of_the_end_of_k_for_every_tile_configuration(oracle, gpu_wrapper):
+    """The last k tiles of a block are fetched by pairs of their own kind (a full tile and nothing, the partial tile,
+    the tile of zeros that completes a pair, nothing at all), chosen by how K ends: an even or odd number of k tiles
+    (of 16 or 32), the last one full or partial, and K shorter than the look-ahead.  Each shape of the end, for each
+    fp32 tile configuration, in blocks inside the matrix and at its edge (M, N = 300, 270), with the column sums that
+    ride on the staging of A (a stage that is stored twice would be summed twice)."""
+    from sharpnet_amd import GPUTensor
+    rng = np.random.default_rng(77)
+    w = gpu_wrapper
+    fp32_cfgs = [c["id"] for c in w.configs() if c["kind"] == "fp32"]
+    M, N = 300, 270
+    try:
+        for K in (5, 16, 33, 60, 64, 70, 80, 90, 96, 100, 128, 136, 150):
+            at = random_tensor(rng, (K, M), -1, 1)   # A read transposed: the dW form, the one that carries the sums
+            a = random_tensor(rng, (M, K), -1, 1)
+            b = random_tensor(rng, (K, N), -1, 1)
+            gat, ga, gb = T(w, at), T(w, a), T(w, b)
+            want_t = oracle.dot(at, True, b, False)
+            want_n = oracle.dot(a, False, b, False)
+            want_cs = at.astype(np.float64).sum(axis=0)
+            for cfg in fp32_cfgs:
+                w.set_tuning(cfg, 1)
+                gc = GPUTensor([M, N], None, w)
+                gcs = GPUTensor([1, M], None, w)
+                gcs.SetValue(float("nan"))
+                gc.GemmEx(transA=1, M=M, N=N, K=K, A=gat, lda=M, B=gb, ldb=N, ldc=N, colsum=gcs)
+                assert np.max(np.abs(gc.ToNumpy() - want_t)) <= bound(K, at, b, 1e-5), (cfg, K, "TN")
+                assert np.max(np.abs(gcs.ToNumpy()[0] - want_cs)) <= 1e-5 * np.sqrt(K) + 1e-6, (cfg, K)
+                gc.GemmEx(transA=0, M=M, N=N, K=K, A=ga, lda=K, B=gb, ldb=N, ldc=N)
+                assert np.max(np.abs(gc.ToNumpy() - want_n)) <= bound(K, a, b, 1e-5), (cfg, K, "NN")
+    finally:
+        w.set_tuning(-1, 0)
+
+
 @pytest.mark.parametrize("rows,in_f,out_f,with_db,wd", [(128, 784, 256, True, 1e-2), (36, 100, 64, False, 0.0),
                                                          (96, 132, 68, True, 0.5), (32, 32, 32, True, 0.0),
                                                          (64, 1000, 128, True, 0.0)])
