@@ -14,8 +14,8 @@ in HBM before the timed region.  Prints ONE JSON line on stdout:
   summary    a handful of figures of the other benchmark configurations.
 The line is strict JSON (no NaN tokens) and short (under 4000 characters): it is the LAST line of
 stdout.  The per-product figures of the other configurations (dense layer, sweep, MLP step, LSTM
-projections, attention matmuls, whole-layer calls) go to stderr and to --extra-out (a JSON file,
-default gpurun_out/bench_extra.json).  Every timed product is checked against the oracle on sampled
+projections, attention matmuls, whole-layer calls) go to stderr and to the JSON file that
+--extra-out names.  Every timed product is checked against the oracle on sampled
 rows of the timed result; a miss ends the run with an error.
 """
 import argparse
