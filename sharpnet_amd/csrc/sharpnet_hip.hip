@@ -157,16 +157,16 @@ constexpr ConfigEntry make_entry_bf16_stored(int occ, double eff_alone, double e
 // TM x TN MFMA tiles of 32x32, a workgroup is WM x WN wavefronts.
 const ConfigEntry kConfigs[] = {
     //                                      occ  alone shared edge
-    make_entry<TileCfg<4, 4, 2, 2, 16>>(1, 0.94, 0.94, 1.25),  // 0: 256 x 256
-    make_entry<TileCfg<2, 4, 2, 2, 16>>(1, 0.91, 0.91, 1.2),   // 1: 128 x 256
-    make_entry<TileCfg<4, 2, 2, 2, 16>>(1, 0.92, 0.92, 1.2),   // 2: 256 x 128
-    make_entry<TileCfg<2, 2, 2, 2, 16>>(2, 0.80, 0.87, 1.1),   // 3: 128 x 128
-    make_entry<TileCfg<1, 2, 2, 2, 16>>(3, 0.70, 0.82, 1.05),  // 4: 64 x 128
-    make_entry<TileCfg<2, 1, 2, 2, 16>>(3, 0.70, 0.82, 1.05),  // 5: 128 x 64
-    make_entry<TileCfg<1, 1, 2, 2, 16>>(5, 0.62, 0.75, 1.05),  // 6: 64 x 64
-    make_entry<TileCfg<2, 2, 2, 2, 32>>(1, 0.82, 0.86, 1.1),   // 7: 128 x 128, BK 32
-    make_entry<TileCfg<2, 1, 2, 2, 32>>(2, 0.72, 0.82, 1.05),  // 8: 128 x 64, BK 32
-    make_entry<TileCfg<1, 1, 2, 2, 32>>(4, 0.60, 0.75, 1.05),  // 9: 64 x 64, BK 32
+    make_entry<TileCfg<4, 4, 2, 2, 16>>(1, 0.990, 0.990, 1.25),  // 0: 256 x 256
+    make_entry<TileCfg<2, 4, 2, 2, 16>>(1, 0.948, 0.948, 1.2),   // 1: 128 x 256
+    make_entry<TileCfg<4, 2, 2, 2, 16>>(1, 0.949, 0.949, 1.2),   // 2: 256 x 128
+    make_entry<TileCfg<2, 2, 2, 2, 16>>(2, 0.897, 0.929, 1.1),   // 3: 128 x 128
+    make_entry<TileCfg<1, 2, 2, 2, 16>>(3, 0.861, 0.906, 1.05),  // 4: 64 x 128
+    make_entry<TileCfg<2, 1, 2, 2, 16>>(3, 0.786, 0.866, 1.05),  // 5: 128 x 64
+    make_entry<TileCfg<1, 1, 2, 2, 16>>(5, 0.758, 0.815, 1.05),  // 6: 64 x 64
+    make_entry<TileCfg<2, 2, 2, 2, 32>>(1, 0.953, 0.953, 1.1),   // 7: 128 x 128, BK 32
+    make_entry<TileCfg<2, 1, 2, 2, 32>>(2, 0.819, 0.878, 1.05),  // 8: 128 x 64, BK 32
+    make_entry<TileCfg<1, 1, 2, 2, 32>>(4, 0.757, 0.813, 1.05),  // 9: 64 x 64, BK 32
     // bf16-input kernels (fp32 operands in memory: bound by the L2 -> LDS path long before the MFMA rate)
     make_entry_bf16<BTileCfg<4, 4, 2, 2, 32>>(1, 0.80, 0.80, 4.0),   // 10: 256 x 256, BK 32
     make_entry_bf16<BTileCfg<2, 2, 2, 2, 32>>(2, 0.60, 0.75, 1.3),   // 11: 128 x 128, BK 32
@@ -339,16 +339,22 @@ struct Choice {
 //  - the per-tile critical path of a workgroup that has the CU to itself (LDS round trip + barrier);
 //  - HBM (unique operand bytes + C, plus the split-K partial sums);
 //  - the L2 -> LDS path (every workgroup re-reads its A and B panels), chip-wide and per CU.
-// Split-K adds a second launch that re-reads the partial sums.  Constants are fits to measurements on MI355X.
+// Split-K adds a second launch that re-reads the partial sums.  The constants (and the efficiencies in kConfigs) are a fit
+// to a sweep on MI355X: every fp32 tile configuration with K split 1, 2 and 4 ways on thirty shapes between 640^3 and
+// 4096^3 (squares, ragged ones, short and long K, tall ones); what the model picks there is within 1.7 % of the fastest
+// measured candidate (0.2 % on average; 9.7 % and 1.6 % with the hand-set constants before).
 double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int splitk, int num_cu) {
     constexpr double kTileLatency = 700.0;     // cycles per k tile when nothing hides the LDS/barrier latency
-    constexpr double kFixed = 5000.0;          // prologue + epilogue of one workgroup
+    constexpr double kFixed = 2290.0;          // prologue + epilogue of one workgroup
     constexpr double kStoreBytesPerCycle = 40; // C write-out rate of one CU
+    constexpr double kChipStoreBytesPerCycle = 1875;  // ... of all of them together (~4.5 TB/s)
     constexpr double kHbmBytesPerCycle = 2000; // ~4.8 TB/s streaming at 2.4 GHz (what a plain copy reaches)
     constexpr double kL2BytesPerCycle = 7000;  // ~17 TB/s aggregate L2 -> CU
     constexpr double kCuBytesPerCycle = 40;    // what one CU can pull from L2 into LDS
-    constexpr double kLaunch = 6000.0;
-    constexpr double kSplitFixed = 20000.0;    // second launch + dependency gap
+    constexpr double kLaunch = 1620.0;
+    constexpr double kSplitFixed = 8650.0;     // second launch + dependency gap
+    constexpr double kSplitPerPart = 500.0;    // what every further part costs beyond its bytes (384 x 384 x 3000: 16 parts
+                                               // 22.4 us, 4 parts 19.3 us)
     const long long tiles_mn = (long long)ceil_div(M, c.BM) * ceil_div(N, c.BN);
     const long long blocks = tiles_mn * batch * splitk;
     const long long per_cu = (blocks + num_cu - 1) / num_cu;
@@ -360,7 +366,15 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
     const double eff = resident >= 2 ? c.eff_shared : c.eff_alone;
     const bool has_edge = (M % c.BM != 0) || (N % c.BN != 0);
     const double edge = !has_edge ? 1.0 : (per_cu <= 2 ? c.edge_slow : 1.0 + (c.edge_slow - 1.0) * 0.15);
-    const double t_mfma = per_cu * nk * mfma_per_tile / eff * edge + kFixed;
+    // A configuration that never shares a compute unit writes every tile out with the matrix pipes idle, and when all
+    // units do so at once they share the chip's write rate: 256 x 256 tiles on 32768 x 2048 x 256 spend 17 of their
+    // 72 us per tile there (286 us; the 128 x 128 tiles, two workgroups per unit, 272 us).  (The write-out of the last
+    // tile of a unit is a cost every configuration has; it stays in kFixed.)
+    const long long writers = blocks < num_cu ? blocks : (long long)num_cu;
+    double store_rate = kChipStoreBytesPerCycle / (double)writers;
+    if (store_rate > kStoreBytesPerCycle) store_rate = kStoreBytesPerCycle;
+    const double t_store = c.occ == 1 ? per_cu * ((double)c.BM * c.BN * 4.0 / store_rate) : 0.0;
+    const double t_mfma = per_cu * nk * mfma_per_tile / eff * edge + t_store + kFixed;
     const double tile_alone = mfma_per_tile / c.eff_alone > kTileLatency ? mfma_per_tile / c.eff_alone : kTileLatency;
     const double t_lat = (double)((per_cu + c.occ - 1) / c.occ) *
                          (nk * tile_alone + kFixed + (double)c.BM * c.BN * 4.0 / kStoreBytesPerCycle);
@@ -378,7 +392,8 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
     const double padded = (double)ceil_div(M, c.BM) * c.BM * (double)ceil_div(N, c.BN) * c.BN / ((double)M * N);
     if (padded > 1.25) t *= padded / 1.25;
     t += kLaunch;
-    if (splitk > 1) t += kSplitFixed + (double)batch * M * N * (2.0 * splitk + 2.0) * 4.0 / kHbmBytesPerCycle;
+    if (splitk > 1)
+        t += kSplitFixed + kSplitPerPart * splitk + (double)batch * M * N * (2.0 * splitk + 2.0) * 4.0 / kHbmBytesPerCycle;
     return t;
 }
 
