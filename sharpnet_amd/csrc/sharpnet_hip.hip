@@ -400,7 +400,10 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
 // kind of kernel that serves a math mode: 0 fp32, 1 bf16-input on fp32 storage, 4 bf16-input on bf16 storage
 inline int kind_of_math(int math) { return math == SNHIP_MATH_BF16_STORED ? 4 : math; }
 
-Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
+// tA / tB: the form of the product.  The efficiencies in kConfigs were measured in the NN form; a product with both operands
+// transposed is the NN product of the transposed result, so an oblong tile then behaves like its mirror image
+// (1280^3 TT: 128 x 64 tiles 41.4 us, 64 x 128 tiles 45.6 us; NN: 44.6 and 41.3 us).  The mixed forms sit in between.
+Choice choose(const Handle* h, int M, int N, int K, int batch, int kind, bool tA = false, bool tB = false) {
     Choice best{kind == 0 ? 6 : (kind == 1 ? 13 : 20), 1};
     double best_cost = 1e300;
     const bool forced = h->force_cfg >= 0 && kConfigs[h->force_cfg].kind == kind;
@@ -429,7 +432,16 @@ Choice choose(const Handle* h, int M, int N, int K, int batch, int kind) {
                 const int kchunk = ceil_div(ceil_div(K, s), e.BK) * e.BK;
                 if ((long long)kchunk * (s - 1) >= K) continue;  // would leave an empty split
             }
-            const double cost = estimate_cycles(e, M, N, K, batch, s, h->num_cu);
+            double cost;
+            const int mirror = (c == 1 || c == 4) ? c + 1 : ((c == 2 || c == 5) ? c - 1 : c);
+            if (tA && tB && mirror != c) {
+                ConfigEntry m = e;
+                m.eff_alone = kConfigs[mirror].eff_alone;
+                m.eff_shared = kConfigs[mirror].eff_shared;
+                cost = estimate_cycles(m, M, N, K, batch, s, h->num_cu);
+            } else {
+                cost = estimate_cycles(e, M, N, K, batch, s, h->num_cu);
+            }
             if (cost < best_cost) {
                 best_cost = cost;
                 best = Choice{c, s};
@@ -841,7 +853,7 @@ int gemm_core(Handle* h, const GemmArgs& g) {
             return gemm_core(h, s);
         }
     }
-    Choice ch = choose(h, M, N, K, batch, kind_of_math(math));
+    Choice ch = choose(h, M, N, K, batch, kind_of_math(math), g.tA, g.tB);
     const int ks_cfg = prefer_ksplit(h, g, math, two_level);
     if (ks_cfg >= 0) ch = Choice{ks_cfg, 1};
     {
