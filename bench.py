@@ -124,9 +124,12 @@ def main():
     def upload(arr):
         return GPUTensor(arr.shape, arr, w)
 
-    def time_gemm(g, a, b, c, steps, warmup, bias=None, min_warm_ms=0.0):
+    def time_gemm(g, a, b, c, steps, warmup, bias=None, min_warm_ms=0.0, groups=1):
         """Returns (wall ms/step, event ms/launch, GPUTensor C, launches): C is what `launches` launches in a row
-        (warm-up included) made of the seeded C, so a product with beta = 1 still has a closed form."""
+        (warm-up included) made of the seeded C, so a product with beta = 1 still has a closed form.
+        groups > 1 (the short products of the other configurations): `steps` launches are timed that many times in a
+        row and the median group counts - the interval between two events includes whatever time the host took to
+        issue the launches, and one descheduled moment inside a window of 0.2 ms is a factor of ten."""
         ga, gb = upload(a), upload(b)
         gc = upload(c) if c is not None else GPUTensor(g.c_shape, None, w)
         gbias = upload(bias) if bias is not None else None
@@ -152,15 +155,18 @@ def main():
                     launch()
                 w.synchronize()
         e0, e1 = w.new_event(), w.new_event()
-        w.synchronize()
-        t0 = time.perf_counter()
-        w.record(e0)
-        for _ in range(steps):
-            launch()
-        w.record(e1)
-        w.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-        ev_ms = w.elapsed_ms(e0, e1) / steps
+        walls, evs = [], []
+        for _ in range(groups):
+            w.synchronize()
+            t0 = time.perf_counter()
+            w.record(e0)
+            for _ in range(steps):
+                launch()
+            w.record(e1)
+            w.synchronize()
+            walls.append((time.perf_counter() - t0) * 1e3 / steps)
+            evs.append(w.elapsed_ms(e0, e1) / steps)
+        wall_ms, ev_ms = float(np.median(walls)), float(np.median(evs))
         w.destroy_event(e0)
         w.destroy_event(e1)
         ga.Dispose()
@@ -544,7 +550,7 @@ def main():
 
         def run(gm, seed, steps=10, warmup=3, bias=None, cpu_reps=0):
             aa, bb, cc = wl.uniform_operands(gm, seed)
-            _, ms, gcx, count = time_gemm(gm, aa, bb, cc, steps, warmup, bias=bias, min_warm_ms=40.0)
+            _, ms, gcx, count = time_gemm(gm, aa, bb, cc, steps, warmup, bias=bias, min_warm_ms=40.0, groups=3)
             err, bound = check_timed_result(gm, aa, bb, cc, gcx.ToNumpy(), count, bias=bias, bf16=bf16_math[0])
             gcx.Dispose()
             tf = gm.flops / (ms * 1e-3) / 1e12
@@ -826,13 +832,16 @@ def layer_timings(w, wl):
         while n < warm or time.perf_counter() - t0 < 0.06:   # clocks take tens of ms to come up after an idle spell
             fn()
             n += 1
-        w.synchronize()
         e0, e1 = w.new_event(), w.new_event()
-        w.record(e0)
-        for _ in range(steps):
-            fn()
-        w.record(e1)
-        ms = w.elapsed_ms(e0, e1) / steps
+        groups = []
+        for _ in range(3):   # the median of three groups: one moment of the host elsewhere does not count
+            w.synchronize()
+            w.record(e0)
+            for _ in range(steps):
+                fn()
+            w.record(e1)
+            groups.append(w.elapsed_ms(e0, e1) / steps)
+        ms = float(np.median(groups))
         w.destroy_event(e0)
         w.destroy_event(e1)
         return round(ms, 4)
