@@ -279,5 +279,14 @@ def test_tile_choice_model_is_sane_without_gpu():
     c, s = ctypes.c_int(), ctypes.c_int()
     assert lib.snhip_query_tuning(None, 8192, 8192, 8192, 1, 0, ctypes.byref(c), ctypes.byref(s)) == 0
     assert (descs[c.value][0], descs[c.value][1], s.value) == (256, 256, 1)
+    # the benchmark's other fp32 shapes go where the sweep of every (configuration, split) pair found the fastest
+    # candidate on MI355X: (BM, BN, BK, split)
+    measured_best = {(4096, 4096, 4096): (256, 256, 16, 1), (1024, 1024, 1024): (64, 64, 32, 1),
+                     (1000, 1000, 1000): (64, 64, 16, 1), (4097, 3001, 2049): (64, 64, 16, 1),
+                     (8192, 64, 8192): (128, 64, 32, 4), (32768, 2048, 256): (128, 128, 16, 1),
+                     (4096, 3072, 4096): (128, 128, 16, 1), (1280, 1280, 1280): (64, 128, 16, 1)}
+    for (M, N, K), want in measured_best.items():
+        assert lib.snhip_query_tuning(None, M, N, K, 1, 0, ctypes.byref(c), ctypes.byref(s)) == 0
+        assert tuple(descs[c.value][:3]) + (s.value,) == want, (M, N, K, descs[c.value][:3], s.value)
     assert lib.snhip_query_tuning(None, 0, 8, 8, 1, 0, ctypes.byref(c), ctypes.byref(s)) == 7
     assert lib.snhip_query_tuning(None, 8, 8, 8, 1, 5, ctypes.byref(c), ctypes.byref(s)) == 7
