@@ -410,15 +410,19 @@ Choice choose(const Handle* h, int M, int N, int K, int batch, int kind, bool tA
     // A tall operand against a narrow one (N <= 64) with a long K streams op(A) from memory once: measured on
     // 8192 x 64 x 8192, all transposes, 128 x 64 tiles with 32-wide k panels (whole 128-byte lines of a k-contiguous
     // operand per row and tile) and one workgroup per compute unit (split 4) take 78-85 us, against 84-92 us for what the
-    // cost model picks (16-wide panels, split 8).
-    if (kind == 0 && !forced && h->force_splitk <= 0 && batch == 1 && N <= 64 && K >= 2048 &&
-        (long long)M * K >= (1LL << 24)) {
-        const ConfigEntry& e = kConfigs[8];
-        const long long tiles = (long long)ceil_div(M, e.BM) * ceil_div(N, e.BN);
-        int s = 1;
-        while (tiles * s < h->num_cu && s < 32 && K / (2 * s) >= 8 * e.BK) s *= 2;
-        const int kchunk = ceil_div(ceil_div(K, s), e.BK) * e.BK;
-        if ((long long)kchunk * (s - 1) < K && (size_t)M * N * s * sizeof(float) <= kMaxWorkspaceBytes) return Choice{8, s};
+    // cost model picks (16-wide panels, split 8).  The bf16 kinds likewise: the model sees the memory time of op(A) either
+    // way and does not split, but half a chip of workgroups does not pull it at that rate (bf16-input, 64 x 64 x 64
+    // tiles: 75.9 us unsplit, 51.7 us split in two).
+    if (!forced && h->force_splitk <= 0 && batch == 1 && N <= 64 && K >= 2048 && (long long)M * K >= (1LL << 24)) {
+        const int cfg = kind == 0 ? 8 : (kind == 1 ? 13 : (kind == 4 ? 20 : -1));
+        if (cfg >= 0) {
+            const ConfigEntry& e = kConfigs[cfg];
+            const long long tiles = (long long)ceil_div(M, e.BM) * ceil_div(N, e.BN);
+            int s = 1;
+            while (tiles * s < h->num_cu && s < 32 && K / (2 * s) >= 8 * e.BK) s *= 2;
+            const int kchunk = ceil_div(ceil_div(K, s), e.BK) * e.BK;
+            if ((long long)kchunk * (s - 1) < K && (size_t)M * N * s * sizeof(float) <= kMaxWorkspaceBytes) return Choice{cfg, s};
+        }
     }
     for (int c = 0; c < kNumConfigs; ++c) {
         const ConfigEntry& e = kConfigs[c];
