@@ -712,3 +712,64 @@ def test_attention_backward_in_bf16_input_mode(oracle, gpu_wrapper, B, H, Tq, Tk
     for name, g, ref in zip(("dS", "dV", "dQ", "dK"), got, (ds_ref, lay(dv_ref, Tk), lay(dq_ref, Tq), lay(dk_ref, Tk))):
         assert np.all(np.isfinite(g)), name
         assert np.max(np.abs(g - ref)) <= 1e-2 * float(np.max(np.abs(ref))), name
+
+
+@pytest.mark.parametrize("tA,tB", [(False, False), (True, True)])
+def test_tall_and_narrow_products_with_a_long_k_are_split_in_every_arithmetic(oracle, gpu_wrapper, tA, tB):
+    """A tall operand against a narrow one with a long K (4096 x 64 x 4096 and a ragged neighbour): the host splits K
+    over enough workgroups to fill the chip - in fp32, with bf16 MFMAs on fp32 operands and with operands stored as
+    bf16 - and the partial sums are added in index order by the reduction kernel.  Result against the oracle at the
+    bar of each arithmetic, twice (the same bits both times)."""
+    from sharpnet_amd import GPUTensor
+    from sharpnet_amd.hiplib import check_status
+    w = gpu_wrapper
+    lib, h = w.lib, w.handle
+    rng = np.random.default_rng(4242 + tA)
+    try:
+        for (M, N, K) in [(4096, 64, 4096), (4100, 50, 4104)]:
+            a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
+            b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
+            c = random_tensor(rng, (M, N), -1, 1)
+            ga, gb = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w)
+            # fp32
+            w.set_math_mode(w.MATH_FP32)
+            outs = []
+            for _ in range(2):
+                gc = GPUTensor([M, N], c, w)
+                gc.Dot(ga, tA, gb, tB, 0.5, 1.0)
+                outs.append(gc.ToNumpy())
+                gc.Dispose()
+            assert w.last_tuning()[1] > 1, w.last_tuning()
+            assert np.array_equal(outs[0], outs[1])
+            ref = oracle.dot(a, tA, b, tB, 0.5, 1.0, c)
+            assert np.max(np.abs(outs[0] - ref)) <= 1e-4 * np.sqrt(K) * 0.5 + 1e-6, (M, N, K)
+            # bf16 MFMAs on the fp32 operands
+            w.set_math_mode(w.MATH_BF16_INPUT)
+            outs = []
+            for _ in range(2):
+                gc = GPUTensor([M, N], c, w)
+                gc.Dot(ga, tA, gb, tB, 0.5, 1.0)
+                outs.append(gc.ToNumpy())
+                gc.Dispose()
+            assert w.last_tuning()[1] > 1, w.last_tuning()
+            assert np.array_equal(outs[0], outs[1])
+            check(oracle, outs[0], a, tA, b, tB, 0.5, 1.0, c, K)
+            w.set_math_mode(w.MATH_FP32)
+            # operands stored as bf16
+            pa, pb = to_bf16_on_device(w, ga), to_bf16_on_device(w, gb)
+            outs = []
+            for _ in range(2):
+                gc = GPUTensor([M, N], c, w)
+                check_status(lib.snhip_dot_bf16_stored(h, pa, a.shape[0], a.shape[1], int(tA), pb, b.shape[0], b.shape[1],
+                                                       int(tB), gc.Pointer, 0.5, 1.0, None))
+                outs.append(gc.ToNumpy())
+                gc.Dispose()
+            assert w.last_tuning()[1] > 1, w.last_tuning()
+            assert np.array_equal(outs[0], outs[1])
+            check(oracle, outs[0], a, tA, b, tB, 0.5, 1.0, c, K)
+            w.release(pa, max(2 * ga.Count, 8))
+            w.release(pb, max(2 * gb.Count, 8))
+            ga.Dispose()
+            gb.Dispose()
+    finally:
+        w.set_math_mode(w.MATH_FP32)
