@@ -413,7 +413,10 @@ Choice choose(const Handle* h, int M, int N, int K, int batch, int kind, bool tA
     // cost model picks (16-wide panels, split 8).  The bf16 kinds likewise: the model sees the memory time of op(A) either
     // way and does not split, but half a chip of workgroups does not pull it at that rate (bf16-input, 64 x 64 x 64
     // tiles: 75.9 us unsplit, 51.7 us split in two).
-    if (!forced && h->force_splitk <= 0 && batch == 1 && N <= 64 && K >= 2048 && (long long)M * K >= (1LL << 24)) {
+    // (When 64 x 64 tiles fill the chip without a split the cost model decides: 16384 x 64 x 4096 takes 74.5 us on them,
+    // 79.6 us on 128 x 64 tiles split in two.)
+    if (!forced && h->force_splitk <= 0 && batch == 1 && N <= 64 && K >= 2048 && (long long)M * K >= (1LL << 24) &&
+        (kind != 0 || (long long)ceil_div(M, 64) * ceil_div(N, 64) < h->num_cu)) {
         const int cfg = kind == 0 ? 8 : (kind == 1 ? 13 : (kind == 4 ? 20 : -1));
         if (cfg >= 0) {
             const ConfigEntry& e = kConfigs[cfg];
@@ -599,6 +602,13 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
     };
     if (!aligned(g.A, g.lda, g.sA, g.tA, g.M) || !aligned(g.B, g.ldb, g.sB, !g.tB, g.N)) return -1;
     if (forced) return h->force_cfg;
+    // A tall operand against one of 32 columns or fewer with a long K: 64-wide tiles would be half padding or more and
+    // need a second launch for their K splits; here the K slices meet inside the workgroup.  Measured: 16384 x 32 x 4096
+    // 61.4 us on 32 x 32 tiles against 75.2 (128 x 64 tiles, split 2), 8192 x 32 x 2048 18.4 against 26.1; on 16 x 16
+    // tiles 8192 x 16 x 8192 45.4 against 74.4, 8192 x 8 x 8192 46.2 against 73.6, 4096 x 32 x 4096 (too few 32 x 32 tiles
+    // for the chip) 22.9 against 26.6.
+    if (h->force_splitk <= 0 && g.batch == 1 && g.N <= 32 && g.K >= 2048 && (long long)g.M * g.K >= (1LL << 24))
+        return (g.N > 16 && ceil_div(g.M, 32) >= h->num_cu) ? kKsplitConfig : kKsplit16Config;
     if (h->force_splitk > 0 || g.K > 1024) return -1;
     // Measured on MI355X: 128 x 256 x 784 8.8 us against 12.8 (64 x 64 tiles, split-K 4 + reduction), 128 x 784 x 256
     // 5.5 against 10.5, 512^3 6.8 against 12.9; a loss when a wavefront's share of K gets long (256 x 256 x 4096:

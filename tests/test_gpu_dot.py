@@ -793,3 +793,34 @@ def test_streaming_kernels_walk_a_two_level_batch(oracle, gpu_wrapper, math, con
     finally:
         w.set_tuning(-1, 0)
         w.set_math_mode(0)
+
+
+@pytest.mark.parametrize("tA,tB", list(itertools.product([False, True], repeat=2)))
+def test_tall_products_with_few_columns_and_a_long_k(oracle, gpu_wrapper, tA, tB):
+    """A tall operand against one of 32 columns or fewer with a long K goes to the kernels that split K inside the
+    workgroup (no padding to 64 columns, no second launch): 32 x 32 tiles when those fill the chip, 16 x 16 tiles
+    otherwise.  Against the oracle, ragged sizes included, C prefilled with NaN for beta = 0."""
+    from sharpnet_amd import GPUTensor
+    w = gpu_wrapper
+    rng = np.random.default_rng(9000 + 2 * tA + tB)
+    kinds = {c["id"]: (c["kind"], c["BM"]) for c in w.configs()}
+    for (M, N, K, want_bm) in [(8192, 32, 2048, 32), (8200, 28, 2052, 32), (4096, 32, 4096, 16), (8192, 8, 2048, 16),
+                               (4100, 12, 4096, 16)]:
+        a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
+        b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
+        c = random_tensor(rng, (M, N), -1, 1)
+        ga, gb = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w)
+        for alpha, beta in ((1.0, 0.0), (0.5, 1.0)):
+            gc = GPUTensor([M, N], c if beta != 0 else None, w)
+            if beta == 0:
+                gc.SetValue(float("nan"))
+            gc.Dot(ga, tA, gb, tB, alpha, beta)
+            cfg, splitk = w.last_tuning()
+            aligned = (M % 4 == 0 or not tA) and (N % 4 == 0 or tB)      # 16-byte pieces along the contiguous direction
+            if aligned:
+                assert kinds[cfg] == ("fp32-ksplit", want_bm) and splitk == 1, (M, N, K, cfg, splitk)
+            ref = oracle.dot(a, tA, b, tB, alpha, beta, c if beta != 0 else None)
+            assert np.max(np.abs(gc.ToNumpy() - ref)) <= 1e-4 * np.sqrt(K) * abs(alpha) + 1e-6, (M, N, K, cfg)
+            gc.Dispose()
+        ga.Dispose()
+        gb.Dispose()
