@@ -609,6 +609,12 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
     // for the chip) 22.9 against 26.6.
     if (h->force_splitk <= 0 && g.batch == 1 && g.N <= 32 && g.K >= 2048 && (long long)g.M * g.K >= (1LL << 24))
         return (g.N > 16 && ceil_div(g.M, 32) >= h->num_cu) ? kKsplitConfig : kKsplit16Config;
+    // The mirror image, a wide operand under one of 32 rows or fewer: 32 x 32 tiles when they fill the chip (32 x 16384 x 4096
+    // 60.6 us against 76.3 on 64 x 128 tiles split in four, 16 x 8192 x 8192 57.0 against 77.9, 32 x 8192 x 2048 18.1
+    // against 25.1; the 16 x 16 tiles gain nothing on this side).
+    if (h->force_splitk <= 0 && g.batch == 1 && g.M <= 32 && g.K >= 2048 && (long long)g.N * g.K >= (1LL << 24) &&
+        ceil_div(g.N, 32) >= h->num_cu)
+        return kKsplitConfig;
     if (h->force_splitk > 0 || g.K > 1024) return -1;
     // Measured on MI355X: 128 x 256 x 784 8.8 us against 12.8 (64 x 64 tiles, split-K 4 + reduction), 128 x 784 x 256
     // 5.5 against 10.5, 512^3 6.8 against 12.9; a loss when a wavefront's share of K gets long (256 x 256 x 4096:

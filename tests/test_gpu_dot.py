@@ -799,13 +799,14 @@ def test_streaming_kernels_walk_a_two_level_batch(oracle, gpu_wrapper, math, con
 def test_tall_products_with_few_columns_and_a_long_k(oracle, gpu_wrapper, tA, tB):
     """A tall operand against one of 32 columns or fewer with a long K goes to the kernels that split K inside the
     workgroup (no padding to 64 columns, no second launch): 32 x 32 tiles when those fill the chip, 16 x 16 tiles
-    otherwise.  Against the oracle, ragged sizes included, C prefilled with NaN for beta = 0."""
+    otherwise; likewise a wide operand under 32 rows or fewer (32 x 32 tiles).  Against the oracle, ragged sizes
+    included, C prefilled with NaN for beta = 0."""
     from sharpnet_amd import GPUTensor
     w = gpu_wrapper
     rng = np.random.default_rng(9000 + 2 * tA + tB)
     kinds = {c["id"]: (c["kind"], c["BM"]) for c in w.configs()}
     for (M, N, K, want_bm) in [(8192, 32, 2048, 32), (8200, 28, 2052, 32), (4096, 32, 4096, 16), (8192, 8, 2048, 16),
-                               (4100, 12, 4096, 16)]:
+                               (4100, 12, 4096, 16), (32, 8192, 2048, 32), (12, 8200, 2052, 32)]:
         a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
         b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
         c = random_tensor(rng, (M, N), -1, 1)
