@@ -618,15 +618,19 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
     if (h->force_splitk > 0 || g.K > 1024) return -1;
     // Measured on MI355X: 128 x 256 x 784 8.8 us against 12.8 (64 x 64 tiles, split-K 4 + reduction), 128 x 784 x 256
     // 5.5 against 10.5, 512^3 6.8 against 12.9; a loss when a wavefront's share of K gets long (256 x 256 x 4096:
-    // 30.5 against 17.2 with split-K 16).  Up to one 32 x 32 tile per compute unit: four K slices; up to one
-    // 32 x 64 tile per compute unit: two.
+    // 30.5 against 17.2 with split-K 16).  Up to one 32 x 32 tile per compute unit: four K slices.
     const long long rows32 = (long long)ceil_div(g.M, 32) * g.batch;
     // 32 x 32 tiles for a quarter of the compute units or fewer, and a K that gives eight wavefronts a few groups of 32
     // each: 16 x 16 tiles, four times the workgroups (128 x 256 x 784: 5.4 us against 8.7 with eight wavefronts on
     // 32 x 32 tiles, 64 x 128 x 1024: 5.4 against 9.1, 128 x 128 x 512: 5.4 against 6.0)
+    // (and up to half of them with a K of 768 or more: 256 x 512 x 1024 8.0 against 10.5 us, 512 x 256 x 768 6.7 against 8.9)
     if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 4 && g.K >= 512) return kKsplit16Config;
+    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 2 && g.K >= 768) return kKsplit16Config;
     if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu) return kKsplitConfig;
-    if (rows32 * ceil_div(g.N, 64) <= (long long)h->num_cu) return kKsplitConfig + 1;
+    // (Up to one 32 x 64 tile per compute unit - two K slices, configuration 15 - used to go here too; since the tail of
+    // the tiled kernels' k loop was shortened the 64 x 64 tiles are ahead on all of those: 512 x 1024 x 256 7.0 against
+    // 8.2 us, 32 x (128 x 128 x 1024) 16.3 against 20.6 us, 256 x 2048 x 512 11.0 against 11.6 us.  The configuration
+    // stays reachable through snhip_set_tuning.)
     return -1;
 }
 

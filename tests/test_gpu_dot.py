@@ -621,15 +621,18 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
         assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, tA, b, tB, 0.5))) <= tol(K, a, b, 0.5)
         gpu_wrapper.set_tuning(-1, 0)
         # automatic choice: the forward product of benchmark configuration 1's Dense layer (32 tiles of 32 x 32: the
-        # 16 x 16-tile kernel), a square product of one 32 x 32 tile per CU, a recurrent step (one 32 x 64 tile per
-        # CU), the layer's dx
+        # 16 x 16-tile kernel), a square product of one 32 x 32 tile per CU, half as many tiles with a long K (16 x 16
+        # tiles again), the layer's dx; a recurrent step (two 32 x 32 tiles per CU) is left to the tiled kernels
         assert len(ks_all) == 4
-        for (M, N, K, want) in [(128, 256, 784, ks_all[3]), (512, 512, 512, ks_all[0]), (256, 2048, 512, ks_all[1]),
-                                (128, 784, 256, ks_all[0])]:
+        for (M, N, K, want) in [(128, 256, 784, ks_all[3]), (512, 512, 512, ks_all[0]), (256, 512, 1024, ks_all[3]),
+                                (128, 784, 256, ks_all[0]), (256, 2048, 512, None)]:
             a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
             b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
             got = gpu_dot(gpu_wrapper, a, tA, b, tB, 1.0, 0.0, c_shape=[M, N], prefill=float("nan"))
-            assert gpu_wrapper.last_tuning() == (want, 1)
+            if want is None:
+                assert gpu_wrapper.last_tuning()[0] not in ks_all
+            else:
+                assert gpu_wrapper.last_tuning() == (want, 1)
             assert np.max(np.abs(got - oracle.dot(a, tA, b, tB))) <= tol(K, a, b)
         # an operand view at an odd element offset cannot be read in 16-byte pieces: another kernel takes over
         big = GPUTensor([128 * 784 + 1], None, gpu_wrapper)
