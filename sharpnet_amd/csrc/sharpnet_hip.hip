@@ -374,7 +374,9 @@ double estimate_cycles(const ConfigEntry& c, int M, int N, int K, int batch, int
     double store_rate = kChipStoreBytesPerCycle / (double)writers;
     if (store_rate > kStoreBytesPerCycle) store_rate = kStoreBytesPerCycle;
     const double t_store = c.occ == 1 ? per_cu * ((double)c.BM * c.BN * 4.0 / store_rate) : 0.0;
-    const double t_mfma = per_cu * nk * mfma_per_tile / eff * edge + t_store + kFixed;
+    // (the last tile of a unit goes out with nothing left to hide it behind, whatever the configuration)
+    const double t_mfma =
+        per_cu * nk * mfma_per_tile / eff * edge + t_store + kFixed + (double)c.BM * c.BN * 4.0 / kStoreBytesPerCycle;
     const double tile_alone = mfma_per_tile / c.eff_alone > kTileLatency ? mfma_per_tile / c.eff_alone : kTileLatency;
     const double t_lat = (double)((per_cu + c.occ - 1) / c.occ) *
                          (nk * tile_alone + kFixed + (double)c.BM * c.BN * 4.0 / kStoreBytesPerCycle);
@@ -646,7 +648,10 @@ int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, 
     if (h->force_cfg >= 0 && !forced) return -1;
     if (h->force_splitk > 1) return -1;
     if (forced) return h->force_cfg;
-    if (g.batch < 8 || g.K > 256 || g.M < 64) return -1;
+    // (fp32: K up to 128 - with 192 and 256 the tiled kernels are level or ahead: 128 x (384 x 384 x 256) 81 against 91 us,
+    // 64 x (512 x 512 x 192) 57 against 60 us, 512 x (256 x 256 x 256) 154 against 151 us.  The bf16 kinds, whose MFMA
+    // time is an eighth, stay streaming up to 256: the probabilities-times-values product of an attention layer.)
+    if (g.batch < 8 || g.K > (math == SNHIP_MATH_FP32 ? 128 : 256) || g.M < 64) return -1;
     const int cfg = g.N <= 64 ? first + 1 : first;
     const long long tiles = (long long)ceil_div(g.M, 128) * ceil_div(g.N, kConfigs[cfg].BN) * g.batch;
     if (tiles < 2LL * h->num_cu) return -1;

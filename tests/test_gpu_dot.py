@@ -682,14 +682,20 @@ def test_streaming_kernel_strided_batches(oracle, gpu_wrapper, tA, tB):
             ga.Dispose()
             gb.Dispose()
         w.set_tuning(-1, 0)
-        # automatic choice: the two attention products of benchmark configuration 5 (fewer matrices, same shape)
-        for (batch, M, N, K, want) in [(256, 256, 256, 64, st_all[0]), (256, 256, 64, 256, st_all[1])]:
+        # automatic choice: the two attention products of benchmark configuration 5 (fewer matrices, same shape) - the
+        # scores (K = 64) stream, the probabilities-times-values product (K = 256) is a few percent faster on the tiled
+        # kernels in fp32 - and a K = 128 product with 64 columns
+        for (batch, M, N, K, want) in [(256, 256, 256, 64, st_all[0]), (256, 256, 64, 256, None),
+                                       (256, 256, 64, 128, st_all[1])]:
             a = random_tensor(rng, (batch, K, M) if tA else (batch, M, K), -1, 1)
             b = random_tensor(rng, (batch, N, K) if tB else (batch, K, N), -1, 1)
             ga, gb, gc = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w), GPUTensor([batch, M, N], None, w)
             gc.SetValue(float("nan"))
             gc.BatchMatrixMultiplication(ga, tA, gb, tB, 1.0, 0.0)
-            assert w.last_tuning() == (want, 1)
+            if want is None:
+                assert w.last_tuning()[0] not in st_all
+            else:
+                assert w.last_tuning() == (want, 1)
             assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, tA, b, tB, 1.0))) <= tol(K, a, b)
             for t in (ga, gb, gc):
                 t.Dispose()
