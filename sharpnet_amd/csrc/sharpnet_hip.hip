@@ -625,9 +625,14 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
     // 32 x 32 tiles for a quarter of the compute units or fewer, and a K that gives eight wavefronts a few groups of 32
     // each: 16 x 16 tiles, four times the workgroups (128 x 256 x 784: 5.4 us against 8.7 with eight wavefronts on
     // 32 x 32 tiles, 64 x 128 x 1024: 5.4 against 9.1, 128 x 128 x 512: 5.4 against 6.0)
-    // (and up to half of them with a K of 768 or more: 256 x 512 x 1024 8.0 against 10.5 us, 512 x 256 x 768 6.7 against 8.9)
+    // (and up to half of them with a K of 256 or more: 256 x 512 x 1024 8.0 against 10.5 us, 512 x 256 x 768 6.7 against 8.9,
+    // 320 x 320 x 512 5.1 against 7.2, 300^3 4.9 against 6.2, 512 x 256 x 256 4.9 against 5.2)
     if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 4 && g.K >= 512) return kKsplit16Config;
-    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 2 && g.K >= 768) return kKsplit16Config;
+    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 2 && g.K >= 256) return kKsplit16Config;
+    // Between half a chip and a whole chip of 32 x 32 tiles, with a K of 384 or more: eight K slices (two wavefronts per
+    // SIMD) instead of four - 512 x 384 x 512 6.1 against 7.2 us, 384 x 384 x 768 7.7 against 8.9, 512 x 512 x 768 8.0
+    // against 9.1, 400 x 400 x 640 7.7 against 8.1.
+    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu && g.K >= 384 && !multi) return kKsplit8Config;
     if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu) return kKsplitConfig;
     // (Up to one 32 x 64 tile per compute unit - two K slices, configuration 15 - used to go here too; since the tail of
     // the tiled kernels' k loop was shortened the 64 x 64 tiles are ahead on all of those: 512 x 1024 x 256 7.0 against
@@ -1178,8 +1183,16 @@ int dense_backward_small(Handle* h, float* dx, float* dW, float* db, const float
     GemmArgs gx;  // dx = dy . W
     gx.M = rows, gx.N = in_features, gx.K = out_features;
     gx.A = dy, gx.lda = out_features, gx.B = W, gx.ldb = in_features, gx.C = dx, gx.ldc = in_features;
-    if (prefer_ksplit(h, gw, SNHIP_MATH_FP32, false) != kKsplitConfig) return kNotTaken;
-    if (prefer_ksplit(h, gx, SNHIP_MATH_FP32, false) != kKsplitConfig) return kNotTaken;
+    // each product: one the K-split kernels take (alignment, K), with at most one 32 x 32 tile per compute unit and not so
+    // few of them that a long K is better cut eight ways on 16 x 16 tiles
+    auto qualifies = [&](const GemmArgs& g) {
+        const int c = prefer_ksplit(h, g, SNHIP_MATH_FP32, false);
+        if (c != kKsplitConfig && c != kKsplit8Config && c != kKsplit16Config) return false;
+        const long long tiles = (long long)ceil_div(g.M, 32) * ceil_div(g.N, 32);
+        if (g.K > 1024 || tiles > h->num_cu) return false;
+        return !(tiles <= h->num_cu / 4 && g.K >= 512);
+    };
+    if (!qualifies(gw) || !qualifies(gx)) return kNotTaken;
     {
         int cur = -1;
         if (hipGetDevice(&cur) != hipSuccess) return SNHIP_STATUS_NOT_INITIALIZED;

@@ -621,11 +621,13 @@ def test_k_split_inside_the_workgroup(oracle, gpu_wrapper, tA, tB):
         assert np.max(np.abs(gc.ToNumpy() - oracle.bmm(a, tA, b, tB, 0.5))) <= tol(K, a, b, 0.5)
         gpu_wrapper.set_tuning(-1, 0)
         # automatic choice: the forward product of benchmark configuration 1's Dense layer (32 tiles of 32 x 32: the
-        # 16 x 16-tile kernel), a square product of one 32 x 32 tile per CU, half as many tiles with a long K (16 x 16
-        # tiles again), the layer's dx; a recurrent step (two 32 x 32 tiles per CU) is left to the tiled kernels
+        # 16 x 16-tile kernel), a square product of one 32 x 32 tile per CU (eight K slices; four with a short K), half
+        # as many tiles (16 x 16 tiles again), the layer's dx (100 tiles: 16 x 16) and dW (200 tiles, K = 128: four
+        # slices); a recurrent step (two 32 x 32 tiles per CU) is left to the tiled kernels
         assert len(ks_all) == 4
-        for (M, N, K, want) in [(128, 256, 784, ks_all[3]), (512, 512, 512, ks_all[0]), (256, 512, 1024, ks_all[3]),
-                                (128, 784, 256, ks_all[0]), (256, 2048, 512, None)]:
+        for (M, N, K, want) in [(128, 256, 784, ks_all[3]), (512, 512, 512, ks_all[2]), (512, 512, 256, ks_all[0]),
+                                (256, 512, 1024, ks_all[3]), (128, 784, 256, ks_all[3]), (256, 784, 128, ks_all[0]),
+                                (256, 2048, 512, None)]:
             a = random_tensor(rng, (K, M) if tA else (M, K), -1, 1)
             b = random_tensor(rng, (N, K) if tB else (K, N), -1, 1)
             got = gpu_dot(gpu_wrapper, a, tA, b, tB, 1.0, 0.0, c_shape=[M, N], prefill=float("nan"))
