@@ -628,11 +628,16 @@ int prefer_ksplit(const Handle* h, const GemmArgs& g, int math, bool two_level) 
     // (and up to half of them with a K of 256 or more: 256 x 512 x 1024 8.0 against 10.5 us, 512 x 256 x 768 6.7 against 8.9,
     // 320 x 320 x 512 5.1 against 7.2, 300^3 4.9 against 6.2, 512 x 256 x 256 4.9 against 5.2)
     if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 4 && g.K >= 512) return kKsplit16Config;
-    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 2 && g.K >= 256) return kKsplit16Config;
+    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu / 2 && g.K >= 256 && !multi) return kKsplit16Config;
     // Between half a chip and a whole chip of 32 x 32 tiles, with a K of 384 or more: eight K slices (two wavefronts per
     // SIMD) instead of four - 512 x 384 x 512 6.1 against 7.2 us, 384 x 384 x 768 7.7 against 8.9, 512 x 512 x 768 8.0
     // against 9.1, 400 x 400 x 640 7.7 against 8.1.
-    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu && g.K >= 384 && !multi) return kKsplit8Config;
+    // (batches of small matrices likewise: 16 x (128 x 128 x 512) 6.2 against 7.3 us, 64 x (64 x 64 x 512) 7.9 against 9.3;
+    // with half a chip of tiles or fewer a batch stays on four slices - 32 x (64 x 64 x 1024) 10.8 us, 11.9 on eight slices,
+    // 12.7 on 16 x 16 tiles)
+    if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu && g.K >= 384 &&
+        (!multi || rows32 * ceil_div(g.N, 32) > (long long)h->num_cu / 2))
+        return kKsplit8Config;
     if (rows32 * ceil_div(g.N, 32) <= (long long)h->num_cu) return kKsplitConfig;
     // (Up to one 32 x 64 tile per compute unit - two K slices, configuration 15 - used to go here too; since the tail of
     // the tiled kernels' k loop was shortened the 64 x 64 tiles are ahead on all of those: 512 x 1024 x 256 7.0 against
