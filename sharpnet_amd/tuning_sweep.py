@@ -2,8 +2,10 @@
 
     python -m sharpnet_amd.tuning_sweep                      # the built-in shape list, NN form
     python -m sharpnet_amd.tuning_sweep --form TT --json out.json 1024x1024x1024 4097x3001x2049
+    python -m sharpnet_amd.tuning_sweep --batch 16 128x128x512 256x256x64     # strided batches of 16 matrices
 
-For each shape (M x N x K, single products through Tensor.Dot) every tiled fp32 configuration is forced through
+For each shape (M x N x K; single products through Tensor.Dot, or strided batches through BatchMatrixMultiplication, which
+also adds the streaming kernels to the candidates) every tiled fp32 configuration is forced through
 snhip_set_tuning with K split 1, 2 and 4 ways (8, 16 and 32 ways too where 64 x 64 tiles would leave the chip mostly idle),
 plus the kernels that split K inside the workgroup, and timed on the wall clock over enough launches to hide the host
 (the minimum of two runs).  Printed per shape: what the library picks by itself, its time, the fastest
@@ -31,6 +33,7 @@ def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("shapes", nargs="*", help="MxNxK, e.g. 1024x1024x1024 (default: a built-in list)")
     ap.add_argument("--form", default="NN", choices=["NN", "NT", "TN", "TT"], help="transposes of A and B")
+    ap.add_argument("--batch", type=int, default=1, help="matrices per strided batch (default: single products)")
     ap.add_argument("--json", default=None, metavar="PATH", help="write every measured time to this file")
     args = ap.parse_args(argv)
     from sharpnet_amd import GPUWrapper, GPUTensor
@@ -41,6 +44,9 @@ def main(argv=None):
     cfgs = w.configs()
     tiled = [c for c in cfgs if c["kind"] == "fp32"]
     inside = [c["id"] for c in cfgs if c["kind"] == "fp32-ksplit"]
+    if args.batch > 1:
+        inside += [c["id"] for c in cfgs if c["kind"] == "fp32-stream"]
+    lead = [args.batch] if args.batch > 1 else []
 
     def timeit(launch, n):
         for _ in range(max(5, n // 4)):
@@ -55,20 +61,24 @@ def main(argv=None):
     everything, regrets = {}, []
     try:
         for (M, N, K) in shapes:
-            a = rng.uniform(-1, 1, (K, M) if tA else (M, K)).astype(np.float32)
-            b = rng.uniform(-1, 1, (N, K) if tB else (K, N)).astype(np.float32)
-            ga, gb, gc = GPUTensor(list(a.shape), a, w), GPUTensor(list(b.shape), b, w), GPUTensor([M, N], None, w)
+            a = rng.uniform(-1, 1, lead + ([K, M] if tA else [M, K])).astype(np.float32)
+            b = rng.uniform(-1, 1, lead + ([N, K] if tB else [K, N])).astype(np.float32)
+            ga, gb = GPUTensor(list(a.shape), a, w), GPUTensor(list(b.shape), b, w)
+            gc = GPUTensor(lead + [M, N], None, w)
 
             def launch():
-                gc.Dot(ga, tA, gb, tB, 1.0, 0.0)
+                if args.batch > 1:
+                    gc.BatchMatrixMultiplication(ga, tA, gb, tB, 1.0, 0.0)
+                else:
+                    gc.Dot(ga, tA, gb, tB, 1.0, 0.0)
             w.set_tuning(-1, 0)
             launch()
             auto = w.last_tuning()
             cands = []
             for c in tiled:
-                tiles = -(-M // c["BM"]) * -(-N // c["BN"])
+                tiles = -(-M // c["BM"]) * -(-N // c["BN"]) * args.batch
                 for s in (1, 2, 4, 8, 16, 32):
-                    if s > 4 and -(-M // 64) * -(-N // 64) * s > 2048:
+                    if s > 4 and -(-M // 64) * -(-N // 64) * s * args.batch > 2048:
                         continue
                     if s > 1 and K // s < 4 * c["BK"]:
                         continue
@@ -109,7 +119,7 @@ def main(argv=None):
         100 * sum(regrets) / len(regrets), 100 * max(regrets), len(regrets)))
     if args.json:
         with open(args.json, "w") as f:
-            json.dump({"form": args.form, "shapes": everything}, f, indent=1)
+            json.dump({"form": args.form, "batch": args.batch, "shapes": everything}, f, indent=1)
     return 0
 
 
