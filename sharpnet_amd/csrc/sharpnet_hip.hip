@@ -665,6 +665,13 @@ int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, 
     const int cfg = g.N <= 64 ? first + 1 : first;
     const long long tiles = (long long)ceil_div(g.M, 128) * ceil_div(g.N, kConfigs[cfg].BN) * g.batch;
     if (tiles < 2LL * h->num_cu) return -1;
+    // fp32, where the tiled kernels are close: only the shapes a sweep has it ahead on - matrices of whole 256-row
+    // blocks (512 x (256 x 256 x 64) 48.8 against 50.6 us, 64 x (512 x 512 x 128) 42.3 against 43.1) and four tiles per
+    // compute unit or more; 8 x (1000 x 1000 x 64) 16.1 us tiled against 19.1, 64 x (384 x 384 x 96) 22.5 against 26.6,
+    // 512 x (64 x 64 x 64) 5.9 against 8.8
+    if (math == SNHIP_MATH_FP32 &&
+        (g.M % 256 != 0 || (g.N % 256 != 0 && g.N > 64) || g.N < 64 || tiles < 4LL * h->num_cu))
+        return -1;
     // mostly-empty tiles waste the streaming they are meant to save
     if ((long long)ceil_div(g.M, 128) * 128 * ceil_div(g.N, kConfigs[cfg].BN) * kConfigs[cfg].BN > 2LL * g.M * g.N) return -1;
     return cfg;

@@ -688,7 +688,7 @@ def test_streaming_kernel_strided_batches(oracle, gpu_wrapper, tA, tB):
         # scores (K = 64) stream, the probabilities-times-values product (K = 256) is a few percent faster on the tiled
         # kernels in fp32 - and a K = 128 product with 64 columns
         for (batch, M, N, K, want) in [(256, 256, 256, 64, st_all[0]), (256, 256, 64, 256, None),
-                                       (256, 256, 64, 128, st_all[1])]:
+                                       (512, 256, 64, 128, st_all[1])]:
             a = random_tensor(rng, (batch, K, M) if tA else (batch, M, K), -1, 1)
             b = random_tensor(rng, (batch, N, K) if tB else (batch, K, N), -1, 1)
             ga, gb, gc = GPUTensor(a.shape, a, w), GPUTensor(b.shape, b, w), GPUTensor([batch, M, N], None, w)
