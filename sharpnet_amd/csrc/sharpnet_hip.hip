@@ -448,6 +448,12 @@ Choice choose(const Handle* h, int M, int N, int K, int batch, int kind, bool tA
                 m.eff_alone = kConfigs[mirror].eff_alone;
                 m.eff_shared = kConfigs[mirror].eff_shared;
                 cost = estimate_cycles(m, M, N, K, batch, s, h->num_cu);
+            } else if (tA != tB && mirror != c) {
+                // one operand transposed: half way (2048^3 TN: 64 x 128 tiles 128 us, 128 x 64 tiles 129 us, 128 x 128 tiles 124 us)
+                ConfigEntry m = e;
+                m.eff_alone = 0.5 * (e.eff_alone + kConfigs[mirror].eff_alone);
+                m.eff_shared = 0.5 * (e.eff_shared + kConfigs[mirror].eff_shared);
+                cost = estimate_cycles(m, M, N, K, batch, s, h->num_cu);
             } else {
                 cost = estimate_cycles(e, M, N, K, batch, s, h->num_cu);
             }
