@@ -106,3 +106,17 @@ def test_traffic_record_names_its_kernel_source():
         if not src["stale"]:
             assert src["kernel_source_sha256_16"] == bench.source_hash(
                 os.path.join(bench.ROOT, "sharpnet_amd", "csrc", "sgemm_mfma.hpp"))
+
+
+def test_tuning_sweep_covers_the_benchmark_shapes_and_parses_its_arguments():
+    """The sweep behind the host's cost model: its built-in list holds every fp32 shape of the benchmark's sweep
+    configuration and the LSTM input projection, and the command line is understood without touching a GPU."""
+    import subprocess
+    import sys
+    from sharpnet_amd import tuning_sweep
+    for shape in [(1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096), (1000, 1000, 1000), (4097, 3001, 2049),
+                  (8192, 64, 8192), (32768, 2048, 256)]:
+        assert shape in tuning_sweep.DEFAULT_SHAPES
+    out = subprocess.run([sys.executable, "-m", "sharpnet_amd.tuning_sweep", "--help"], capture_output=True, text=True,
+                         timeout=120)
+    assert out.returncode == 0 and "--batch" in out.stdout and "--form" in out.stdout
