@@ -29,17 +29,24 @@
 
 namespace snhip {
 
-struct BDtlCfg {
-    static constexpr int BM = 256, BN = 256, BK = 32, NT = 256, TM = 4, TN = 4, WN = 2;
+// T: MFMA tiles per wavefront along each dimension.  T = 4: the 256 x 256 tile described above; T = 2: 128 x 128 (64 x 64
+// per wavefront, 16 KB stages), for products with too few 256 x 256 tiles to fill the chip.
+template <int T>
+struct BDtlCfgT {
+    static constexpr int TM = T, TN = T, WN = 2, NT = 256;
+    static constexpr int ROWS = 64 * T;  // rows of an operand tile
+    static constexpr int BM = ROWS, BN = ROWS, BK = 32;
     static constexpr int STAGES = 4;
     static constexpr int ROW_BYTES = BK * 2, CPR = ROW_BYTES / 16;  // chunks of 16 bytes per row
-    static constexpr int OPND_BYTES = 256 * ROW_BYTES, STAGE_BYTES = 2 * OPND_BYTES;
+    static constexpr int OPND_BYTES = ROWS * ROW_BYTES, STAGE_BYTES = 2 * OPND_BYTES;
     static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
     static constexpr int ROWS_PER_INST = 1024 / ROW_BYTES;       // physical rows one wavefront instruction fills
-    static constexpr int ROUNDS = 256 / (4 * ROWS_PER_INST);     // instructions per thread, operand and tile
+    static constexpr int ROUNDS = ROWS / (4 * ROWS_PER_INST);    // instructions per thread, operand and tile
     static constexpr int L = 2 * ROUNDS;                         // loads per thread and tile
     static constexpr int KSTEPS = BK / 16;
+    static_assert(TM * TN >= TM + TN, "one fragment read per MFMA slot of a k step");
 };
+using BDtlCfg = BDtlCfgT<4>;
 
 __device__ __forceinline__ int bdtl_swizzle(int phys_row) { return (phys_row >> 1) & (BDtlCfg::CPR - 1); }
 
@@ -50,8 +57,16 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
 }
 
-__global__ void __launch_bounds__(BDtlCfg::NT) bgemm_nt_dtl_kernel(const GemmParams p) {
-    using C = BDtlCfg;
+// 16 bytes per lane from global memory to LDS at dst + 16 * lane.  (A function of its own: with the builtin inside a lambda
+// of the kernel template the host pass drops the instantiation without a word, and the library then lacks the kernel's stub.)
+__device__ __forceinline__ void bdtl_load16(const __bf16* src, char* dst) {
+    __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+}
+
+template <int T>
+__global__ void __launch_bounds__(256) bgemm_nt_dtl_kernel(const GemmParams p) {
+    static_assert(BDtlCfgT<T>::NT == 256, "launch bounds");
+    using C = BDtlCfgT<T>;
     constexpr int TM = C::TM, TN = C::TN, WN = C::WN, BK = C::BK, S = C::STAGES, L = C::L, KSTEPS = C::KSTEPS;
     extern __shared__ __attribute__((aligned(1024))) char smem_dtl[];
     char* const smem = smem_dtl;
@@ -85,8 +100,7 @@ __global__ void __launch_bounds__(BDtlCfg::NT) bgemm_nt_dtl_kernel(const GemmPar
         const int tt = t < KT ? t : KT - 1;
         const int o = x / C::ROUNDS, j = x % C::ROUNDS;
         char* dst = smem + st * C::STAGE_BYTES + o * C::OPND_BYTES + (j * 4 + wave) * 1024;
-        __builtin_amdgcn_global_load_lds(gsrc[o][j] + (long long)tt * BK, (__attribute__((address_space(3))) void*)dst, 16,
-                                         0, 0);
+        bdtl_load16(gsrc[o][j] + (long long)tt * BK, dst);
     };
 
     f32x16 acc[TM][TN];
@@ -163,7 +177,7 @@ __global__ void __launch_bounds__(BDtlCfg::NT) bgemm_nt_dtl_kernel(const GemmPar
     }
     wait_vmcnt<0>();  // the trailing reloads must have landed before this workgroup's LDS is handed on
 
-    store_accumulators_plain<TM, TN, true>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, batch, batch,
+    store_accumulators_plain<TM, TN>(acc, p, m0 + wm * (TM * 32), n0 + wn * (TN * 32) + TN * l32, lhi, batch, batch,
                                            wc.tile_m * p.tiles_n + wc.tile_n);
 }
 

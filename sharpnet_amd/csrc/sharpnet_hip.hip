@@ -251,13 +251,17 @@ const ConfigEntry kConfigs[] = {
     // bf16 storage, both operands k-contiguous, tiles through global -> LDS direct loads (bgemm_dtl.hpp): one form
     // only (A plain, B transposed), shapes that are whole tiles; see prefer_dtl()
     ConfigEntry{BDtlCfg::BM, BDtlCfg::BN, BDtlCfg::BK, BDtlCfg::NT, BDtlCfg::LDS_BYTES, 16, 7,
-                {{nullptr, bgemm_nt_dtl_kernel}, {nullptr, nullptr}},
+                {{nullptr, bgemm_nt_dtl_kernel<4>}, {nullptr, nullptr}},
                 {{nullptr, nullptr}, {nullptr, nullptr}},
                 1, 0.9, 0.9, 1.0},  // 27: 256 x 256, k panels of 32, four LDS stages
+    ConfigEntry{BDtlCfgT<2>::BM, BDtlCfgT<2>::BN, BDtlCfgT<2>::BK, BDtlCfgT<2>::NT, BDtlCfgT<2>::LDS_BYTES, 4, 7,
+                {{nullptr, bgemm_nt_dtl_kernel<2>}, {nullptr, nullptr}},
+                {{nullptr, nullptr}, {nullptr, nullptr}},
+                2, 0.7, 0.8, 1.0},  // 28: 128 x 128, the same kernel with 64 x 64 per wavefront
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 constexpr int kKsplit16Config = 26;
-constexpr int kBDtlConfig = 27;
+constexpr int kBDtlConfig = 27;       // and kBDtlConfig + 1 (128 x 128 tiles)
 constexpr int kKsplitConfig = 14;   // and kKsplitConfig + 1
 constexpr int kStreamConfig = 16;   // and kStreamConfig + 1
 constexpr int kKsplit8Config = 21;
@@ -690,15 +694,29 @@ int prefer_stream(const Handle* h, const GemmArgs& g, int math, bool two_level, 
 // MI355X, 8192^3, U(-1, 1) operands: 1.19-1.21 PFLOP/s against 1.12-1.15 for the register-staged 256 x 256 kernel.
 int prefer_dtl(const Handle* h, const GemmArgs& g, int math, bool wants_ext) {
     if (math != SNHIP_MATH_BF16_STORED || g.tA || !g.tB || wants_ext) return -1;
-    if (h->force_cfg >= 0 && h->force_cfg != kBDtlConfig) return -1;
+    if (h->force_cfg >= 0 && h->force_cfg != kBDtlConfig && h->force_cfg != kBDtlConfig + 1) return -1;
     if (h->force_splitk > 1) return -1;
-    if (g.M % BDtlCfg::BM != 0 || g.N % BDtlCfg::BN != 0 || g.K % BDtlCfg::BK != 0 || g.K < BDtlCfg::BK) return -1;
     if ((uintptr_t)g.A % 16 != 0 || (uintptr_t)g.B % 16 != 0 || g.lda % 8 != 0 || g.ldb % 8 != 0) return -1;
     if (g.batch > 1 && (g.sA % 8 != 0 || g.sB % 8 != 0)) return -1;
-    if (h->force_cfg == kBDtlConfig) return kBDtlConfig;
-    const long long tiles = (long long)(g.M / BDtlCfg::BM) * (g.N / BDtlCfg::BN) * g.batch;
-    if (tiles < h->num_cu || g.K < 8 * BDtlCfg::BK) return -1;
-    return kBDtlConfig;
+    // the 128 x 128 form of the kernel: whole 128-wide tiles
+    const bool small_ok = g.M % BDtlCfgT<2>::BM == 0 && g.N % BDtlCfgT<2>::BN == 0 && g.K % BDtlCfgT<2>::BK == 0 &&
+                          g.K >= BDtlCfgT<2>::BK;
+    if (h->force_cfg == kBDtlConfig + 1) return small_ok ? kBDtlConfig + 1 : -1;
+    const bool big_ok = g.M % BDtlCfg::BM == 0 && g.N % BDtlCfg::BN == 0 && g.K % BDtlCfg::BK == 0 && g.K >= BDtlCfg::BK;
+    if (h->force_cfg == kBDtlConfig) return big_ok ? kBDtlConfig : -1;
+    if (g.K < 8 * BDtlCfg::BK) return -1;
+    // 256 x 256 tiles from a little over half a chip of them: 3072^3 (144 tiles) 59.5 us against 75.0 on the
+    // register-staged 128 x 128 tiles; level at 128 tiles (4096 x 2048 x 2048: 43.7 against 42.9), behind at 100.
+    if (big_ok && 2LL * (g.M / BDtlCfg::BM) * (g.N / BDtlCfg::BN) * g.batch > h->num_cu) return kBDtlConfig;
+    // 128 x 128 tiles when they number between a quarter of a chip and a chip and K is not long: 2048^3 24.7 us against
+    // 27.6, 1536^3 17.1 against 20.9, 2048 x 1024 x 1024 10.9 against 15.2, 1024^3 10.0 against 12.1 (64 x 64 x 128 tiles);
+    // with more tiles the register-staged kernel shares the compute unit better (2560^3 45.5 against 50.8), with a long K
+    // and few tiles the 64 x 64 tiles win (1024 x 1024 x 4096: 21.9 against 36.0).
+    if (small_ok && g.K <= 2048) {
+        const long long t128 = (long long)(g.M / BDtlCfgT<2>::BM) * (g.N / BDtlCfgT<2>::BN) * g.batch;
+        if (4 * t128 >= h->num_cu && t128 <= h->num_cu) return kBDtlConfig + 1;
+    }
+    return -1;
 }
 
 // Operand pointers travel as const float* whatever the storage; A and B of SNHIP_MATH_BF16_STORED hold 2-byte

@@ -325,8 +325,8 @@ def test_bf16_stored_direct_to_lds_kernel(oracle, gpu_wrapper):
     w = gpu_wrapper
     lib, h = w.lib, w.handle
     dtl = [c["id"] for c in w.configs() if c["kind"] == "bf16-stored-dtl"]
-    assert len(dtl) == 1
-    dtl = dtl[0]
+    assert len(dtl) == 2                      # 256 x 256 tiles and the same kernel with 128 x 128 tiles
+    dtl, dtl_small = dtl
     rng = np.random.default_rng(2700)
 
     def run(a, b, c0, alpha, beta, bias, force):
@@ -370,6 +370,27 @@ def test_bf16_stored_direct_to_lds_kernel(oracle, gpu_wrapper):
         other, tuning2 = run(a, b, c0, alpha, beta, bias, -1)          # small shapes: the cost model's own choice
         assert tuning2[0] != dtl
         assert float(np.max(np.abs(got - other))) <= bound
+    # the 128 x 128 form: one tile and one k panel, fewer k panels than stages, several tiles, a strided batch, a long K
+    for (batch, M, N, K, alpha, beta, with_bias) in [(1, 128, 128, 32, 1.0, 0.0, False), (1, 128, 384, 64, -0.5, 1.0, True),
+                                                     (1, 384, 128, 96, 1.0, 0.0, True), (3, 128, 256, 160, 1.0, 1.0, True),
+                                                     (2, 256, 256, 2048, 1.0, 0.0, False),
+                                                     (1, 640, 384, 1024, 0.25, 0.5, False)]:
+        print("direct-to-LDS 128 x 128 case", batch, M, N, K, alpha, beta, with_bias, flush=True)
+        a, b = random_tensor(rng, (batch, M, K), -1, 1), random_tensor(rng, (batch, N, K), -1, 1)
+        c0 = random_tensor(rng, (batch, M, N), -1, 1)
+        bias = random_tensor(rng, (N,), -1, 1) if with_bias else None
+        got, tuning = run(a, b, c0, alpha, beta, bias, dtl_small)
+        assert tuning == (dtl_small, 1), tuning
+        ref = oracle.bmm(oracle.round_to_bf16(a), False, oracle.round_to_bf16(b), True, alpha, beta, c0 if beta else None)
+        if bias is not None:
+            ref = ref + bias
+        assert np.all(np.isfinite(got))
+        assert float(np.max(np.abs(got - ref))) <= 1e-4 * np.sqrt(K) * abs(alpha) + 1e-6 * (abs(beta) + 1), (batch, M, N, K)
+    for (M, N, K) in [(300, 128, 64), (128, 128, 48), (128, 120, 64)]:
+        a, b = random_tensor(rng, (1, M, K), -1, 1), random_tensor(rng, (1, N, K), -1, 1)
+        got, tuning = run(a, b, None, 1.0, 0.0, None, dtl_small)
+        assert tuning[0] != dtl_small
+        assert float(np.max(np.abs(got - oracle.bmm(oracle.round_to_bf16(a), False, oracle.round_to_bf16(b), True)))) <= 1e-4 * np.sqrt(K)
     # shapes the kernel does not take run on another configuration even when it is forced
     for (M, N, K) in [(300, 256, 64), (256, 256, 48), (256, 250, 64)]:
         a, b = random_tensor(rng, (1, M, K), -1, 1), random_tensor(rng, (1, N, K), -1, 1)
