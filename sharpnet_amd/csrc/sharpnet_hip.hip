@@ -160,11 +160,11 @@ const ConfigEntry kConfigs[] = {
     make_entry<TileCfg<4, 4, 2, 2, 16>>(1, 0.990, 0.990, 1.25),  // 0: 256 x 256
     make_entry<TileCfg<2, 4, 2, 2, 16>>(1, 0.948, 0.948, 1.2),   // 1: 128 x 256
     make_entry<TileCfg<4, 2, 2, 2, 16>>(1, 0.949, 0.949, 1.2),   // 2: 256 x 128
-    make_entry<TileCfg<2, 2, 2, 2, 16>>(2, 0.897, 0.929, 1.1),   // 3: 128 x 128
+    make_entry<TileCfg<2, 2, 2, 2, 16>>(2, 0.897, 0.929, 1.05),  // 3: 128 x 128
     make_entry<TileCfg<1, 2, 2, 2, 16>>(3, 0.861, 0.906, 1.05),  // 4: 64 x 128
     make_entry<TileCfg<2, 1, 2, 2, 16>>(3, 0.786, 0.866, 1.05),  // 5: 128 x 64
     make_entry<TileCfg<1, 1, 2, 2, 16>>(5, 0.758, 0.815, 1.05),  // 6: 64 x 64
-    make_entry<TileCfg<2, 2, 2, 2, 32>>(1, 0.935, 0.935, 1.1),   // 7: 128 x 128, BK 32
+    make_entry<TileCfg<2, 2, 2, 2, 32>>(1, 0.935, 0.935, 1.05),  // 7: 128 x 128, BK 32
     make_entry<TileCfg<2, 1, 2, 2, 32>>(2, 0.819, 0.878, 1.05),  // 8: 128 x 64, BK 32
     make_entry<TileCfg<1, 1, 2, 2, 32>>(4, 0.757, 0.813, 1.05),  // 9: 64 x 64, BK 32
     // bf16-input kernels (fp32 operands in memory: bound by the L2 -> LDS path long before the MFMA rate)
