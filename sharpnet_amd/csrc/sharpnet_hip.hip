@@ -470,7 +470,11 @@ Choice choose(const Handle* h, int M, int N, int K, int batch, int kind, bool tA
     // 64 x 64 tiles with at most one workgroup per compute unit: when K is a whole number of 32-wide k panels, the
     // configuration with those panels is 3-5 % ahead of the one with 16-wide panels (1024^3 in all four forms 19.2-19.7
     // against 20.2-20.3 us, 1024 x 1024 x 256 ... 2048, 512 x 512 x 2048); with a ragged K (1000, 1040, 700) it is not.
-    if (kind == 0 && !forced && best.cfg == 6 && K % 32 == 0 && K / best.splitk >= 256 &&
+    // (With both operands transposed also for a ragged K whose 16-wide panels are an odd number - the loop then multiplies
+    // a panel of zeros to complete its last pair - while its 32-wide panels are an even number: 1000^3 TT 22.2 against
+    // 23.2 us, 960 x 1024 x 1000 20.5 against 20.9; not K = 1040, 700, 1100, 500.)
+    const bool odd_pairs_tt = tA && tB && best.splitk == 1 && ceil_div(K, 16) % 2 == 1 && ceil_div(K, 32) % 2 == 0;
+    if (kind == 0 && !forced && best.cfg == 6 && (K % 32 == 0 || odd_pairs_tt) && K / best.splitk >= 256 &&
         (long long)ceil_div(M, 64) * ceil_div(N, 64) * batch * best.splitk <= h->num_cu) {
         const int kchunk = ceil_div(ceil_div(K, best.splitk), 32) * 32;
         if ((long long)kchunk * (best.splitk - 1) < K) best.cfg = 9;
