@@ -1212,7 +1212,6 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     // MODE 1: a full-k tile of an edge block (branch-free loads through the precomputed edge facts ea / eb);
     // MODE 2: the last tiles of an interior block (each fetch decides between unchecked loads and, at or past the
     //         end of K, checked ones);
-    // MODE 7: tile `fetch` is the tile of zeros that completes a pair of tiles (no loads: the stage is cleared);
     // MODE 3: the last tiles of an edge block (edge loads for full-k tiles, fully checked loads otherwise);
     // MODE 4: MODE 1 for a block none of whose vectors arrives shifted (M and N multiples of 4, or the operand is
     //         k-contiguous): plain LDS stores.  The element selects of the shifted store, executed for nothing, made
@@ -1221,6 +1220,8 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     //         fetched: the register stage is stored to LDS and not refilled.  Without any load in it the pair costs what
     //         a pair of the main loop costs (1361 cycles with 64 x 64 tiles); as a pair of MODE 2, whose every slot
     //         chooses between two kinds of load (of tiles beyond the end: zeros), it took 2361.
+    // MODE 9: the very last tile of an interior block with an odd number of tiles: nothing is stored and nothing fetched
+    //         (there is no tile after it; the tile of zeros that used to complete the last pair is no longer multiplied).
     // R: the register stage that holds the next tile (it is stored to LDS buffer P ^ 1 and refilled).
     auto k_tile = [&](auto parity, auto stage, auto mode, const typename StageA::Edge& ea,
                       const typename StageB::Edge& eb) {
@@ -1273,7 +1274,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                     }
                     // - the staging work items (store piece q to LDS, then refill its registers
                     //   from global memory), item w in slot w*G/NW;
-                    if (gslot < G) {
+                    if (MODE != 9 && gslot < G) {
 #pragma unroll
                         for (int w = 0; w < NW; ++w) {
                             if ((w * G) / NW != gslot) continue;
@@ -1282,7 +1283,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                             if (q < StageA::NV) {
                                 const int v = q < StageA::NV ? q : 0;
                                 if (is_store) {
-                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4 || MODE == 5 || MODE == 7) {
+                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4 || MODE == 5) {
                                         sa.store_lds_vec(as_next, ra[R][v], v);
                                         if constexpr (COLSUM) {
                                             if (sum_stored) cs += ra[R][v];
@@ -1296,8 +1297,6 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                                     }
                                 } else if constexpr (MODE == 5 || MODE == 6) {
                                     // nothing left to fetch
-                                } else if constexpr (MODE == 7) {
-                                    ra[R][v] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
                                 } else if (MODE == 1 || MODE == 4 || edge_fast)
                                     sa.load_edge_vec(ra[R][v], v, ea);
                                 else if (fast)
@@ -1307,14 +1306,12 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                             } else {
                                 const int v = q >= StageA::NV ? q - StageA::NV : 0;
                                 if (is_store) {
-                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4 || MODE == 5 || MODE == 7)
+                                    if constexpr (MODE == 0 || MODE == 2 || MODE == 4 || MODE == 5)
                                         sb.store_lds_vec(bs_next, rb[R][v], v);
                                     else
                                         sb.store_lds_vec_shifted(bs_next, rb[R][v], v, sh_b[R], any_rot_b);
                                 } else if constexpr (MODE == 5 || MODE == 6) {
                                     // nothing left to fetch
-                                } else if constexpr (MODE == 7) {
-                                    rb[R][v] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
                                 } else if (MODE == 1 || MODE == 4 || edge_fast)
                                     sb.load_edge_vec(rb[R][v], v, eb);
                                 else if (fast)
@@ -1374,9 +1371,10 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         wait_for_all_loads();
         for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 0>{}, kt, kNoLimit, std::integral_constant<int, 0>{});
         if constexpr (SPLIT_TAIL) {
-            // The pairs whose fetches reach the end of K.  An even number of full tiles: the last tile is fetched by
-            // the first tile of a pair whose second tile fetches nothing.
-            if (kt + NS + 1 < nk_full && kt + 2 * NS >= nk_even) {
+            // The pairs whose fetches reach the end of K (tiles at or beyond nk are not fetched: an odd number of tiles ends
+            // with a tile on its own, below).  An even number of full tiles: the last tile is fetched by the first tile of
+            // a pair whose second tile fetches nothing.
+            if (kt + NS + 1 < nk_full && kt + 2 * NS >= nk) {
                 tiles(std::integral_constant<int, 0>{}, kt, kNoLimit, std::integral_constant<int, 5>{});
                 kt += NS;
             }
@@ -1387,13 +1385,11 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
                 tiles(std::integral_constant<int, 2>{}, kt, nk, std::integral_constant<int, 5>{});
                 kt += NS;
             }
-            // an odd number of tiles: the tile of zeros that completes the last pair
-            if (kt + NS + 1 < nk_even) {
-                tiles(std::integral_constant<int, 7>{}, kt, nk, std::integral_constant<int, 5>{});
-                kt += NS;
-            }
-            // what is left has nothing to fetch
-            for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 5>{}, kt, nk, std::integral_constant<int, 5>{});
+            // whole pairs that have nothing to fetch
+            for (; kt + 1 < nk; kt += NS) tiles(std::integral_constant<int, 5>{}, kt, nk, std::integral_constant<int, 5>{});
+            // an odd number of tiles: the last one by itself (it reads LDS buffer 0: its index is even)
+            if (kt < nk)
+                k_tile(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 9>{}, ea, eb);
         } else {
             for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 2>{}, kt, nk, std::integral_constant<int, 2>{});
         }
