@@ -1220,7 +1220,7 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
     //         fetched: the register stage is stored to LDS and not refilled.  Without any load in it the pair costs what
     //         a pair of the main loop costs (1361 cycles with 64 x 64 tiles); as a pair of MODE 2, whose every slot
     //         chooses between two kinds of load (of tiles beyond the end: zeros), it took 2361.
-    // MODE 9: the very last tile of an interior block with an odd number of tiles: nothing is stored and nothing fetched
+    // MODE 9: the very last tile of a block with an odd number of tiles: nothing is stored and nothing fetched
     //         (there is no tile after it; the tile of zeros that used to complete the last pair is no longer multiplied).
     // R: the register stage that holds the next tile (it is stored to LDS buffer P ^ 1 and refilled).
     auto k_tile = [&](auto parity, auto stage, auto mode, const typename StageA::Edge& ea,
@@ -1349,9 +1349,8 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
         }
     };
     constexpr int kNoLimit = 0x7fffffff;
-    // a pair of tiles fetches the tiles NS + 1 and NS + 2 ahead of its first one; the loop multiplies nk tiles rounded up
-    // to a whole pair: once the first of those fetches lies beyond that, nothing needs fetching any more
-    const int nk_even = nk + (nk & 1);
+    // a pair of tiles fetches the tiles NS + 1 and NS + 2 ahead of its first one; once the first of those fetches lies at
+    // or beyond nk, nothing needs fetching any more
     static_assert(NS == 2, "the tail loops are written for pairs of tiles");
     // The 256 x 256 tiles, which use every register there is, keep one kind of pair for the whole tail (MODE 2 / 3): with
     // more kinds of pair the compiler spilled 1.2 KB per lane there.  (For the smaller tiles, too, the kinds of pair are
@@ -1401,8 +1400,12 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_mfma_kernel(const GemmParams p)
             for (; kt + 2 * NS < nk_full; kt += NS) tiles(std::integral_constant<int, 4>{}, kt, kNoLimit, std::integral_constant<int, 4>{});
         }
         if constexpr (SPLIT_TAIL) {
-            for (; kt + NS + 1 < nk_even; kt += NS) tiles(std::integral_constant<int, 3>{}, kt, nk, std::integral_constant<int, 3>{});
-            for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 6>{}, kt, nk, std::integral_constant<int, 6>{});
+            // pairs whose first tile still has a tile to fetch, whole pairs that fetch nothing, and - an odd number of
+            // tiles - the last tile by itself, as in interior blocks
+            for (; kt + NS + 1 < nk; kt += NS) tiles(std::integral_constant<int, 3>{}, kt, nk, std::integral_constant<int, 3>{});
+            for (; kt + 1 < nk; kt += NS) tiles(std::integral_constant<int, 6>{}, kt, nk, std::integral_constant<int, 6>{});
+            if (kt < nk)
+                k_tile(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 9>{}, ea, eb);
         } else {
             for (; kt < nk; kt += NS) tiles(std::integral_constant<int, 3>{}, kt, nk, std::integral_constant<int, 3>{});
         }
